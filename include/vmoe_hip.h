@@ -1,0 +1,284 @@
+/* vmoe_hip.h -- C ABI of libvmoe_hip.so: the inference-time V-MoE layer on one
+ * MI355X (gfx950).
+ *
+ * The reference (google-research/vmoe) is pure Python on JAX/XLA and has no
+ * native interface; each entry point below replaces a group of XLA ops of the
+ * reference, cited as file:line relative to the reference checkout.  These are
+ * the symbols a jax.ffi custom-call shim or a ctypes binding attaches to.
+ *
+ * Conventions
+ *  - All pointers are DEVICE pointers unless stated; arrays are dense,
+ *    row-major, in the shapes given.  The caller owns every buffer, including
+ *    workspaces; no entry point allocates, frees or synchronises the host.
+ *  - `stream` is a hipStream_t passed as void* (0 = the null stream).
+ *  - Return value: 0 on success, a negative VMOE_E_* code for rejected
+ *    arguments (nothing was launched), a positive value is a hipError_t.
+ *  - dtype: VMOE_F32 (float) or VMOE_BF16 (bfloat16 storage, float32 math).
+ *  - Symbols: G groups, S items per group, E experts, K selected experts per
+ *    item, C capacity (slots per expert per group), D item width, M hidden
+ *    width of the expert MLP, T = G*S.
+ *  - A "slot row" is the flat row index e*(G*C) + r(g,c) into the expert
+ *    buffer (E, G*C, ...), where r(g,c) is the row order produced by
+ *    vmoe/moe.py:488-500 (_dispatch): ((g % Q)*E + g / Q)*C + c with Q = G/E
+ *    when G % E == 0, else g*C + c.
+ *  - Re-entrant: calls on distinct streams with distinct buffers may overlap.
+ */
+#ifndef VMOE_HIP_H_
+#define VMOE_HIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define VMOE_ABI_VERSION 1
+
+typedef void* vmoe_stream_t;
+
+enum { VMOE_F32 = 0, VMOE_BF16 = 1 };
+enum { VMOE_GELU_TANH = 0, VMOE_GELU_ERF = 1 };
+
+enum {
+  VMOE_OK = 0,
+  VMOE_E_NULL = -1,        /* a required pointer is null */
+  VMOE_E_SHAPE = -2,       /* a size is < 1, or K > E, or sizes disagree */
+  VMOE_E_DTYPE = -3,       /* unknown dtype / enum value */
+  VMOE_E_ALIGN = -4,       /* row width not a multiple of 16 bytes, or pointer misaligned */
+  VMOE_E_OVERFLOW = -5,    /* an index would not fit in int32 */
+  VMOE_E_UNSUPPORTED = -6, /* valid, but outside what the kernels cover (see each call) */
+  VMOE_E_WORKSPACE = -7    /* workspace missing or too small */
+};
+
+int vmoe_abi_version(void);
+const char* vmoe_error_string(int code);
+
+/* ------------------------------------------------------------------ gating
+ * Replaces vmoe/nn/routing.py:73-80 (nn.Dense without bias + softmax) fused
+ * with the jax.lax.top_k of vmoe/moe.py:567.
+ * logits = x @ w (float32 accumulate, rounded to dtype), gates = softmax over E
+ * (float32 internals, rounded to dtype), then the K largest gates per item in
+ * descending order, equal gates -> lower expert index first.
+ * Limits: E <= 128; D % 8 == 0 (bf16) / D % 4 == 0 (f32).
+ */
+typedef struct {
+  const void* x;           /* (G*S, D) dtype */
+  const void* w;           /* (D, E) dtype: Router/dense/kernel */
+  const float* logit_bias; /* optional (E,) float32 added to the logits; null = reference behaviour */
+  void* gates;             /* optional out (G*S, E) dtype */
+  float* topk_val;         /* out (G*S, K) float32 (values are exact dtype values) */
+  int32_t* topk_idx;       /* out (G*S, K) */
+  int32_t num_items;       /* T = G*S */
+  int32_t D, E, K;
+  int32_t dtype;
+} VmoeGateTopkParams;
+int vmoe_gate_topk(const VmoeGateTopkParams* p, vmoe_stream_t stream);
+
+/* Top-k alone on given gates (G*S, E) float32: the jax.lax.top_k of
+ * vmoe/moe.py:567.  Bit-exact selection; E <= 1024. */
+typedef struct {
+  const float* gates;
+  float* topk_val;   /* (num_items, K) */
+  int32_t* topk_idx; /* (num_items, K) */
+  int32_t num_items, E, K;
+} VmoeTopkParams;
+int vmoe_topk(const VmoeTopkParams* p, vmoe_stream_t stream);
+
+/* ------------------------------------------------------------------ metrics
+ * Replaces vmoe/nn/routing.py:81-91,133-157,247-252: per group,
+ * importance_loss = (std/mean)^2 of sum_s gates[s,:] (population std),
+ * gshard_loss = mean_e(mean_s onehot(top1) * mean_s gates) * E^2,
+ * auxiliary_loss = sum of weight*loss over weights > 0.  E <= 1024.
+ */
+typedef struct {
+  const void* gates;        /* (G, S, E) dtype */
+  const int32_t* top1_idx;  /* first-choice expert of item i at top1_idx[i*top1_stride] */
+  float* importance_loss;   /* out (G,) */
+  float* gshard_loss;       /* out (G,) */
+  float* auxiliary_loss;    /* out (G,) */
+  float gshard_loss_weight, importance_loss_weight;
+  int32_t G, S, E, top1_stride;
+  int32_t dtype;
+} VmoeRouterMetricsParams;
+int vmoe_router_metrics(const VmoeRouterMetricsParams* p, vmoe_stream_t stream);
+
+/* ------------------------------------------------------------------ slot assignment
+ * Replaces vmoe/moe.py:568-589 + :646-648 (_get_top_experts_per_item_common and
+ * the indices dispatcher builder), for all groups at once (the jax.vmap of
+ * vmoe/nn/routing.py:123-128).  Integer work, bit-exact:
+ * position(s,k) = number of (s',k') of the same group with the same expert and
+ * (k' < k, or k' == k and s' before s in priority order); priority order is
+ * the item index, or with batch_priority the stable descending order of
+ * topk_val[:,0].  Positions are not clipped; an assignment is kept iff
+ * position < C.  Experts outside [0,E) get position -1.
+ * Limits: 8*pow2ceil(S) + 8*E*ceil(S*K/32) + 4*S + 4*E bytes of LDS <= 160 KiB.
+ */
+typedef struct {
+  const float* topk_val;   /* (G, S, K); only [:, :, 0] is read, and only with batch_priority */
+  const int32_t* topk_idx; /* (G, S, K) */
+  int32_t* indices;        /* out (G, S, K, 2): (expert, position) */
+  int32_t* token_slot;     /* out (G, S, K): slot row of the assignment, -1 if dropped */
+  int32_t* slot_token;     /* out (E*G*C,): flat item index g*S+s feeding the slot row, -1 if empty */
+  int32_t* fill;           /* optional out (G, E): min(C, demand) */
+  int32_t G, S, E, K, C;
+  int32_t batch_priority;
+} VmoeRouteAssignParams;
+int vmoe_route_assign(const VmoeRouteAssignParams* p, vmoe_stream_t stream);
+
+/* Builds the two slot maps from hand-made (expert, position) indices, as
+ * vmoe/moe.py:190-197 and :202-206 interpret them: entries with expert >= E or
+ * position >= C are dropped.  Negative entries are counted in
+ * *num_invalid; slots targeted by more than one item are counted in
+ * *num_duplicates (the reference would accumulate them; these kernels do not,
+ * callers must treat a non-zero count as an error).  Both counters are device
+ * int32 and must be zeroed by the caller. */
+typedef struct {
+  const int32_t* indices; /* (G, S, K, 2) */
+  int32_t* token_slot;    /* out (G, S, K) */
+  int32_t* slot_token;    /* out (E*G*C,) */
+  int32_t* num_duplicates;
+  int32_t* num_invalid;
+  int32_t G, S, E, K, C;
+} VmoeIndicesToSlotsParams;
+int vmoe_indices_to_slots(const VmoeIndicesToSlotsParams* p, vmoe_stream_t stream);
+
+/* ------------------------------------------------------------------ dispatch / combine
+ * dispatch replaces ExpertIndicesDispatcher.dispatch (vmoe/moe.py:190-197:
+ * repeat + scatter_nd into zeros + _dispatch layout): out[slot] = x[item] for
+ * kept assignments, 0 for empty slots.  Exact copy.
+ * combine replaces ExpertIndicesDispatcher.combine (vmoe/moe.py:199-209):
+ * out[item] = sum_k weights[item,k] * (slot >= 0 ? y[slot] : 0), products and
+ * sums in float32 in k order, rounded once to dtype.
+ * Row width D*sizeof(dtype) must be a multiple of 16 bytes.
+ */
+typedef struct {
+  const void* x;             /* (num_items, D) dtype */
+  const int32_t* token_slot; /* (num_items, K) */
+  const int32_t* slot_token; /* (num_slots,) */
+  void* out;                 /* (num_slots, D) dtype */
+  int32_t num_items, num_slots, K, D;
+  int32_t dtype;
+} VmoeDispatchParams;
+int vmoe_dispatch(const VmoeDispatchParams* p, vmoe_stream_t stream);
+
+typedef struct {
+  const void* y;             /* (num_slots, D) dtype */
+  const int32_t* token_slot; /* (num_items, K) */
+  const float* weights;      /* (num_items, K) float32 */
+  void* out;                 /* (num_items, D) dtype */
+  int32_t num_items, num_slots, K, D;
+  int32_t dtype;
+} VmoeCombineParams;
+int vmoe_combine(const VmoeCombineParams* p, vmoe_stream_t stream);
+
+/* Dense (G,S,E,C) view of a sparse assignment, for callers that read
+ * EinsumDispatcher.combine_weights / dispatch_weights (vmoe/moe.py:609-619):
+ * combine[g,s,e,c] = weight of the kept assignment (s -> e,c), else 0;
+ * dispatch[g,s,e,c] = 1 where an assignment is kept.  Outputs must be zeroed by
+ * the caller; either may be null. */
+typedef struct {
+  const int32_t* indices; /* (G, S, K, 2) */
+  const float* weights;   /* (G, S, K) */
+  float* combine;         /* out (G, S, E, C) float32 */
+  uint8_t* dispatch;      /* out (G, S, E, C) bool */
+  int32_t G, S, E, K, C;
+} VmoeDensifyParams;
+int vmoe_densify(const VmoeDensifyParams* p, vmoe_stream_t stream);
+
+/* ------------------------------------------------------------------ expert MLP
+ * Replaces the expert vmap of vmoe/moe.py:434-439 over
+ * vit_jax.models_vit.MlpBlock (called from vmoe/nn/vit_moe.py:38-45), dropout
+ * off: for every expert e, y = gelu(x @ w0[e] + b0[e]) @ w1[e] + b1[e], all rows.
+ * bf16: bf16 operands, float32 accumulate, results rounded to bf16 after each
+ * matmul, after each bias add and after the GELU.
+ * bf16 needs the kernels in K-contiguous order: pass w0t (E,M,D) / w1t (E,D,M)
+ * made once by vmoe_pack_expert_weights; if they are null the call packs
+ * w0/w1 into `workspace` first (extra HBM pass).  D % 8 == 0 and M % 8 == 0.
+ */
+typedef struct {
+  const void* x;    /* (E, R, D) dtype */
+  const void* w0;   /* (E, D, M) dtype: Mlp/Dense_0/kernel (may be null when w0t is given) */
+  const void* b0;   /* (E, M) dtype or null */
+  const void* w1;   /* (E, M, D) dtype: Mlp/Dense_1/kernel (may be null when w1t is given) */
+  const void* b1;   /* (E, D) dtype or null */
+  const void* w0t;  /* optional (E, M, D) dtype: w0 transposed per expert */
+  const void* w1t;  /* optional (E, D, M) dtype: w1 transposed per expert */
+  void* out;        /* (E, R, D) dtype */
+  void* workspace;  /* vmoe_expert_mlp_workspace_bytes() bytes */
+  size_t workspace_bytes;
+  int32_t E, R, D, M;
+  int32_t dtype;
+  int32_t gelu;     /* VMOE_GELU_TANH (flax default) or VMOE_GELU_ERF */
+} VmoeExpertMlpParams;
+size_t vmoe_expert_mlp_workspace_bytes(const VmoeExpertMlpParams* p);
+int vmoe_expert_mlp(const VmoeExpertMlpParams* p, vmoe_stream_t stream);
+
+/* (batch, rows, cols) -> (batch, cols, rows), 2- or 4-byte elements. */
+typedef struct {
+  const void* in;
+  void* out;
+  int32_t batch, rows, cols;
+  int32_t dtype;
+} VmoeTransposeParams;
+int vmoe_pack_expert_weights(const VmoeTransposeParams* p, vmoe_stream_t stream);
+
+/* ------------------------------------------------------------------ Soft MoE
+ * soft_route replaces vmoe/projects/soft_moe/router.py:57-96 (no noise):
+ * unit-normalise items and slot parameters (eps 1e-6 inside the rsqrt), scale
+ * the smaller operand, logits[g,m,n] = x_hat . mu_hat, dispatch = softmax over
+ * items m, combine = softmax over slots n.  N = num_experts*num_slots <= 1024,
+ * the (S x N) logits of a group must fit the 160 KiB LDS as float32.
+ */
+typedef struct {
+  const void* x;      /* (G, S, D) dtype */
+  const void* mu;     /* (D, N) dtype: Router/mu reshaped (D, n*p) */
+  float scale;        /* Router/scale */
+  void* dispatch_w;   /* out (G, S, N) dtype */
+  void* combine_w;    /* out (G, S, N) dtype */
+  void* logits;       /* optional out (G, S, N) dtype */
+  void* workspace;    /* D*N*sizeof(float) bytes for the unit-norm, scaled mu */
+  size_t workspace_bytes;
+  int32_t G, S, D, N;
+  int32_t dtype;
+} VmoeSoftRouteParams;
+size_t vmoe_soft_route_workspace_bytes(const VmoeSoftRouteParams* p);
+int vmoe_soft_route(const VmoeSoftRouteParams* p, vmoe_stream_t stream);
+
+/* EinsumDispatcher.dispatch / .combine with dense weights
+ * (vmoe/moe.py:148-161): per group,
+ *   dispatch: out[slot(g,n)] = sum_s w[g,s,n] * x[g,s,:]
+ *   combine:  out[g,s,:]     = sum_n w[g,s,n] * y[slot(g,n)]
+ * with N = E*C and slot(g, n=e*C+c) the slot row defined at the top.
+ * float32 accumulate, result rounded to out_dtype.  `w` is float32, bf16 or
+ * bool (dispatch only; w_dtype = 2).
+ */
+enum { VMOE_W_F32 = 0, VMOE_W_BF16 = 1, VMOE_W_BOOL = 2 };
+typedef struct {
+  const void* w;     /* (G, S, E*C) */
+  const void* data;  /* dispatch: (G, S, D); combine: (E*G*C, D) */
+  void* out;         /* dispatch: (E*G*C, D); combine: (G, S, D) */
+  int32_t G, S, E, C, D;
+  int32_t w_dtype, data_dtype, out_dtype;
+} VmoeEinsumParams;
+int vmoe_einsum_dispatch(const VmoeEinsumParams* p, vmoe_stream_t stream);
+int vmoe_einsum_combine(const VmoeEinsumParams* p, vmoe_stream_t stream);
+
+/* Elementwise float32 <-> bfloat16 conversion (round to nearest even):
+ * the _cast_to_bfloat16 / astype pair of Bfloat16Dispatcher, vmoe/moe.py:212-227. */
+typedef struct {
+  const void* in;
+  void* out;
+  size_t n;
+  int32_t in_dtype, out_dtype;
+} VmoeCastParams;
+int vmoe_cast(const VmoeCastParams* p, vmoe_stream_t stream);
+
+/* Plain device copy kernel of n bytes (n % 16 == 0); the measured HBM ceiling
+ * that bandwidth figures are compared with. */
+int vmoe_copy_bytes(const void* in, void* out, size_t n, vmoe_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* VMOE_HIP_H_ */

@@ -1,0 +1,86 @@
+"""CPU-side checks of the drop-in boundary: the shared library loads, exports
+every symbol declared in include/vmoe_hip.h, and the ctypes structs match the
+header's layout.  No compute call is made (there may be no GPU)."""
+import ctypes
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "vmoe_hip.h")
+
+
+def _declared_functions():
+  text = open(HEADER).read()
+  text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+  return sorted(set(re.findall(r"\b(vmoe_[a-z0-9_]+)\s*\(", text)))
+
+
+def _lib():
+  from vmoe_amd import _hip
+  if not os.path.exists(_hip.lib_path()):
+    from vmoe_amd.csrc import build
+    build.build(verbose=False)
+  return ctypes.CDLL(_hip.lib_path())
+
+
+def test_header_functions_are_exported():
+  lib = _lib()
+  names = _declared_functions()
+  assert len(names) >= 18
+  for n in names:
+    assert hasattr(lib, n), f"{n} declared in vmoe_hip.h but not exported"
+
+
+def test_python_export_list_matches_header():
+  from vmoe_amd import _hip
+  assert sorted(_hip.EXPORTS) == _declared_functions()
+
+
+def test_version_and_error_strings():
+  lib = _lib()
+  assert lib.vmoe_abi_version() == 1
+  lib.vmoe_error_string.restype = ctypes.c_char_p
+  assert lib.vmoe_error_string(0) == b"ok"
+  for code in range(-7, 0):
+    assert lib.vmoe_error_string(code) != b"unknown vmoe error"
+
+
+def test_struct_layouts_match_header():
+  """Field order/types of each ctypes struct follow the header's typedef."""
+  from vmoe_amd import _hip
+  text = open(HEADER).read()
+  text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+  structs = {n: b for b, n in re.findall(r"typedef struct \{(.*?)\}\s*(\w+);", text, flags=re.S)}
+  cmap = {"int32_t": ctypes.c_int32, "float": ctypes.c_float, "size_t": ctypes.c_size_t}
+  py = {"VmoeGateTopkParams": _hip.GateTopkParams, "VmoeTopkParams": _hip.TopkParams,
+        "VmoeRouterMetricsParams": _hip.RouterMetricsParams,
+        "VmoeRouteAssignParams": _hip.RouteAssignParams,
+        "VmoeIndicesToSlotsParams": _hip.IndicesToSlotsParams,
+        "VmoeDispatchParams": _hip.DispatchParams, "VmoeCombineParams": _hip.CombineParams,
+        "VmoeDensifyParams": _hip.DensifyParams, "VmoeExpertMlpParams": _hip.ExpertMlpParams,
+        "VmoeTransposeParams": _hip.TransposeParams, "VmoeSoftRouteParams": _hip.SoftRouteParams,
+        "VmoeEinsumParams": _hip.EinsumParams, "VmoeCastParams": _hip.CastParams}
+  assert set(py) == set(structs)
+  for name, body in structs.items():
+    want = []
+    for decl in body.split(";"):
+      decl = decl.strip()
+      if not decl:
+        continue
+      m = re.match(r"(const\s+)?(\w+)\s*(\*?)\s*(.*)", decl)
+      base, star, names = m.group(2), m.group(3), m.group(4)
+      for nm in names.split(","):
+        nm = nm.strip()
+        is_ptr = bool(star) or nm.startswith("*")
+        want.append(ctypes.c_void_p if is_ptr else cmap[base])
+    got = [t for _, t in py[name]._fields_]
+    assert got == want, name
+
+
+def test_null_params_are_rejected_without_a_gpu():
+  lib = _lib()
+  for fn in ("vmoe_gate_topk", "vmoe_route_assign", "vmoe_dispatch", "vmoe_combine",
+             "vmoe_expert_mlp", "vmoe_soft_route", "vmoe_einsum_dispatch", "vmoe_cast"):
+    assert getattr(lib, fn)(None, None) == -1

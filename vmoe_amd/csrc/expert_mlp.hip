@@ -1,0 +1,213 @@
+// Expert MLPs (Dense -> GELU -> Dense per expert) for gfx950.
+//
+// Replaces the expert vmap of vmoe/moe.py:434-439 over
+// vit_jax.models_vit.MlpBlock (vmoe/nn/vit_moe.py:38-45): a GEMM batched over
+// the expert axis with the bias add and the GELU fused into the epilogue of the
+// first product and the bias add into the second.
+#include "gemm_bf16.h"
+
+namespace vmoe {
+namespace {
+
+// ---------------------------------------------------------------- float32 path
+// C[b] (R x N) = epi(A[b] (R x Kd) . B[b] (Kd x N) + bias[b]) with
+// v_mfma_f32_32x32x2_f32 (IEEE float32 multiply-add).  64x64 tile, 4 waves,
+// B is consumed in the reference's (in, out) order: a lane's B operand is one
+// scalar B[k][n], so no transposition is needed.
+constexpr int kF32Tile = 64, kF32BK = 16;
+
+template <int EPI>
+__global__ __launch_bounds__(256) void gemm_f32_kernel(
+    const float* __restrict__ A, const float* __restrict__ B, const float* __restrict__ bias,
+    float* __restrict__ C, int R, int N, int Kd, int tiles_m, int tiles_n) {
+  __shared__ float sa[kF32Tile][kF32BK + 1];
+  __shared__ float sb[kF32BK][kF32Tile + 4];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  const int m = lane & 31, h = lane >> 5;
+  const int per_batch = tiles_m * tiles_n;
+  const int b = blockIdx.x / per_batch;
+  const int rem = blockIdx.x - b * per_batch;
+  const int tile_n = rem / tiles_m, tile_m = rem - tile_n * tiles_m;
+  const int row0 = tile_m * kF32Tile, col0 = tile_n * kF32Tile;
+  const float* Ab = A + (size_t)b * R * Kd;
+  const float* Bb = B + (size_t)b * Kd * N;
+  floatx16 acc;
+#pragma unroll
+  for (int v = 0; v < 16; ++v) acc[v] = 0.f;
+  const int ar = tid >> 2, akc = (tid & 3) * 4;   // A: 64 rows x 4 float4
+  const int bk = tid >> 4, bn = (tid & 15) * 4;   // B: 16 rows x 16 float4
+  for (int k0 = 0; k0 < Kd; k0 += kF32BK) {
+    float4 va = make_float4(0.f, 0.f, 0.f, 0.f), vb = va;
+    {
+      int gr = row0 + ar;
+      if (gr >= R) gr = R - 1;
+      if (k0 + akc + 4 <= Kd) va = *reinterpret_cast<const float4*>(Ab + (size_t)gr * Kd + k0 + akc);
+      int gk = k0 + bk, gn = col0 + bn;
+      if (gk < Kd && gn + 4 <= N) vb = *reinterpret_cast<const float4*>(Bb + (size_t)gk * N + gn);
+    }
+    __syncthreads();
+    sa[ar][akc + 0] = va.x; sa[ar][akc + 1] = va.y; sa[ar][akc + 2] = va.z; sa[ar][akc + 3] = va.w;
+    sb[bk][bn + 0] = vb.x; sb[bk][bn + 1] = vb.y; sb[bk][bn + 2] = vb.z; sb[bk][bn + 3] = vb.w;
+    __syncthreads();
+#pragma unroll
+    for (int ks = 0; ks < kF32BK / 2; ++ks) {
+      float a = sa[wm * 32 + m][ks * 2 + h];
+      float bb = sb[ks * 2 + h][wn * 32 + m];
+      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a, bb, acc, 0, 0, 0);
+    }
+  }
+  const int col = col0 + wn * 32 + m;
+  const bool col_ok = col < N;
+  const float bv = (bias != nullptr && col_ok) ? bias[(size_t)b * N + col] : 0.f;
+  float* Cb = C + (size_t)b * R * N;
+#pragma unroll
+  for (int v = 0; v < 16; ++v) {
+    const int row = row0 + wm * 32 + (v >> 2) * 8 + h * 4 + (v & 3);
+    float o = acc[v] + bv;
+    if (EPI == kEpiBiasGeluTanh) o = gelu_tanh(o);
+    if (EPI == kEpiBiasGeluErf) o = gelu_erf(o);
+    if (row < R && col_ok) Cb[(size_t)row * N + col] = o;
+  }
+}
+
+template <int EPI>
+int launch_gemm_f32(const float* A, const float* B, const float* bias, float* C, int batch, int R,
+                    int N, int Kd, hipStream_t stream) {
+  const int tiles_m = (R + kF32Tile - 1) / kF32Tile, tiles_n = (N + kF32Tile - 1) / kF32Tile;
+  const long long blocks = (long long)batch * tiles_m * tiles_n;
+  if (blocks > 0x7fffffffLL) return VMOE_E_OVERFLOW;
+  hipLaunchKernelGGL(gemm_f32_kernel<EPI>, dim3((unsigned)blocks), dim3(256), 0, stream, A, B, bias,
+                     C, R, N, Kd, tiles_m, tiles_n);
+  return launch_status();
+}
+
+// ---------------------------------------------------------------- transpose
+template <typename T>
+__global__ __launch_bounds__(256) void transpose_kernel(const T* __restrict__ in,
+                                                        T* __restrict__ out, int rows, int cols) {
+  __shared__ T tile[64][64 + 2];
+  const int b = blockIdx.z;
+  const int r0 = blockIdx.y * 64, c0 = blockIdx.x * 64;
+  const T* src = in + (size_t)b * rows * cols;
+  T* dst = out + (size_t)b * rows * cols;
+  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+  for (int i = ty; i < 64; i += 4) {
+    int r = r0 + i, c = c0 + tx;
+    if (r < rows && c < cols) tile[i][tx] = src[(size_t)r * cols + c];
+  }
+  __syncthreads();
+  for (int i = ty; i < 64; i += 4) {
+    int c = c0 + i, r = r0 + tx;
+    if (r < rows && c < cols) dst[(size_t)c * rows + r] = tile[tx][i];
+  }
+}
+
+int transpose(const void* in, void* out, int batch, int rows, int cols, int dtype,
+              hipStream_t stream) {
+  dim3 grid((cols + 63) / 64, (rows + 63) / 64, batch);
+  if (dtype == VMOE_BF16)
+    hipLaunchKernelGGL(transpose_kernel<bf16_t>, grid, dim3(256), 0, stream, (const bf16_t*)in,
+                       (bf16_t*)out, rows, cols);
+  else
+    hipLaunchKernelGGL(transpose_kernel<float>, grid, dim3(256), 0, stream, (const float*)in,
+                       (float*)out, rows, cols);
+  return launch_status();
+}
+
+using CfgBig = GemmCfg<256, 256, 2, 2>;
+
+size_t align256(size_t v) { return (v + 255) / 256 * 256; }
+
+}  // namespace
+}  // namespace vmoe
+
+using namespace vmoe;
+
+static int check_mlp(const VmoeExpertMlpParams* p) {
+  if (p == nullptr || p->x == nullptr || p->out == nullptr) return VMOE_E_NULL;
+  if (p->E < 1 || p->R < 1 || p->D < 1 || p->M < 1) return VMOE_E_SHAPE;
+  if (p->dtype != VMOE_F32 && p->dtype != VMOE_BF16) return VMOE_E_DTYPE;
+  if (p->gelu != VMOE_GELU_TANH && p->gelu != VMOE_GELU_ERF) return VMOE_E_DTYPE;
+  if (p->dtype == VMOE_BF16) {
+    if ((p->w0 == nullptr && p->w0t == nullptr) || (p->w1 == nullptr && p->w1t == nullptr))
+      return VMOE_E_NULL;
+    if (p->D % 8 != 0 || p->M % 8 != 0) return VMOE_E_ALIGN;
+  } else {
+    if (p->w0 == nullptr || p->w1 == nullptr) return VMOE_E_NULL;
+    if (p->D % 4 != 0 || p->M % 4 != 0) return VMOE_E_ALIGN;
+  }
+  if (!aligned16(p->x) || !aligned16(p->out)) return VMOE_E_ALIGN;
+  if ((int64_t)p->E * p->R >= INT32_MAX) return VMOE_E_OVERFLOW;
+  return VMOE_OK;
+}
+
+extern "C" size_t vmoe_expert_mlp_workspace_bytes(const VmoeExpertMlpParams* p) {
+  if (p == nullptr || p->E < 1 || p->R < 1 || p->D < 1 || p->M < 1) return 0;
+  const size_t b = p->dtype == VMOE_BF16 ? 2 : 4;
+  size_t bytes = align256((size_t)p->E * p->R * p->M * b);  // hidden activations
+  if (p->dtype == VMOE_BF16) {
+    if (p->w0t == nullptr) bytes += align256((size_t)p->E * p->D * p->M * b);
+    if (p->w1t == nullptr) bytes += align256((size_t)p->E * p->D * p->M * b);
+  }
+  return bytes;
+}
+
+extern "C" int vmoe_expert_mlp(const VmoeExpertMlpParams* p, vmoe_stream_t stream_) {
+  int rc = check_mlp(p);
+  if (rc != VMOE_OK) return rc;
+  const size_t need = vmoe_expert_mlp_workspace_bytes(p);
+  if (p->workspace == nullptr || p->workspace_bytes < need || !aligned16(p->workspace))
+    return VMOE_E_WORKSPACE;
+  hipStream_t stream = as_stream(stream_);
+  unsigned char* ws = static_cast<unsigned char*>(p->workspace);
+  const size_t b = p->dtype == VMOE_BF16 ? 2 : 4;
+  void* hidden = ws;
+  ws += align256((size_t)p->E * p->R * p->M * b);
+  const bool tanh_gelu = p->gelu == VMOE_GELU_TANH;
+  if (p->dtype == VMOE_BF16) {
+    const void* w0t = p->w0t;
+    const void* w1t = p->w1t;
+    if (w0t == nullptr) {
+      rc = transpose(p->w0, ws, p->E, p->D, p->M, VMOE_BF16, stream);
+      if (rc != VMOE_OK) return rc;
+      w0t = ws;
+      ws += align256((size_t)p->E * p->D * p->M * b);
+    }
+    if (w1t == nullptr) {
+      rc = transpose(p->w1, ws, p->E, p->M, p->D, VMOE_BF16, stream);
+      if (rc != VMOE_OK) return rc;
+      w1t = ws;
+    }
+    if (tanh_gelu)
+      rc = launch_gemm_bf16<CfgBig, kEpiBiasGeluTanh>((const bf16_t*)p->x, (const bf16_t*)w0t,
+                                                      (const bf16_t*)p->b0, (bf16_t*)hidden, p->E,
+                                                      p->R, p->M, p->D, stream);
+    else
+      rc = launch_gemm_bf16<CfgBig, kEpiBiasGeluErf>((const bf16_t*)p->x, (const bf16_t*)w0t,
+                                                     (const bf16_t*)p->b0, (bf16_t*)hidden, p->E,
+                                                     p->R, p->M, p->D, stream);
+    if (rc != VMOE_OK) return rc;
+    return launch_gemm_bf16<CfgBig, kEpiBias>((const bf16_t*)hidden, (const bf16_t*)w1t,
+                                              (const bf16_t*)p->b1, (bf16_t*)p->out, p->E, p->R,
+                                              p->D, p->M, stream);
+  }
+  if (tanh_gelu)
+    rc = launch_gemm_f32<kEpiBiasGeluTanh>((const float*)p->x, (const float*)p->w0,
+                                           (const float*)p->b0, (float*)hidden, p->E, p->R, p->M,
+                                           p->D, stream);
+  else
+    rc = launch_gemm_f32<kEpiBiasGeluErf>((const float*)p->x, (const float*)p->w0,
+                                          (const float*)p->b0, (float*)hidden, p->E, p->R, p->M,
+                                          p->D, stream);
+  if (rc != VMOE_OK) return rc;
+  return launch_gemm_f32<kEpiBias>((const float*)hidden, (const float*)p->w1, (const float*)p->b1,
+                                   (float*)p->out, p->E, p->R, p->D, p->M, stream);
+}
+
+extern "C" int vmoe_pack_expert_weights(const VmoeTransposeParams* p, vmoe_stream_t stream) {
+  if (p == nullptr || p->in == nullptr || p->out == nullptr) return VMOE_E_NULL;
+  if (p->batch < 1 || p->rows < 1 || p->cols < 1 || p->batch > 65535) return VMOE_E_SHAPE;
+  if (p->dtype != VMOE_F32 && p->dtype != VMOE_BF16) return VMOE_E_DTYPE;
+  return transpose(p->in, p->out, p->batch, p->rows, p->cols, p->dtype, as_stream(stream));
+}

@@ -1,0 +1,401 @@
+// Fused router gating for gfx950: logits = x @ W on the matrix cores, softmax
+// over experts and top-K selection in registers with cross-lane reductions.
+//
+// Replaces vmoe/nn/routing.py:73-80 and the jax.lax.top_k of vmoe/moe.py:567.
+//
+// Work split: a wave owns a tile of 32 items.  The router kernel W (D x E) is
+// staged once per workgroup in LDS (bf16: transposed to [expert][k] so that a
+// lane's MFMA B fragment is one 16-byte read; f32: kept [k][expert]).  Item rows
+// stream from HBM with 16-byte loads, 64 contiguous bytes per lane per step.
+// After the K loop a 32x32 accumulator tile holds, per lane, one expert column
+// for 16 item rows; the softmax and the top-K run across the 32 lanes of a
+// half-wave with xor shuffles, 16 rows at a time.
+#include "vmoe_common.h"
+
+namespace vmoe {
+namespace {
+
+constexpr int kGateThreads = 256;
+constexpr int kGateWaves = kGateThreads / kWave;
+
+__device__ __forceinline__ float inv_orderable(uint32_t u) {
+  uint32_t b = (u & 0x80000000u) ? (u & 0x7fffffffu) : ~u;
+  return __builtin_bit_cast(float, b);
+}
+
+template <int MASK>
+__device__ __forceinline__ float xor_max(float v) {
+  return fmaxf(v, __shfl_xor(v, MASK, kWave));
+}
+
+__device__ __forceinline__ float half_wave_max(float v) {
+  v = fmaxf(v, __shfl_xor(v, 1, kWave));
+  v = fmaxf(v, __shfl_xor(v, 2, kWave));
+  v = fmaxf(v, __shfl_xor(v, 4, kWave));
+  v = fmaxf(v, __shfl_xor(v, 8, kWave));
+  v = fmaxf(v, __shfl_xor(v, 16, kWave));
+  return v;
+}
+__device__ __forceinline__ float half_wave_sum(float v) {
+  v += __shfl_xor(v, 1, kWave);
+  v += __shfl_xor(v, 2, kWave);
+  v += __shfl_xor(v, 4, kWave);
+  v += __shfl_xor(v, 8, kWave);
+  v += __shfl_xor(v, 16, kWave);
+  return v;
+}
+__device__ __forceinline__ uint64_t half_wave_max_u64(uint64_t v) {
+#pragma unroll
+  for (int m = 1; m < 32; m <<= 1) {
+    uint32_t lo = __shfl_xor((uint32_t)v, m, kWave);
+    uint32_t hi = __shfl_xor((uint32_t)(v >> 32), m, kWave);
+    uint64_t o = ((uint64_t)hi << 32) | lo;
+    v = o > v ? o : v;
+  }
+  return v;
+}
+
+// LDS row stride (in elements) of the staged router kernel.
+template <typename T> __host__ __device__ constexpr int w_stride(int kc, int epad) {
+  return sizeof(T) == 2 ? kc + 8 : epad;
+}
+
+template <typename T, int NT>
+__global__ __launch_bounds__(kGateThreads) void gate_topk_kernel(
+    const T* __restrict__ x, const T* __restrict__ w, const float* __restrict__ bias,
+    T* __restrict__ gates, float* __restrict__ topk_val, int32_t* __restrict__ topk_idx,
+    int num_items, int D, int E, int K, int KC, int num_chunks, int num_tiles) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  T* wl = reinterpret_cast<T*>(smem);
+  constexpr int EP = NT * 32;
+  constexpr bool kBf16 = sizeof(T) == 2;
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int m = lane & 31;
+  const int h = lane >> 5;
+  const int stride = w_stride<T>(KC, EP);
+  const int tiles_per_iter = gridDim.x * kGateWaves;
+  const int iters = (num_tiles + tiles_per_iter - 1) / tiles_per_iter;
+
+  for (int it = 0; it < iters; ++it) {
+    const int tile = it * tiles_per_iter + blockIdx.x * kGateWaves + wave;
+    const bool active = tile < num_tiles;
+    const int row0 = tile * 32;
+    int r = row0 + m;
+    if (r >= num_items) r = num_items - 1;
+    if (r < 0) r = 0;
+    const T* xrow = x + (size_t)r * D;
+
+    floatx16 acc[NT];
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) acc[nt][i] = 0.f;
+
+    for (int c = 0; c < num_chunks; ++c) {
+      const int k0 = c * KC;
+      if (num_chunks > 1 || it == 0) {
+        __syncthreads();
+        // Stage W[k0 : k0+KC, :] into LDS, zero padded in both directions.
+        for (int idx = tid; idx < KC * EP; idx += kGateThreads) {
+          int k = idx / EP, n = idx - k * EP;
+          T v = 0;
+          if (k0 + k < D && n < E) v = w[(size_t)(k0 + k) * E + n];
+          if (kBf16) wl[n * stride + k] = v; else wl[k * stride + n] = v;
+        }
+        __syncthreads();
+      }
+      if (!active) continue;
+      if constexpr (kBf16) {
+        const int nkb = KC / 64;
+        for (int kb = 0; kb < nkb; ++kb) {
+          const int kl = kb * 64 + h * 32;  // this lane's 32 k's inside the chunk
+          uint4 a[4];
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            int kg = k0 + kl + j * 8;
+            a[j] = (kg + 8 <= D) ? *reinterpret_cast<const uint4*>(xrow + kg) : make_uint4(0, 0, 0, 0);
+          }
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            bf16x8 af = __builtin_bit_cast(bf16x8, a[j]);
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) {
+              uint4 b = *reinterpret_cast<const uint4*>(wl + (nt * 32 + m) * stride + kl + j * 8);
+              acc[nt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af, __builtin_bit_cast(bf16x8, b),
+                                                                acc[nt], 0, 0, 0);
+            }
+          }
+        }
+      } else {
+        const int nkb = KC / 16;
+        for (int kb = 0; kb < nkb; ++kb) {
+          const int kl = kb * 16 + h * 8;
+          float a[8];
+#pragma unroll
+          for (int j = 0; j < 2; ++j) {
+            int kg = k0 + kl + j * 4;
+            float4 v = (kg + 4 <= D) ? *reinterpret_cast<const float4*>(xrow + kg)
+                                     : make_float4(0.f, 0.f, 0.f, 0.f);
+            a[j * 4 + 0] = v.x; a[j * 4 + 1] = v.y; a[j * 4 + 2] = v.z; a[j * 4 + 3] = v.w;
+          }
+#pragma unroll
+          for (int i = 0; i < 8; ++i) {
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) {
+              float b = wl[(kl + i) * stride + nt * 32 + m];
+              acc[nt] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], b, acc[nt], 0, 0, 0);
+            }
+          }
+        }
+      }
+    }
+    if (!active) continue;
+
+    // Epilogue: 16 accumulator registers = 16 item rows per half-wave.
+    float bn[NT];
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+      int n = nt * 32 + m;
+      bn[nt] = (bias != nullptr && n < E) ? bias[n] : 0.f;
+    }
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const int row = row0 + (i >> 2) * 8 + h * 4 + (i & 3);
+      float g[NT];
+      float mx = -INFINITY;
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt) {
+        float v = Elt<T>::round(acc[nt][i]);
+        if (bias != nullptr) v = Elt<T>::round(v + bn[nt]);
+        g[nt] = (nt * 32 + m < E) ? v : -INFINITY;
+        mx = fmaxf(mx, g[nt]);
+      }
+      mx = half_wave_max(mx);
+      float sum = 0.f;
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt) {
+        g[nt] = (nt * 32 + m < E) ? expf(g[nt] - mx) : 0.f;
+        sum += g[nt];
+      }
+      sum = half_wave_sum(sum);
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt) g[nt] = Elt<T>::round(g[nt] / sum);
+      const bool row_ok = row < num_items;
+      if (gates != nullptr && row_ok) {
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt)
+          if (nt * 32 + m < E) Elt<T>::store(gates + (size_t)row * E + nt * 32 + m, g[nt]);
+      }
+      uint32_t taken = 0;
+      for (int kk = 0; kk < K; ++kk) {
+        uint64_t best = 0;
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) {
+          int n = nt * 32 + m;
+          if (n < E && !(taken >> nt & 1u)) {
+            uint64_t key = ((uint64_t)orderable(g[nt]) << 32) | (uint32_t)(0xFFFFFFFFu - (uint32_t)n);
+            best = key > best ? key : best;
+          }
+        }
+        best = half_wave_max_u64(best);
+        const int n_star = (int)(0xFFFFFFFFu - (uint32_t)best);
+        if ((n_star & 31) == m) taken |= 1u << (n_star >> 5);
+        if (m == 0 && row_ok) {
+          topk_val[(size_t)row * K + kk] = inv_orderable((uint32_t)(best >> 32));
+          topk_idx[(size_t)row * K + kk] = n_star;
+        }
+      }
+    }
+  }
+}
+
+// Top-K of given float32 gates, one wave per item, E <= 1024.
+__global__ __launch_bounds__(256) void topk_kernel(const float* __restrict__ gates,
+                                                   float* __restrict__ topk_val,
+                                                   int32_t* __restrict__ topk_idx,
+                                                   int num_items, int E, int K) {
+  const int lane = threadIdx.x & 63;
+  const int item = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+  if (item >= num_items) return;
+  const float* g = gates + (size_t)item * E;
+  float v[16];
+#pragma unroll
+  for (int j = 0; j < 16; ++j) {
+    int n = j * 64 + lane;
+    v[j] = n < E ? g[n] : 0.f;
+  }
+  uint32_t taken = 0;
+  for (int kk = 0; kk < K; ++kk) {
+    uint64_t best = 0;
+#pragma unroll
+    for (int j = 0; j < 16; ++j) {
+      int n = j * 64 + lane;
+      if (n < E && !(taken >> j & 1u)) {
+        uint64_t key = ((uint64_t)orderable(v[j]) << 32) | (uint32_t)(0xFFFFFFFFu - (uint32_t)n);
+        best = key > best ? key : best;
+      }
+    }
+#pragma unroll
+    for (int msk = 1; msk < 64; msk <<= 1) {
+      uint32_t lo = __shfl_xor((uint32_t)best, msk, kWave);
+      uint32_t hi = __shfl_xor((uint32_t)(best >> 32), msk, kWave);
+      uint64_t o = ((uint64_t)hi << 32) | lo;
+      best = o > best ? o : best;
+    }
+    const int n_star = (int)(0xFFFFFFFFu - (uint32_t)best);
+    if ((n_star & 63) == lane) taken |= 1u << (n_star >> 6);
+    if (lane == 0) {
+      // Return the stored bits of the winner (keeps -0.0 / payloads intact).
+      topk_val[(size_t)item * K + kk] = g[n_star];
+      topk_idx[(size_t)item * K + kk] = n_star;
+    }
+  }
+}
+
+// Per-group auxiliary losses.  One workgroup per group; thread (r, e) sums
+// column e over rows r, r+R, ... in a fixed order, partial sums are combined in
+// a fixed order, so results are run-to-run identical.
+template <typename T>
+__global__ __launch_bounds__(256) void router_metrics_kernel(
+    const T* __restrict__ gates, const int32_t* __restrict__ top1, float* __restrict__ imp_loss,
+    float* __restrict__ gsh_loss, float* __restrict__ aux_loss, float w_gsh, float w_imp,
+    int S, int E, int top1_stride) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  float* part = reinterpret_cast<float*>(smem);              // (R, E)
+  const int tid = threadIdx.x;
+  const int g = blockIdx.x;
+  const int cols = E < 256 ? E : 256;
+  const int R = 256 / cols;                                  // rows handled per pass
+  int* count = reinterpret_cast<int*>(part + (size_t)R * E);   // (E,)
+  float* imp = reinterpret_cast<float*>(count + E);          // (E,)
+  for (int e = tid; e < E; e += 256) count[e] = 0;
+  __syncthreads();
+  const int r = tid / cols;
+  const int c = tid - r * cols;
+  if (r < R) {
+    for (int e = c; e < E; e += cols) {
+      float s = 0.f;
+      for (int i = r; i < S; i += R) s += Elt<T>::load(gates + ((size_t)g * S + i) * E + e);
+      part[r * E + e] = s;
+    }
+  }
+  for (int i = tid; i < S; i += 256) {
+    int t = top1[((size_t)g * S + i) * top1_stride];
+    if (t >= 0 && t < E) atomicAdd(&count[t], 1);
+  }
+  __syncthreads();
+  for (int e = tid; e < E; e += 256) {
+    float s = 0.f;
+    for (int rr = 0; rr < R; ++rr) s += part[rr * E + e];
+    imp[e] = s;
+  }
+  __syncthreads();
+  if (tid == 0) {
+    float mean = 0.f;
+    for (int e = 0; e < E; ++e) mean += imp[e];
+    mean /= (float)E;
+    float var = 0.f, gs = 0.f;
+    for (int e = 0; e < E; ++e) {
+      float d = imp[e] - mean;
+      var += d * d;
+      gs += ((float)count[e] / (float)S) * (imp[e] / (float)S);
+    }
+    var /= (float)E;
+    float il = var / (mean * mean);
+    float gl = gs / (float)E * (float)E * (float)E;
+    imp_loss[g] = il;
+    gsh_loss[g] = gl;
+    float a = 0.f;
+    if (w_gsh > 0.f) a += gl * w_gsh;
+    if (w_imp > 0.f) a += il * w_imp;
+    aux_loss[g] = a;
+  }
+}
+
+template <typename T>
+int launch_gate(const VmoeGateTopkParams* p, hipStream_t stream) {
+  const int nt = (p->E + 31) / 32;
+  const int ep = (nt == 3 ? 4 : nt) * 32;
+  const int gran = sizeof(T) == 2 ? 64 : 16;
+  const int dpad = (p->D + gran - 1) / gran * gran;
+  // Keep the staged router kernel within 96 KiB of LDS; split D otherwise.
+  const size_t budget = 96 * 1024;
+  int kc = dpad;
+  while ((size_t)(sizeof(T) == 2 ? ep * (kc + 8) : kc * ep) * sizeof(T) > budget && kc > gran)
+    kc = ((kc / 2) + gran - 1) / gran * gran;
+  const int num_chunks = (dpad + kc - 1) / kc;
+  const size_t lds = (size_t)(sizeof(T) == 2 ? ep * (kc + 8) : kc * ep) * sizeof(T);
+  const int num_tiles = (p->num_items + 31) / 32;
+  int blocks = (num_tiles + kGateWaves - 1) / kGateWaves;
+  if (blocks > 1024) blocks = 1024;
+  auto run = [&](auto kern) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return (int)e;
+    hipLaunchKernelGGL(kern, dim3(blocks), dim3(kGateThreads), lds, stream,
+                       (const T*)p->x, (const T*)p->w, p->logit_bias, (T*)p->gates, p->topk_val,
+                       p->topk_idx, p->num_items, p->D, p->E, p->K, kc, num_chunks, num_tiles);
+    return launch_status();
+  };
+  switch (nt) {
+    case 1: return run(gate_topk_kernel<T, 1>);
+    case 2: return run(gate_topk_kernel<T, 2>);
+    default: return run(gate_topk_kernel<T, 4>);
+  }
+}
+
+}  // namespace
+}  // namespace vmoe
+
+using namespace vmoe;
+
+extern "C" int vmoe_gate_topk(const VmoeGateTopkParams* p, vmoe_stream_t stream) {
+  if (p == nullptr || p->x == nullptr || p->w == nullptr || p->topk_val == nullptr ||
+      p->topk_idx == nullptr)
+    return VMOE_E_NULL;
+  if (p->num_items < 1 || p->D < 1 || p->E < 1 || p->K < 1 || p->K > p->E) return VMOE_E_SHAPE;
+  if (p->dtype != VMOE_F32 && p->dtype != VMOE_BF16) return VMOE_E_DTYPE;
+  if (p->E > 128) return VMOE_E_UNSUPPORTED;
+  const int vec = p->dtype == VMOE_BF16 ? 8 : 4;
+  if (p->D % vec != 0 || !aligned16(p->x)) return VMOE_E_ALIGN;
+  if ((int64_t)p->num_items * (p->D > p->E * p->K ? p->D : p->E * p->K) >= (int64_t)1 << 40)
+    return VMOE_E_OVERFLOW;
+  return p->dtype == VMOE_BF16 ? launch_gate<bf16_t>(p, as_stream(stream))
+                               : launch_gate<float>(p, as_stream(stream));
+}
+
+extern "C" int vmoe_topk(const VmoeTopkParams* p, vmoe_stream_t stream) {
+  if (p == nullptr || p->gates == nullptr || p->topk_val == nullptr || p->topk_idx == nullptr)
+    return VMOE_E_NULL;
+  if (p->num_items < 1 || p->E < 1 || p->K < 1 || p->K > p->E) return VMOE_E_SHAPE;
+  if (p->E > 1024) return VMOE_E_UNSUPPORTED;
+  const int blocks = (p->num_items + 3) / 4;
+  hipLaunchKernelGGL(topk_kernel, dim3(blocks), dim3(256), 0, as_stream(stream), p->gates,
+                     p->topk_val, p->topk_idx, p->num_items, p->E, p->K);
+  return launch_status();
+}
+
+extern "C" int vmoe_router_metrics(const VmoeRouterMetricsParams* p, vmoe_stream_t stream) {
+  if (p == nullptr || p->gates == nullptr || p->top1_idx == nullptr ||
+      p->importance_loss == nullptr || p->gshard_loss == nullptr || p->auxiliary_loss == nullptr)
+    return VMOE_E_NULL;
+  if (p->G < 1 || p->S < 1 || p->E < 1 || p->top1_stride < 1) return VMOE_E_SHAPE;
+  if (p->dtype != VMOE_F32 && p->dtype != VMOE_BF16) return VMOE_E_DTYPE;
+  if (p->E > 1024) return VMOE_E_UNSUPPORTED;
+  const int cols = p->E < 256 ? p->E : 256;
+  const int R = 256 / cols;
+  const size_t lds = ((size_t)R * p->E + 2 * (size_t)p->E) * 4;
+  if (p->dtype == VMOE_BF16)
+    hipLaunchKernelGGL(router_metrics_kernel<bf16_t>, dim3(p->G), dim3(256), lds, as_stream(stream),
+                       (const bf16_t*)p->gates, p->top1_idx, p->importance_loss, p->gshard_loss,
+                       p->auxiliary_loss, p->gshard_loss_weight, p->importance_loss_weight, p->S,
+                       p->E, p->top1_stride);
+  else
+    hipLaunchKernelGGL(router_metrics_kernel<float>, dim3(p->G), dim3(256), lds, as_stream(stream),
+                       (const float*)p->gates, p->top1_idx, p->importance_loss, p->gshard_loss,
+                       p->auxiliary_loss, p->gshard_loss_weight, p->importance_loss_weight, p->S,
+                       p->E, p->top1_stride);
+  return launch_status();
+}

@@ -1,0 +1,231 @@
+// Capacity-bounded slot assignment with Batch Priority Routing for gfx950.
+//
+// Replaces vmoe/moe.py:568-589 (+ :646-648): the reference sorts items by their
+// first-choice gate, flattens the (K, S) choices K-major, takes a one-hot over
+// experts and a cumulative sum down the K*S rows.  Here one workgroup owns a
+// group and works entirely in LDS:
+//   1. 64-bit keys (descending-gate order bits << 32 | item) are bitonic-sorted;
+//      the item index in the low word makes the order stable by construction.
+//   2. every (item, choice) sets bit  k*S + rank(item)  in its expert's bitmap
+//      (integer LDS atomics: order-independent result);
+//   3. an exclusive prefix of per-word popcounts turns "how many set bits come
+//      before mine" -- the cumsum of the one-hot column -- into one table
+//      lookup plus one masked popcount.
+// The kernel also emits the two maps the data-movement kernels use: item ->
+// slot row (-1 when over capacity) and slot row -> item (-1 when empty).
+#include "vmoe_common.h"
+
+namespace vmoe {
+namespace {
+
+constexpr int kRouteThreads = 1024;
+
+__host__ __device__ inline int pow2ceil(int v) {
+  int p = 1;
+  while (p < v) p <<= 1;
+  return p;
+}
+
+__global__ __launch_bounds__(kRouteThreads) void route_assign_kernel(
+    const float* __restrict__ topk_val, const int32_t* __restrict__ topk_idx,
+    int32_t* __restrict__ indices, int32_t* __restrict__ token_slot,
+    int32_t* __restrict__ slot_token, int32_t* __restrict__ fill, int G, int S, int E, int K,
+    int C, int bpr, int SP, int W) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  // Layout: keys[SP] (u64, only with bpr) | bitmap[E*W] | prefix[E*W] | rank[S] | total[E]
+  uint64_t* keys = reinterpret_cast<uint64_t*>(smem);
+  uint32_t* bitmap = reinterpret_cast<uint32_t*>(smem + (bpr ? (size_t)SP * 8 : 0));
+  uint32_t* prefix = bitmap + (size_t)E * W;
+  int32_t* rank = reinterpret_cast<int32_t*>(prefix + (size_t)E * W);
+  int32_t* total = rank + S;
+  const int tid = threadIdx.x;
+  const int g = blockIdx.x;
+  const float* val = topk_val + (size_t)g * S * K;
+  const int32_t* idx = topk_idx + (size_t)g * S * K;
+
+  for (int i = tid; i < E * W; i += kRouteThreads) bitmap[i] = 0u;
+  if (bpr) {
+    for (int s = tid; s < SP; s += kRouteThreads) {
+      uint64_t key = ~0ull;
+      if (s < S) key = ((uint64_t)(~orderable(val[(size_t)s * K])) << 32) | (uint32_t)s;
+      keys[s] = key;
+    }
+    __syncthreads();
+    // Bitonic sort, ascending.
+    for (int size = 2; size <= SP; size <<= 1) {
+      for (int stride = size >> 1; stride > 0; stride >>= 1) {
+        for (int t = tid; t < (SP >> 1); t += kRouteThreads) {
+          int lo = 2 * t - (t & (stride - 1));
+          int hi = lo + stride;
+          bool up = (lo & size) == 0;
+          uint64_t a = keys[lo], b = keys[hi];
+          if ((a > b) == up) { keys[lo] = b; keys[hi] = a; }
+        }
+        __syncthreads();
+      }
+    }
+    for (int r = tid; r < S; r += kRouteThreads) rank[(uint32_t)keys[r]] = r;
+  } else {
+    for (int s = tid; s < S; s += kRouteThreads) rank[s] = s;
+  }
+  __syncthreads();
+
+  const int SK = S * K;
+  for (int i = tid; i < SK; i += kRouteThreads) {
+    int s = i / K, k = i - s * K;
+    int e = idx[i];
+    if (e >= 0 && e < E) {
+      int bit = k * S + rank[s];
+      atomicOr(&bitmap[(size_t)e * W + (bit >> 5)], 1u << (bit & 31));
+    }
+  }
+  __syncthreads();
+  // Exclusive prefix of popcounts per expert: one wave per expert, 64 words per step.
+  {
+    const int lane = tid & 63, wave = tid >> 6, nwaves = kRouteThreads >> 6;
+    for (int e = wave; e < E; e += nwaves) {
+      int carry = 0;
+      for (int w0 = 0; w0 < W; w0 += 64) {
+        int w = w0 + lane;
+        int c = w < W ? __popc(bitmap[(size_t)e * W + w]) : 0;
+        int incl = c;
+#pragma unroll
+        for (int d = 1; d < 64; d <<= 1) {
+          int o = __shfl_up(incl, d, kWave);
+          if (lane >= d) incl += o;
+        }
+        if (w < W) prefix[(size_t)e * W + w] = (uint32_t)(carry + incl - c);
+        carry += __shfl(incl, 63, kWave);
+      }
+      if (lane == 0) total[e] = carry;
+    }
+  }
+  __syncthreads();
+
+  for (int i = tid; i < SK; i += kRouteThreads) {
+    int s = i / K, k = i - s * K;
+    int e = idx[i];
+    int pos = -1, slot = -1;
+    if (e >= 0 && e < E) {
+      int bit = k * S + rank[s];
+      int w = bit >> 5;
+      pos = (int)prefix[(size_t)e * W + w] +
+            __popc(bitmap[(size_t)e * W + w] & ((1u << (bit & 31)) - 1u));
+      if (pos < C) {
+        slot = slot_row(e, g, pos, G, E, C);
+        slot_token[slot] = g * S + s;
+      }
+    }
+    size_t o = (size_t)g * SK + i;
+    indices[2 * o] = e;
+    indices[2 * o + 1] = pos;
+    token_slot[o] = slot;
+  }
+  // Slots nobody claimed.
+  for (int i = tid; i < E * C; i += kRouteThreads) {
+    int e = i / C, c = i - e * C;
+    if (c >= total[e]) slot_token[slot_row(e, g, c, G, E, C)] = -1;
+  }
+  if (fill != nullptr)
+    for (int e = tid; e < E; e += kRouteThreads) fill[(size_t)g * E + e] = total[e] < C ? total[e] : C;
+}
+
+__global__ __launch_bounds__(256) void fill_i32_kernel(int32_t* p, size_t n, int32_t v) {
+  size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) p[i] = v;
+}
+
+__global__ __launch_bounds__(256) void indices_to_slots_kernel(
+    const int32_t* __restrict__ indices, int32_t* __restrict__ token_slot,
+    int32_t* __restrict__ slot_token, int32_t* __restrict__ num_dup, int32_t* __restrict__ num_inv,
+    int G, int S, int E, int K, int C) {
+  size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  size_t n = (size_t)G * S * K;
+  if (i >= n) return;
+  int e = indices[2 * i], c = indices[2 * i + 1];
+  int slot = -1;
+  if (e < 0 || c < 0) {
+    atomicAdd(num_inv, 1);
+  } else if (e < E && c < C) {
+    size_t item = i / K;
+    int g = (int)(item / S);
+    slot = slot_row(e, g, c, G, E, C);
+    int prev = atomicExch(&slot_token[slot], (int)item);
+    if (prev >= 0) atomicAdd(num_dup, 1);
+  }
+  token_slot[i] = slot;
+}
+
+__global__ __launch_bounds__(256) void densify_kernel(
+    const int32_t* __restrict__ indices, const float* __restrict__ weights,
+    float* __restrict__ combine, uint8_t* __restrict__ dispatch, int G, int S, int E, int K, int C) {
+  size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  size_t n = (size_t)G * S * K;
+  if (i >= n) return;
+  int e = indices[2 * i], c = indices[2 * i + 1];
+  if (e < 0 || c < 0 || e >= E || c >= C) return;
+  size_t item = i / K;
+  size_t o = (item * E + e) * C + c;
+  if (combine != nullptr) combine[o] = weights[i];
+  if (dispatch != nullptr) dispatch[o] = 1;
+}
+
+}  // namespace
+}  // namespace vmoe
+
+using namespace vmoe;
+
+static int check_route_shapes(int G, int S, int E, int K, int C) {
+  if (G < 1 || S < 1 || E < 1 || K < 1 || C < 1 || K > E) return VMOE_E_SHAPE;
+  if ((int64_t)G * S * K * 2 >= INT32_MAX || (int64_t)E * G * C >= INT32_MAX) return VMOE_E_OVERFLOW;
+  return VMOE_OK;
+}
+
+extern "C" int vmoe_route_assign(const VmoeRouteAssignParams* p, vmoe_stream_t stream) {
+  if (p == nullptr || p->topk_idx == nullptr || p->indices == nullptr ||
+      p->token_slot == nullptr || p->slot_token == nullptr)
+    return VMOE_E_NULL;
+  if (p->batch_priority && p->topk_val == nullptr) return VMOE_E_NULL;
+  int rc = check_route_shapes(p->G, p->S, p->E, p->K, p->C);
+  if (rc != VMOE_OK) return rc;
+  const int SP = pow2ceil(p->S);
+  const int W = (p->S * p->K + 31) / 32;
+  const size_t lds = (p->batch_priority ? (size_t)SP * 8 : 0) + (size_t)p->E * W * 8 +
+                     (size_t)p->S * 4 + (size_t)p->E * 4;
+  if (lds > 160 * 1024) return VMOE_E_UNSUPPORTED;
+  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(route_assign_kernel),
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+  if (e != hipSuccess) return (int)e;
+  hipLaunchKernelGGL(route_assign_kernel, dim3(p->G), dim3(kRouteThreads), lds, as_stream(stream),
+                     p->topk_val, p->topk_idx, p->indices, p->token_slot, p->slot_token, p->fill,
+                     p->G, p->S, p->E, p->K, p->C, p->batch_priority ? 1 : 0, SP, W);
+  return launch_status();
+}
+
+extern "C" int vmoe_indices_to_slots(const VmoeIndicesToSlotsParams* p, vmoe_stream_t stream) {
+  if (p == nullptr || p->indices == nullptr || p->token_slot == nullptr ||
+      p->slot_token == nullptr || p->num_duplicates == nullptr || p->num_invalid == nullptr)
+    return VMOE_E_NULL;
+  if (p->G < 1 || p->S < 1 || p->E < 1 || p->K < 1 || p->C < 1) return VMOE_E_SHAPE;
+  if ((int64_t)p->G * p->S * p->K * 2 >= INT32_MAX || (int64_t)p->E * p->G * p->C >= INT32_MAX)
+    return VMOE_E_OVERFLOW;
+  const size_t ns = (size_t)p->E * p->G * p->C;
+  const size_t n = (size_t)p->G * p->S * p->K;
+  hipLaunchKernelGGL(fill_i32_kernel, dim3((unsigned)((ns + 255) / 256)), dim3(256), 0,
+                     as_stream(stream), p->slot_token, ns, -1);
+  hipLaunchKernelGGL(indices_to_slots_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0,
+                     as_stream(stream), p->indices, p->token_slot, p->slot_token,
+                     p->num_duplicates, p->num_invalid, p->G, p->S, p->E, p->K, p->C);
+  return launch_status();
+}
+
+extern "C" int vmoe_densify(const VmoeDensifyParams* p, vmoe_stream_t stream) {
+  if (p == nullptr || p->indices == nullptr) return VMOE_E_NULL;
+  if (p->combine != nullptr && p->weights == nullptr) return VMOE_E_NULL;
+  if (p->G < 1 || p->S < 1 || p->E < 1 || p->K < 1 || p->C < 1) return VMOE_E_SHAPE;
+  const size_t n = (size_t)p->G * p->S * p->K;
+  hipLaunchKernelGGL(densify_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0,
+                     as_stream(stream), p->indices, p->weights, p->combine, p->dispatch, p->G,
+                     p->S, p->E, p->K, p->C);
+  return launch_status();
+}

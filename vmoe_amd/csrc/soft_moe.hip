@@ -1,0 +1,355 @@
+// Soft MoE routing and dense (einsum) dispatch / combine for gfx950.
+//
+// soft_route replaces vmoe/projects/soft_moe/router.py:57-96: one workgroup per
+// group normalises the item rows, multiplies them with the unit-norm slot
+// parameters on the matrix cores, keeps the (S x N) logits of the group in LDS
+// and takes both softmaxes (over items for the dispatch weights, over slots for
+// the combine weights) from that one copy.
+//
+// einsum_dispatch / einsum_combine replace EinsumDispatcher.dispatch/.combine
+// (vmoe/moe.py:148-161) for dense weights, including the expert-buffer row
+// order of _dispatch/_receive (moe.py:488-519).  They run on
+// v_mfma_f32_32x32x2_f32: the weights keep full float32 precision (the
+// reference promotes bf16 data to the weights' dtype), and a lane's operands
+// are single scalars, so neither the (S, N) weights nor the (rows, D) data need
+// a transposed copy.
+#include "vmoe_common.h"
+
+namespace vmoe {
+namespace {
+
+constexpr float kNormEps = 1e-6f;
+
+__device__ __forceinline__ float load_any(const void* p, size_t i, int dtype) {
+  return dtype == VMOE_F32 ? reinterpret_cast<const float*>(p)[i]
+                           : bf2f(reinterpret_cast<const bf16_t*>(p)[i]);
+}
+__device__ __forceinline__ float load_w(const void* p, size_t i, int wdtype) {
+  if (wdtype == VMOE_W_F32) return reinterpret_cast<const float*>(p)[i];
+  if (wdtype == VMOE_W_BF16) return bf2f(reinterpret_cast<const bf16_t*>(p)[i]);
+  return reinterpret_cast<const uint8_t*>(p)[i] ? 1.f : 0.f;
+}
+__device__ __forceinline__ void store_any(void* p, size_t i, float v, int dtype) {
+  if (dtype == VMOE_F32) reinterpret_cast<float*>(p)[i] = v;
+  else reinterpret_cast<bf16_t*>(p)[i] = f2bf(v);
+}
+
+// Unit-normalise the columns of mu (D, N) and apply the scale when it belongs to
+// mu.  bf16: writes muT (N, D) so that a column's k run is contiguous;
+// f32: writes (D, N).
+template <typename T>
+__global__ __launch_bounds__(256) void soft_prep_mu_kernel(const T* __restrict__ mu,
+                                                           T* __restrict__ out, float scale,
+                                                           int scale_mu, int D, int N) {
+  __shared__ float red[256];
+  const int n = blockIdx.x, tid = threadIdx.x;
+  float s = 0.f;
+  for (int d = tid; d < D; d += 256) {
+    float v = Elt<T>::load(mu + (size_t)d * N + n);
+    s += v * v;
+  }
+  red[tid] = s;
+  __syncthreads();
+  for (int o = 128; o > 0; o >>= 1) {
+    if (tid < o) red[tid] += red[tid + o];
+    __syncthreads();
+  }
+  const float inv = 1.0f / sqrtf(red[0] + kNormEps);
+  const float sc = Elt<T>::round(scale);
+  for (int d = tid; d < D; d += 256) {
+    float v = Elt<T>::round(Elt<T>::load(mu + (size_t)d * N + n) * inv);
+    if (scale_mu) v = Elt<T>::round(v * sc);
+    if (sizeof(T) == 2) Elt<T>::store(out + (size_t)n * D + d, v);
+    else Elt<T>::store(out + (size_t)d * N + n, v);
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void soft_route_kernel(
+    const T* __restrict__ x, const T* __restrict__ muw, T* __restrict__ dispatch_w,
+    T* __restrict__ combine_w, T* __restrict__ logits_out, float scale, int scale_x, int S, int D,
+    int N, int SP, int NP) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  float* inv_norm = reinterpret_cast<float*>(smem);                  // SP
+  T* lg = reinterpret_cast<T*>(smem + (size_t)SP * 4);               // SP x LDW
+  const int LDW = NP + (sizeof(T) == 2 ? 2 : 1);
+  constexpr bool kBf16 = sizeof(T) == 2;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int m = lane & 31, h = lane >> 5;
+  const int g = blockIdx.x;
+  const T* xg = x + (size_t)g * S * D;
+  const float sc = Elt<T>::round(scale);
+
+  // Phase 1: 1/sqrt(sum x^2 + eps) per item row.
+  for (int s = wave; s < SP; s += 4) {
+    float acc = 0.f;
+    if (s < S)
+      for (int d = lane; d < D; d += 64) {
+        float v = Elt<T>::load(xg + (size_t)s * D + d);
+        acc += v * v;
+      }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) acc += __shfl_xor(acc, o, kWave);
+    if (lane == 0) inv_norm[s] = s < S ? 1.0f / sqrtf(acc + kNormEps) : 0.f;
+  }
+  __syncthreads();
+
+  // Phase 2: logits tile by tile (32 items x 32 slots per MFMA accumulator).
+  const int row_tiles = SP / 32, col_tiles = NP / 32;
+  for (int rt = wave; rt < row_tiles; rt += 4) {
+    int r = rt * 32 + m;
+    const float inv = inv_norm[r];
+    if (r >= S) r = S - 1;
+    const T* xrow = xg + (size_t)r * D;
+    for (int ct0 = 0; ct0 < col_tiles; ct0 += 4) {
+      floatx16 acc[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[j][v] = 0.f;
+      if constexpr (kBf16) {
+        for (int k0 = 0; k0 < D; k0 += 16) {
+          const int k = k0 + h * 8;
+          bf16x8 af;
+          if (k + 8 <= D) {
+            uint4 raw = *reinterpret_cast<const uint4*>(xrow + k);
+            const uint32_t w4[4] = {raw.x, raw.y, raw.z, raw.w};
+            uint32_t o4[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+              float lo = bf16r(__builtin_bit_cast(float, w4[i] << 16) * inv);
+              float hi = bf16r(__builtin_bit_cast(float, w4[i] & 0xffff0000u) * inv);
+              if (scale_x) { lo = bf16r(lo * sc); hi = bf16r(hi * sc); }
+              o4[i] = (uint32_t)f2bf(lo) | ((uint32_t)f2bf(hi) << 16);
+            }
+            af = __builtin_bit_cast(bf16x8, make_uint4(o4[0], o4[1], o4[2], o4[3]));
+          } else {
+            af = __builtin_bit_cast(bf16x8, make_uint4(0, 0, 0, 0));
+          }
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            const int n = (ct0 + j) * 32 + m;
+            uint4 braw = make_uint4(0, 0, 0, 0);
+            if (ct0 + j < col_tiles && n < N && k + 8 <= D)
+              braw = *reinterpret_cast<const uint4*>(muw + (size_t)n * D + k);
+            acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af, __builtin_bit_cast(bf16x8, braw),
+                                                             acc[j], 0, 0, 0);
+          }
+        }
+      } else {
+        for (int k0 = 0; k0 < D; k0 += 2) {
+          const int k = k0 + h;
+          float a = 0.f;
+          if (k < D) {
+            a = Elt<T>::load(xrow + k) * inv;
+            if (scale_x) a = a * sc;
+          }
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            const int n = (ct0 + j) * 32 + m;
+            float bv = 0.f;
+            if (ct0 + j < col_tiles && n < N && k < D) bv = Elt<T>::load(muw + (size_t)k * N + n);
+            acc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, bv, acc[j], 0, 0, 0);
+          }
+        }
+      }
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        if (ct0 + j >= col_tiles) continue;
+        const int col = (ct0 + j) * 32 + m;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          const int row = rt * 32 + (v >> 2) * 8 + h * 4 + (v & 3);
+          Elt<T>::store(lg + (size_t)row * LDW + col, acc[j][v]);
+        }
+      }
+    }
+  }
+  __syncthreads();
+
+  // Phase 3: combine weights = softmax over the N slots of each item (wave per row).
+  for (int s = wave; s < S; s += 4) {
+    const T* row = lg + (size_t)s * LDW;
+    float mx = -INFINITY;
+    for (int n = lane; n < N; n += 64) mx = fmaxf(mx, Elt<T>::load(row + n));
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o, kWave));
+    float sum = 0.f;
+    for (int n = lane; n < N; n += 64) sum += expf(Elt<T>::load(row + n) - mx);
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) sum += __shfl_xor(sum, o, kWave);
+    const size_t base = ((size_t)g * S + s) * N;
+    for (int n = lane; n < N; n += 64) {
+      float l = Elt<T>::load(row + n);
+      Elt<T>::store(combine_w + base + n, expf(l - mx) / sum);
+      if (logits_out != nullptr) Elt<T>::store(logits_out + base + n, l);
+    }
+  }
+  // Phase 4: dispatch weights = softmax over the S items of each slot (thread per column).
+  for (int n = tid; n < N; n += 256) {
+    float mx = -INFINITY;
+    for (int s = 0; s < S; ++s) mx = fmaxf(mx, Elt<T>::load(lg + (size_t)s * LDW + n));
+    float sum = 0.f;
+    for (int s = 0; s < S; ++s) sum += expf(Elt<T>::load(lg + (size_t)s * LDW + n) - mx);
+    for (int s = 0; s < S; ++s) {
+      float l = Elt<T>::load(lg + (size_t)s * LDW + n);
+      Elt<T>::store(dispatch_w + ((size_t)g * S + s) * N + n, expf(l - mx) / sum);
+    }
+  }
+}
+
+// Dense einsum between per-group weights and data on the float32 matrix cores.
+//   DISPATCH: out[slot(g,mm)] = sum_s w[g,s,mm] * data[g,s,:]      (M = E*C, Kd = S)
+//   COMBINE:  out[g,mm,:]     = sum_n w[g,mm,n] * data[slot(g,n)]  (M = S,   Kd = E*C)
+template <bool DISPATCH>
+__global__ __launch_bounds__(256) void einsum_kernel(const void* __restrict__ w,
+                                                     const void* __restrict__ data,
+                                                     void* __restrict__ out, int G, int S, int E,
+                                                     int C, int D, int wdt, int ddt, int odt) {
+  __shared__ float sa[64][16 + 1];
+  __shared__ float sb[16][64 + 4];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  const int m = lane & 31, h = lane >> 5;
+  const int g = blockIdx.z;
+  const int N = E * C;
+  const int M = DISPATCH ? N : S;
+  const int Kd = DISPATCH ? S : N;
+  const int row0 = blockIdx.y * 64, col0 = blockIdx.x * 64;
+  const size_t wbase = (size_t)g * S * N;
+  floatx16 acc;
+#pragma unroll
+  for (int v = 0; v < 16; ++v) acc[v] = 0.f;
+  for (int k0 = 0; k0 < Kd; k0 += 16) {
+    float va[4], vb[4];
+    if (DISPATCH) {
+      const int kk = k0 + (tid >> 4), m4 = row0 + (tid & 15) * 4;
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        va[i] = (kk < Kd && m4 + i < M) ? load_w(w, wbase + (size_t)kk * N + m4 + i, wdt) : 0.f;
+    } else {
+      const int mm = row0 + (tid >> 2), k4 = k0 + (tid & 3) * 4;
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        va[i] = (mm < M && k4 + i < Kd) ? load_w(w, wbase + (size_t)mm * N + k4 + i, wdt) : 0.f;
+    }
+    {
+      const int kk = k0 + (tid >> 4), n4 = col0 + (tid & 15) * 4;
+      size_t rowi = 0;
+      if (kk < Kd) rowi = DISPATCH ? (size_t)g * S + kk : (size_t)slot_row(kk / C, g, kk % C, G, E, C);
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        vb[i] = (kk < Kd && n4 + i < D) ? load_any(data, rowi * D + n4 + i, ddt) : 0.f;
+    }
+    __syncthreads();
+    if (DISPATCH) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) sa[(tid & 15) * 4 + i][tid >> 4] = va[i];
+    } else {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) sa[tid >> 2][(tid & 3) * 4 + i] = va[i];
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) sb[tid >> 4][(tid & 15) * 4 + i] = vb[i];
+    __syncthreads();
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks)
+      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(sa[wm * 32 + m][ks * 2 + h],
+                                                 sb[ks * 2 + h][wn * 32 + m], acc, 0, 0, 0);
+  }
+  const int col = col0 + wn * 32 + m;
+#pragma unroll
+  for (int v = 0; v < 16; ++v) {
+    const int mm = row0 + wm * 32 + (v >> 2) * 8 + h * 4 + (v & 3);
+    if (mm < M && col < D) {
+      size_t orow = DISPATCH ? (size_t)slot_row(mm / C, g, mm % C, G, E, C) : (size_t)g * S + mm;
+      store_any(out, orow * D + col, acc[v], odt);
+    }
+  }
+}
+
+int check_einsum(const VmoeEinsumParams* p, bool dispatch) {
+  if (p == nullptr || p->w == nullptr || p->data == nullptr || p->out == nullptr) return VMOE_E_NULL;
+  if (p->G < 1 || p->S < 1 || p->E < 1 || p->C < 1 || p->D < 1) return VMOE_E_SHAPE;
+  if (p->G > 65535) return VMOE_E_UNSUPPORTED;
+  if (p->w_dtype < VMOE_W_F32 || p->w_dtype > VMOE_W_BOOL) return VMOE_E_DTYPE;
+  if (!dispatch && p->w_dtype == VMOE_W_BOOL) return VMOE_E_DTYPE;
+  if ((p->data_dtype != VMOE_F32 && p->data_dtype != VMOE_BF16) ||
+      (p->out_dtype != VMOE_F32 && p->out_dtype != VMOE_BF16))
+    return VMOE_E_DTYPE;
+  if ((int64_t)p->E * p->G * p->C >= INT32_MAX || (int64_t)p->G * p->S >= INT32_MAX)
+    return VMOE_E_OVERFLOW;
+  return VMOE_OK;
+}
+
+}  // namespace
+}  // namespace vmoe
+
+using namespace vmoe;
+
+extern "C" size_t vmoe_soft_route_workspace_bytes(const VmoeSoftRouteParams* p) {
+  if (p == nullptr || p->D < 1 || p->N < 1) return 0;
+  return (size_t)p->D * p->N * sizeof(float);
+}
+
+extern "C" int vmoe_soft_route(const VmoeSoftRouteParams* p, vmoe_stream_t stream_) {
+  if (p == nullptr || p->x == nullptr || p->mu == nullptr || p->dispatch_w == nullptr ||
+      p->combine_w == nullptr)
+    return VMOE_E_NULL;
+  if (p->G < 1 || p->S < 1 || p->D < 1 || p->N < 1) return VMOE_E_SHAPE;
+  if (p->dtype != VMOE_F32 && p->dtype != VMOE_BF16) return VMOE_E_DTYPE;
+  if (p->N > 1024) return VMOE_E_UNSUPPORTED;
+  if (p->dtype == VMOE_BF16 && (p->D % 8 != 0 || !aligned16(p->x))) return VMOE_E_ALIGN;
+  if (p->workspace == nullptr || p->workspace_bytes < vmoe_soft_route_workspace_bytes(p) ||
+      !aligned16(p->workspace))
+    return VMOE_E_WORKSPACE;
+  const size_t esz = p->dtype == VMOE_BF16 ? 2 : 4;
+  const int SP = (p->S + 31) / 32 * 32, NP = (p->N + 31) / 32 * 32;
+  const int LDW = NP + (esz == 2 ? 2 : 1);
+  const size_t lds = (size_t)SP * 4 + (size_t)SP * LDW * esz;
+  if (lds > 160 * 1024) return VMOE_E_UNSUPPORTED;
+  hipStream_t stream = as_stream(stream_);
+  // router.py:79-82: the scale multiplies whichever of the two operands is smaller.
+  const int scale_x = ((int64_t)p->G * p->S * p->D < (int64_t)p->D * p->N) ? 1 : 0;
+  if (p->dtype == VMOE_BF16) {
+    hipLaunchKernelGGL(soft_prep_mu_kernel<bf16_t>, dim3(p->N), dim3(256), 0, stream,
+                       (const bf16_t*)p->mu, (bf16_t*)p->workspace, p->scale, !scale_x, p->D, p->N);
+    auto kern = soft_route_kernel<bf16_t>;
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return (int)e;
+    hipLaunchKernelGGL(kern, dim3(p->G), dim3(256), lds, stream, (const bf16_t*)p->x,
+                       (const bf16_t*)p->workspace, (bf16_t*)p->dispatch_w, (bf16_t*)p->combine_w,
+                       (bf16_t*)p->logits, p->scale, scale_x, p->S, p->D, p->N, SP, NP);
+  } else {
+    hipLaunchKernelGGL(soft_prep_mu_kernel<float>, dim3(p->N), dim3(256), 0, stream,
+                       (const float*)p->mu, (float*)p->workspace, p->scale, !scale_x, p->D, p->N);
+    auto kern = soft_route_kernel<float>;
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return (int)e;
+    hipLaunchKernelGGL(kern, dim3(p->G), dim3(256), lds, stream, (const float*)p->x,
+                       (const float*)p->workspace, (float*)p->dispatch_w, (float*)p->combine_w,
+                       (float*)p->logits, p->scale, scale_x, p->S, p->D, p->N, SP, NP);
+  }
+  return launch_status();
+}
+
+extern "C" int vmoe_einsum_dispatch(const VmoeEinsumParams* p, vmoe_stream_t stream) {
+  int rc = check_einsum(p, true);
+  if (rc != VMOE_OK) return rc;
+  const int M = p->E * p->C;
+  dim3 grid((p->D + 63) / 64, (M + 63) / 64, p->G);
+  hipLaunchKernelGGL(einsum_kernel<true>, grid, dim3(256), 0, as_stream(stream), p->w, p->data,
+                     p->out, p->G, p->S, p->E, p->C, p->D, p->w_dtype, p->data_dtype, p->out_dtype);
+  return launch_status();
+}
+
+extern "C" int vmoe_einsum_combine(const VmoeEinsumParams* p, vmoe_stream_t stream) {
+  int rc = check_einsum(p, false);
+  if (rc != VMOE_OK) return rc;
+  dim3 grid((p->D + 63) / 64, (p->S + 63) / 64, p->G);
+  hipLaunchKernelGGL(einsum_kernel<false>, grid, dim3(256), 0, as_stream(stream), p->w, p->data,
+                     p->out, p->G, p->S, p->E, p->C, p->D, p->w_dtype, p->data_dtype, p->out_dtype);
+  return launch_status();
+}

@@ -1,0 +1,82 @@
+// Shared device helpers for the gfx950 kernels of libvmoe_hip.so.
+#ifndef VMOE_COMMON_H_
+#define VMOE_COMMON_H_
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "vmoe_hip.h"
+
+namespace vmoe {
+
+constexpr int kWave = 64;
+
+typedef uint16_t bf16_t;  // bfloat16 storage
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+
+// float32 -> bfloat16, round to nearest even (v_cvt_pk_bf16_f32 on gfx950).
+__device__ __forceinline__ bf16_t f2bf(float f) {
+  __bf16 b = (__bf16)f;
+  return __builtin_bit_cast(bf16_t, b);
+}
+__device__ __forceinline__ float bf2f(bf16_t h) {
+  return __builtin_bit_cast(float, (uint32_t)h << 16);
+}
+// Round a float32 to the nearest bfloat16 value, kept as float32.
+__device__ __forceinline__ float bf16r(float f) { return bf2f(f2bf(f)); }
+
+template <typename T> struct Elt;
+template <> struct Elt<float> {
+  static constexpr int dtype = VMOE_F32;
+  __device__ static __forceinline__ float load(const float* p) { return *p; }
+  __device__ static __forceinline__ void store(float* p, float v) { *p = v; }
+  __device__ static __forceinline__ float round(float v) { return v; }
+};
+template <> struct Elt<bf16_t> {
+  static constexpr int dtype = VMOE_BF16;
+  __device__ static __forceinline__ float load(const bf16_t* p) { return bf2f(*p); }
+  __device__ static __forceinline__ void store(bf16_t* p, float v) { *p = f2bf(v); }
+  __device__ static __forceinline__ float round(float v) { return bf16r(v); }
+};
+
+__device__ __forceinline__ float gelu_tanh(float x) {
+  const float c = 0.7978845608028654f;  // sqrt(2/pi)
+  float inner = c * (x + 0.044715f * (x * x * x));
+  return 0.5f * x * (1.0f + tanhf(inner));
+}
+__device__ __forceinline__ float gelu_erf(float x) {
+  return 0.5f * x * (1.0f + erff(x * 0.7071067811865476f));
+}
+
+// Monotone map float32 -> uint32 (larger float -> larger uint); -0.0 == +0.0.
+__device__ __forceinline__ uint32_t orderable(float f) {
+  uint32_t u = __builtin_bit_cast(uint32_t, f);
+  if (u == 0x80000000u) u = 0u;
+  return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+}
+
+// Slot row of (expert e, group g, position c) in the (E, G*C) expert buffer.
+__device__ __forceinline__ int slot_row(int e, int g, int c, int G, int E, int C) {
+  int r;
+  if (G % E == 0) {
+    int q = G / E;
+    r = ((g % q) * E + g / q) * C + c;
+  } else {
+    r = g * C + c;
+  }
+  return e * (G * C) + r;
+}
+
+inline hipStream_t as_stream(vmoe_stream_t s) { return reinterpret_cast<hipStream_t>(s); }
+
+inline int launch_status() {
+  hipError_t err = hipGetLastError();
+  return err == hipSuccess ? VMOE_OK : (int)err;
+}
+
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+}  // namespace vmoe
+#endif  // VMOE_COMMON_H_

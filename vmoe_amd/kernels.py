@@ -1,0 +1,253 @@
+"""Functional wrappers of the C ABI: allocate outputs with torch, call the HIP kernels.
+
+Each function maps to one entry point of include/vmoe_hip.h.  Tensors must live
+on a ROCm device and are used as raw device pointers on torch's current stream.
+"""
+from __future__ import annotations
+
+from typing import Optional, Tuple
+
+import torch
+
+from vmoe_amd import _hip as H
+
+
+def _i32(*shape, device):
+  return torch.empty(shape, dtype=torch.int32, device=device)
+
+
+def _f32(*shape, device):
+  return torch.empty(shape, dtype=torch.float32, device=device)
+
+
+def gate_topk(x: torch.Tensor, w: torch.Tensor, num_selected_experts: int,
+              logit_bias: Optional[torch.Tensor] = None, return_gates: bool = True):
+  """x (G,S,D), w (D,E) -> gates (G,S,E) or None, topk_val (G,S,K) f32, topk_idx (G,S,K) i32."""
+  G, S, D = x.shape
+  E = w.shape[1]
+  K = num_selected_experts
+  x = x.contiguous()
+  w = w.to(x.dtype).contiguous()
+  gates = torch.empty((G, S, E), dtype=x.dtype, device=x.device) if return_gates else None
+  val = _f32(G, S, K, device=x.device)
+  idx = _i32(G, S, K, device=x.device)
+  if logit_bias is not None:
+    logit_bias = logit_bias.to(torch.float32).contiguous()
+  p = H.GateTopkParams(H.ptr(x), H.ptr(w), H.ptr(logit_bias), H.ptr(gates), H.ptr(val), H.ptr(idx),
+                       G * S, D, E, K, H.dtype_code(x.dtype))
+  H.call("vmoe_gate_topk", p)
+  return gates, val, idx
+
+
+def topk(gates: torch.Tensor, k: int):
+  """gates (..., E) float32 -> values (..., K) f32, indices (..., K) i32; ties -> lower index."""
+  E = gates.shape[-1]
+  g = gates.to(torch.float32).contiguous()
+  n = g.numel() // E
+  val = _f32(*gates.shape[:-1], k, device=g.device)
+  idx = _i32(*gates.shape[:-1], k, device=g.device)
+  H.call("vmoe_topk", H.TopkParams(H.ptr(g), H.ptr(val), H.ptr(idx), n, E, k))
+  return val, idx
+
+
+def router_metrics(gates: torch.Tensor, topk_idx: torch.Tensor, gshard_loss_weight: float,
+                   importance_loss_weight: float):
+  """gates (G,S,E), topk_idx (G,S,K) -> importance_loss, gshard_loss, auxiliary_loss, each (G,) f32."""
+  G, S, E = gates.shape
+  gates = gates.contiguous()
+  topk_idx = topk_idx.contiguous()
+  imp, gsh, aux = (_f32(G, device=gates.device) for _ in range(3))
+  p = H.RouterMetricsParams(H.ptr(gates), H.ptr(topk_idx), H.ptr(imp), H.ptr(gsh), H.ptr(aux),
+                            float(gshard_loss_weight), float(importance_loss_weight), G, S, E,
+                            topk_idx.shape[-1], H.dtype_code(gates.dtype))
+  H.call("vmoe_router_metrics", p)
+  return imp, gsh, aux
+
+
+def route_assign(topk_val: Optional[torch.Tensor], topk_idx: torch.Tensor, num_experts: int,
+                 capacity: int, batch_priority: bool):
+  """topk_idx (G,S,K) -> indices (G,S,K,2), token_slot (G,S,K), slot_token (E*G*C,), fill (G,E)."""
+  G, S, K = topk_idx.shape
+  dev = topk_idx.device
+  topk_idx = topk_idx.contiguous()
+  if topk_val is not None:
+    topk_val = topk_val.to(torch.float32).contiguous()
+  indices = _i32(G, S, K, 2, device=dev)
+  token_slot = _i32(G, S, K, device=dev)
+  slot_token = _i32(num_experts * G * capacity, device=dev)
+  fill = _i32(G, num_experts, device=dev)
+  p = H.RouteAssignParams(H.ptr(topk_val), H.ptr(topk_idx), H.ptr(indices), H.ptr(token_slot),
+                          H.ptr(slot_token), H.ptr(fill), G, S, num_experts, K, capacity,
+                          int(bool(batch_priority)))
+  H.call("vmoe_route_assign", p)
+  return indices, token_slot, slot_token, fill
+
+
+def indices_to_slots(indices: torch.Tensor, num_experts: int, capacity: int):
+  """indices (G,S,K,2) -> token_slot (G,S,K), slot_token (E*G*C,), counters (2,) [dups, invalid]."""
+  G, S, K, _ = indices.shape
+  dev = indices.device
+  indices = indices.to(torch.int32).contiguous()
+  token_slot = _i32(G, S, K, device=dev)
+  slot_token = _i32(num_experts * G * capacity, device=dev)
+  counters = torch.zeros(2, dtype=torch.int32, device=dev)
+  p = H.IndicesToSlotsParams(H.ptr(indices), H.ptr(token_slot), H.ptr(slot_token),
+                             H.c_void_p(counters.data_ptr()), H.c_void_p(counters.data_ptr() + 4),
+                             G, S, num_experts, K, capacity)
+  H.call("vmoe_indices_to_slots", p)
+  return token_slot, slot_token, counters
+
+
+def dispatch(x: torch.Tensor, token_slot: torch.Tensor, slot_token: torch.Tensor,
+             out: Optional[torch.Tensor] = None) -> torch.Tensor:
+  """x (T,D), token_slot (T,K), slot_token (NS,) -> (NS, D)."""
+  T, D = x.shape
+  K = token_slot.shape[-1]
+  NS = slot_token.numel()
+  x = x.contiguous()
+  if out is None:
+    out = torch.empty((NS, D), dtype=x.dtype, device=x.device)
+  p = H.DispatchParams(H.ptr(x), H.ptr(token_slot), H.ptr(slot_token), H.ptr(out), T, NS, K, D,
+                       H.dtype_code(x.dtype))
+  H.call("vmoe_dispatch", p)
+  return out
+
+
+def combine(y: torch.Tensor, token_slot: torch.Tensor, weights: torch.Tensor,
+            out: Optional[torch.Tensor] = None) -> torch.Tensor:
+  """y (NS,D), token_slot (T,K), weights (T,K) f32 -> (T, D)."""
+  NS, D = y.shape
+  T, K = token_slot.shape
+  y = y.contiguous()
+  weights = weights.to(torch.float32).contiguous()
+  if out is None:
+    out = torch.empty((T, D), dtype=y.dtype, device=y.device)
+  p = H.CombineParams(H.ptr(y), H.ptr(token_slot), H.ptr(weights), H.ptr(out), T, NS, K, D,
+                      H.dtype_code(y.dtype))
+  H.call("vmoe_combine", p)
+  return out
+
+
+def densify(indices: torch.Tensor, weights: torch.Tensor, num_experts: int, capacity: int):
+  """indices (G,S,K,2), weights (G,S,K) -> combine (G,S,E,C) f32, dispatch (G,S,E,C) bool."""
+  G, S, K, _ = indices.shape
+  dev = indices.device
+  cw = torch.zeros((G, S, num_experts, capacity), dtype=torch.float32, device=dev)
+  dw = torch.zeros((G, S, num_experts, capacity), dtype=torch.uint8, device=dev)
+  weights = weights.to(torch.float32).contiguous()
+  p = H.DensifyParams(H.ptr(indices.contiguous()), H.ptr(weights), H.ptr(cw), H.ptr(dw), G, S,
+                      num_experts, K, capacity)
+  H.call("vmoe_densify", p)
+  return cw, dw.view(torch.bool)
+
+
+def pack_expert_weights(w: torch.Tensor) -> torch.Tensor:
+  """(E, rows, cols) -> (E, cols, rows), contiguous."""
+  E, rows, cols = w.shape
+  w = w.contiguous()
+  out = torch.empty((E, cols, rows), dtype=w.dtype, device=w.device)
+  p = H.TransposeParams(H.ptr(w), H.ptr(out), E, rows, cols, H.dtype_code(w.dtype))
+  H.call("vmoe_pack_expert_weights", p)
+  return out
+
+
+def expert_mlp(x: torch.Tensor, w0, b0, w1, b1, w0t=None, w1t=None, approximate_gelu: bool = True,
+               workspace: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None):
+  """x (E,R,D) -> (E,R,D): gelu(x @ w0 + b0) @ w1 + b1 per expert."""
+  E, R, D = x.shape
+  M = (w0.shape[2] if w0 is not None else w0t.shape[1])
+  x = x.contiguous()
+  if out is None:
+    out = torch.empty_like(x)
+  p = H.ExpertMlpParams(H.ptr(x), H.ptr(w0), H.ptr(b0), H.ptr(w1), H.ptr(b1), H.ptr(w0t),
+                        H.ptr(w1t), H.ptr(out), None, 0, E, R, D, M, H.dtype_code(x.dtype),
+                        H.GELU_TANH if approximate_gelu else H.GELU_ERF)
+  need = H.lib().vmoe_expert_mlp_workspace_bytes(H.ctypes.byref(p))
+  if workspace is None or workspace.numel() * workspace.element_size() < need:
+    workspace = torch.empty(need, dtype=torch.uint8, device=x.device)
+  p.workspace = H.ptr(workspace)
+  p.workspace_bytes = workspace.numel() * workspace.element_size()
+  H.call("vmoe_expert_mlp", p)
+  return out
+
+
+def expert_mlp_workspace_bytes(E, R, D, M, dtype, prepacked: bool) -> int:
+  one = H.c_void_p(16)
+  p = H.ExpertMlpParams(one, one, None, one, None, one if prepacked else None,
+                        one if prepacked else None, one, None, 0, E, R, D, M,
+                        H.dtype_code(dtype), 0)
+  return int(H.lib().vmoe_expert_mlp_workspace_bytes(H.ctypes.byref(p)))
+
+
+def soft_route(x: torch.Tensor, mu: torch.Tensor, scale: float, return_logits: bool = False):
+  """x (G,S,D), mu (D,N) -> dispatch_w (G,S,N), combine_w (G,S,N) [, logits]."""
+  G, S, D = x.shape
+  N = mu.shape[1]
+  x = x.contiguous()
+  mu = mu.to(x.dtype).contiguous()
+  dw = torch.empty((G, S, N), dtype=x.dtype, device=x.device)
+  cw = torch.empty_like(dw)
+  logits = torch.empty_like(dw) if return_logits else None
+  p = H.SoftRouteParams(H.ptr(x), H.ptr(mu), float(scale), H.ptr(dw), H.ptr(cw), H.ptr(logits),
+                        None, 0, G, S, D, N, H.dtype_code(x.dtype))
+  need = H.lib().vmoe_soft_route_workspace_bytes(H.ctypes.byref(p))
+  ws = torch.empty(max(need, 16), dtype=torch.uint8, device=x.device)
+  p.workspace = H.ptr(ws)
+  p.workspace_bytes = ws.numel()
+  H.call("vmoe_soft_route", p)
+  return (dw, cw, logits) if return_logits else (dw, cw)
+
+
+def _w_code(w: torch.Tensor) -> int:
+  if w.dtype == torch.float32:
+    return H.W_F32
+  if w.dtype == torch.bfloat16:
+    return H.W_BF16
+  if w.dtype == torch.bool:
+    return H.W_BOOL
+  raise TypeError(f"Unsupported weight dtype {w.dtype}")
+
+
+def einsum_dispatch(w: torch.Tensor, data: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
+  """w (G,S,E,C), data (G,S,D) -> (E*G*C, D) in the expert buffer's row order."""
+  G, S, E, C = w.shape
+  D = data.shape[-1]
+  w = w.contiguous()
+  data = data.contiguous()
+  out = torch.empty((E * G * C, D), dtype=out_dtype, device=data.device)
+  wv = w.view(torch.uint8) if w.dtype == torch.bool else w
+  p = H.EinsumParams(H.ptr(wv), H.ptr(data), H.ptr(out), G, S, E, C, D, _w_code(w),
+                     H.dtype_code(data.dtype), H.dtype_code(out_dtype))
+  H.call("vmoe_einsum_dispatch", p)
+  return out
+
+
+def einsum_combine(w: torch.Tensor, data: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
+  """w (G,S,E,C), data (E*G*C, D) -> (G,S,D)."""
+  G, S, E, C = w.shape
+  D = data.shape[-1]
+  w = w.contiguous()
+  data = data.contiguous()
+  out = torch.empty((G, S, D), dtype=out_dtype, device=data.device)
+  p = H.EinsumParams(H.ptr(w), H.ptr(data), H.ptr(out), G, S, E, C, D, _w_code(w),
+                     H.dtype_code(data.dtype), H.dtype_code(out_dtype))
+  H.call("vmoe_einsum_combine", p)
+  return out
+
+
+def cast(x: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
+  """float32 <-> bfloat16 with the library's conversion kernel."""
+  if x.dtype == dtype:
+    return x
+  x = x.contiguous()
+  out = torch.empty(x.shape, dtype=dtype, device=x.device)
+  if x.numel():
+    p = H.CastParams(H.ptr(x), H.ptr(out), x.numel(), H.dtype_code(x.dtype), H.dtype_code(dtype))
+    H.call("vmoe_cast", p)
+  return out
+
+
+def copy_bytes(src: torch.Tensor, dst: torch.Tensor) -> None:
+  n = src.numel() * src.element_size()
+  H.check(H.lib().vmoe_copy_bytes(H.ptr(src), H.ptr(dst), H.c_size_t(n), H.stream()),
+          "vmoe_copy_bytes")
