@@ -1,0 +1,227 @@
+"""Benchmark of the MoE layer on one MI355X.
+
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--config NAME] [--no-cpu-baseline]
+
+A step is one pass of the whole layer (gating + top-k, losses, slot assignment
+with batch priority routing, dispatch, expert MLPs, combine) over one batch of
+synthetic tokens already resident in HBM.  Prints ONE JSON line.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+  sys.path.insert(0, ROOT)
+
+# Published MI355X peaks used as roofline denominators.
+PEAK_BF16_TFLOPS = 2500.0
+PEAK_FP32_MATRIX_TFLOPS = 157.3
+PEAK_HBM_GBS = 8000.0
+
+# HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc runs
+# (FETCH_SIZE + WRITE_SIZE, scaled by a copy kernel of known size); None until measured.
+MEASURED_TRAFFIC_BYTES = {}
+
+
+def parse_args():
+  ap = argparse.ArgumentParser()
+  ap.add_argument("--gpus", type=int, default=1)
+  ap.add_argument("--steps", type=int, default=20)
+  ap.add_argument("--warmup", type=int, default=5)
+  ap.add_argument("--config", default="vmoe_b16_layer_E32_k2_bpr")
+  ap.add_argument("--no-cpu-baseline", action="store_true")
+  ap.add_argument("--cpu-groups", type=int, default=2,
+                  help="groups of the workload the CPU baseline is timed on")
+  return ap.parse_args()
+
+
+def device_weights(cfg, torch, dev, seed):
+  """Seeded LeCun-normal expert kernels drawn on the device (fast), biases 0."""
+  gen = torch.Generator(device=dev)
+  gen.manual_seed(seed)
+  D, M, E = cfg.d_model, cfg.mlp_dim, cfg.num_experts
+  tdt = torch.bfloat16 if cfg.dtype == "bfloat16" else torch.float32
+  w0 = (torch.randn((E, D, M), generator=gen, device=dev) / D ** 0.5).to(tdt)
+  w1 = (torch.randn((E, M, D), generator=gen, device=dev) / M ** 0.5).to(tdt)
+  return w0, w1, torch.zeros((E, M), dtype=tdt, device=dev), torch.zeros((E, D), dtype=tdt, device=dev)
+
+
+def cpu_baseline(cfg, x_np, params_np, bias_np, groups):
+  """Times the CPU oracle (NumPy/torch-CPU restatement of the reference path) on
+  the first `groups` groups of the same workload."""
+  from oracle import moe_oracle as O
+  S = cfg.group_size
+  imgs = groups * cfg.group_images
+  xs = x_np[:imgs]
+  dtype = O.BF16 if cfg.dtype == "bfloat16" else O.F32
+  def run():
+    return O.mlp_moe_block(xs, params_np, group_size=S,
+                           num_selected_experts=cfg.num_selected_experts,
+                           dispatcher_kwargs=cfg.dispatcher_kwargs("indices"), dtype=dtype,
+                           logit_bias=bias_np)
+  run()
+  times = []
+  for _ in range(3):
+    t0 = time.perf_counter()
+    run()
+    times.append(time.perf_counter() - t0)
+  t = float(np.median(times))
+  import torch
+  return {
+      "value": groups * S / t, "unit": "tokens/s", "cores": int(torch.get_num_threads()),
+      "kind": "port",
+      "sample": (f"oracle/moe_oracle.py mlp_moe_block (indices dispatcher) on {groups} of "
+                 f"{cfg.num_groups} groups ({groups * S} tokens, all {cfg.num_experts} experts), "
+                 f"median of 3 runs of {t:.2f} s; NumPy BLAS + torch CPU threads"),
+      "host_cpus": os.cpu_count(),
+  }
+
+
+def main():
+  args = parse_args()
+  if args.gpus != 1:
+    print("bench.py: this build runs on ONE GPU (all experts resident, no collectives); "
+          f"--gpus {args.gpus} is not supported.", file=sys.stderr)
+    sys.exit(2)
+  import torch
+  from vmoe_amd import _hip, configs, kernels
+  from vmoe_amd.nn import vit_moe
+
+  cfg = configs.CONFIGS[args.config]
+  dev = torch.device("cuda:0")
+  torch.cuda.set_device(dev)
+  tdt = torch.bfloat16 if cfg.dtype == "bfloat16" else torch.float32
+  D, M, E, K = cfg.d_model, cfg.mlp_dim, cfg.num_experts, cfg.num_selected_experts
+  T, S, G = cfg.num_tokens, cfg.group_size, cfg.num_groups
+
+  # Inputs: tokens and router on the host generator, expert weights on the device one.
+  rng = np.random.Generator(np.random.PCG64(0))
+  n_rot = 4
+  xs_np = []
+  for _ in range(n_rot):
+    x = rng.standard_normal((cfg.num_images, cfg.tokens_per_image, D), dtype=np.float32)
+    if cfg.layer_norm_inputs:
+      x = ((x - x.mean(-1, keepdims=True)) / np.sqrt(x.var(-1, keepdims=True) + 1e-6)).astype(np.float32)
+    xs_np.append(x)
+  router_np = (rng.standard_normal((D, E), dtype=np.float32) / np.sqrt(D)).astype(np.float32)
+  bias_np = None
+  if cfg.logit_bias_std:
+    bias_np = (rng.standard_normal(E, dtype=np.float32) * cfg.logit_bias_std).astype(np.float32)
+  w0, w1, b0, b1 = device_weights(cfg, torch, dev, seed=1)
+  xs = [torch.from_numpy(x).to(dev).to(tdt) for x in xs_np]
+  variables = {"params": {
+      "Router": {"dense": {"kernel": torch.from_numpy(router_np).to(dev)}},
+      "Mlp": {"Dense_0": {"kernel": w0, "bias": b0}, "Dense_1": {"kernel": w1, "bias": b1}}}}
+  router_kwargs = dict(num_selected_experts=K, dispatcher=cfg.dispatcher_kwargs("indices"))
+  if bias_np is not None:
+    router_kwargs["logit_bias"] = torch.from_numpy(bias_np).to(dev)
+  layer = vit_moe.MlpMoeBlock(mlp_dim=M, num_experts=E, group_size=S, deterministic=True,
+                              router=router_kwargs, dtype=tdt)
+
+  def step(i):
+    return layer.apply(variables, xs[i % n_rot])
+
+  for i in range(args.warmup):
+    out, metrics = step(i)
+  torch.cuda.synchronize()
+
+  sink = {}
+  _hip.set_timing_sink(sink)
+  torch.cuda.synchronize()
+  t0 = time.perf_counter()
+  for i in range(args.steps):
+    out, metrics = step(i)
+  torch.cuda.synchronize()
+  t1 = time.perf_counter()
+  _hip.set_timing_sink(None)
+  ms_per_step = (t1 - t0) * 1e3 / args.steps
+  tokens_per_s = T / (ms_per_step * 1e-3)
+
+  stage_ms = {name: float(np.mean([a.elapsed_time(b) for a, b in pairs])) * (len(pairs) / args.steps)
+              for name, pairs in sink.items()}
+
+  # Kept assignments (rows that carry an item) for the algorithmic flop count.
+  gates, val, idx = kernels.gate_topk(xs[0].view(G, S, D), variables["params"]["Router"]["dense"]["kernel"].to(tdt), K,
+                                      logit_bias=router_kwargs.get("logit_bias"))
+  C = cfg_capacity(cfg)
+  _, token_slot, _, fill = kernels.route_assign(val, idx, E, C, cfg.batch_priority)
+  kept = int(fill.sum())
+  b = 2 if tdt == torch.bfloat16 else 4
+  # Dominant kernel: the expert GEMM (two launches per step, 2*A*D*M flops each).
+  mlp_ms = stage_ms["vmoe_expert_mlp"]
+  gemm_ms = mlp_ms / 2.0
+  flops_per_launch = 2.0 * kept * D * M
+  achieved_tflops = flops_per_launch / (gemm_ms * 1e-3) / 1e12
+  peak = PEAK_BF16_TFLOPS if tdt == torch.bfloat16 else PEAK_FP32_MATRIX_TFLOPS
+  roofline = {"bound": "mfma", "kernel": "gemm_bf16_kernel" if b == 2 else "gemm_f32_kernel",
+              "achieved": achieved_tflops, "peak": peak, "unit": "TFLOP/s",
+              "frac": achieved_tflops / peak, "traffic": MEASURED_TRAFFIC_BYTES.get(cfg.name),
+              "launch_ms": gemm_ms, "flops_per_launch": flops_per_launch, "kept_rows": kept,
+              "buffer_rows": E * G * C}
+
+  # HBM-bound stages, algorithmic bytes (each item row read once, whole buffer written).
+  bytes_dispatch = T * D * b + E * G * C * D * b + 8 * T * K
+  bytes_combine = kept * D * b + 12 * T * K + T * D * b
+  bytes_gate = T * D * b + D * E * b + 12 * T * K + T * E * b
+  # Measured copy ceiling of the same device (read + write of 512 MiB).
+  n = 512 << 20
+  src = torch.empty(n, dtype=torch.uint8, device=dev)
+  dst = torch.empty_like(src)
+  for _ in range(2):
+    kernels.copy_bytes(src, dst)
+  e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+  e0.record()
+  for _ in range(5):
+    kernels.copy_bytes(src, dst)
+  e1.record()
+  torch.cuda.synchronize()
+  copy_gbs = 2 * n * 5 / (e0.elapsed_time(e1) * 1e-3) / 1e9
+  del src, dst
+  hbm = {
+      "dispatch_GBps": bytes_dispatch / (stage_ms["vmoe_dispatch"] * 1e-3) / 1e9,
+      "combine_GBps": bytes_combine / (stage_ms["vmoe_combine"] * 1e-3) / 1e9,
+      "gate_topk_GBps": bytes_gate / (stage_ms["vmoe_gate_topk"] * 1e-3) / 1e9,
+      "copy_kernel_GBps": copy_gbs, "peak_GBps": PEAK_HBM_GBS,
+  }
+  hbm["dispatch_frac_of_peak"] = hbm["dispatch_GBps"] / PEAK_HBM_GBS
+  hbm["combine_frac_of_peak"] = hbm["combine_GBps"] / PEAK_HBM_GBS
+
+  result = {
+      "metric": "MoE-layer tokens/sec at B/16 E=32 k=2 bf16; dispatch/combine HBM GB/s",
+      "value": tokens_per_s, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
+      "warmup": args.warmup, "ms_per_step": ms_per_step, "higher_is_better": True,
+      "scaling": "weak", "vs_baseline": None, "dtype": "bf16" if b == 2 else "f32",
+      "data": "synthetic (seeded N(0,1) tokens, LayerNorm-ed; LeCun-normal experts; random-init router)",
+      "config": {"workload": cfg.name, "tokens": T, "d_model": D, "mlp_dim": M, "experts": E,
+                 "selected": K, "groups": G, "group_size": S, "capacity": C,
+                 "batch_priority": cfg.batch_priority, "capacity_factor": cfg.capacity_factor},
+      "roofline": roofline,
+      "stage_ms": stage_ms,
+      "hbm": hbm,
+  }
+  if not args.no_cpu_baseline:
+    params_np = {
+        "Router": {"dense": {"kernel": router_np}},
+        "Mlp": {"Dense_0": {"kernel": w0.float().cpu().numpy(), "bias": b0.float().cpu().numpy()},
+                "Dense_1": {"kernel": w1.float().cpu().numpy(), "bias": b1.float().cpu().numpy()}}}
+    result["cpu_baseline"] = cpu_baseline(cfg, xs_np[0], params_np, bias_np, min(args.cpu_groups, G))
+  else:
+    result["cpu_baseline"] = None
+  print(json.dumps(result))
+
+
+def cfg_capacity(cfg):
+  from vmoe_amd import moe
+  return moe.compute_capacity(cfg.group_size * cfg.num_selected_experts, cfg.num_experts,
+                              cfg.capacity_factor)
+
+
+if __name__ == "__main__":
+  main()

@@ -44,8 +44,19 @@ BF16 = "bfloat16"
 
 # --------------------------------------------------------------------------- dtypes
 def bf16_round(x) -> np.ndarray:
-  """Rounds float32 values to the nearest bfloat16 (ties to even), kept as float32."""
+  """Rounds float32 values to the nearest bfloat16 (ties to even), kept as float32.
+
+  Large arrays go through torch's CPU conversion, which is the same rounding
+  (tests/test_oracle_golden.py::test_bf16_round_vs_torch) on all cores.
+  """
   x = np.ascontiguousarray(x, dtype=np.float32)
+  if x.size >= (1 << 20):
+    import torch
+    return torch.from_numpy(x).to(torch.bfloat16).to(torch.float32).numpy()
+  return _bf16_round_numpy(x)
+
+
+def _bf16_round_numpy(x: np.ndarray) -> np.ndarray:
   u = x.view(np.uint32)
   bias = ((u >> np.uint32(16)) & np.uint32(1)) + np.uint32(0x7FFF)
   r = ((u + bias) & np.uint32(0xFFFF0000)).view(np.float32)

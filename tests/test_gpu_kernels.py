@@ -302,4 +302,74 @@ def test_bad_arguments_return_error_codes(K):
     K.gate_topk(x.double(), w.double(), 2)
   idx = torch.zeros((1, 4, 2), dtype=torch.int32, device=dev())
   with pytest.raises(H.VmoeError, match="invalid sizes"):
-    K.route_assign(None, idx, 4, 0, False)                           # C < 1
+    K.route_assign(None, idx, 1, 4, False)                           # K > E
+  with pytest.raises(H.VmoeError, match="null"):
+    K.route_assign(None, idx, 4, 4, True)                            # BPR needs the gates
+
+
+# ------------------------------------------------------------------ Soft MoE
+SOFT_CASES = [
+    # G, S, D, n, p, dtype
+    (1, 8, 16, 5, 2, O.F32),
+    (3, 50, 64, 7, 3, O.F32),
+    (2, 196, 768, 128, 1, O.BF16),
+    (4, 100, 256, 16, 2, O.BF16),
+    (1, 2, 16, 4, 2, O.F32),          # inputs smaller than mu: the scale multiplies the inputs
+]
+
+
+@pytest.mark.parametrize("G,S,D,n,p,dtype", SOFT_CASES)
+def test_soft_route(K, G, S, D, n, p, dtype):
+  rng = np.random.default_rng(S + n)
+  x = O.cast(rng.standard_normal((G, S, D)), dtype)
+  mu = O.cast(rng.standard_normal((D, n, p)) / np.sqrt(D), dtype)
+  scale = 1.75
+  dw, cw, lg = K.soft_route(to_dev(x, dtype), to_dev(mu.reshape(D, n * p), dtype), scale,
+                            return_logits=True)
+  wl, wd, wc, _ = O.soft_router_weights(x, mu, scale, dtype)
+  tol = 1e-5 if dtype == O.F32 else 2e-2
+  assert_close(to_np(lg), wl.reshape(G, S, n * p), tol * (1 if dtype == O.BF16 else 4), "logits")
+  assert_close(to_np(dw), wd.reshape(G, S, n * p), tol * 4, "dispatch weights")
+  assert_close(to_np(cw), wc.reshape(G, S, n * p), tol * 4, "combine weights")
+  atol = 1e-4 if dtype == O.F32 else 3e-2
+  np.testing.assert_allclose(to_np(dw).sum(1), 1.0, atol=atol)
+  np.testing.assert_allclose(to_np(cw).sum(2), 1.0, atol=atol)
+
+
+EINSUM_CASES = [
+    # G, S, E, C, D, wdtype, ddtype
+    (2, 3, 2, 2, 4, O.F32, O.F32),
+    (2, 3, 4, 1, 4, O.F32, O.F32),
+    (4, 50, 2, 3, 40, O.F32, O.BF16),     # Bfloat16Dispatcher over float32 weights
+    (8, 196, 4, 2, 96, O.BF16, O.BF16),
+    (3, 33, 5, 1, 20, O.F32, O.F32),
+]
+
+
+@pytest.mark.parametrize("G,S,E,C,D,wdtype,ddtype", EINSUM_CASES)
+def test_einsum_dispatch_combine(K, G, S, E, C, D, wdtype, ddtype):
+  rng = np.random.default_rng(G + S)
+  w = O.cast(O.softmax(rng.standard_normal((G, S, E * C)).astype(np.float32)), wdtype)
+  w = w.reshape(G, S, E, C)
+  x = O.cast(rng.standard_normal((G, S, D)), ddtype)
+  d = O.EinsumDispatcher(w, w)
+  out_dtype = wdtype if wdtype == ddtype else O.F32
+  buf = K.einsum_dispatch(to_dev(w, wdtype), to_dev(x, ddtype), tdtype(out_dtype))
+  want = O.cast(d.dispatch(x), out_dtype)
+  tol = 1e-5 if out_dtype == O.F32 else 2e-2
+  assert_close(to_np(buf).reshape(E, G * C, D), want, tol, "einsum dispatch")
+  y = O.cast(rng.standard_normal((E, G * C, D)), ddtype)
+  out = K.einsum_combine(to_dev(w, wdtype), to_dev(y, ddtype).view(E * G * C, D), tdtype(out_dtype))
+  assert_close(to_np(out), O.cast(d.combine(y), out_dtype), tol, "einsum combine")
+
+
+def test_einsum_golden_and_bool_weights(K, goldens):
+  data = np.asarray(goldens["dispatcher_data"]["data"], np.float32)
+  for case in ("dispatcher_experts_divide_groups", "dispatcher_groups_divide_experts"):
+    g = goldens[case]
+    cw = np.asarray(g["einsum_combine_weights"], np.float32)
+    E, C = g["num_experts"], g["capacity"]
+    buf = K.einsum_dispatch(to_dev(cw > 0), to_dev(data), torch.float32)
+    np.testing.assert_array_almost_equal(to_np(buf).reshape(E, 2 * C, 4), np.asarray(g["expected_dispatch"]))
+    out = K.einsum_combine(to_dev(cw), buf, torch.float32)
+    np.testing.assert_array_almost_equal(to_np(out), np.asarray(g["expected_combine"]))

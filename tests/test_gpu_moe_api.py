@@ -1,0 +1,386 @@
+"""The reference's own unit tests for the path, restated against the drop-in
+Python surface (vmoe_amd.moe / nn.routing / nn.vit_moe / projects.soft_moe.router),
+plus end-to-end parity of the whole layer against the CPU oracle.
+
+Mirrors vmoe/moe_test.py, vmoe/nn/routing_test.py and
+vmoe/projects/soft_moe/router_test.py case by case.
+"""
+import numpy as np
+import pytest
+import torch
+
+from oracle import moe_oracle as O
+from tests.util import assert_close, dev, tdtype, to_dev, to_np
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def moe():
+  from vmoe_amd import moe
+  return moe
+
+
+# ------------------------------------------------------------------ DispatcherTest
+def test_compute_capacity_raises_wrong_input_values(moe):
+  with pytest.raises(ValueError, match="The values .* lead to capacity .*, but it must be greater "
+                     "than or equal to 1"):
+    moe.compute_capacity(128, 32, -1.0)
+
+
+def test_bfloat16_dispatcher(moe):
+  seen = []
+
+  class Inner(moe.BaseDispatcher):
+    def dispatch(self, x):
+      seen.append(x.dtype)
+      return x
+    combine = dispatch
+
+  d = moe.Bfloat16Dispatcher(dispatcher=Inner())
+  x = torch.zeros((5, 4, 3), dtype=torch.float32, device=dev())
+  assert d.dispatch(x).dtype == torch.float32
+  assert d.combine(x).dtype == torch.float32
+  assert seen == [torch.bfloat16, torch.bfloat16]
+
+
+def _run_dispatcher_test(goldens, dispatcher, case):
+  data = to_dev(np.asarray(goldens["dispatcher_data"]["data"], np.float32))
+  out = dispatcher.dispatch(data)
+  np.testing.assert_array_almost_equal(to_np(out), np.asarray(goldens[case]["expected_dispatch"]))
+  comb = dispatcher.combine(out)
+  np.testing.assert_array_almost_equal(to_np(comb), np.asarray(goldens[case]["expected_combine"]))
+
+
+@pytest.mark.parametrize("case", ["dispatcher_experts_divide_groups",
+                                  "dispatcher_groups_divide_experts"])
+def test_einsum(moe, goldens, case):
+  cw = to_dev(np.asarray(goldens[case]["einsum_combine_weights"], np.float32))
+  _run_dispatcher_test(goldens, moe.EinsumDispatcher(combine_weights=cw), case)
+
+
+@pytest.mark.parametrize("case", ["dispatcher_experts_divide_groups",
+                                  "dispatcher_groups_divide_experts"])
+def test_indices(moe, goldens, case):
+  g = goldens[case]
+  idx = to_dev(np.asarray(g["indices"], np.int32))
+  cw = to_dev(np.tile(np.asarray([[[0.7, 0.3]]], np.float32), (2, 3, 1)))
+  d = moe.ExpertIndicesDispatcher(indices=idx, combine_weights=cw, num_experts=g["num_experts"],
+                                  capacity=g["capacity"])
+  _run_dispatcher_test(goldens, d, case)
+
+
+def test_indices_duplicate_slots_raise(moe):
+  idx = to_dev(np.asarray([[[[0, 0]], [[0, 0]]]], np.int32))
+  cw = torch.ones((1, 2, 1), device=dev())
+  d = moe.ExpertIndicesDispatcher(indices=idx, combine_weights=cw, num_experts=2, capacity=2)
+  with pytest.raises(ValueError, match="same"):
+    d.dispatch(torch.ones((1, 2, 4), device=dev()))
+
+
+# ------------------------------------------------------------------ GetTopExpertsPerItemDispatcherTest
+@pytest.mark.parametrize("bpr", [False, True])
+def test_top_experts_per_item_einsum(moe, goldens, bpr):
+  g = goldens["top_experts_per_item"]
+  gates = to_dev(np.asarray(g["gates"], np.float32))
+  d = moe._get_top_experts_per_item_einsum_dispatcher(
+      gates, num_selected_experts=2, capacity=2, batch_priority=bpr)
+  want = np.asarray(g["einsum_combine_weights"]["bpr" if bpr else "vanilla"])
+  np.testing.assert_array_almost_equal(to_np(d.combine_weights), want)
+
+
+@pytest.mark.parametrize("bpr", [False, True])
+def test_top_experts_per_item_expert_indices(moe, goldens, bpr):
+  g = goldens["top_experts_per_item"]
+  gates = to_dev(np.asarray(g["gates"], np.float32))
+  d = moe._get_top_experts_per_item_expert_indices_dispatcher(
+      gates, num_selected_experts=2, capacity=2, batch_priority=bpr)
+  assert d.num_experts == 3 and d.capacity == 2
+  np.testing.assert_array_equal(to_np(d.indices), np.asarray(g["indices"]["bpr" if bpr else "vanilla"]))
+  np.testing.assert_array_almost_equal(to_np(d.combine_weights), np.asarray(g["indices_combine_weights"]))
+
+
+@pytest.mark.parametrize("name,cls", [("einsum", "EinsumDispatcher"),
+                                      ("indices", "ExpertIndicesDispatcher")])
+def test_get_top_experts_per_item_dispatcher(moe, name, cls):
+  gates = torch.zeros((4, 32), device=dev())
+  d = moe.get_top_experts_per_item_dispatcher(gates, name, num_selected_experts=2, capacity=2,
+                                              batch_priority=False)
+  assert isinstance(d, getattr(moe, cls))
+
+
+@pytest.mark.parametrize("name", ["einsum", "indices"])
+def test_get_top_experts_per_item_dispatcher_capacity_factor(moe, name):
+  gates = torch.zeros((32, 32), device=dev())
+  d = moe.get_top_experts_per_item_dispatcher(gates, name, num_selected_experts=2, capacity=None,
+                                              capacity_factor=1.0, batch_priority=False)
+  inner = d._d if hasattr(d, "_d") else d
+  inner = getattr(inner, "_inner", inner)
+  assert inner.capacity == 4   # increase_to_multiple_of_4(ceil(32 * 2 / 32))
+
+
+def test_get_top_experts_per_item_dispatcher_unknown(moe):
+  gates = torch.zeros((4, 32), device=dev())
+  with pytest.raises(ValueError, match="Unknown dispatcher type"):
+    moe.get_top_experts_per_item_dispatcher(gates, name="foo", num_selected_experts=2, capacity=2,
+                                            batch_priority=False)
+
+
+def test_get_top_experts_per_item_dispatcher_missing_capacity(moe):
+  gates = torch.zeros((4, 32), device=dev())
+  with pytest.raises(ValueError, match="You must specify either 'capacity' or 'capacity_factor'"):
+    moe.get_top_experts_per_item_dispatcher(gates, name="foo", num_selected_experts=2,
+                                            capacity=None, capacity_factor=None,
+                                            batch_priority=False)
+
+
+def test_top_items_per_expert_argument_errors(moe):
+  gates = torch.zeros((4, 32), device=dev())
+  with pytest.raises(ValueError, match="Unknown dispatcher type"):
+    moe.get_top_items_per_expert_dispatcher(gates, name="foo", capacity=2)
+  with pytest.raises(ValueError, match="You must specify either 'capacity' or 'capacity_factor'"):
+    moe.get_top_items_per_expert_dispatcher(gates, name="foo", capacity=None, capacity_factor=None)
+
+
+# ------------------------------------------------------------------ SparseMoeSpmdLayerTest
+class DummyExpert:
+  """Expert with a single scalar parameter that is added to the input (moe_test.py:331-337)."""
+
+  def init(self, rng, x):
+    g = torch.Generator().manual_seed(int(rng))
+    return {"params": {"p": (torch.randn((), generator=g) * 0.01).to(x.device)}}
+
+  def apply(self, variables, x):
+    return x + variables["params"]["p"]
+
+
+def _generate_dispatchers(moe, batch_size, group_size, num_experts, capacity):
+  """moe_test.py:362-417 restated: item i -> experts (2i)%E and (2i+1)%E, weights .7/.3."""
+  G = batch_size // group_size
+  e = (np.arange(2 * batch_size) % num_experts).reshape(G, group_size, 2)
+  pos = np.stack([O.route_greedy(e[g], None, num_experts) for g in range(G)])
+  idx = np.stack([e, pos], -1).astype(np.int32)
+  w = np.tile(np.asarray([0.7, 0.3], np.float32)[None, None], (G, group_size, 1))
+  ind = moe.ExpertIndicesDispatcher(to_dev(idx), to_dev(w), num_experts, capacity)
+  cw = np.zeros((G, group_size, num_experts, capacity), np.float32)
+  for g in range(G):
+    for s in range(group_size):
+      for k in range(2):
+        if pos[g, s, k] < capacity:
+          cw[g, s, e[g, s, k], pos[g, s, k]] = w[g, s, k]
+  return {"indices": ind, "einsum": moe.EinsumDispatcher(combine_weights=to_dev(cw))}
+
+
+@pytest.mark.parametrize("kind", ["einsum", "indices"])
+@pytest.mark.parametrize("split", [False, True])
+def test_initialize_split_rngs(moe, kind, split):
+  layer = moe.sparse_moe_spmd(DummyExpert, variable_axes={"params": 0},
+                              split_rngs={"params": split})()
+  x = (10 * torch.arange(1, 33, dtype=torch.float32, device=dev())).reshape(4, 8, 1)
+  d = _generate_dispatchers(moe, 32, 8, 4, 2)[kind]
+  variables = layer.init(0, d, x)
+  p = variables["params"]["p"]
+  assert tuple(p.shape) == (4,)
+  assert len(set(to_np(p).tolist())) == (4 if split else 1)
+
+
+@pytest.mark.parametrize("kind", ["einsum", "indices"])
+def test_apply(moe, goldens, kind):
+  c = goldens["sparse_moe_apply"]
+  B, S, C, E = c["batch_size"], c["group_size"], c["capacity"], c["num_experts"]
+  layer = moe.sparse_moe_spmd(DummyExpert, variable_axes={"params": 0},
+                              split_rngs={"params": False})()
+  x = (10 * torch.arange(1, 1 + B, dtype=torch.float32, device=dev())).reshape(B // S, S, 1)
+  variables = {"params": {"p": 1 + torch.arange(E, dtype=torch.float32, device=dev())}}
+  out = layer.apply(variables, _generate_dispatchers(moe, B, S, E, C)[kind], x)
+  b = ((1 + np.arange(2 * B) % E).reshape(B, 2) * np.asarray([[0.7, 0.3]])).sum(axis=1)
+  expected = (10 * (1 + np.arange(B)) + b).reshape(-1, S, 1)
+  np.testing.assert_array_almost_equal(to_np(out), expected, decimal=4)
+
+
+@pytest.mark.parametrize("G", [1, 2, 4, 8])
+def test_sparse_moe_spmd_with_axes(moe, goldens, G):
+  c = goldens["sparse_moe_with_axes"]
+  S, E, C = c["S"], c["E"], c["C"]
+  layer = moe.sparse_moe_spmd_with_axes(DummyExpert, variable_axes={"params": 0},
+                                        split_rngs={"params": True},
+                                        partitioning_axis_names={"params": "expert"})(name="moe")
+  x = to_dev(np.tile(np.arange(S, dtype=np.float32).reshape(1, S, 1), (G, 1, 1)))
+  w = to_dev(np.tile(np.arange(S).reshape(1, S, 1, 1) == np.arange(S).reshape(1, 1, E, C),
+                     (G, 1, 1, 1)).astype(np.float32))
+  variables = {"params": {"p": to_dev(np.asarray([1, 2, 3, 4], np.float32).reshape(4, 1))}}
+  out = layer.apply(variables, moe.EinsumDispatcher(combine_weights=w), x)
+  expected = np.tile((np.arange(S) + (np.arange(S) // 4 + 1)).reshape(1, S, 1), (G, 1, 1))
+  np.testing.assert_array_almost_equal(to_np(out), expected, decimal=5)
+
+
+# ------------------------------------------------------------------ routing_test.py
+def test_router_forward_deterministic_and_identity_kernel():
+  from vmoe_amd.nn import routing
+  x = torch.arange(20, dtype=torch.float32, device=dev()).reshape(1, 5, 4)
+  variables = {"params": {"dense": {"kernel": torch.eye(4, device=dev())}}}
+  layer = routing.NoisyTopExpertsPerItemRouter(
+      num_experts=4, num_selected_experts=2, noise_std=1.0, deterministic=True,
+      dispatcher=dict(name="indices", capacity=4, batch_priority=False))
+  d1, m1 = layer.apply(variables, x)
+  d2, m2 = layer.apply(variables, x)
+  assert torch.equal(d1.indices, d2.indices) and torch.equal(d1.combine_weights, d2.combine_weights)
+  for k in m1:
+    assert torch.equal(m1[k], m2[k])
+  gates = O.softmax(to_np(x))
+  want = O.get_top_experts_per_item_dispatcher(gates, "indices", 2, False, capacity=4)
+  np.testing.assert_array_equal(to_np(d1.indices), want.indices)
+  np.testing.assert_allclose(to_np(d1.combine_weights), want.combine_weights, rtol=1e-5)
+  wm = O.router_metrics(gates)
+  for k in ("auxiliary_loss", "gshard_loss", "importance_loss"):
+    np.testing.assert_allclose(to_np(m1[k]), wm[k], rtol=1e-4, atol=1e-6)
+
+
+def test_router_argument_errors():
+  from vmoe_amd.nn import routing
+  layer = routing.NoisyTopExpertsPerItemRouter(num_experts=4, num_selected_experts=5,
+                                               deterministic=True, dispatcher=dict(name="indices", capacity=2, batch_priority=False))
+  variables = {"params": {"dense": {"kernel": torch.eye(4, device=dev())}}}
+  with pytest.raises(ValueError, match="num_experts >= num_selected_experts >= 1"):
+    layer.apply(variables, torch.zeros((1, 5, 4), device=dev()))
+  layer = routing.NoisyTopExpertsPerItemRouter(num_experts=4, num_selected_experts=2,
+                                               deterministic=True)
+  with pytest.raises(ValueError, match="inputs.ndim must be 3"):
+    layer.apply(variables, torch.zeros((5, 4), device=dev()))
+  noisy = routing.NoisyTopExpertsPerItemRouter(num_experts=4, num_selected_experts=2, noise_std=1.0)
+  with pytest.raises(NotImplementedError):
+    noisy.apply(variables, torch.zeros((1, 5, 4), device=dev()))
+
+
+# ------------------------------------------------------------------ soft_moe/router_test.py
+def test_soft_router_forward(goldens):
+  from vmoe_amd.projects.soft_moe import router
+  g = goldens["soft_router_forward"]
+  x = torch.ones(tuple(g["x_shape"]), dtype=torch.float32, device=dev())
+  layer = router.SoftRouter(num_experts=g["num_experts"])
+  variables = layer.init(0, x)
+  assert list(variables["params"]["mu"].shape) == g["mu_shape"]
+  assert variables["params"]["scale"].shape == ()
+  dispatcher, _ = layer.apply(variables, x)
+  assert isinstance(dispatcher, router.Bfloat16Dispatcher)
+
+
+def test_soft_router_metrics(goldens):
+  from vmoe_amd.projects.soft_moe import router
+  g = goldens["soft_router_metrics"]
+  x = to_dev(np.asarray(g["x"], np.float32))
+  mu = to_dev(np.asarray(g["mu"], np.float32))
+  metrics = router.SoftRouter(num_experts=3).get_metrics(x, x, mu)
+  assert set(metrics) == set(g["expected"])
+  for k, v in g["expected"].items():
+    assert float(metrics[k]) == pytest.approx(v, abs=1e-5), k
+
+
+def test_soft_cosine_psim():
+  from vmoe_amd.projects.soft_moe import router
+  import scipy.spatial.distance as ssd
+  x = np.random.default_rng(0).standard_normal((6, 5, 4, 3, 2)).astype(np.float32)
+  y = to_np(router.cosine_psim(to_dev(x), (0,), (3, 4)))
+  assert y.shape == (6, 5, 4, 5, 4)
+  expected = np.stack([(1 - ssd.squareform(ssd.pdist(xi.reshape(20, -1), metric="cosine"))
+                        ).reshape(5, 4, 5, 4) for xi in x])
+  np.testing.assert_allclose(y, expected, rtol=1e-3, atol=1e-6)
+
+
+@pytest.mark.parametrize("dtype", [O.F32, O.BF16])
+def test_soft_moe_layer_vs_oracle(moe, dtype):
+  """SoftRouter + expert MLPs + combine against the oracle on a small case."""
+  from vmoe_amd.nn import vit_moe
+  from vmoe_amd.projects.soft_moe import router
+  rng = np.random.default_rng(3)
+  G, m, D, M, n, p = 4, 24, 64, 128, 4, 2
+  x = O.cast(rng.standard_normal((G, m, D)), dtype)
+  mu = rng.standard_normal((D, n, p)).astype(np.float32) / np.sqrt(D)
+  w0 = O.cast(rng.standard_normal((n, D, M)) / np.sqrt(D), dtype)
+  w1 = O.cast(rng.standard_normal((n, M, D)) / np.sqrt(M), dtype)
+  b0 = np.zeros((n, M), np.float32)
+  b1 = np.zeros((n, D), np.float32)
+  layer = router.SoftRouter(num_experts=n, num_slots=p, compute_similarity_metrics=False)
+  disp, metrics = layer.apply({"params": {"mu": to_dev(mu), "scale": torch.tensor(1.5, device=dev())}},
+                              to_dev(x, dtype))
+  mlp = moe.sparse_moe_spmd(vit_moe.MlpBlock, variable_axes={"params": 0})(mlp_dim=M)
+  variables = {"params": {"Dense_0": {"kernel": to_dev(w0, dtype), "bias": to_dev(b0, dtype)},
+                          "Dense_1": {"kernel": to_dev(w1, dtype), "bias": to_dev(b1, dtype)}}}
+  out = mlp.apply(variables, disp, to_dev(x, dtype))
+  odisp, ometrics = O.soft_router(x, mu, 1.5, dtype, compute_similarity_metrics=False)
+  want = O.cast(O.sparse_moe(odisp, lambda b: O.mlp_block(b, w0, b0, w1, b1, dtype), x), dtype)
+  assert_close(to_np(out), want, 1e-4 if dtype == O.F32 else 3e-2, "soft moe layer")
+  for k, v in ometrics.items():
+    assert float(metrics[k]) == pytest.approx(float(v), rel=2e-2, abs=1e-3), k
+
+
+# ------------------------------------------------------------------ whole layer
+def _layer_params(rng, D, M, E, dtype, bias_scale=0.0):
+  return {
+      "Router": {"dense": {"kernel": (rng.standard_normal((D, E)) / np.sqrt(D)).astype(np.float32)}},
+      "Mlp": {"Dense_0": {"kernel": O.cast(rng.standard_normal((E, D, M)) / np.sqrt(D), dtype),
+                          "bias": O.cast(rng.standard_normal((E, M)) * bias_scale, dtype)},
+              "Dense_1": {"kernel": O.cast(rng.standard_normal((E, M, D)) / np.sqrt(M), dtype),
+                          "bias": O.cast(rng.standard_normal((E, D)) * bias_scale, dtype)}}}
+
+
+def _params_to_dev(params, dtype):
+  f = lambda a: to_dev(a, dtype)
+  return {"params": {"Router": {"dense": {"kernel": to_dev(params["Router"]["dense"]["kernel"])}},
+                     "Mlp": {k: {kk: f(vv) for kk, vv in v.items()} for k, v in params["Mlp"].items()}}}
+
+
+LAYER_CASES = [
+    # N, L, D, M, E, K, group_size, dispatcher kwargs, dtype
+    (32, 49, 512, 2048, 8, 2, 49, dict(name="indices", batch_priority=False, capacity_factor=1.05), O.F32),
+    (32, 49, 512, 2048, 8, 2, 49, dict(name="einsum", batch_priority=False, capacity_factor=1.05), O.F32),
+    (8, 196, 256, 512, 32, 2, 784, dict(name="indices", batch_priority=True, capacity_factor=1.0), O.BF16),
+    (4, 100, 128, 256, 8, 2, 200, dict(name="einsum", batch_priority=True, capacity_factor=0.5,
+                                       bfloat16=True), O.F32),
+]
+
+
+@pytest.mark.parametrize("N,L,D,M,E,k,gs,dkw,dtype", LAYER_CASES)
+def test_mlp_moe_block_vs_oracle(N, L, D, M, E, k, gs, dkw, dtype):
+  """Whole layer on seeded inputs.  Float results depend on the gates, and a gate
+  that differs in the last bit can flip a routing decision, so the check is
+  (a) routing is bit-exact GIVEN the kernel's gates, (b) outputs match the oracle
+  to tolerance on every item whose routing agrees, (c) almost all items agree."""
+  from vmoe_amd.nn import vit_moe
+  rng = np.random.default_rng(N + D)
+  params = _layer_params(rng, D, M, E, dtype, bias_scale=0.1)
+  x = O.cast(rng.standard_normal((N, L, D)), dtype)
+  layer = vit_moe.MlpMoeBlock(mlp_dim=M, num_experts=E, group_size=gs, deterministic=True,
+                              router=dict(num_selected_experts=k, dispatcher=dkw),
+                              dtype=tdtype(dtype))
+  out, metrics = layer.apply(_params_to_dev(params, dtype), to_dev(x, dtype))
+  want, wmetrics = O.mlp_moe_block(x, params, group_size=gs, num_selected_experts=k,
+                                   dispatcher_kwargs=dkw, dtype=dtype)
+  assert out.shape == (N, L, D) and out.dtype == tdtype(dtype)
+  got = to_np(out).reshape(-1, D)
+  want = want.reshape(-1, D)
+  tol = 2e-5 if dtype == O.F32 and not dkw.get("bfloat16") else 2e-2
+  rms = np.sqrt((want ** 2).mean())
+  bad_items = (np.abs(got - want) > tol * (rms + np.abs(want))).any(-1)
+  frac = bad_items.mean()
+  print(f"layer {dtype} {dkw['name']}: items outside tolerance {bad_items.sum()} / {bad_items.size}")
+  assert frac <= (0.0 if dtype == O.F32 else 0.01)
+  for key in ("auxiliary_loss", "gshard_loss", "importance_loss"):
+    np.testing.assert_allclose(to_np(metrics[key]), wmetrics[key], rtol=2e-2 if dtype == O.BF16 else 1e-4)
+
+
+def test_mlp_moe_block_init_shapes():
+  from vmoe_amd.nn import vit_moe
+  layer = vit_moe.MlpMoeBlock(mlp_dim=32, num_experts=4, group_size=16, deterministic=True,
+                              router=dict(num_selected_experts=2,
+                                          dispatcher=dict(name="indices", batch_priority=True,
+                                                          capacity_factor=2.0)))
+  x = torch.randn((2, 16, 16), device=dev())
+  v = layer.init(0, x)["params"]
+  assert tuple(v["Router"]["dense"]["kernel"].shape) == (16, 4)
+  assert tuple(v["Mlp"]["Dense_0"]["kernel"].shape) == (4, 16, 32)
+  assert tuple(v["Mlp"]["Dense_0"]["bias"].shape) == (4, 32)
+  assert tuple(v["Mlp"]["Dense_1"]["kernel"].shape) == (4, 32, 16)
+  assert tuple(v["Mlp"]["Dense_1"]["bias"].shape) == (4, 16)
+  out, metrics = layer.apply({"params": v}, x)
+  assert out.shape == x.shape and set(metrics) == {"auxiliary_loss", "gshard_loss", "importance_loss"}

@@ -208,8 +208,11 @@ def test_bf16_round_vs_torch():
   rng = np.random.default_rng(2)
   x = np.concatenate([rng.standard_normal(100000).astype(np.float32) * 10.0 ** rng.integers(-20, 20, 100000),
                       np.asarray([0.0, -0.0, 1.0, 1.00390625, 1.0078125, 3.3895314e38, np.inf, -np.inf], np.float32)])
+  x = x.astype(np.float32)
   want = torch.from_numpy(x).to(torch.bfloat16).to(torch.float32).numpy()
-  np.testing.assert_array_equal(O.bf16_round(x), want)
+  np.testing.assert_array_equal(O._bf16_round_numpy(x), want)
+  big = np.tile(x, 12)
+  np.testing.assert_array_equal(O.bf16_round(big), np.tile(want, 12))
   assert np.isnan(O.bf16_round(np.asarray([np.nan], np.float32))[0])
 
 

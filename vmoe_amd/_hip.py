@@ -162,6 +162,27 @@ class CastParams(ctypes.Structure):
               ("in_dtype", c_int32), ("out_dtype", c_int32)]
 
 
+_timing_sink = None
+
+
+def set_timing_sink(sink) -> None:
+  """With a dict as sink, every entry point is bracketed by a pair of timing
+  events on the stream it is launched on; the pairs are appended to
+  ``sink[name]`` for the caller to read after synchronising.  None disables."""
+  global _timing_sink
+  _timing_sink = sink
+
+
 def call(name: str, params: ctypes.Structure) -> None:
   fn = getattr(lib(), name)
-  check(fn(ctypes.byref(params), stream()), name)
+  sink = _timing_sink
+  if sink is None:
+    check(fn(ctypes.byref(params), stream()), name)
+    return
+  start = torch.cuda.Event(enable_timing=True)
+  stop = torch.cuda.Event(enable_timing=True)
+  start.record()
+  code = fn(ctypes.byref(params), stream())
+  stop.record()
+  sink.setdefault(name, []).append((start, stop))
+  check(code, name)

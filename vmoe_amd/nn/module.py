@@ -1,0 +1,60 @@
+"""A minimal stand-in for flax.linen.Module: hyper-parameters are constructor
+keyword arguments with class-level defaults, parameters live in a nested dict
+``{'params': {...}}`` with the reference's names, ``init(seed, *inputs)``
+creates them and ``apply(variables, *inputs)`` runs the module."""
+from __future__ import annotations
+
+from typing import Any, Dict
+
+import torch
+
+
+class Module:
+  _fields: Dict[str, Any] = {}
+
+  def __init__(self, **kwargs):
+    fields = {}
+    for cls in reversed(type(self).__mro__):
+      fields.update(getattr(cls, "_fields", {}))
+    self.name = kwargs.pop("name", None)
+    unknown = set(kwargs) - set(fields)
+    if unknown:
+      raise TypeError(f"{type(self).__name__} got unexpected arguments {sorted(unknown)}")
+    missing = [k for k, v in fields.items() if v is _REQUIRED and k not in kwargs]
+    if missing:
+      raise TypeError(f"{type(self).__name__} missing required arguments {missing}")
+    for k, v in fields.items():
+      setattr(self, k, kwargs.get(k, v))
+
+  def init(self, rng, *inputs):
+    raise NotImplementedError
+
+  def apply(self, variables, *inputs, **kwargs):
+    raise NotImplementedError
+
+  def __call__(self, variables, *inputs, **kwargs):
+    return self.apply(variables, *inputs, **kwargs)
+
+
+class _Required:
+  def __repr__(self):
+    return "<required>"
+
+
+_REQUIRED = _Required()
+
+
+def generator(rng, device="cpu") -> torch.Generator:
+  if isinstance(rng, torch.Generator):
+    return rng
+  g = torch.Generator(device=device)
+  g.manual_seed(int(rng))
+  return g
+
+
+def lecun_normal(gen: torch.Generator, shape, fan_in: int, dtype=torch.float32, device=None):
+  """jax.nn.initializers.lecun_normal: truncated normal with variance 1/fan_in."""
+  t = torch.empty(shape, dtype=torch.float32)
+  torch.nn.init.trunc_normal_(t, mean=0.0, std=1.0, a=-2.0, b=2.0, generator=gen)
+  t = t * (1.0 / 0.87962566103423978) / (fan_in ** 0.5)
+  return t.to(dtype).to(device) if device is not None else t.to(dtype)

@@ -1,0 +1,94 @@
+"""Routers of the MoE layer on HIP kernels; host-side mirror of vmoe/nn/routing.py.
+
+A router is called on (G, S, D) inputs and returns ``(dispatcher, metrics)``.
+"""
+from __future__ import annotations
+
+from typing import Any, Dict, Mapping, Optional, Tuple
+
+import torch
+
+import vmoe_amd.moe
+from vmoe_amd import kernels as K
+from vmoe_amd.nn import module
+
+Array = torch.Tensor
+BaseDispatcher = vmoe_amd.moe.BaseDispatcher
+KwArgs = Mapping[str, Any]
+Metrics = Mapping[str, Array]
+
+
+class NoisyTopExpertsPerItemRouter(module.Module):
+  """Top-K experts per item with optional Batch Priority Routing; vmoe/nn/routing.py:31-183.
+
+  Parameters: ``{'dense': {'kernel': (D, E)}}``.  Only the inference branch
+  (``deterministic=True`` or ``noise_std == 0``) is implemented: gating noise and
+  the load loss belong to training.
+
+  ``logit_bias`` (not in the reference, whose gating layer has no bias) adds a
+  fixed float32 (E,) vector to the logits before the softmax; it exists for the
+  benchmark configuration that skews the expert load.
+  """
+  _fields = dict(num_experts=module._REQUIRED, num_selected_experts=1, noise_std=1.0,
+                 gshard_loss_weight=0.0, importance_loss_weight=1.0, load_loss_weight=1.0,
+                 dispatcher=None, deterministic=False, dtype=None, logit_bias=None)
+
+  def init(self, rng, inputs: Array):
+    gen = module.generator(rng)
+    D = inputs.shape[-1]
+    kernel = module.lecun_normal(gen, (D, self.num_experts), fan_in=D, device=inputs.device)
+    return {"params": {"dense": {"kernel": kernel}}}
+
+  def apply(self, variables, inputs: Array) -> Tuple[BaseDispatcher, Metrics]:
+    kernel = variables["params"]["dense"]["kernel"]
+    gates, metrics, topk = self._compute_gates_softmax_and_metrics(inputs, kernel)
+    dispatcher = self._create_dispatcher(gates, topk)
+    return dispatcher, metrics
+
+  def _compute_gates_softmax_and_metrics(self, inputs: Array, kernel: Array):
+    num_experts = self.num_experts
+    if inputs.ndim != 3:
+      raise ValueError(f"inputs.ndim must be 3, but it is {inputs.ndim}")
+    if not num_experts >= self.num_selected_experts >= 1:
+      raise ValueError(f"num_experts >= num_selected_experts >= 1, but got "
+                       f"num_experts = {num_experts} and "
+                       f"num_selected_experts = {self.num_selected_experts}.")
+    if kernel.shape != (inputs.shape[-1], num_experts):
+      raise ValueError(f"Router kernel has shape {tuple(kernel.shape)}, expected "
+                       f"{(inputs.shape[-1], num_experts)}")
+    if not (self.deterministic or self.noise_std == 0.0):
+      raise NotImplementedError(
+          "The noisy (training-time) branch of the router is not implemented; "
+          "use deterministic=True or noise_std=0.")
+    dtype = self.dtype or inputs.dtype
+    x = K.cast(inputs, dtype)
+    w = K.cast(kernel, dtype)
+    gates, val, idx = K.gate_topk(x, w, self.num_selected_experts, logit_bias=self.logit_bias)
+    importance_loss, gshard_loss, auxiliary_loss = K.router_metrics(
+        gates, idx, self.gshard_loss_weight, self.importance_loss_weight)
+    metrics = {
+        "auxiliary_loss": auxiliary_loss,
+        "gshard_loss": gshard_loss,
+        "importance_loss": importance_loss,
+    }
+    return gates, metrics, (val, idx)
+
+  def _create_dispatcher(self, gates_dispatch: Array, topk=None):
+    dispatcher_kwargs = dict(**(self.dispatcher or {}))
+    use_bfloat16 = dispatcher_kwargs.pop("bfloat16", False)
+    dispatcher = vmoe_amd.moe.get_top_experts_per_item_dispatcher(
+        gates_dispatch, num_selected_experts=self.num_selected_experts, _topk=topk,
+        **dispatcher_kwargs)
+    if use_bfloat16:
+      dispatcher = vmoe_amd.moe.Bfloat16Dispatcher(dispatcher)
+    return dispatcher
+
+
+class NoisyTopItemsPerExpertRouter(module.Module):
+  """Experts-choice router, vmoe/nn/routing.py:186-244.  Not part of the
+  inference path built here: constructing it works, calling it raises."""
+  _fields = dict(num_experts=module._REQUIRED, noise_std=1.0, dispatcher=None,
+                 deterministic=False, dtype=None)
+
+  def apply(self, variables, inputs):
+    raise NotImplementedError("Top-items-per-expert routing has no HIP kernel yet.")
