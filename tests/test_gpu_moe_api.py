@@ -295,7 +295,7 @@ def test_soft_moe_layer_vs_oracle(moe, dtype):
   rng = np.random.default_rng(3)
   G, m, D, M, n, p = 4, 24, 64, 128, 4, 2
   x = O.cast(rng.standard_normal((G, m, D)), dtype)
-  mu = rng.standard_normal((D, n, p)).astype(np.float32) / np.sqrt(D)
+  mu = (rng.standard_normal((D, n, p)) / np.sqrt(D)).astype(np.float32)
   w0 = O.cast(rng.standard_normal((n, D, M)) / np.sqrt(D), dtype)
   w1 = O.cast(rng.standard_normal((n, M, D)) / np.sqrt(M), dtype)
   b0 = np.zeros((n, M), np.float32)
