@@ -115,7 +115,11 @@ int transpose(const void* in, void* out, int batch, int rows, int cols, int dtyp
   return launch_status();
 }
 
-using CfgBig = GemmCfg<256, 256, 2, 2>;
+// First product (short K = D, GELU epilogue): two 128x256 workgroups per CU so one
+// workgroup's epilogue overlaps the other's MFMAs.  Second product (long K = M):
+// one 256x256 workgroup per CU for the highest arithmetic intensity.
+using CfgUp = GemmCfg<128, 256, 2, 2, 32, 3, 2>;
+using CfgDown = GemmCfg<256, 256, 2, 2, 32, 4, 1>;
 
 size_t align256(size_t v) { return (v + 255) / 256 * 256; }
 
@@ -180,15 +184,15 @@ extern "C" int vmoe_expert_mlp(const VmoeExpertMlpParams* p, vmoe_stream_t strea
       w1t = ws;
     }
     if (tanh_gelu)
-      rc = launch_gemm_bf16<CfgBig, kEpiBiasGeluTanh>((const bf16_t*)p->x, (const bf16_t*)w0t,
+      rc = launch_gemm_bf16<CfgUp, kEpiBiasGeluTanh>((const bf16_t*)p->x, (const bf16_t*)w0t,
                                                       (const bf16_t*)p->b0, (bf16_t*)hidden, p->E,
                                                       p->R, p->M, p->D, stream);
     else
-      rc = launch_gemm_bf16<CfgBig, kEpiBiasGeluErf>((const bf16_t*)p->x, (const bf16_t*)w0t,
+      rc = launch_gemm_bf16<CfgUp, kEpiBiasGeluErf>((const bf16_t*)p->x, (const bf16_t*)w0t,
                                                      (const bf16_t*)p->b0, (bf16_t*)hidden, p->E,
                                                      p->R, p->M, p->D, stream);
     if (rc != VMOE_OK) return rc;
-    return launch_gemm_bf16<CfgBig, kEpiBias>((const bf16_t*)hidden, (const bf16_t*)w1t,
+    return launch_gemm_bf16<CfgDown, kEpiBias>((const bf16_t*)hidden, (const bf16_t*)w1t,
                                               (const bf16_t*)p->b1, (bf16_t*)p->out, p->E, p->R,
                                               p->D, p->M, stream);
   }

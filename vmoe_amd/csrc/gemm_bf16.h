@@ -7,9 +7,22 @@
 // (BM/WM) x (BN/WN) of it as a grid of 32x32 v_mfma_f32_32x32x16_bf16 tiles held
 // in accumulator registers.  K advances in steps of BK = 64 through two LDS
 // stages: the global loads of step k+1 are issued into registers before the
-// MFMAs of step k and written to the other stage after them, one barrier per
-// step.  LDS rows are padded by 16 bytes so that the eight lanes served per
-// clock hit all 32 banks.
+// MFMAs of step k and written to the other stage while the last MFMAs of step k
+// run, one barrier per step.  Inside a step the LDS fragment reads of the next
+// 16-wide k slice are issued before the MFMAs of the current one (double
+// buffered fragment registers).  LDS rows are padded by 16 bytes so that the
+// eight lanes served per clock hit all 32 banks.
+//
+// The MFMA is issued with the weight fragment as its first operand, so the
+// accumulator tile is C^T: a lane ends up with 4 consecutive output columns of
+// one output row, which the epilogue packs into 8-byte LDS writes; the tile is
+// then streamed out with 16-byte, row-contiguous global stores.
+//
+// Workgroup -> tile mapping: hardware hands consecutive workgroups to the 8 XCDs
+// round-robin, each XCD has a private L2.  Workgroup w is therefore given
+// logical tile (w % 8) * ceil(tiles/8) + w / 8, so that an XCD walks a contiguous
+// run of tiles (whole experts), and within an expert tiles are ordered in panels
+// of 8 row tiles so that the tiles in flight on an XCD share A and B panels.
 #ifndef VMOE_GEMM_BF16_H_
 #define VMOE_GEMM_BF16_H_
 
@@ -19,72 +32,147 @@ namespace vmoe {
 
 enum { kEpiBias = 0, kEpiBiasGeluTanh = 1, kEpiBiasGeluErf = 2 };
 
-template <int BM_, int BN_, int WM_, int WN_>
+constexpr int kNumXcd = 8;
+constexpr int kPanelRows = 8;   // row tiles per panel in the tile order
+
+// 0.5 x (1 + tanh(c (x + 0.044715 x^3))) = x * sigmoid(2 c (x + 0.044715 x^3)),
+// with the hardware exp2 and reciprocal (relative error ~1e-7, far inside bf16).
+__device__ __forceinline__ float gelu_tanh_fast(float x) {
+  const float k0 = -2.0f * 0.7978845608028654f * 1.4426950408889634f;
+  const float k1 = k0 * 0.044715f;
+  float z = x * fmaf(k1, x * x, k0);
+  float e = __builtin_amdgcn_exp2f(z);
+  return x * __builtin_amdgcn_rcpf(1.0f + e);
+}
+
+template <int EPI>
+__device__ __forceinline__ float apply_epilogue(float acc, float bias, bool has_bias) {
+  float o = bf16r(acc);
+  if (has_bias) o = bf16r(o + bias);
+  if (EPI == kEpiBiasGeluTanh) o = gelu_tanh_fast(o);
+  if (EPI == kEpiBiasGeluErf) o = gelu_erf(o);
+  return o;
+}
+
+template <int BM_, int BN_, int WM_, int WN_, int BK_ = 32, int NSTAGE_ = 4, int BLOCKS_PER_CU_ = 1>
 struct GemmCfg {
-  static constexpr int BM = BM_, BN = BN_, BK = 64, WM = WM_, WN = WN_;
-  static constexpr int kThreads = 64 * WM * WN;
+  static constexpr int BM = BM_, BN = BN_, BK = BK_, WM = WM_, WN = WN_, NSTAGE = NSTAGE_;
+  static constexpr int kBlocksPerCu = BLOCKS_PER_CU_;
+  static constexpr int kWaves = WM * WN;
+  static constexpr int kThreads = 64 * kWaves;
   static constexpr int TM = BM / WM, TN = BN / WN;   // wave tile
   static constexpr int FM = TM / 32, FN = TN / 32;   // 32x32 MFMA tiles per wave
-  static constexpr int kLd = BK + 8;                 // padded LDS row, elements
-  static constexpr int kStageElems = (BM + BN) * kLd;
-  static constexpr size_t kLdsBytes = 2ull * kStageElems * sizeof(bf16_t);
-  static constexpr int kChunksPerRow = BK / 8;
-  static constexpr int kAChunks = BM * kChunksPerRow / kThreads;  // 16-byte loads per thread
-  static constexpr int kBChunks = BN * kChunksPerRow / kThreads;
+  static constexpr int kRowBytes = BK * 2;           // LDS row of one k tile, XOR-swizzled 16-byte chunks
+  static constexpr int kChunksPerRow = BK / 8;       // 4 (BK=32) or 8 (BK=64)
+  static constexpr int kRowsPerLoad = 64 / kChunksPerRow;   // rows filled by one wave-wide DMA load
+  // The gfx950 LDS serves 16 lanes of a 128-bit read per clock from 64 banks (256
+  // bytes): the swizzle must spread 16 consecutive rows over all of them.
+  static constexpr int kSwzShift = BK == 32 ? 2 : 1;  // log2(rows per 256-byte bank line)
+  static constexpr int kStageBytes = (BM + BN) * kRowBytes;
+  static constexpr int kOutLd = TN + 8;              // padded row of the staged output tile
+  static constexpr size_t kMainBytes = (size_t)NSTAGE * kStageBytes;
+  static constexpr size_t kOutBytes = (size_t)kWaves * TM * kOutLd * sizeof(bf16_t);
+  static constexpr size_t kLdsBytes = kMainBytes > kOutBytes ? kMainBytes : kOutBytes;
+  static constexpr int kAIssues = BM / kRowsPerLoad / kWaves;
+  static constexpr int kBIssues = BN / kRowsPerLoad / kWaves;
+  static constexpr int kLoads = kAIssues + kBIssues;  // DMA instructions per wave per k tile
+  static_assert(BK == 32 || BK == 64, "BK");
+  static_assert(NSTAGE >= 2 && (NSTAGE - 1) * kLoads < 64, "vmcnt is a 6-bit counter");
   static_assert(BM % (WM * 32) == 0 && BN % (WN * 32) == 0, "wave tile must be 32-aligned");
-  static_assert((BM * kChunksPerRow) % kThreads == 0 && (BN * kChunksPerRow) % kThreads == 0,
+  static_assert(BM % (kRowsPerLoad * kWaves) == 0 && BN % (kRowsPerLoad * kWaves) == 0,
                 "tile loads must divide evenly");
+  static_assert(kLdsBytes * kBlocksPerCu <= 160 * 1024, "LDS budget");
 };
 
+// s_waitcnt vmcnt(N) with lgkmcnt/expcnt left at their maxima.
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {
+  __builtin_amdgcn_s_waitcnt(0x0f70 | (N & 15) | ((N >> 4) << 14));
+}
+__device__ __forceinline__ void wait_lgkmcnt0() { __builtin_amdgcn_s_waitcnt(0xc07f); }
+
+#ifdef VMOE_GEMM_DEBUG_SAME_TILE
+#define VMOE_DBG_ROW(x) 0
+#define VMOE_DBG_BATCH(x) 0
+#else
+#define VMOE_DBG_ROW(x) (x)
+#define VMOE_DBG_BATCH(x) (x)
+#endif
+#ifdef VMOE_GEMM_DEBUG_NO_XCD
+#define VMOE_DBG_LOGICAL(expr) ((int)blockIdx.x)
+#else
+#define VMOE_DBG_LOGICAL(expr) (expr)
+#endif
+
+typedef const __attribute__((address_space(1))) void* global_ptr_t;
+typedef __attribute__((address_space(3))) void* lds_ptr_t;
+
+// Fast path: Kd % 64 == 0.  Global tiles go straight into LDS
+// (global_load_lds_dwordx4: lane L of a wave lands at base + 16*L), so lane L
+// fetches the global chunk that the XOR swizzle assigns to LDS slot L:
+// row = L/8, slot = L%8, chunk = slot ^ (row & 7).
 template <typename Cfg, int EPI>
-__global__ __launch_bounds__(Cfg::kThreads) void gemm_bf16_kernel(
+__global__ __launch_bounds__(Cfg::kThreads, Cfg::kBlocksPerCu) void gemm_bf16_kernel(
     const bf16_t* __restrict__ A, const bf16_t* __restrict__ Bt, const bf16_t* __restrict__ bias,
-    bf16_t* __restrict__ C, int R, int N, int Kd, int tiles_m, int tiles_n) {
-  extern __shared__ __align__(16) unsigned char smem[];
-  bf16_t* lds = reinterpret_cast<bf16_t*>(smem);
-  constexpr int BM = Cfg::BM, BN = Cfg::BN, BK = Cfg::BK, LD = Cfg::kLd;
+    bf16_t* __restrict__ C, int R, int N, int Kd, int tiles_m, int tiles_n, int num_tiles,
+    int tiles_per_xcd) {
+  extern __shared__ __align__(1024) unsigned char smem[];
+  constexpr int BM = Cfg::BM, BN = Cfg::BN, BK = Cfg::BK;
   constexpr int FM = Cfg::FM, FN = Cfg::FN;
+  constexpr int RB = Cfg::kRowBytes;
   const int tid = threadIdx.x;
   const int lane = tid & 63;
-  const int wave = tid >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave / Cfg::WN, wn = wave % Cfg::WN;
   const int m = lane & 31, h = lane >> 5;
 
-  // Tile order: consecutive workgroups share the same weight columns (tile_n)
-  // and walk down the rows, so a weight tile stays in L2 while it is reused.
+  // XCD-aware logical tile id.
+  const int logical = VMOE_DBG_LOGICAL((blockIdx.x % kNumXcd) * tiles_per_xcd + blockIdx.x / kNumXcd);
+  if (blockIdx.x / kNumXcd >= tiles_per_xcd || logical >= num_tiles) return;
   const int per_batch = tiles_m * tiles_n;
-  const int b = blockIdx.x / per_batch;
-  const int rem = blockIdx.x - b * per_batch;
-  const int tile_n = rem / tiles_m;
-  const int tile_m = rem - tile_n * tiles_m;
+  const int b = logical / per_batch;
+  const int rem = logical - b * per_batch;
+  const int panel = rem / (kPanelRows * tiles_n);
+  const int in_panel = rem - panel * kPanelRows * tiles_n;
+  const int rows_here = min(kPanelRows, tiles_m - panel * kPanelRows);
+  const int tile_n = in_panel / rows_here;
+  const int tile_m = panel * kPanelRows + in_panel - tile_n * rows_here;
   const int row0 = tile_m * BM, col0 = tile_n * BN;
-  const bf16_t* Ab = A + (size_t)b * R * Kd;
-  const bf16_t* Bb = Bt + (size_t)b * N * Kd;
+  const unsigned char* Ab = reinterpret_cast<const unsigned char*>(A + (size_t)VMOE_DBG_BATCH(b) * R * Kd);
+  const unsigned char* Bb = reinterpret_cast<const unsigned char*>(Bt + (size_t)VMOE_DBG_BATCH(b) * N * Kd);
 
-  // Per-thread global chunk coordinates (fixed over the K loop).
-  const bf16_t* a_src[Cfg::kAChunks];
-  const bf16_t* b_src[Cfg::kBChunks];
-  int a_dst[Cfg::kAChunks], b_dst[Cfg::kBChunks], a_kc[Cfg::kAChunks], b_kc[Cfg::kBChunks];
+  // Byte offsets of this lane's chunk in each of its load instructions.  Lane L
+  // of a DMA load lands in LDS slot L: row L / CPR, chunk slot L % CPR; it
+  // therefore fetches global chunk  slot ^ swz(row).
+  constexpr int CPR = Cfg::kChunksPerRow;
+  constexpr int RPL = Cfg::kRowsPerLoad;
+  const int lrow = lane / CPR;
+  // (RPL * kWaves is a multiple of the swizzle period, so the row inside a wave's
+  // load group determines the swizzle up to the wave's own offset.)
+  const int chunk = (lane % CPR) ^ (((wave * RPL + lrow) >> Cfg::kSwzShift) & (CPR - 1));
+  uint32_t a_goff[Cfg::kAIssues], b_goff[Cfg::kBIssues];
 #pragma unroll
-  for (int i = 0; i < Cfg::kAChunks; ++i) {
-    int c = tid + i * Cfg::kThreads;
-    int r = c / Cfg::kChunksPerRow, kc = c % Cfg::kChunksPerRow;
-    int gr = row0 + r;
-    if (gr >= R) gr = R - 1;
-    a_src[i] = Ab + (size_t)gr * Kd + kc * 8;
-    a_dst[i] = r * LD + kc * 8;
-    a_kc[i] = kc * 8;
+  for (int i = 0; i < Cfg::kAIssues; ++i) {
+    int r = (i * Cfg::kWaves + wave) * RPL + lrow;
+    a_goff[i] = (uint32_t)min(VMOE_DBG_ROW(row0) + r, R - 1) * (uint32_t)Kd * 2u + chunk * 16;
   }
 #pragma unroll
-  for (int i = 0; i < Cfg::kBChunks; ++i) {
-    int c = tid + i * Cfg::kThreads;
-    int r = c / Cfg::kChunksPerRow, kc = c % Cfg::kChunksPerRow;
-    int gn = col0 + r;
-    if (gn >= N) gn = N - 1;
-    b_src[i] = Bb + (size_t)gn * Kd + kc * 8;
-    b_dst[i] = BM * LD + r * LD + kc * 8;
-    b_kc[i] = kc * 8;
+  for (int i = 0; i < Cfg::kBIssues; ++i) {
+    int r = (i * Cfg::kWaves + wave) * RPL + lrow;
+    b_goff[i] = (uint32_t)min(VMOE_DBG_ROW(col0) + r, N - 1) * (uint32_t)Kd * 2u + chunk * 16;
   }
+  auto load_tile = [&](int stage, int k0) {
+    unsigned char* s = smem + stage * Cfg::kStageBytes;
+#pragma unroll
+    for (int i = 0; i < Cfg::kAIssues; ++i)
+      __builtin_amdgcn_global_load_lds((global_ptr_t)(Ab + a_goff[i] + (size_t)k0 * 2),
+                                       (lds_ptr_t)(s + (i * Cfg::kWaves + wave) * RPL * RB), 16, 0, 0);
+#pragma unroll
+    for (int i = 0; i < Cfg::kBIssues; ++i)
+      __builtin_amdgcn_global_load_lds((global_ptr_t)(Bb + b_goff[i] + (size_t)k0 * 2),
+                                       (lds_ptr_t)(s + BM * RB + (i * Cfg::kWaves + wave) * RPL * RB),
+                                       16, 0, 0);
+  };
 
   floatx16 acc[FM][FN];
 #pragma unroll
@@ -94,90 +182,267 @@ __global__ __launch_bounds__(Cfg::kThreads) void gemm_bf16_kernel(
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
 
-  uint4 ra[Cfg::kAChunks], rb[Cfg::kBChunks];
-  auto load_global = [&](int k0) {
+  bf16x8 fa[2][FM], fb[2][FN];
+  const int a_row_off = (wm * Cfg::TM + m) * RB;
+  const int b_row_off = BM * RB + (wn * Cfg::TN + m) * RB;
+  const int swz = (m >> Cfg::kSwzShift) & (CPR - 1);
+  auto load_frags = [&](int buf, int stage, int ks) {
+    const unsigned char* s = smem + stage * Cfg::kStageBytes + (((2 * ks + h) ^ swz) * 16);
 #pragma unroll
-    for (int i = 0; i < Cfg::kAChunks; ++i)
-      ra[i] = (k0 + a_kc[i] + 8 <= Kd) ? *reinterpret_cast<const uint4*>(a_src[i] + k0)
-                                       : make_uint4(0, 0, 0, 0);
+    for (int i = 0; i < FM; ++i)
+      fa[buf][i] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(s + a_row_off + i * 32 * RB));
 #pragma unroll
-    for (int i = 0; i < Cfg::kBChunks; ++i)
-      rb[i] = (k0 + b_kc[i] + 8 <= Kd) ? *reinterpret_cast<const uint4*>(b_src[i] + k0)
-                                       : make_uint4(0, 0, 0, 0);
-  };
-  auto store_lds = [&](int stage) {
-    bf16_t* s = lds + stage * Cfg::kStageElems;
-#pragma unroll
-    for (int i = 0; i < Cfg::kAChunks; ++i) *reinterpret_cast<uint4*>(s + a_dst[i]) = ra[i];
-#pragma unroll
-    for (int i = 0; i < Cfg::kBChunks; ++i) *reinterpret_cast<uint4*>(s + b_dst[i]) = rb[i];
+    for (int j = 0; j < FN; ++j)
+      fb[buf][j] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(s + b_row_off + j * 32 * RB));
   };
 
-  const int nk = (Kd + BK - 1) / BK;
-  load_global(0);
-  store_lds(0);
-  __syncthreads();
-  for (int kt = 0; kt < nk; ++kt) {
-    const bool more = kt + 1 < nk;
-    if (more) load_global((kt + 1) * BK);
-    const bf16_t* sa = lds + (kt & 1) * Cfg::kStageElems + (wm * Cfg::TM + m) * LD + h * 8;
-    const bf16_t* sb = lds + (kt & 1) * Cfg::kStageElems + BM * LD + (wn * Cfg::TN + m) * LD + h * 8;
+  // Main loop: a ring of NSTAGE LDS stages, the DMA loads run PD = NSTAGE-1 k
+  // tiles ahead of the MFMAs and are never drained: the wait in front of the
+  // tile barrier only covers the tile needed next (vmcnt leaves the younger
+  // loads in flight).  The fragment reads of k slice s+1 are interleaved with
+  // the MFMAs of slice s; the barrier of a tile sits before its last slice, so
+  // the first fragments of the next tile are fetched under that slice's MFMAs.
+  auto mfma_slice = [&](int buf) {
 #pragma unroll
-    for (int ks = 0; ks < BK / 16; ++ks) {
-      bf16x8 fa[FM], fb[FN];
-#pragma unroll
-      for (int i = 0; i < FM; ++i)
-        fa[i] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(sa + i * 32 * LD + ks * 16));
+    for (int i = 0; i < FM; ++i)
 #pragma unroll
       for (int j = 0; j < FN; ++j)
-        fb[j] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(sb + j * 32 * LD + ks * 16));
+        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[buf][j], fa[buf][i], acc[i][j], 0, 0, 0);
+  };
+  constexpr int KS = BK / 16;
+  constexpr int NS = Cfg::NSTAGE, PD = NS - 1, L = Cfg::kLoads;
+  constexpr int kReads = FM + FN;
+  constexpr int kMfmas = FM * FN;
+  static_assert(KS >= 2, "slice schedule");
+  // Scheduling hints for one k slice (its own scheduling region): the LDS reads
+  // of the next slice go out behind the first MFMAs (an MFMA leads, so the wait
+  // for the previous slice's reads never covers a new read); the DMA loads
+  // (first slice only) are spread over the remaining MFMAs.
+  auto slice_schedule = [&](bool with_vmem) {
+    constexpr int kLead = kReads < kMfmas ? kReads : kMfmas;
+    constexpr int kReadsPer = (kReads + kLead - 1) / kLead;
+    constexpr int kRest = kMfmas - kLead;
 #pragma unroll
-      for (int i = 0; i < FM; ++i)
-#pragma unroll
-        for (int j = 0; j < FN; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i], fb[j], acc[i][j], 0, 0, 0);
+    for (int g = 0; g < kLead; ++g) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, kReadsPer, 0);
     }
-    if (more) store_lds((kt + 1) & 1);
-    __syncthreads();
-  }
+    if (with_vmem) {
+      if constexpr (kRest > 0) {
+        constexpr int kPer = (L + kRest - 1) / kRest;
+#pragma unroll
+        for (int g = 0; g < kRest; ++g) {
+          __builtin_amdgcn_sched_group_barrier(0x020, kPer, 0);
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        }
+      } else {
+        __builtin_amdgcn_sched_group_barrier(0x020, L, 0);
+      }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  // Waits until k tile `next` has landed: only the tiles issued after it
+  // (at most PD-1, fewer at the end of the K loop) may stay in flight.
+  auto wait_tile = [&](int younger) {
+    if (younger >= PD - 1) wait_vmcnt<(PD - 1) * L>();
+    else if (PD >= 3 && younger == PD - 2) wait_vmcnt<(PD >= 3 ? PD - 2 : 0) * L>();
+    else if (PD >= 4 && younger == PD - 3) wait_vmcnt<(PD >= 4 ? PD - 3 : 0) * L>();
+    else wait_vmcnt<0>();
+  };
+  static_assert(PD <= 4, "wait_tile covers up to 4 tiles of prefetch");
 
-  // Epilogue: lane holds column (col0 + ... + m) for rows (v/4)*8 + h*4 + v%4.
+  const int nk = Kd / BK;
+#pragma unroll
+  for (int t = 0; t < PD; ++t)
+    if (t < nk) load_tile(t, t * BK);
+  wait_tile(min(PD, nk) - 1);
+  __builtin_amdgcn_s_barrier();
+  __builtin_amdgcn_sched_barrier(0);
+  load_frags(0, 0, 0);
+  int stage = 0;
+  for (int kt = 0; kt < nk; ++kt) {
+    const int next_stage = stage + 1 == NS ? 0 : stage + 1;
+    const int load_stage = stage == 0 ? NS - 1 : stage - 1;   // (kt + PD) % NS
+    const bool do_load = kt + PD < nk;
+    const bool has_next = kt + 1 < nk;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      if (ks + 1 < KS) {
+#ifndef VMOE_DBG_NO_FRAGS
+        load_frags((ks + 1) & 1, stage, ks + 1);
+#endif
+#ifndef VMOE_DBG_NO_DMA
+        if (ks == 0 && do_load) load_tile(load_stage, (kt + PD) * BK);
+#endif
+      } else if (has_next) {
+        // Tiles kt+2 .. min(kt+PD, nk-1) were issued after tile kt+1.
+        wait_tile(min(kt + PD, nk - 1) - (kt + 1));
+        wait_lgkmcnt0();
+#ifndef VMOE_DBG_NO_BARRIER
+        __builtin_amdgcn_s_barrier();
+#endif
+        __builtin_amdgcn_sched_barrier(0);
+#ifndef VMOE_DBG_NO_FRAGS
+        load_frags(0, next_stage, 0);
+#endif
+      }
+      mfma_slice(ks & 1);
+      slice_schedule(ks == 0);
+    }
+    stage = next_stage;
+  }
+  wait_lgkmcnt0();
+  __syncthreads();   // all waves are done with the operand tiles: LDS is reused below
+
+  // Epilogue.  acc[i][j][v] = C[row0 + wm*TM + i*32 + m][col0 + wn*TN + j*32 + (v/4)*8 + h*4 + v%4].
+  const bf16_t* biasb = bias != nullptr ? bias + (size_t)b * N : nullptr;
+  bf16_t* Cb = C + (size_t)b * R * N;
+  constexpr int OLD = Cfg::kOutLd;
+  bf16_t* so = reinterpret_cast<bf16_t*>(smem) + (size_t)wave * Cfg::TM * OLD;
+#pragma unroll
+  for (int j = 0; j < FN; ++j) {
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const int cl = j * 32 + q * 8 + h * 4;          // column inside the wave tile
+      const int col = col0 + wn * Cfg::TN + cl;
+      float bv[4] = {0.f, 0.f, 0.f, 0.f};
+      if (biasb != nullptr) {
+#pragma unroll
+        for (int t = 0; t < 4; ++t) bv[t] = bf2f(biasb[min(col + t, N - 1)]);
+      }
+#pragma unroll
+      for (int i = 0; i < FM; ++i) {
+        uint32_t p[2];
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+          float o0 = apply_epilogue<EPI>(acc[i][j][q * 4 + 2 * t], bv[2 * t], biasb != nullptr);
+          float o1 = apply_epilogue<EPI>(acc[i][j][q * 4 + 2 * t + 1], bv[2 * t + 1], biasb != nullptr);
+          p[t] = (uint32_t)f2bf(o0) | ((uint32_t)f2bf(o1) << 16);
+        }
+        *reinterpret_cast<uint2*>(so + (i * 32 + m) * OLD + cl) = make_uint2(p[0], p[1]);
+      }
+    }
+  }
+  // Each wave reads back only what it wrote (LDS operations of a wave complete in order).
+  constexpr int kChunksOut = Cfg::TN / 8;             // 16-byte chunks per staged row
+  constexpr int kRowsPerPass = 64 / kChunksOut;
+  static_assert(64 % kChunksOut == 0, "wave tile width must divide a wave");
+  const int oc = (lane % kChunksOut) * 8;
+  const int orow = lane / kChunksOut;
+#pragma unroll
+  for (int r0 = 0; r0 < Cfg::TM; r0 += kRowsPerPass) {
+    const int rl = r0 + orow;
+    const int row = row0 + wm * Cfg::TM + rl;
+    const int col = col0 + wn * Cfg::TN + oc;
+    uint4 v = *reinterpret_cast<const uint4*>(so + rl * OLD + oc);
+    if (row < R && col + 8 <= N) *reinterpret_cast<uint4*>(Cb + (size_t)row * N + col) = v;
+  }
+}
+
+// Generic path (any Kd % 8 == 0): 128x128 tile, operands staged through
+// registers into padded LDS rows, out-of-range k chunks zero-filled.
+template <int EPI>
+__global__ __launch_bounds__(256) void gemm_bf16_generic_kernel(
+    const bf16_t* __restrict__ A, const bf16_t* __restrict__ Bt, const bf16_t* __restrict__ bias,
+    bf16_t* __restrict__ C, int R, int N, int Kd, int tiles_m, int tiles_n) {
+  constexpr int BM = 128, BN = 128, BK = 64, LD = BK + 8, NCH = 4;
+  __shared__ __align__(16) bf16_t lds[(BM + BN) * LD];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  const int m = lane & 31, h = lane >> 5;
+  const int per_batch = tiles_m * tiles_n;
+  const int b = blockIdx.x / per_batch;
+  const int rem = blockIdx.x - b * per_batch;
+  const int tile_n = rem / tiles_m, tile_m = rem - tile_n * tiles_m;
+  const int row0 = tile_m * BM, col0 = tile_n * BN;
+  const bf16_t* Ab = A + (size_t)b * R * Kd;
+  const bf16_t* Bb = Bt + (size_t)b * N * Kd;
+  const int kc8 = (tid & 7) * 8;
+  floatx16 acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+  for (int k0 = 0; k0 < Kd; k0 += BK) {
+    const bool ok = k0 + kc8 + 8 <= Kd;
+    const int kk = ok ? k0 + kc8 : Kd - 8;
+    uint4 ra[NCH], rb[NCH];
+#pragma unroll
+    for (int i = 0; i < NCH; ++i) {
+      const int r = (tid >> 3) + i * 32;
+      ra[i] = *reinterpret_cast<const uint4*>(Ab + (size_t)min(row0 + r, R - 1) * Kd + kk);
+      rb[i] = *reinterpret_cast<const uint4*>(Bb + (size_t)min(col0 + r, N - 1) * Kd + kk);
+      if (!ok) { ra[i] = make_uint4(0, 0, 0, 0); rb[i] = make_uint4(0, 0, 0, 0); }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < NCH; ++i) {
+      const int r = (tid >> 3) + i * 32;
+      *reinterpret_cast<uint4*>(lds + r * LD + kc8) = ra[i];
+      *reinterpret_cast<uint4*>(lds + (BM + r) * LD + kc8) = rb[i];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int ks = 0; ks < BK / 16; ++ks) {
+      bf16x8 fa[2], fb[2];
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        fa[i] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(
+            lds + (wm * 64 + i * 32 + m) * LD + ks * 16 + h * 8));
+        fb[i] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(
+            lds + (BM + wn * 64 + i * 32 + m) * LD + ks * 16 + h * 8));
+      }
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[j], fa[i], acc[i][j], 0, 0, 0);
+    }
+  }
   const bf16_t* biasb = bias != nullptr ? bias + (size_t)b * N : nullptr;
   bf16_t* Cb = C + (size_t)b * R * N;
 #pragma unroll
-  for (int j = 0; j < FN; ++j) {
-    const int col = col0 + wn * Cfg::TN + j * 32 + m;
-    const bool col_ok = col < N;
-    const float bv = (biasb != nullptr && col_ok) ? bf2f(biasb[col]) : 0.f;
+  for (int i = 0; i < 2; ++i) {
+    const int row = row0 + wm * 64 + i * 32 + m;
 #pragma unroll
-    for (int i = 0; i < FM; ++i) {
+    for (int j = 0; j < 2; ++j)
 #pragma unroll
       for (int v = 0; v < 16; ++v) {
-        const int row = row0 + wm * Cfg::TM + i * 32 + (v >> 2) * 8 + h * 4 + (v & 3);
-        float o = bf16r(acc[i][j][v]);
-        if (biasb != nullptr) o = bf16r(o + bv);
-        if (EPI == kEpiBiasGeluTanh) o = gelu_tanh(o);
-        if (EPI == kEpiBiasGeluErf) o = gelu_erf(o);
-        if (row < R && col_ok) Cb[(size_t)row * N + col] = f2bf(o);
+        const int col = col0 + wn * 64 + j * 32 + (v >> 2) * 8 + h * 4 + (v & 3);
+        if (row < R && col < N) {
+          float bv = biasb != nullptr ? bf2f(biasb[col]) : 0.f;
+          Cb[(size_t)row * N + col] = f2bf(apply_epilogue<EPI>(acc[i][j][v], bv, biasb != nullptr));
+        }
       }
-    }
   }
 }
 
 template <typename Cfg, int EPI>
 int launch_gemm_bf16(const bf16_t* A, const bf16_t* Bt, const bf16_t* bias, bf16_t* C, int batch,
                      int R, int N, int Kd, hipStream_t stream) {
+  if (Kd % Cfg::BK != 0 || (uint64_t)(R > N ? R : N) * Kd * 2 >= (1ull << 32)) {
+    const int tiles_m = (R + 127) / 128, tiles_n = (N + 127) / 128;
+    const long long blocks = (long long)batch * tiles_m * tiles_n;
+    if (blocks > 0x7fffffffLL) return VMOE_E_OVERFLOW;
+    hipLaunchKernelGGL(gemm_bf16_generic_kernel<EPI>, dim3((unsigned)blocks), dim3(256), 0, stream,
+                       A, Bt, bias, C, R, N, Kd, tiles_m, tiles_n);
+    return launch_status();
+  }
   const int tiles_m = (R + Cfg::BM - 1) / Cfg::BM;
   const int tiles_n = (N + Cfg::BN - 1) / Cfg::BN;
-  const long long blocks = (long long)batch * tiles_m * tiles_n;
-  if (blocks > 0x7fffffffLL) return VMOE_E_OVERFLOW;
+  const long long tiles = (long long)batch * tiles_m * tiles_n;
+  if (tiles > 0x7ffffff0LL) return VMOE_E_OVERFLOW;
+  const int tiles_per_xcd = (int)((tiles + kNumXcd - 1) / kNumXcd);
+  const unsigned blocks = (unsigned)tiles_per_xcd * kNumXcd;
   auto kern = gemm_bf16_kernel<Cfg, EPI>;
   hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                      hipFuncAttributeMaxDynamicSharedMemorySize,
                                      (int)Cfg::kLdsBytes);
   if (e != hipSuccess) return (int)e;
-  hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(Cfg::kThreads), Cfg::kLdsBytes, stream, A,
-                     Bt, bias, C, R, N, Kd, tiles_m, tiles_n);
+  hipLaunchKernelGGL(kern, dim3(blocks), dim3(Cfg::kThreads), Cfg::kLdsBytes, stream, A, Bt, bias,
+                     C, R, N, Kd, tiles_m, tiles_n, (int)tiles, tiles_per_xcd);
   return launch_status();
 }
 
