@@ -97,34 +97,60 @@ __global__ __launch_bounds__(kGateThreads) void gate_topk_kernel(
       const int k0 = c * KC;
       if (num_chunks > 1 || it == 0) {
         __syncthreads();
-        // Stage W[k0 : k0+KC, :] into LDS, zero padded in both directions.
-        for (int idx = tid; idx < KC * EP; idx += kGateThreads) {
-          int k = idx / EP, n = idx - k * EP;
-          T v = 0;
-          if (k0 + k < D && n < E) v = w[(size_t)(k0 + k) * E + n];
-          if (kBf16) wl[n * stride + k] = v; else wl[k * stride + n] = v;
+        // Stage W[k0 : k0+KC, :] into LDS, zero padded in both directions.  When
+        // a row of W is a whole number of 16-byte vectors the loads are vector
+        // loads, all independent, so the staging costs one memory round trip.
+        constexpr int VW = 16 / (int)sizeof(T);
+        if (E % VW == 0 && (reinterpret_cast<uintptr_t>(w) & 15u) == 0) {
+          const int vec_per_row = EP / VW;
+          for (int idx = tid; idx < KC * vec_per_row; idx += kGateThreads) {
+            const int k = idx / vec_per_row, n0 = (idx - k * vec_per_row) * VW;
+            uint4 raw = make_uint4(0, 0, 0, 0);
+            if (k0 + k < D && n0 < E)
+              raw = *reinterpret_cast<const uint4*>(w + (size_t)(k0 + k) * E + n0);
+            const T* v = reinterpret_cast<const T*>(&raw);
+#pragma unroll
+            for (int t = 0; t < VW; ++t) {
+              if (kBf16) wl[(n0 + t) * stride + k] = v[t]; else wl[k * stride + n0 + t] = v[t];
+            }
+          }
+        } else {
+          for (int idx = tid; idx < KC * EP; idx += kGateThreads) {
+            int k = idx / EP, n = idx - k * EP;
+            T v = 0;
+            if (k0 + k < D && n < E) v = w[(size_t)(k0 + k) * E + n];
+            if (kBf16) wl[n * stride + k] = v; else wl[k * stride + n] = v;
+          }
         }
         __syncthreads();
       }
       if (!active) continue;
       if constexpr (kBf16) {
         const int nkb = KC / 64;
-        for (int kb = 0; kb < nkb; ++kb) {
-          const int kl = kb * 64 + h * 32;  // this lane's 32 k's inside the chunk
-          uint4 a[4];
+        constexpr int UB = 3;   // 64-k blocks in flight per step (12 x 16-byte loads per lane)
+        for (int kb0 = 0; kb0 < nkb; kb0 += UB) {
+          uint4 a[UB][4];
 #pragma unroll
-          for (int j = 0; j < 4; ++j) {
-            int kg = k0 + kl + j * 8;
-            a[j] = (kg + 8 <= D) ? *reinterpret_cast<const uint4*>(xrow + kg) : make_uint4(0, 0, 0, 0);
-          }
+          for (int u = 0; u < UB; ++u)
 #pragma unroll
-          for (int j = 0; j < 4; ++j) {
-            bf16x8 af = __builtin_bit_cast(bf16x8, a[j]);
+            for (int j = 0; j < 4; ++j) {
+              int kg = k0 + (kb0 + u) * 64 + h * 32 + j * 8;
+              a[u][j] = (kb0 + u < nkb && kg + 8 <= D) ? *reinterpret_cast<const uint4*>(xrow + kg)
+                                                       : make_uint4(0, 0, 0, 0);
+            }
 #pragma unroll
-            for (int nt = 0; nt < NT; ++nt) {
-              uint4 b = *reinterpret_cast<const uint4*>(wl + (nt * 32 + m) * stride + kl + j * 8);
-              acc[nt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af, __builtin_bit_cast(bf16x8, b),
-                                                                acc[nt], 0, 0, 0);
+          for (int u = 0; u < UB; ++u) {
+            if (kb0 + u >= nkb) break;
+            const int kl = (kb0 + u) * 64 + h * 32;  // this lane's 32 k's inside the chunk
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+              bf16x8 af = __builtin_bit_cast(bf16x8, a[u][j]);
+#pragma unroll
+              for (int nt = 0; nt < NT; ++nt) {
+                uint4 b = *reinterpret_cast<const uint4*>(wl + (nt * 32 + m) * stride + kl + j * 8);
+                acc[nt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af, __builtin_bit_cast(bf16x8, b),
+                                                                  acc[nt], 0, 0, 0);
+              }
             }
           }
         }
@@ -254,43 +280,66 @@ __global__ __launch_bounds__(256) void topk_kernel(const float* __restrict__ gat
   }
 }
 
-// Per-group auxiliary losses.  One workgroup per group; thread (r, e) sums
-// column e over rows r, r+R, ... in a fixed order, partial sums are combined in
-// a fixed order, so results are run-to-run identical.
+// Per-group auxiliary losses.  One workgroup of 1024 threads per group; thread
+// (r, q) sums a strip of V expert columns over rows r, r+R, ... in a fixed
+// order, the R partial sums per column are then added in a fixed order, so
+// results are run-to-run identical.
+constexpr int kMetricThreads = 1024;
+
 template <typename T>
-__global__ __launch_bounds__(256) void router_metrics_kernel(
+__global__ __launch_bounds__(kMetricThreads) void router_metrics_kernel(
     const T* __restrict__ gates, const int32_t* __restrict__ top1, float* __restrict__ imp_loss,
     float* __restrict__ gsh_loss, float* __restrict__ aux_loss, float w_gsh, float w_imp,
-    int S, int E, int top1_stride) {
+    int S, int E, int top1_stride, int V) {
   extern __shared__ __align__(16) unsigned char smem[];
-  float* part = reinterpret_cast<float*>(smem);              // (R, E)
   const int tid = threadIdx.x;
   const int g = blockIdx.x;
-  const int cols = E < 256 ? E : 256;
-  const int R = 256 / cols;                                  // rows handled per pass
-  int* count = reinterpret_cast<int*>(part + (size_t)R * E);   // (E,)
+  const int strips = (E + V - 1) / V;                        // column strips per row
+  const int R = kMetricThreads / strips > 0 ? kMetricThreads / strips : 1;   // row lanes
+  float* part = reinterpret_cast<float*>(smem);              // (R, strips * V)
+  const int EW = strips * V;
+  int* count = reinterpret_cast<int*>(part + (size_t)R * EW);  // (E,)
   float* imp = reinterpret_cast<float*>(count + E);          // (E,)
-  for (int e = tid; e < E; e += 256) count[e] = 0;
+  for (int e = tid; e < E; e += kMetricThreads) count[e] = 0;
   __syncthreads();
-  const int r = tid / cols;
-  const int c = tid - r * cols;
+  const int r = tid / strips;
+  const int q = tid - r * strips;
   if (r < R) {
-    for (int e = c; e < E; e += cols) {
-      float s = 0.f;
-      for (int i = r; i < S; i += R) s += Elt<T>::load(gates + ((size_t)g * S + i) * E + e);
-      part[r * E + e] = s;
+    float s[8];
+#pragma unroll
+    for (int t = 0; t < 8; ++t) s[t] = 0.f;
+    const T* base = gates + (size_t)g * S * E + q * V;
+    if (V == 16 / (int)sizeof(T)) {
+      // One 16-byte load per row (E is a multiple of V and rows are 16-byte aligned).
+      for (int i = r; i < S; i += R) {
+        const uint4 raw = *reinterpret_cast<const uint4*>(base + (size_t)i * E);
+        const T* v = reinterpret_cast<const T*>(&raw);
+#pragma unroll
+        for (int t = 0; t < (int)(16 / sizeof(T)); ++t) s[t] += Elt<T>::load(&v[t]);
+      }
+    } else {
+      for (int i = r; i < S; i += R)
+        for (int t = 0; t < V; ++t)
+          if (q * V + t < E) s[t] += Elt<T>::load(base + (size_t)i * E + t);
     }
+    for (int t = 0; t < V; ++t) part[(size_t)r * EW + q * V + t] = s[t];
   }
-  for (int i = tid; i < S; i += 256) {
+  for (int i = tid; i < S; i += kMetricThreads) {
     int t = top1[((size_t)g * S + i) * top1_stride];
     if (t >= 0 && t < E) atomicAdd(&count[t], 1);
   }
   __syncthreads();
-  for (int e = tid; e < E; e += 256) {
-    float s = 0.f;
-    for (int rr = 0; rr < R; ++rr) s += part[rr * E + e];
-    imp[e] = s;
+  // Fixed-order tree over the row lanes.
+  int span = 1;
+  while (span < R) span <<= 1;
+  for (int off = span >> 1; off > 0; off >>= 1) {
+    for (int idx = tid; idx < off * EW; idx += kMetricThreads) {
+      int rr = idx / EW, c = idx - rr * EW;
+      if (rr + off < R) part[(size_t)rr * EW + c] += part[(size_t)(rr + off) * EW + c];
+    }
+    __syncthreads();
   }
+  for (int e = tid; e < E; e += kMetricThreads) imp[e] = part[e];
   __syncthreads();
   if (tid == 0) {
     float mean = 0.f;
@@ -384,18 +433,23 @@ extern "C" int vmoe_router_metrics(const VmoeRouterMetricsParams* p, vmoe_stream
   if (p->G < 1 || p->S < 1 || p->E < 1 || p->top1_stride < 1) return VMOE_E_SHAPE;
   if (p->dtype != VMOE_F32 && p->dtype != VMOE_BF16) return VMOE_E_DTYPE;
   if (p->E > 1024) return VMOE_E_UNSUPPORTED;
-  const int cols = p->E < 256 ? p->E : 256;
-  const int R = 256 / cols;
-  const size_t lds = ((size_t)R * p->E + 2 * (size_t)p->E) * 4;
+  const int esz = p->dtype == VMOE_BF16 ? 2 : 4;
+  const int vec = 16 / esz;
+  const bool vec_ok = p->E % vec == 0 && aligned16(p->gates);
+  const int V = vec_ok ? vec : 1;
+  const int strips = (p->E + V - 1) / V;
+  const int R = kMetricThreads / strips > 0 ? kMetricThreads / strips : 1;
+  const size_t lds = ((size_t)R * strips * V + 2 * (size_t)p->E) * 4;
+  if (lds > 64 * 1024) return VMOE_E_UNSUPPORTED;
   if (p->dtype == VMOE_BF16)
-    hipLaunchKernelGGL(router_metrics_kernel<bf16_t>, dim3(p->G), dim3(256), lds, as_stream(stream),
-                       (const bf16_t*)p->gates, p->top1_idx, p->importance_loss, p->gshard_loss,
-                       p->auxiliary_loss, p->gshard_loss_weight, p->importance_loss_weight, p->S,
-                       p->E, p->top1_stride);
+    hipLaunchKernelGGL(router_metrics_kernel<bf16_t>, dim3(p->G), dim3(kMetricThreads), lds,
+                       as_stream(stream), (const bf16_t*)p->gates, p->top1_idx, p->importance_loss,
+                       p->gshard_loss, p->auxiliary_loss, p->gshard_loss_weight,
+                       p->importance_loss_weight, p->S, p->E, p->top1_stride, V);
   else
-    hipLaunchKernelGGL(router_metrics_kernel<float>, dim3(p->G), dim3(256), lds, as_stream(stream),
-                       (const float*)p->gates, p->top1_idx, p->importance_loss, p->gshard_loss,
-                       p->auxiliary_loss, p->gshard_loss_weight, p->importance_loss_weight, p->S,
-                       p->E, p->top1_stride);
+    hipLaunchKernelGGL(router_metrics_kernel<float>, dim3(p->G), dim3(kMetricThreads), lds,
+                       as_stream(stream), (const float*)p->gates, p->top1_idx, p->importance_loss,
+                       p->gshard_loss, p->auxiliary_loss, p->gshard_loss_weight,
+                       p->importance_loss_weight, p->S, p->E, p->top1_stride, V);
   return launch_status();
 }

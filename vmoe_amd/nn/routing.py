@@ -62,7 +62,7 @@ class NoisyTopExpertsPerItemRouter(module.Module):
           "use deterministic=True or noise_std=0.")
     dtype = self.dtype or inputs.dtype
     x = K.cast(inputs, dtype)
-    w = K.cast(kernel, dtype)
+    w = self._cast_kernel(kernel, dtype)
     gates, val, idx = K.gate_topk(x, w, self.num_selected_experts, logit_bias=self.logit_bias)
     importance_loss, gshard_loss, auxiliary_loss = K.router_metrics(
         gates, idx, self.gshard_loss_weight, self.importance_loss_weight)
@@ -72,6 +72,18 @@ class NoisyTopExpertsPerItemRouter(module.Module):
         "importance_loss": importance_loss,
     }
     return gates, metrics, (val, idx)
+
+  def _cast_kernel(self, kernel: Array, dtype) -> Array:
+    """The router kernel in the compute dtype; the cast of a parameter tensor is
+    done once and reused until the tensor changes."""
+    if kernel.dtype == dtype:
+      return kernel
+    key = (kernel.data_ptr(), kernel._version, dtype)
+    cached = getattr(self, "_kernel_cache", None)
+    if cached is None or cached[0] != key:
+      cached = (key, K.cast(kernel, dtype))
+      self._kernel_cache = cached
+    return cached[1]
 
   def _create_dispatcher(self, gates_dispatch: Array, topk=None):
     dispatcher_kwargs = dict(**(self.dispatcher or {}))
