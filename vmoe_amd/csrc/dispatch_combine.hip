@@ -12,18 +12,76 @@
 // so there are no atomics and the result is bit-deterministic.
 // combine is item-major as well: <= K row reads, float32 multiply and add in k
 // order (no fused multiply-add, to match a float32 einsum), one rounded store.
-// One wave moves kRows rows per step with 16-byte accesses per lane, all loads
-// of a step issued before the first store.
+// Work is flattened over (row, 16-byte chunk), eight rows per workgroup, so all
+// lanes carry data for any row width; accesses carry the non-temporal hint.
 #include "vmoe_common.h"
 
 namespace vmoe {
 namespace {
 
-constexpr int kRows = 4;          // rows per wave per step
-constexpr int kZeroSlots = 16;    // slots checked per zero-fill wave
+constexpr int kRowsPerBlock = 8;   // item rows (or slot rows) moved by one workgroup
 constexpr int kMoveThreads = 256;
+constexpr int kMaxK = 8;           // choices per item held in LDS; larger K takes the generic kernels
 
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+
+// Streaming accesses: every row is touched once per kernel, so loads and stores
+// carry the non-temporal hint.
+__device__ __forceinline__ uint4 load_stream(const uint4* p) {
+  return __builtin_bit_cast(uint4, __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p)));
+}
+__device__ __forceinline__ void store_stream(uint4* p, const uint4& v) {
+  __builtin_nontemporal_store(__builtin_bit_cast(u32x4, v), reinterpret_cast<u32x4*>(p));
+}
+
+// idx / cpr for idx < 2^16 with magic = ceil(2^32 / cpr); magic == 0 encodes cpr == 1.
+__device__ __forceinline__ int div_chunks(int idx, uint32_t magic) {
+  return magic == 0 ? idx : (int)__umulhi((uint32_t)idx, magic);
+}
+
+// Work is flattened over (row, 16-byte chunk) so that every lane of every wave
+// moves data whatever the row width: thread t of a workgroup handles chunks
+// t, t+256, ... of the workgroup's kRowsPerBlock rows.
 __global__ __launch_bounds__(kMoveThreads) void dispatch_kernel(
+    const uint4* __restrict__ x, const int32_t* __restrict__ token_slot,
+    const int32_t* __restrict__ slot_token, uint4* __restrict__ out, int num_items, int num_slots,
+    int K, int cpr, uint32_t magic, int item_blocks) {
+  __shared__ int32_t slots[kRowsPerBlock * kMaxK];
+  const int tid = threadIdx.x;
+  const int total = kRowsPerBlock * cpr;
+  if ((int)blockIdx.x < item_blocks) {
+    const int t0 = blockIdx.x * kRowsPerBlock;
+    if (tid < kRowsPerBlock * K) {
+      const int r = tid / K;
+      slots[tid] = t0 + r < num_items ? token_slot[(size_t)t0 * K + tid] : -1;
+    }
+    __syncthreads();
+    for (int idx = tid; idx < total; idx += kMoveThreads) {
+      const int r = div_chunks(idx, magic);
+      const int ch = idx - r * cpr;
+      if (t0 + r >= num_items) continue;
+      const uint4 v = load_stream(x + (size_t)(t0 + r) * cpr + ch);
+      for (int k = 0; k < K; ++k) {
+        const int slot = slots[r * K + k];
+        if (slot >= 0) store_stream(out + (size_t)slot * cpr + ch, v);
+      }
+    }
+  } else {
+    // Zero-fill of the slots no item claimed.
+    const int s0 = (blockIdx.x - item_blocks) * kRowsPerBlock;
+    if (tid < kRowsPerBlock) slots[tid] = s0 + tid < num_slots ? slot_token[s0 + tid] : 0;
+    __syncthreads();
+    const uint4 z = make_uint4(0, 0, 0, 0);
+    for (int idx = tid; idx < total; idx += kMoveThreads) {
+      const int r = div_chunks(idx, magic);
+      const int ch = idx - r * cpr;
+      if (slots[r] < 0) store_stream(out + (size_t)(s0 + r) * cpr + ch, z);
+    }
+  }
+}
+
+// Any K (choices read from global memory), one wave per item row.
+__global__ __launch_bounds__(kMoveThreads) void dispatch_generic_kernel(
     const uint4* __restrict__ x, const int32_t* __restrict__ token_slot,
     const int32_t* __restrict__ slot_token, uint4* __restrict__ out, int num_items, int num_slots,
     int K, int cpr, int item_waves) {
@@ -31,30 +89,17 @@ __global__ __launch_bounds__(kMoveThreads) void dispatch_kernel(
   const int wave = __builtin_amdgcn_readfirstlane(
       (int)((blockIdx.x * (unsigned)kMoveThreads + threadIdx.x) >> 6));
   if (wave < item_waves) {
-    const int t0 = wave * kRows;
     for (int ch = lane; ch < cpr; ch += kWave) {
-      uint4 v[kRows];
-#pragma unroll
-      for (int r = 0; r < kRows; ++r)
-        if (t0 + r < num_items) v[r] = x[(size_t)(t0 + r) * cpr + ch];
-#pragma unroll
-      for (int r = 0; r < kRows; ++r) {
-        if (t0 + r < num_items) {
-          for (int k = 0; k < K; ++k) {
-            int slot = token_slot[(size_t)(t0 + r) * K + k];
-            if (slot >= 0) out[(size_t)slot * cpr + ch] = v[r];
-          }
-        }
+      const uint4 v = x[(size_t)wave * cpr + ch];
+      for (int k = 0; k < K; ++k) {
+        int slot = token_slot[(size_t)wave * K + k];
+        if (slot >= 0) out[(size_t)slot * cpr + ch] = v;
       }
     }
   } else {
-    const int s0 = (wave - item_waves) * kZeroSlots;
-    const uint4 z = make_uint4(0, 0, 0, 0);
-    for (int i = 0; i < kZeroSlots; ++i) {
-      int s = s0 + i;
-      if (s < num_slots && slot_token[s] < 0)
-        for (int ch = lane; ch < cpr; ch += kWave) out[(size_t)s * cpr + ch] = z;
-    }
+    const int s = wave - item_waves;
+    if (s < num_slots && slot_token[s] < 0)
+      for (int ch = lane; ch < cpr; ch += kWave) out[(size_t)s * cpr + ch] = make_uint4(0, 0, 0, 0);
   }
 }
 
@@ -88,82 +133,102 @@ template <> struct Chunk<bf16_t> {
   }
 };
 
-constexpr int kMaxK = 8;  // register-resident fast path; larger K takes the generic loop
-
 template <typename T>
 __global__ __launch_bounds__(kMoveThreads) void combine_kernel(
+    const uint4* __restrict__ y, const int32_t* __restrict__ token_slot,
+    const float* __restrict__ weights, uint4* __restrict__ out, int num_items, int K, int cpr,
+    uint32_t magic) {
+  constexpr int N = Chunk<T>::n;
+  __shared__ int32_t slots[kRowsPerBlock * kMaxK];
+  __shared__ float wts[kRowsPerBlock * kMaxK];
+  const int tid = threadIdx.x;
+  const int t0 = blockIdx.x * kRowsPerBlock;
+  if (tid < kRowsPerBlock * K) {
+    const int r = tid / K;
+    const bool ok = t0 + r < num_items;
+    slots[tid] = ok ? token_slot[(size_t)t0 * K + tid] : -1;
+    wts[tid] = ok ? weights[(size_t)t0 * K + tid] : 0.f;
+  }
+  __syncthreads();
+  const int total = kRowsPerBlock * cpr;
+  for (int idx = tid; idx < total; idx += kMoveThreads) {
+    const int r = div_chunks(idx, magic);
+    const int ch = idx - r * cpr;
+    if (t0 + r >= num_items) continue;
+    float acc[N];
+    if (K == 2) {
+      // Both reads in flight before any arithmetic.
+      const int s0 = slots[r * 2], s1 = slots[r * 2 + 1];
+      uint4 v0 = make_uint4(0, 0, 0, 0), v1 = v0;
+      if (s0 >= 0) v0 = load_stream(y + (size_t)s0 * cpr + ch);
+      if (s1 >= 0) v1 = load_stream(y + (size_t)s1 * cpr + ch);
+      float a[N], b[N];
+      Chunk<T>::unpack(v0, a);
+      Chunk<T>::unpack(v1, b);
+      const float w0 = wts[r * 2], w1 = wts[r * 2 + 1];
+#pragma unroll
+      for (int j = 0; j < N; ++j) {
+        float p0 = s0 >= 0 ? __fmul_rn(w0, a[j]) : 0.f;
+        float p1 = s1 >= 0 ? __fmul_rn(w1, b[j]) : 0.f;
+        acc[j] = __fadd_rn(p0, p1);
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < N; ++j) acc[j] = 0.f;
+      for (int k = 0; k < K; ++k) {
+        const int slot = slots[r * K + k];
+        if (slot < 0) continue;
+        const float w = wts[r * K + k];
+        float a[N];
+        Chunk<T>::unpack(load_stream(y + (size_t)slot * cpr + ch), a);
+#pragma unroll
+        for (int j = 0; j < N; ++j) acc[j] = __fadd_rn(acc[j], __fmul_rn(w, a[j]));
+      }
+    }
+    store_stream(out + (size_t)(t0 + r) * cpr + ch, Chunk<T>::pack(acc));
+  }
+}
+
+// Any K, one wave per item row.
+template <typename T>
+__global__ __launch_bounds__(kMoveThreads) void combine_generic_kernel(
     const uint4* __restrict__ y, const int32_t* __restrict__ token_slot,
     const float* __restrict__ weights, uint4* __restrict__ out, int num_items, int K, int cpr) {
   constexpr int N = Chunk<T>::n;
   const int lane = threadIdx.x & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(
+  const int t = __builtin_amdgcn_readfirstlane(
       (int)((blockIdx.x * (unsigned)kMoveThreads + threadIdx.x) >> 6));
-  const int t0 = wave * kRows;
-  if (t0 >= num_items) return;
-  if (K == 2) {
-    // The common case: both reads of all rows in flight before any arithmetic.
-    for (int ch = lane; ch < cpr; ch += kWave) {
-      uint4 v[kRows][2];
-      int slot[kRows][2];
-      float w[kRows][2];
+  if (t >= num_items) return;
+  for (int ch = lane; ch < cpr; ch += kWave) {
+    float acc[N];
 #pragma unroll
-      for (int r = 0; r < kRows; ++r)
+    for (int j = 0; j < N; ++j) acc[j] = 0.f;
+    for (int k = 0; k < K; ++k) {
+      int slot = token_slot[(size_t)t * K + k];
+      if (slot < 0) continue;
+      float w = weights[(size_t)t * K + k];
+      float a[N];
+      Chunk<T>::unpack(y[(size_t)slot * cpr + ch], a);
 #pragma unroll
-        for (int k = 0; k < 2; ++k) {
-          bool ok = t0 + r < num_items;
-          slot[r][k] = ok ? token_slot[(size_t)(t0 + r) * 2 + k] : -1;
-          w[r][k] = ok ? weights[(size_t)(t0 + r) * 2 + k] : 0.f;
-          v[r][k] = make_uint4(0, 0, 0, 0);
-          if (slot[r][k] >= 0) v[r][k] = y[(size_t)slot[r][k] * cpr + ch];
-        }
-#pragma unroll
-      for (int r = 0; r < kRows; ++r) {
-        if (t0 + r >= num_items) continue;
-        float a[N], b[N], o[N];
-        Chunk<T>::unpack(v[r][0], a);
-        Chunk<T>::unpack(v[r][1], b);
-#pragma unroll
-        for (int j = 0; j < N; ++j) {
-          float p0 = slot[r][0] >= 0 ? __fmul_rn(w[r][0], a[j]) : 0.f;
-          float p1 = slot[r][1] >= 0 ? __fmul_rn(w[r][1], b[j]) : 0.f;
-          o[j] = __fadd_rn(p0, p1);
-        }
-        out[(size_t)(t0 + r) * cpr + ch] = Chunk<T>::pack(o);
-      }
+      for (int j = 0; j < N; ++j) acc[j] = __fadd_rn(acc[j], __fmul_rn(w, a[j]));
     }
-    return;
-  }
-  for (int r = 0; r < kRows; ++r) {
-    const int t = t0 + r;
-    if (t >= num_items) break;
-    for (int ch = lane; ch < cpr; ch += kWave) {
-      float acc[N];
-#pragma unroll
-      for (int j = 0; j < N; ++j) acc[j] = 0.f;
-      for (int k = 0; k < K; ++k) {
-        int slot = token_slot[(size_t)t * K + k];
-        if (slot < 0) continue;
-        float w = weights[(size_t)t * K + k];
-        float a[N];
-        Chunk<T>::unpack(y[(size_t)slot * cpr + ch], a);
-#pragma unroll
-        for (int j = 0; j < N; ++j) acc[j] = __fadd_rn(acc[j], __fmul_rn(w, a[j]));
-      }
-      out[(size_t)t * cpr + ch] = Chunk<T>::pack(acc);
-    }
+    out[(size_t)t * cpr + ch] = Chunk<T>::pack(acc);
   }
 }
 
+// Grid-stride streaming copy: the bandwidth yardstick.
 __global__ __launch_bounds__(256) void copy_kernel(const uint4* __restrict__ in,
                                                    uint4* __restrict__ out, size_t n16) {
-  size_t i = (size_t)blockIdx.x * 256 * 4 + threadIdx.x;
-  uint4 v[4];
+  const size_t stride = (size_t)gridDim.x * 256 * 4;
+  for (size_t i = (size_t)blockIdx.x * 256 * 4 + threadIdx.x; i < n16; i += stride) {
+    uint4 v[4];
 #pragma unroll
-  for (int j = 0; j < 4; ++j)
-    if (i + j * 256 < n16) v[j] = in[i + j * 256];
+    for (int j = 0; j < 4; ++j)
+      if (i + j * 256 < n16) v[j] = load_stream(in + i + j * 256);
 #pragma unroll
-  for (int j = 0; j < 4; ++j)
-    if (i + j * 256 < n16) out[i + j * 256] = v[j];
+    for (int j = 0; j < 4; ++j)
+      if (i + j * 256 < n16) store_stream(out + i + j * 256, v[j]);
+  }
 }
 
 __global__ __launch_bounds__(256) void cast_f32_to_bf16_kernel(const float* __restrict__ in,
@@ -209,18 +274,30 @@ int check_move(const void* a, const void* b, const void* c, int num_items, int n
 
 using namespace vmoe;
 
+static uint32_t chunk_magic(int cpr) {
+  return cpr == 1 ? 0u : (uint32_t)(((1ull << 32) + cpr - 1) / cpr);
+}
+
 extern "C" int vmoe_dispatch(const VmoeDispatchParams* p, vmoe_stream_t stream) {
   if (p == nullptr || p->token_slot == nullptr || p->slot_token == nullptr) return VMOE_E_NULL;
   int rc = check_move(p->x, p->token_slot, p->out, p->num_items, p->num_slots, p->K, p->D, p->dtype);
   if (rc != VMOE_OK) return rc;
   const int cpr = (int)((size_t)p->D * (p->dtype == VMOE_BF16 ? 2 : 4) / 16);
-  const int item_waves = (p->num_items + kRows - 1) / kRows;
-  const int zero_waves = (p->num_slots + kZeroSlots - 1) / kZeroSlots;
-  const int waves_per_block = kMoveThreads / kWave;
-  const int blocks = (item_waves + zero_waves + waves_per_block - 1) / waves_per_block;
-  hipLaunchKernelGGL(dispatch_kernel, dim3(blocks), dim3(kMoveThreads), 0, as_stream(stream),
-                     (const uint4*)p->x, p->token_slot, p->slot_token, (uint4*)p->out,
-                     p->num_items, p->num_slots, p->K, cpr, item_waves);
+  if (p->K <= kMaxK && kRowsPerBlock * cpr < 65536) {
+    const int item_blocks = (p->num_items + kRowsPerBlock - 1) / kRowsPerBlock;
+    const int zero_blocks = (p->num_slots + kRowsPerBlock - 1) / kRowsPerBlock;
+    hipLaunchKernelGGL(dispatch_kernel, dim3(item_blocks + zero_blocks), dim3(kMoveThreads), 0,
+                       as_stream(stream), (const uint4*)p->x, p->token_slot, p->slot_token,
+                       (uint4*)p->out, p->num_items, p->num_slots, p->K, cpr, chunk_magic(cpr),
+                       item_blocks);
+  } else {
+    const long long waves = (long long)p->num_items + p->num_slots;
+    const long long blocks = (waves + 3) / 4;
+    if (blocks > 0x7fffffffLL) return VMOE_E_OVERFLOW;
+    hipLaunchKernelGGL(dispatch_generic_kernel, dim3((unsigned)blocks), dim3(kMoveThreads), 0,
+                       as_stream(stream), (const uint4*)p->x, p->token_slot, p->slot_token,
+                       (uint4*)p->out, p->num_items, p->num_slots, p->K, cpr, p->num_items);
+  }
   return launch_status();
 }
 
@@ -229,17 +306,28 @@ extern "C" int vmoe_combine(const VmoeCombineParams* p, vmoe_stream_t stream) {
   int rc = check_move(p->y, p->token_slot, p->out, p->num_items, p->num_slots, p->K, p->D, p->dtype);
   if (rc != VMOE_OK) return rc;
   const int cpr = (int)((size_t)p->D * (p->dtype == VMOE_BF16 ? 2 : 4) / 16);
-  const int waves = (p->num_items + kRows - 1) / kRows;
-  const int waves_per_block = kMoveThreads / kWave;
-  const int blocks = (waves + waves_per_block - 1) / waves_per_block;
-  if (p->dtype == VMOE_BF16)
-    hipLaunchKernelGGL(combine_kernel<bf16_t>, dim3(blocks), dim3(kMoveThreads), 0,
-                       as_stream(stream), (const uint4*)p->y, p->token_slot, p->weights,
-                       (uint4*)p->out, p->num_items, p->K, cpr);
-  else
-    hipLaunchKernelGGL(combine_kernel<float>, dim3(blocks), dim3(kMoveThreads), 0,
-                       as_stream(stream), (const uint4*)p->y, p->token_slot, p->weights,
-                       (uint4*)p->out, p->num_items, p->K, cpr);
+  const bool bf16 = p->dtype == VMOE_BF16;
+  if (p->K <= kMaxK && kRowsPerBlock * cpr < 65536) {
+    const int blocks = (p->num_items + kRowsPerBlock - 1) / kRowsPerBlock;
+    if (bf16)
+      hipLaunchKernelGGL(combine_kernel<bf16_t>, dim3(blocks), dim3(kMoveThreads), 0,
+                         as_stream(stream), (const uint4*)p->y, p->token_slot, p->weights,
+                         (uint4*)p->out, p->num_items, p->K, cpr, chunk_magic(cpr));
+    else
+      hipLaunchKernelGGL(combine_kernel<float>, dim3(blocks), dim3(kMoveThreads), 0,
+                         as_stream(stream), (const uint4*)p->y, p->token_slot, p->weights,
+                         (uint4*)p->out, p->num_items, p->K, cpr, chunk_magic(cpr));
+  } else {
+    const int blocks = (p->num_items + 3) / 4;
+    if (bf16)
+      hipLaunchKernelGGL(combine_generic_kernel<bf16_t>, dim3(blocks), dim3(kMoveThreads), 0,
+                         as_stream(stream), (const uint4*)p->y, p->token_slot, p->weights,
+                         (uint4*)p->out, p->num_items, p->K, cpr);
+    else
+      hipLaunchKernelGGL(combine_generic_kernel<float>, dim3(blocks), dim3(kMoveThreads), 0,
+                         as_stream(stream), (const uint4*)p->y, p->token_slot, p->weights,
+                         (uint4*)p->out, p->num_items, p->K, cpr);
+  }
   return launch_status();
 }
 
@@ -247,8 +335,8 @@ extern "C" int vmoe_copy_bytes(const void* in, void* out, size_t n, vmoe_stream_
   if (in == nullptr || out == nullptr) return VMOE_E_NULL;
   if (n == 0 || n % 16 != 0 || !aligned16(in) || !aligned16(out)) return VMOE_E_ALIGN;
   const size_t n16 = n / 16;
-  const size_t blocks = (n16 + 1023) / 1024;
-  if (blocks > 0x7fffffffull) return VMOE_E_OVERFLOW;
+  size_t blocks = (n16 + 1023) / 1024;
+  if (blocks > 4096) blocks = 4096;
   hipLaunchKernelGGL(copy_kernel, dim3((unsigned)blocks), dim3(256), 0, as_stream(stream),
                      (const uint4*)in, (uint4*)out, n16);
   return launch_status();

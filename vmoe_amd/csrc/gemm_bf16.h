@@ -5,13 +5,20 @@
 //
 // Tiling: a workgroup of WM x WN waves computes a BM x BN tile; each wave owns
 // (BM/WM) x (BN/WN) of it as a grid of 32x32 v_mfma_f32_32x32x16_bf16 tiles held
-// in accumulator registers.  K advances in steps of BK = 64 through two LDS
-// stages: the global loads of step k+1 are issued into registers before the
-// MFMAs of step k and written to the other stage while the last MFMAs of step k
-// run, one barrier per step.  Inside a step the LDS fragment reads of the next
-// 16-wide k slice are issued before the MFMAs of the current one (double
-// buffered fragment registers).  LDS rows are padded by 16 bytes so that the
-// eight lanes served per clock hit all 32 banks.
+// in accumulator registers.
+//
+// Operand path: global memory -> LDS directly (global_load_lds_dwordx4), no
+// staging registers and no LDS write instructions.  A wave-wide load fills 1 KiB
+// of consecutive LDS, lane L landing at base + 16*L, so each lane fetches the
+// global 16-byte chunk that an XOR swizzle assigns to its LDS slot; the swizzle
+// makes the 128-bit fragment reads conflict-free on the 64 LDS banks.
+//
+// Pipeline: K advances in BK-wide tiles through a ring of NSTAGE LDS stages; the
+// DMA loads run NSTAGE-1 tiles ahead and are never drained (s_waitcnt vmcnt(n)
+// covers only the tile needed next).  Inside a tile the fragment reads of the
+// next 16-wide k slice are issued under the MFMAs of the current one (double
+// buffered fragment registers), and the tile's one barrier sits before its last
+// slice so that the next tile's first fragments are fetched under MFMAs too.
 //
 // The MFMA is issued with the weight fragment as its first operand, so the
 // accumulator tile is C^T: a lane ends up with 4 consecutive output columns of
@@ -90,24 +97,91 @@ __device__ __forceinline__ void wait_vmcnt() {
   __builtin_amdgcn_s_waitcnt(0x0f70 | (N & 15) | ((N >> 4) << 14));
 }
 __device__ __forceinline__ void wait_lgkmcnt0() { __builtin_amdgcn_s_waitcnt(0xc07f); }
-
-#ifdef VMOE_GEMM_DEBUG_SAME_TILE
-#define VMOE_DBG_ROW(x) 0
-#define VMOE_DBG_BATCH(x) 0
-#else
-#define VMOE_DBG_ROW(x) (x)
-#define VMOE_DBG_BATCH(x) (x)
-#endif
-#ifdef VMOE_GEMM_DEBUG_NO_XCD
-#define VMOE_DBG_LOGICAL(expr) ((int)blockIdx.x)
-#else
-#define VMOE_DBG_LOGICAL(expr) (expr)
-#endif
+// Workgroup barrier without the implicit "wait for every outstanding memory
+// operation" of __syncthreads(): callers wait for exactly what they need first.
+// The asm clobbers keep the compiler from moving LDS accesses across it.
+__device__ __forceinline__ void raw_barrier() {
+  asm volatile("" ::: "memory");
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
+  __builtin_amdgcn_sched_barrier(0);
+}
 
 typedef const __attribute__((address_space(1))) void* global_ptr_t;
 typedef __attribute__((address_space(3))) void* lds_ptr_t;
 
-// Fast path: Kd % 64 == 0.  Global tiles go straight into LDS
+// Epilogue of one wave: acc[i][j][v] = C[wrow0 + i*32 + m][wcol0 + j*32 + (v/4)*8 + h*4 + v%4]
+// (the MFMA was issued with the weight fragment first, so a lane holds 4
+// consecutive columns of one row).  Bias, rounding, GELU and the bf16 pack happen
+// in registers; the wave tile is staged in a wave-private LDS region and leaves
+// as 16-byte, row-contiguous global stores.
+template <int EPI, int TM, int TN>
+__device__ __forceinline__ void store_tile(floatx16 (&acc)[TM / 32][TN / 32], unsigned char* smem,
+                                           int wave, int lane, const bf16_t* __restrict__ bias,
+                                           bf16_t* __restrict__ C, int b, int R, int N, int wrow0,
+                                           int wcol0) {
+  constexpr int FM = TM / 32, FN = TN / 32, OLD = TN + 8;
+  const int m = lane & 31, h = lane >> 5;
+  const bf16_t* biasb = bias != nullptr ? bias + (size_t)b * N : nullptr;
+  bf16_t* Cb = C + (size_t)b * R * N;
+  bf16_t* so = reinterpret_cast<bf16_t*>(smem) + (size_t)wave * TM * OLD;
+#pragma unroll
+  for (int j = 0; j < FN; ++j) {
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const int cl = j * 32 + q * 8 + h * 4;          // column inside the wave tile
+      const int col = wcol0 + cl;
+      float bv[4] = {0.f, 0.f, 0.f, 0.f};
+      if (biasb != nullptr) {
+#pragma unroll
+        for (int t = 0; t < 4; ++t) bv[t] = bf2f(biasb[min(col + t, N - 1)]);
+      }
+#pragma unroll
+      for (int i = 0; i < FM; ++i) {
+        uint32_t p[2];
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+          float o0 = apply_epilogue<EPI>(acc[i][j][q * 4 + 2 * t], bv[2 * t], biasb != nullptr);
+          float o1 = apply_epilogue<EPI>(acc[i][j][q * 4 + 2 * t + 1], bv[2 * t + 1], biasb != nullptr);
+          p[t] = (uint32_t)f2bf(o0) | ((uint32_t)f2bf(o1) << 16);
+        }
+        *reinterpret_cast<uint2*>(so + (i * 32 + m) * OLD + cl) = make_uint2(p[0], p[1]);
+      }
+    }
+  }
+  // Each wave reads back only what it wrote (LDS operations of a wave complete in order).
+  constexpr int kChunksOut = TN / 8;                  // 16-byte chunks per staged row
+  constexpr int kRowsPerPass = 64 / kChunksOut;
+  static_assert(64 % kChunksOut == 0, "wave tile width must divide a wave");
+  const int oc = (lane % kChunksOut) * 8;
+  const int orow = lane / kChunksOut;
+#pragma unroll
+  for (int r0 = 0; r0 < TM; r0 += kRowsPerPass) {
+    const int rl = r0 + orow;
+    const int row = wrow0 + rl;
+    const int col = wcol0 + oc;
+    uint4 v = *reinterpret_cast<const uint4*>(so + rl * OLD + oc);
+    if (row < R && col + 8 <= N) *reinterpret_cast<uint4*>(Cb + (size_t)row * N + col) = v;
+  }
+}
+
+// XCD-aware workgroup -> (batch, tile_m, tile_n); returns false for padding workgroups.
+__device__ __forceinline__ bool map_tile(int tiles_m, int tiles_n, int num_tiles, int tiles_per_xcd,
+                                         int& b, int& tile_m, int& tile_n) {
+  const int logical = (blockIdx.x % kNumXcd) * tiles_per_xcd + blockIdx.x / kNumXcd;
+  if (blockIdx.x / kNumXcd >= tiles_per_xcd || logical >= num_tiles) return false;
+  const int per_batch = tiles_m * tiles_n;
+  b = logical / per_batch;
+  const int rem = logical - b * per_batch;
+  const int panel = rem / (kPanelRows * tiles_n);
+  const int in_panel = rem - panel * kPanelRows * tiles_n;
+  const int rows_here = min(kPanelRows, tiles_m - panel * kPanelRows);
+  tile_n = in_panel / rows_here;
+  tile_m = panel * kPanelRows + in_panel - tile_n * rows_here;
+  return true;
+}
+
+// Fast path: Kd % BK == 0.  Global tiles go straight into LDS
 // (global_load_lds_dwordx4: lane L of a wave lands at base + 16*L), so lane L
 // fetches the global chunk that the XOR swizzle assigns to LDS slot L:
 // row = L/8, slot = L%8, chunk = slot ^ (row & 7).
@@ -126,20 +200,11 @@ __global__ __launch_bounds__(Cfg::kThreads, Cfg::kBlocksPerCu) void gemm_bf16_ke
   const int wm = wave / Cfg::WN, wn = wave % Cfg::WN;
   const int m = lane & 31, h = lane >> 5;
 
-  // XCD-aware logical tile id.
-  const int logical = VMOE_DBG_LOGICAL((blockIdx.x % kNumXcd) * tiles_per_xcd + blockIdx.x / kNumXcd);
-  if (blockIdx.x / kNumXcd >= tiles_per_xcd || logical >= num_tiles) return;
-  const int per_batch = tiles_m * tiles_n;
-  const int b = logical / per_batch;
-  const int rem = logical - b * per_batch;
-  const int panel = rem / (kPanelRows * tiles_n);
-  const int in_panel = rem - panel * kPanelRows * tiles_n;
-  const int rows_here = min(kPanelRows, tiles_m - panel * kPanelRows);
-  const int tile_n = in_panel / rows_here;
-  const int tile_m = panel * kPanelRows + in_panel - tile_n * rows_here;
+  int b, tile_m, tile_n;
+  if (!map_tile(tiles_m, tiles_n, num_tiles, tiles_per_xcd, b, tile_m, tile_n)) return;
   const int row0 = tile_m * BM, col0 = tile_n * BN;
-  const unsigned char* Ab = reinterpret_cast<const unsigned char*>(A + (size_t)VMOE_DBG_BATCH(b) * R * Kd);
-  const unsigned char* Bb = reinterpret_cast<const unsigned char*>(Bt + (size_t)VMOE_DBG_BATCH(b) * N * Kd);
+  const unsigned char* Ab = reinterpret_cast<const unsigned char*>(A + (size_t)b * R * Kd);
+  const unsigned char* Bb = reinterpret_cast<const unsigned char*>(Bt + (size_t)b * N * Kd);
 
   // Byte offsets of this lane's chunk in each of its load instructions.  Lane L
   // of a DMA load lands in LDS slot L: row L / CPR, chunk slot L % CPR; it
@@ -154,12 +219,12 @@ __global__ __launch_bounds__(Cfg::kThreads, Cfg::kBlocksPerCu) void gemm_bf16_ke
 #pragma unroll
   for (int i = 0; i < Cfg::kAIssues; ++i) {
     int r = (i * Cfg::kWaves + wave) * RPL + lrow;
-    a_goff[i] = (uint32_t)min(VMOE_DBG_ROW(row0) + r, R - 1) * (uint32_t)Kd * 2u + chunk * 16;
+    a_goff[i] = (uint32_t)min(row0 + r, R - 1) * (uint32_t)Kd * 2u + chunk * 16;
   }
 #pragma unroll
   for (int i = 0; i < Cfg::kBIssues; ++i) {
     int r = (i * Cfg::kWaves + wave) * RPL + lrow;
-    b_goff[i] = (uint32_t)min(VMOE_DBG_ROW(col0) + r, N - 1) * (uint32_t)Kd * 2u + chunk * 16;
+    b_goff[i] = (uint32_t)min(col0 + r, N - 1) * (uint32_t)Kd * 2u + chunk * 16;
   }
   auto load_tile = [&](int stage, int k0) {
     unsigned char* s = smem + stage * Cfg::kStageBytes;
@@ -256,8 +321,7 @@ __global__ __launch_bounds__(Cfg::kThreads, Cfg::kBlocksPerCu) void gemm_bf16_ke
   for (int t = 0; t < PD; ++t)
     if (t < nk) load_tile(t, t * BK);
   wait_tile(min(PD, nk) - 1);
-  __builtin_amdgcn_s_barrier();
-  __builtin_amdgcn_sched_barrier(0);
+  raw_barrier();
   load_frags(0, 0, 0);
   int stage = 0;
   for (int kt = 0; kt < nk; ++kt) {
@@ -268,23 +332,14 @@ __global__ __launch_bounds__(Cfg::kThreads, Cfg::kBlocksPerCu) void gemm_bf16_ke
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
       if (ks + 1 < KS) {
-#ifndef VMOE_DBG_NO_FRAGS
         load_frags((ks + 1) & 1, stage, ks + 1);
-#endif
-#ifndef VMOE_DBG_NO_DMA
         if (ks == 0 && do_load) load_tile(load_stage, (kt + PD) * BK);
-#endif
       } else if (has_next) {
         // Tiles kt+2 .. min(kt+PD, nk-1) were issued after tile kt+1.
         wait_tile(min(kt + PD, nk - 1) - (kt + 1));
         wait_lgkmcnt0();
-#ifndef VMOE_DBG_NO_BARRIER
-        __builtin_amdgcn_s_barrier();
-#endif
-        __builtin_amdgcn_sched_barrier(0);
-#ifndef VMOE_DBG_NO_FRAGS
+        raw_barrier();
         load_frags(0, next_stage, 0);
-#endif
       }
       mfma_slice(ks & 1);
       slice_schedule(ks == 0);
@@ -294,49 +349,8 @@ __global__ __launch_bounds__(Cfg::kThreads, Cfg::kBlocksPerCu) void gemm_bf16_ke
   wait_lgkmcnt0();
   __syncthreads();   // all waves are done with the operand tiles: LDS is reused below
 
-  // Epilogue.  acc[i][j][v] = C[row0 + wm*TM + i*32 + m][col0 + wn*TN + j*32 + (v/4)*8 + h*4 + v%4].
-  const bf16_t* biasb = bias != nullptr ? bias + (size_t)b * N : nullptr;
-  bf16_t* Cb = C + (size_t)b * R * N;
-  constexpr int OLD = Cfg::kOutLd;
-  bf16_t* so = reinterpret_cast<bf16_t*>(smem) + (size_t)wave * Cfg::TM * OLD;
-#pragma unroll
-  for (int j = 0; j < FN; ++j) {
-#pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      const int cl = j * 32 + q * 8 + h * 4;          // column inside the wave tile
-      const int col = col0 + wn * Cfg::TN + cl;
-      float bv[4] = {0.f, 0.f, 0.f, 0.f};
-      if (biasb != nullptr) {
-#pragma unroll
-        for (int t = 0; t < 4; ++t) bv[t] = bf2f(biasb[min(col + t, N - 1)]);
-      }
-#pragma unroll
-      for (int i = 0; i < FM; ++i) {
-        uint32_t p[2];
-#pragma unroll
-        for (int t = 0; t < 2; ++t) {
-          float o0 = apply_epilogue<EPI>(acc[i][j][q * 4 + 2 * t], bv[2 * t], biasb != nullptr);
-          float o1 = apply_epilogue<EPI>(acc[i][j][q * 4 + 2 * t + 1], bv[2 * t + 1], biasb != nullptr);
-          p[t] = (uint32_t)f2bf(o0) | ((uint32_t)f2bf(o1) << 16);
-        }
-        *reinterpret_cast<uint2*>(so + (i * 32 + m) * OLD + cl) = make_uint2(p[0], p[1]);
-      }
-    }
-  }
-  // Each wave reads back only what it wrote (LDS operations of a wave complete in order).
-  constexpr int kChunksOut = Cfg::TN / 8;             // 16-byte chunks per staged row
-  constexpr int kRowsPerPass = 64 / kChunksOut;
-  static_assert(64 % kChunksOut == 0, "wave tile width must divide a wave");
-  const int oc = (lane % kChunksOut) * 8;
-  const int orow = lane / kChunksOut;
-#pragma unroll
-  for (int r0 = 0; r0 < Cfg::TM; r0 += kRowsPerPass) {
-    const int rl = r0 + orow;
-    const int row = row0 + wm * Cfg::TM + rl;
-    const int col = col0 + wn * Cfg::TN + oc;
-    uint4 v = *reinterpret_cast<const uint4*>(so + rl * OLD + oc);
-    if (row < R && col + 8 <= N) *reinterpret_cast<uint4*>(Cb + (size_t)row * N + col) = v;
-  }
+  store_tile<EPI, Cfg::TM, Cfg::TN>(acc, smem, wave, lane, bias, C, b, R, N, row0 + wm * Cfg::TM,
+                                    col0 + wn * Cfg::TN);
 }
 
 // Generic path (any Kd % 8 == 0): 128x128 tile, operands staged through
