@@ -88,12 +88,81 @@ def cpu_baseline(cfg, x_np, params_np, bias_np, groups):
   }
 
 
+def soft_main(args):
+  """Soft MoE layer (SoftRouter + expert MLPs), same protocol as the sparse layer."""
+  import torch
+  from vmoe_amd import _hip, configs, kernels, moe
+  from vmoe_amd.nn import vit_moe
+  from vmoe_amd.projects.soft_moe import router as soft_router
+
+  cfg = configs.SOFT_B16
+  dev = torch.device("cuda:0")
+  torch.cuda.set_device(dev)
+  tdt = torch.bfloat16
+  D, M, n, p = cfg.d_model, cfg.mlp_dim, cfg.num_experts, cfg.num_slots
+  G, m = cfg.num_images, cfg.tokens_per_image
+  rng = np.random.Generator(np.random.PCG64(0))
+  xs = [torch.from_numpy(rng.standard_normal((G, m, D), dtype=np.float32)).to(dev).to(tdt)
+        for _ in range(4)]
+  mu = torch.from_numpy((rng.standard_normal((D, n, p), dtype=np.float32) / np.sqrt(D)).astype(np.float32)).to(dev)
+  gen = torch.Generator(device=dev)
+  gen.manual_seed(1)
+  w0 = (torch.randn((n, D, M), generator=gen, device=dev) / D ** 0.5).to(tdt)
+  w1 = (torch.randn((n, M, D), generator=gen, device=dev) / M ** 0.5).to(tdt)
+  rvars = {"params": {"mu": mu, "scale": torch.ones((), device=dev)}}
+  mvars = {"params": {"Dense_0": {"kernel": w0, "bias": torch.zeros((n, M), dtype=tdt, device=dev)},
+                      "Dense_1": {"kernel": w1, "bias": torch.zeros((n, D), dtype=tdt, device=dev)}}}
+  layer = soft_router.SoftRouter(num_experts=n, num_slots=p, compute_similarity_metrics=False, dtype=tdt)
+  mlp = moe.sparse_moe_spmd(vit_moe.MlpBlock, variable_axes={"params": 0})(mlp_dim=M, dtype=tdt)
+
+  def step(i):
+    dispatcher, metrics = layer.apply(rvars, xs[i % 4])
+    return mlp.apply(mvars, dispatcher, xs[i % 4])
+
+  for i in range(args.warmup):
+    step(i)
+  torch.cuda.synchronize()
+  sink = {}
+  _hip.set_timing_sink(sink)
+  t0 = time.perf_counter()
+  for i in range(args.steps):
+    step(i)
+  torch.cuda.synchronize()
+  t1 = time.perf_counter()
+  _hip.set_timing_sink(None)
+  ms = (t1 - t0) * 1e3 / args.steps
+  stage_ms = {name: float(np.mean([a.elapsed_time(b) for a, b in pairs])) * (len(pairs) / args.steps)
+              for name, pairs in sink.items()}
+  T = G * m
+  # Dominant kernel: the expert GEMM, weight-bandwidth bound here (1.2 GB of weights
+  # for 309 GFLOP): algorithmic bytes = weights + slot activations in and out + hidden.
+  rows = G * p
+  bytes_mlp = 2 * (2 * n * D * M + 2 * n * rows * D + 2 * n * rows * M)
+  mlp_ms = stage_ms["vmoe_expert_mlp"]
+  achieved = bytes_mlp / (mlp_ms * 1e-3) / 1e9
+  result = {
+      "metric": "Soft MoE layer tokens/sec at B/16, 128 experts x 1 slot, bf16",
+      "value": T / (ms * 1e-3), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
+      "warmup": args.warmup, "ms_per_step": ms, "higher_is_better": True, "scaling": "weak",
+      "vs_baseline": None, "dtype": "bf16", "data": "synthetic (seeded N(0,1) tokens and parameters)",
+      "config": {"workload": cfg.name, "tokens": T, "d_model": D, "mlp_dim": M, "experts": n,
+                 "slots_per_expert": p, "groups": G, "group_size": m},
+      "roofline": {"bound": "hbm", "kernel": "gemm_bf16_kernel", "achieved": achieved,
+                   "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": achieved / PEAK_HBM_GBS,
+                   "traffic": None, "launch_ms": mlp_ms / 2, "bytes_per_layer": bytes_mlp},
+      "stage_ms": stage_ms, "cpu_baseline": None,
+  }
+  print(json.dumps(result))
+
+
 def main():
   args = parse_args()
   if args.gpus != 1:
     print("bench.py: this build runs on ONE GPU (all experts resident, no collectives); "
           f"--gpus {args.gpus} is not supported.", file=sys.stderr)
     sys.exit(2)
+  if args.config == "soft_moe_b16_128x1":
+    return soft_main(args)
   import torch
   from vmoe_amd import _hip, configs, kernels
   from vmoe_amd.nn import vit_moe
