@@ -39,7 +39,6 @@ namespace vmoe {
 
 enum { kEpiBias = 0, kEpiBiasGeluTanh = 1, kEpiBiasGeluErf = 2 };
 
-constexpr int kNumXcd = 8;
 constexpr int kPanelRows = 8;   // row tiles per panel in the tile order
 
 // 0.5 x (1 + tanh(c (x + 0.044715 x^3))) = x * sigmoid(2 c (x + 0.044715 x^3)),
@@ -90,22 +89,6 @@ struct GemmCfg {
                 "tile loads must divide evenly");
   static_assert(kLdsBytes * kBlocksPerCu <= 160 * 1024, "LDS budget");
 };
-
-// s_waitcnt vmcnt(N) with lgkmcnt/expcnt left at their maxima.
-template <int N>
-__device__ __forceinline__ void wait_vmcnt() {
-  __builtin_amdgcn_s_waitcnt(0x0f70 | (N & 15) | ((N >> 4) << 14));
-}
-__device__ __forceinline__ void wait_lgkmcnt0() { __builtin_amdgcn_s_waitcnt(0xc07f); }
-// Workgroup barrier without the implicit "wait for every outstanding memory
-// operation" of __syncthreads(): callers wait for exactly what they need first.
-// The asm clobbers keep the compiler from moving LDS accesses across it.
-__device__ __forceinline__ void raw_barrier() {
-  asm volatile("" ::: "memory");
-  __builtin_amdgcn_s_barrier();
-  asm volatile("" ::: "memory");
-  __builtin_amdgcn_sched_barrier(0);
-}
 
 typedef const __attribute__((address_space(1))) void* global_ptr_t;
 typedef __attribute__((address_space(3))) void* lds_ptr_t;

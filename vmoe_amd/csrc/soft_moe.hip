@@ -14,6 +14,7 @@
 // are single scalars, so neither the (S, N) weights nor the (rows, D) data need
 // a transposed copy.
 #include "vmoe_common.h"
+#include "einsum_bf16.h"
 
 namespace vmoe {
 namespace {
@@ -198,6 +199,258 @@ __global__ __launch_bounds__(256) void soft_route_kernel(
   }
 }
 
+// bfloat16 soft routing, fast path (N <= 128 slots, D <= 32 * 2 * KSW).
+//
+// One workgroup of eight waves per group, with the unit-norm slot parameters held
+// in registers for the whole kernel: wave (j, kh) keeps the B fragments of column
+// tile j (32 slots) for half kh of the contraction.  The item rows then stream
+// through once, 32 at a time: each wave loads four whole rows (coalesced), takes
+// their norms from its registers, and writes the normalised rows into an LDS tile
+// while the loads of the next 32 rows are already in flight; every wave multiplies
+// the tile with its half of k, the two halves meet in LDS, and the logits of the
+// group collect in LDS as bfloat16.  Both softmaxes (over slots for the combine
+// weights, over items for the dispatch weights) are taken from that one copy, so
+// memory sees the items once and each weight once.
+constexpr int kSrThreads = 512;
+constexpr int kSrRows = 32;
+
+struct SoftLds {
+  size_t xs, part, red, cmx, csum, lg, total;
+};
+inline SoftLds soft_lds_layout(int D, int SP, int NP) {
+  SoftLds l;
+  l.xs = 0;
+  l.part = l.xs + (size_t)kSrRows * (D + 8) * 2;
+  l.red = l.part + 4 * 4 * 64 * 4 * sizeof(float);
+  l.cmx = l.red + kSrThreads * sizeof(float);
+  l.csum = l.cmx + 128 * sizeof(float);
+  l.lg = l.csum + 128 * sizeof(float);
+  l.total = l.lg + (size_t)SP * (NP + 8) * 2;
+  return l;
+}
+
+// exp(l - mx) / sum as exp2(l * log2e - mx * log2e) * (1 / sum) with the hardware
+// exp2 and reciprocal: relative error ~1e-6, against 4e-3 for the bfloat16 result.
+constexpr float kLog2e = 1.4426950408889634f;
+
+template <int KSW>
+__global__ __launch_bounds__(kSrThreads) void soft_route_bf16_kernel(
+    const bf16_t* __restrict__ x, const bf16_t* __restrict__ muw, bf16_t* __restrict__ dispatch_w,
+    bf16_t* __restrict__ combine_w, bf16_t* __restrict__ logits_out, float scale, int scale_x, int S,
+    int D, int N, int SP, int NP, SoftLds L) {
+  constexpr int CP = KSW / 8;   // 16-byte pieces of an item row per lane of a half wave
+  extern __shared__ __align__(16) unsigned char smem[];
+  bf16_t* xs = reinterpret_cast<bf16_t*>(smem + L.xs);
+  float4* part = reinterpret_cast<float4*>(smem + L.part);
+  float* red = reinterpret_cast<float*>(smem + L.red);
+  float* cmx = reinterpret_cast<float*>(smem + L.cmx);
+  float* csum = reinterpret_cast<float*>(smem + L.csum);
+  bf16_t* lg = reinterpret_cast<bf16_t*>(smem + L.lg);
+  const int LDX = D + 8, LDW = NP + 8;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int m = lane & 31, h = lane >> 5;
+  const int j = wave & 3, kh = wave >> 2;
+  const int g = blockIdx.x;
+  const bf16_t* xg = x + (size_t)g * S * D;
+  const float sc = bf16r(scale);
+  const int row_chunks = D / 8, row_tiles = SP / kSrRows, col_tiles = NP / 32;
+  const int ks_total = D / 16, ks_half = (ks_total + 1) / 2;
+  const int ks0 = kh * ks_half, nks = min(ks_half, ks_total - ks0);
+  const bool mma_on = j < col_tiles;
+
+  // Slot parameters of this wave: column tile j, k steps ks0 .. ks0 + nks.
+  bf16x8 bfr[KSW];
+  {
+    const bf16_t* brow = muw + (size_t)min(j * 32 + m, N - 1) * D + h * 8;
+#pragma unroll
+    for (int i = 0; i < KSW; ++i)
+      bfr[i] = __builtin_bit_cast(
+          bf16x8, *reinterpret_cast<const uint4*>(brow + min(ks0 + i, ks_total - 1) * 16));
+  }
+
+  // Four item rows per wave and tile, one row per half wave at a time (rows
+  // wave*4 + 2*i + h); rows past S re-read row S-1 and are written as zeros.
+  uint4 raw[2][CP];
+  auto load_rows = [&](int t) {
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int r = min(t * kSrRows + wave * 4 + 2 * i + h, S - 1);
+#pragma unroll
+      for (int ps = 0; ps < CP; ++ps) {
+        const int c = min(ps * 32 + m, row_chunks - 1);
+        raw[i][ps] = *reinterpret_cast<const uint4*>(xg + (size_t)r * D + c * 8);
+      }
+    }
+  };
+  load_rows(0);
+
+  for (int t = 0; t < row_tiles; ++t) {
+    // norms from the registers, normalised rows into the LDS tile
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      float sq = 0.f;
+#pragma unroll
+      for (int ps = 0; ps < CP; ++ps) {
+        const uint32_t w4[4] = {raw[i][ps].x, raw[i][ps].y, raw[i][ps].z, raw[i][ps].w};
+        float tsum = 0.f;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const float lo = bf_lo(w4[q]), hi = bf_hi(w4[q]);
+          tsum = fmaf(lo, lo, tsum);
+          tsum = fmaf(hi, hi, tsum);
+        }
+        if (ps * 32 + m < row_chunks) sq += tsum;
+      }
+#pragma unroll
+      for (int o = 16; o > 0; o >>= 1) sq += __shfl_xor(sq, o, kWave);
+      const int lrow = wave * 4 + 2 * i + h;
+      const float inv = t * kSrRows + lrow < S ? 1.0f / sqrtf(sq + kNormEps) : 0.f;
+#pragma unroll
+      for (int ps = 0; ps < CP; ++ps) {
+        const int c = ps * 32 + m;
+        const uint32_t w4[4] = {raw[i][ps].x, raw[i][ps].y, raw[i][ps].z, raw[i][ps].w};
+        uint32_t o4[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          float lo = bf_lo(w4[q]) * inv, hi = bf_hi(w4[q]) * inv;
+          if (scale_x) { lo = bf16r(lo) * sc; hi = bf16r(hi) * sc; }
+          o4[q] = pack_bf16x2(lo, hi);
+        }
+        if (c < row_chunks)
+          *reinterpret_cast<uint4*>(xs + (size_t)lrow * LDX + c * 8) = make_uint4(o4[0], o4[1], o4[2], o4[3]);
+      }
+    }
+    wait_lgkmcnt0();
+    raw_barrier();
+    if (t + 1 < row_tiles) load_rows(t + 1);
+
+    floatx16 acc;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) acc[v] = 0.f;
+    if (mma_on) {
+      const bf16_t* arow = xs + (size_t)m * LDX + ks0 * 16 + h * 8;
+#pragma unroll
+      for (int i = 0; i < KSW; ++i) {
+        if (i < nks) {
+          const bf16x8 af = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(arow + i * 16));
+          acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af, bfr[i], acc, 0, 0, 0);
+        }
+      }
+      if (kh == 1) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+          part[(j * 4 + q) * 64 + lane] = make_float4(acc[q * 4], acc[q * 4 + 1], acc[q * 4 + 2], acc[q * 4 + 3]);
+      }
+    }
+    wait_lgkmcnt0();
+    raw_barrier();
+    if (mma_on && kh == 0) {
+      const int col = j * 32 + m;
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const float4 o = part[(j * 4 + q) * 64 + lane];
+        const float ov[4] = {o.x, o.y, o.z, o.w};
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          const int row = t * kSrRows + q * 8 + h * 4 + u;
+          lg[(size_t)row * LDW + col] = f2bf(acc[q * 4 + u] + ov[u]);
+        }
+      }
+    }
+  }
+  __syncthreads();
+
+  // Combine weights: softmax over the N slots of each item.  Half wave = one row,
+  // lane = four consecutive slots.
+  for (int s0 = wave * 2; s0 < S; s0 += 16) {
+    const int s = s0 + h;
+    const int c = m * 4;
+    float l[4] = {-INFINITY, -INFINITY, -INFINITY, -INFINITY};
+    if (s < S && c < N) {
+      const uint2 pr = *reinterpret_cast<const uint2*>(lg + (size_t)s * LDW + c);
+      l[0] = bf_lo(pr.x); l[1] = bf_hi(pr.x); l[2] = bf_lo(pr.y); l[3] = bf_hi(pr.y);
+    }
+    float mx = fmaxf(fmaxf(l[0], l[1]), fmaxf(l[2], l[3]));
+#pragma unroll
+    for (int o = 16; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o, kWave));
+    const float mb = mx * kLog2e;
+    float e[4], sum = 0.f;
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      e[u] = __builtin_amdgcn_exp2f(fmaf(l[u], kLog2e, -mb));   // exp2(-inf) = 0 past N
+      sum += e[u];
+    }
+#pragma unroll
+    for (int o = 16; o > 0; o >>= 1) sum += __shfl_xor(sum, o, kWave);
+    const float rs = __builtin_amdgcn_rcpf(sum);
+    if (s < S && c < N)
+      *reinterpret_cast<uint2*>(combine_w + ((size_t)g * S + s) * N + c) =
+          make_uint2(pack_bf16x2(e[0] * rs, e[1] * rs), pack_bf16x2(e[2] * rs, e[3] * rs));
+  }
+
+  // Thread -> (16-byte piece c of a weights row, rows s = sr, sr + rpp, ...).
+  const int lchunks = N / 8, rpp = kSrThreads / lchunks;
+  const int sr = tid / lchunks, pc = tid - sr * lchunks;
+  if (logits_out != nullptr && sr < rpp) {
+    for (int s = sr; s < S; s += rpp)
+      *reinterpret_cast<uint4*>(logits_out + ((size_t)g * S + s) * N + pc * 8) =
+          *reinterpret_cast<const uint4*>(lg + (size_t)s * LDW + pc * 8);
+  }
+
+  // Dispatch weights: softmax over the S items of each slot.  For the maxima and
+  // sums a column is shared by RG threads that take every RG-th row and meet in LDS.
+  {
+    const int RG = kSrThreads / NP;
+    const int n = tid % NP, rg = tid / NP;
+    const bool act = rg < RG;
+    float mx = -INFINITY;
+    if (act)
+      for (int s = rg; s < S; s += RG) mx = fmaxf(mx, bf2f(lg[(size_t)s * LDW + n]));
+    red[tid] = mx;
+    __syncthreads();
+    if (act) {
+      mx = -INFINITY;
+      for (int q = 0; q < RG; ++q) mx = fmaxf(mx, red[q * NP + n]);
+    }
+    __syncthreads();
+    const float mb = mx * kLog2e;
+    float sum = 0.f;
+    if (act)
+      for (int s = rg; s < S; s += RG)
+        sum += __builtin_amdgcn_exp2f(fmaf(bf2f(lg[(size_t)s * LDW + n]), kLog2e, -mb));
+    red[tid] = sum;
+    __syncthreads();
+    if (act && rg == 0) {
+      sum = 0.f;
+      for (int q = 0; q < RG; ++q) sum += red[q * NP + n];
+      cmx[n] = mb;
+      csum[n] = __builtin_amdgcn_rcpf(sum);
+    }
+    __syncthreads();
+    if (sr < rpp) {
+      float cm[8], cr[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        cm[u] = cmx[pc * 8 + u];
+        cr[u] = csum[pc * 8 + u];
+      }
+      for (int s = sr; s < S; s += rpp) {
+        const uint4 rawl = *reinterpret_cast<const uint4*>(lg + (size_t)s * LDW + pc * 8);
+        const uint32_t w4[4] = {rawl.x, rawl.y, rawl.z, rawl.w};
+        uint32_t o4[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          const float lo = __builtin_amdgcn_exp2f(fmaf(bf_lo(w4[u]), kLog2e, -cm[2 * u])) * cr[2 * u];
+          const float hi = __builtin_amdgcn_exp2f(fmaf(bf_hi(w4[u]), kLog2e, -cm[2 * u + 1])) * cr[2 * u + 1];
+          o4[u] = pack_bf16x2(lo, hi);
+        }
+        *reinterpret_cast<uint4*>(dispatch_w + ((size_t)g * S + s) * N + pc * 8) =
+            make_uint4(o4[0], o4[1], o4[2], o4[3]);
+      }
+    }
+  }
+}
+
 // Dense einsum between per-group weights and data on the float32 matrix cores.
 //   DISPATCH: out[slot(g,mm)] = sum_s w[g,s,mm] * data[g,s,:]      (M = E*C, Kd = S)
 //   COMBINE:  out[g,mm,:]     = sum_n w[g,mm,n] * data[slot(g,n)]  (M = S,   Kd = E*C)
@@ -307,11 +560,25 @@ extern "C" int vmoe_soft_route(const VmoeSoftRouteParams* p, vmoe_stream_t strea
   const int SP = (p->S + 31) / 32 * 32, NP = (p->N + 31) / 32 * 32;
   const int LDW = NP + (esz == 2 ? 2 : 1);
   const size_t lds = (size_t)SP * 4 + (size_t)SP * LDW * esz;
-  if (lds > 160 * 1024) return VMOE_E_UNSUPPORTED;
   hipStream_t stream = as_stream(stream_);
   // router.py:79-82: the scale multiplies whichever of the two operands is smaller.
   const int scale_x = ((int64_t)p->G * p->S * p->D < (int64_t)p->D * p->N) ? 1 : 0;
-  if (p->dtype == VMOE_BF16) {
+  const SoftLds L = soft_lds_layout(p->D, SP, NP);
+  if (p->dtype == VMOE_BF16 && p->N <= 128 && p->N % 8 == 0 && p->D % 16 == 0 && p->D <= 1024 &&
+      L.total <= 160 * 1024 && aligned16(p->dispatch_w) && aligned16(p->combine_w) &&
+      (p->logits == nullptr || aligned16(p->logits))) {
+    hipLaunchKernelGGL(soft_prep_mu_kernel<bf16_t>, dim3(p->N), dim3(256), 0, stream,
+                       (const bf16_t*)p->mu, (bf16_t*)p->workspace, p->scale, !scale_x, p->D, p->N);
+    auto kern = p->D <= 768 ? soft_route_bf16_kernel<24> : soft_route_bf16_kernel<32>;
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)L.total);
+    if (e != hipSuccess) return (int)e;
+    hipLaunchKernelGGL(kern, dim3(p->G), dim3(kSrThreads), L.total, stream, (const bf16_t*)p->x,
+                       (const bf16_t*)p->workspace, (bf16_t*)p->dispatch_w, (bf16_t*)p->combine_w,
+                       (bf16_t*)p->logits, p->scale, scale_x, p->S, p->D, p->N, SP, NP, L);
+  } else if (lds > 160 * 1024) {
+    return VMOE_E_UNSUPPORTED;
+  } else if (p->dtype == VMOE_BF16) {
     hipLaunchKernelGGL(soft_prep_mu_kernel<bf16_t>, dim3(p->N), dim3(256), 0, stream,
                        (const bf16_t*)p->mu, (bf16_t*)p->workspace, p->scale, !scale_x, p->D, p->N);
     auto kern = soft_route_kernel<bf16_t>;
@@ -338,6 +605,7 @@ extern "C" int vmoe_soft_route(const VmoeSoftRouteParams* p, vmoe_stream_t strea
 extern "C" int vmoe_einsum_dispatch(const VmoeEinsumParams* p, vmoe_stream_t stream) {
   int rc = check_einsum(p, true);
   if (rc != VMOE_OK) return rc;
+  if (ein::dispatch_fast_ok(p)) return ein::launch_dispatch_fast(p, as_stream(stream));
   const int M = p->E * p->C;
   dim3 grid((p->D + 63) / 64, (M + 63) / 64, p->G);
   hipLaunchKernelGGL(einsum_kernel<true>, grid, dim3(256), 0, as_stream(stream), p->w, p->data,
@@ -348,6 +616,7 @@ extern "C" int vmoe_einsum_dispatch(const VmoeEinsumParams* p, vmoe_stream_t str
 extern "C" int vmoe_einsum_combine(const VmoeEinsumParams* p, vmoe_stream_t stream) {
   int rc = check_einsum(p, false);
   if (rc != VMOE_OK) return rc;
+  if (ein::combine_fast_ok(p)) return ein::launch_combine_fast(p, as_stream(stream));
   dim3 grid((p->D + 63) / 64, (p->S + 63) / 64, p->G);
   hipLaunchKernelGGL(einsum_kernel<false>, grid, dim3(256), 0, as_stream(stream), p->w, p->data,
                      p->out, p->G, p->S, p->E, p->C, p->D, p->w_dtype, p->data_dtype, p->out_dtype);

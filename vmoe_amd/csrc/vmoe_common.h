@@ -24,6 +24,15 @@ __device__ __forceinline__ bf16_t f2bf(float f) {
 __device__ __forceinline__ float bf2f(bf16_t h) {
   return __builtin_bit_cast(float, (uint32_t)h << 16);
 }
+// Two float32 -> two bfloat16 in one dword (lo in bits 0..15): one v_cvt_pk_bf16_f32.
+typedef float floatx2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+  floatx2 v = {lo, hi};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2));
+}
+__device__ __forceinline__ float bf_lo(uint32_t w) { return __builtin_bit_cast(float, w << 16); }
+__device__ __forceinline__ float bf_hi(uint32_t w) { return __builtin_bit_cast(float, w & 0xffff0000u); }
 // Round a float32 to the nearest bfloat16 value, kept as float32.
 __device__ __forceinline__ float bf16r(float f) { return bf2f(f2bf(f)); }
 
@@ -67,6 +76,26 @@ __device__ __forceinline__ int slot_row(int e, int g, int c, int G, int E, int C
     r = g * C + c;
   }
   return e * (G * C) + r;
+}
+
+// Accelerator complex dies of the device; workgroup i is placed on die i % kNumXcd,
+// and each die has its own L2.
+constexpr int kNumXcd = 8;
+
+// s_waitcnt vmcnt(N) with lgkmcnt/expcnt left at their maxima.
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {
+  __builtin_amdgcn_s_waitcnt(0x0f70 | (N & 15) | ((N >> 4) << 14));
+}
+__device__ __forceinline__ void wait_lgkmcnt0() { __builtin_amdgcn_s_waitcnt(0xc07f); }
+// Workgroup barrier without the implicit "wait for every outstanding memory
+// operation" of __syncthreads(): callers wait for exactly what they need first.
+// The asm clobbers keep the compiler from moving LDS accesses across it.
+__device__ __forceinline__ void raw_barrier() {
+  asm volatile("" ::: "memory");
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
+  __builtin_amdgcn_sched_barrier(0);
 }
 
 inline hipStream_t as_stream(vmoe_stream_t s) { return reinterpret_cast<hipStream_t>(s); }
