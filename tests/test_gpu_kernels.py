@@ -315,6 +315,14 @@ SOFT_CASES = [
     (2, 196, 768, 128, 1, O.BF16),
     (4, 100, 256, 16, 2, O.BF16),
     (1, 2, 16, 4, 2, O.F32),          # inputs smaller than mu: the scale multiplies the inputs
+    # every model width of the register-resident bf16 path, ragged S and N
+    (3, 77, 384, 24, 1, O.BF16),
+    (2, 130, 512, 8, 5, O.BF16),
+    (2, 33, 1024, 128, 1, O.BF16),
+    (1, 300, 256, 104, 1, O.BF16),
+    (1, 20, 768, 64, 2, O.BF16),      # inputs smaller than mu on the bf16 path
+    (2, 64, 768, 20, 1, O.BF16),      # N % 8 != 0: generic path
+    (2, 64, 320, 16, 1, O.BF16),      # width outside the fast path
 ]
 
 

@@ -202,17 +202,20 @@ __global__ __launch_bounds__(256) void soft_route_kernel(
 // bfloat16 soft routing, fast path (N <= 128 slots, D <= 32 * 2 * KSW).
 //
 // One workgroup of eight waves per group, with the unit-norm slot parameters held
-// in registers for the whole kernel: wave (j, kh) keeps the B fragments of column
-// tile j (32 slots) for half kh of the contraction.  The item rows then stream
+// in registers for the whole kernel: wave w keeps the B fragments of 16 slots for
+// the whole contraction (v_mfma_f32_16x16x32_bf16).  The item rows then stream
 // through once, 32 at a time: each wave loads four whole rows (coalesced), takes
 // their norms from its registers, and writes the normalised rows into an LDS tile
-// while the loads of the next 32 rows are already in flight; every wave multiplies
-// the tile with its half of k, the two halves meet in LDS, and the logits of the
-// group collect in LDS as bfloat16.  Both softmaxes (over slots for the combine
-// weights, over items for the dispatch weights) are taken from that one copy, so
-// memory sees the items once and each weight once.
+// while the loads of the next 64 rows are already in flight; every wave multiplies
+// the tile with its slots, and the logits of the group collect in LDS as
+// bfloat16.  Both softmaxes (over slots for the combine weights, over items for
+// the dispatch weights) are taken from that one copy, so memory sees the items
+// once and each weight once.
 constexpr int kSrThreads = 512;
 constexpr int kSrRows = 32;
+
+// Model widths the register-resident fast path is instantiated for.
+inline bool soft_fast_width(int D) { return D == 256 || D == 384 || D == 512 || D == 768 || D == 1024; }
 
 struct SoftLds {
   size_t xs, part, red, cmx, csum, lg, total;
@@ -221,7 +224,7 @@ inline SoftLds soft_lds_layout(int D, int SP, int NP) {
   SoftLds l;
   l.xs = 0;
   l.part = l.xs + (size_t)kSrRows * (D + 8) * 2;
-  l.red = l.part + 4 * 4 * 64 * 4 * sizeof(float);
+  l.red = l.part;
   l.cmx = l.red + kSrThreads * sizeof(float);
   l.csum = l.cmx + 128 * sizeof(float);
   l.lg = l.csum + 128 * sizeof(float);
@@ -238,10 +241,9 @@ __global__ __launch_bounds__(kSrThreads) void soft_route_bf16_kernel(
     const bf16_t* __restrict__ x, const bf16_t* __restrict__ muw, bf16_t* __restrict__ dispatch_w,
     bf16_t* __restrict__ combine_w, bf16_t* __restrict__ logits_out, float scale, int scale_x, int S,
     int D, int N, int SP, int NP, SoftLds L) {
-  constexpr int CP = KSW / 8;   // 16-byte pieces of an item row per lane of a half wave
+  constexpr int CP = (KSW + 7) / 8;   // 16-byte pieces of an item row per lane of a half wave
   extern __shared__ __align__(16) unsigned char smem[];
   bf16_t* xs = reinterpret_cast<bf16_t*>(smem + L.xs);
-  float4* part = reinterpret_cast<float4*>(smem + L.part);
   float* red = reinterpret_cast<float*>(smem + L.red);
   float* cmx = reinterpret_cast<float*>(smem + L.cmx);
   float* csum = reinterpret_cast<float*>(smem + L.csum);
@@ -249,29 +251,73 @@ __global__ __launch_bounds__(kSrThreads) void soft_route_bf16_kernel(
   const int LDX = D + 8, LDW = NP + 8;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int m = lane & 31, h = lane >> 5;
-  const int j = wave & 3, kh = wave >> 2;
   const int g = blockIdx.x;
   const bf16_t* xg = x + (size_t)g * S * D;
   const float sc = bf16r(scale);
-  const int row_chunks = D / 8, row_tiles = SP / kSrRows, col_tiles = NP / 32;
-  const int ks_total = D / 16, ks_half = (ks_total + 1) / 2;
-  const int ks0 = kh * ks_half, nks = min(ks_half, ks_total - ks0);
-  const bool mma_on = j < col_tiles;
+  const int row_chunks = D / 8, row_tiles = SP / kSrRows;
+  const int r16 = lane & 15, kq = lane >> 4;   // 16x16x32 fragment: row / column, k quarter
+  const bool mma_on = wave * 16 < NP;
 
-  // Slot parameters of this wave: column tile j, k steps ks0 .. ks0 + nks.
+  // Slot parameters of this wave: slots wave*16 .. +16, every k step (D == 32 * KSW).
   bf16x8 bfr[KSW];
   {
-    const bf16_t* brow = muw + (size_t)min(j * 32 + m, N - 1) * D + h * 8;
+    const bf16_t* brow = muw + (size_t)min(wave * 16 + r16, N - 1) * D + kq * 8;
 #pragma unroll
     for (int i = 0; i < KSW; ++i)
-      bfr[i] = __builtin_bit_cast(
-          bf16x8, *reinterpret_cast<const uint4*>(brow + min(ks0 + i, ks_total - 1) * 16));
+      bfr[i] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(brow + i * 32));
   }
+
+  // Combine weights of the item rows [s_begin, s_end): softmax over the N slots.
+  // Half wave = one row, lane = four consecutive slots; two rows per half wave at a
+  // time so that the two shuffle chains overlap.
+  auto combine_rows = [&](int s_begin, int s_end) {
+    for (int s0 = s_begin + wave * 4; s0 < s_end; s0 += 32) {
+      const int c = m * 4;
+      float l[2][4], mx[2];
+#pragma unroll
+      for (int r = 0; r < 2; ++r) {
+        const int s = s0 + 2 * r + h;
+#pragma unroll
+        for (int u = 0; u < 4; ++u) l[r][u] = -INFINITY;
+        if (s < s_end && c < N) {
+          const uint2 pr = *reinterpret_cast<const uint2*>(lg + (size_t)s * LDW + c);
+          l[r][0] = bf_lo(pr.x); l[r][1] = bf_hi(pr.x); l[r][2] = bf_lo(pr.y); l[r][3] = bf_hi(pr.y);
+        }
+        mx[r] = fmaxf(fmaxf(l[r][0], l[r][1]), fmaxf(l[r][2], l[r][3]));
+      }
+#pragma unroll
+      for (int o = 16; o > 0; o >>= 1)
+#pragma unroll
+        for (int r = 0; r < 2; ++r) mx[r] = fmaxf(mx[r], __shfl_xor(mx[r], o, kWave));
+      float e[2][4], sum[2];
+#pragma unroll
+      for (int r = 0; r < 2; ++r) {
+        const float mb = mx[r] * kLog2e;
+        sum[r] = 0.f;
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          e[r][u] = __builtin_amdgcn_exp2f(fmaf(l[r][u], kLog2e, -mb));   // exp2(-inf) = 0 past N
+          sum[r] += e[r][u];
+        }
+      }
+#pragma unroll
+      for (int o = 16; o > 0; o >>= 1)
+#pragma unroll
+        for (int r = 0; r < 2; ++r) sum[r] += __shfl_xor(sum[r], o, kWave);
+#pragma unroll
+      for (int r = 0; r < 2; ++r) {
+        const int s = s0 + 2 * r + h;
+        const float rs = __builtin_amdgcn_rcpf(sum[r]);
+        if (s < s_end && c < N)
+          *reinterpret_cast<uint2*>(combine_w + ((size_t)g * S + s) * N + c) = make_uint2(
+              pack_bf16x2(e[r][0] * rs, e[r][1] * rs), pack_bf16x2(e[r][2] * rs, e[r][3] * rs));
+      }
+    }
+  };
 
   // Four item rows per wave and tile, one row per half wave at a time (rows
   // wave*4 + 2*i + h); rows past S re-read row S-1 and are written as zeros.
-  uint4 raw[2][CP];
-  auto load_rows = [&](int t) {
+  auto load_rows = [&](uint4 (&raw)[2][CP], int t) {
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
       const int r = min(t * kSrRows + wave * 4 + 2 * i + h, S - 1);
@@ -282,9 +328,9 @@ __global__ __launch_bounds__(kSrThreads) void soft_route_bf16_kernel(
       }
     }
   };
-  load_rows(0);
 
-  for (int t = 0; t < row_tiles; ++t) {
+  // One tile of 32 item rows, held in raw; its registers then take the tile after next.
+  auto tile = [&](uint4 (&raw)[2][CP], int t) {
     // norms from the registers, normalised rows into the LDS tile
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
@@ -322,71 +368,52 @@ __global__ __launch_bounds__(kSrThreads) void soft_route_bf16_kernel(
     }
     wait_lgkmcnt0();
     raw_barrier();
-    if (t + 1 < row_tiles) load_rows(t + 1);
+    if (t + 2 < row_tiles) load_rows(raw, t + 2);
+    // the logits of the previous tile are complete: their combine weights fill the
+    // time the loads are in flight
+    if (t > 0) combine_rows((t - 1) * kSrRows, min(t * kSrRows, S));
 
-    floatx16 acc;
-#pragma unroll
-    for (int v = 0; v < 16; ++v) acc[v] = 0.f;
     if (mma_on) {
-      const bf16_t* arow = xs + (size_t)m * LDX + ks0 * 16 + h * 8;
+      floatx4 acc[2];
+#pragma unroll
+      for (int rh = 0; rh < 2; ++rh)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) acc[rh][v] = 0.f;
+      const bf16_t* arow = xs + (size_t)r16 * LDX + kq * 8;
 #pragma unroll
       for (int i = 0; i < KSW; ++i) {
-        if (i < nks) {
-          const bf16x8 af = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(arow + i * 16));
-          acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af, bfr[i], acc, 0, 0, 0);
-        }
-      }
-      if (kh == 1) {
+        const int ko = i * 32;
 #pragma unroll
-        for (int q = 0; q < 4; ++q)
-          part[(j * 4 + q) * 64 + lane] = make_float4(acc[q * 4], acc[q * 4 + 1], acc[q * 4 + 2], acc[q * 4 + 3]);
+        for (int rh = 0; rh < 2; ++rh) {
+          const bf16x8 af = __builtin_bit_cast(
+              bf16x8, *reinterpret_cast<const uint4*>(arow + (size_t)rh * 16 * LDX + ko));
+          acc[rh] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af, bfr[i], acc[rh], 0, 0, 0);
+        }
+        // bound how many fragment reads the scheduler hoists (register pressure)
+        if ((i & 3) == 3) __builtin_amdgcn_sched_barrier(0);
       }
+      const int col = wave * 16 + r16;
+#pragma unroll
+      for (int rh = 0; rh < 2; ++rh)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+          const int row = t * kSrRows + rh * 16 + kq * 4 + v;
+          lg[(size_t)row * LDW + col] = f2bf(acc[rh][v]);
+        }
     }
     wait_lgkmcnt0();
     raw_barrier();
-    if (mma_on && kh == 0) {
-      const int col = j * 32 + m;
-#pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const float4 o = part[(j * 4 + q) * 64 + lane];
-        const float ov[4] = {o.x, o.y, o.z, o.w};
-#pragma unroll
-        for (int u = 0; u < 4; ++u) {
-          const int row = t * kSrRows + q * 8 + h * 4 + u;
-          lg[(size_t)row * LDW + col] = f2bf(acc[q * 4 + u] + ov[u]);
-        }
-      }
-    }
+  };
+
+  uint4 raw0[2][CP], raw1[2][CP];
+  load_rows(raw0, 0);
+  if (row_tiles > 1) load_rows(raw1, 1);
+  for (int t = 0; t < row_tiles; t += 2) {
+    tile(raw0, t);
+    if (t + 1 < row_tiles) tile(raw1, t + 1);
   }
   __syncthreads();
-
-  // Combine weights: softmax over the N slots of each item.  Half wave = one row,
-  // lane = four consecutive slots.
-  for (int s0 = wave * 2; s0 < S; s0 += 16) {
-    const int s = s0 + h;
-    const int c = m * 4;
-    float l[4] = {-INFINITY, -INFINITY, -INFINITY, -INFINITY};
-    if (s < S && c < N) {
-      const uint2 pr = *reinterpret_cast<const uint2*>(lg + (size_t)s * LDW + c);
-      l[0] = bf_lo(pr.x); l[1] = bf_hi(pr.x); l[2] = bf_lo(pr.y); l[3] = bf_hi(pr.y);
-    }
-    float mx = fmaxf(fmaxf(l[0], l[1]), fmaxf(l[2], l[3]));
-#pragma unroll
-    for (int o = 16; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o, kWave));
-    const float mb = mx * kLog2e;
-    float e[4], sum = 0.f;
-#pragma unroll
-    for (int u = 0; u < 4; ++u) {
-      e[u] = __builtin_amdgcn_exp2f(fmaf(l[u], kLog2e, -mb));   // exp2(-inf) = 0 past N
-      sum += e[u];
-    }
-#pragma unroll
-    for (int o = 16; o > 0; o >>= 1) sum += __shfl_xor(sum, o, kWave);
-    const float rs = __builtin_amdgcn_rcpf(sum);
-    if (s < S && c < N)
-      *reinterpret_cast<uint2*>(combine_w + ((size_t)g * S + s) * N + c) =
-          make_uint2(pack_bf16x2(e[0] * rs, e[1] * rs), pack_bf16x2(e[2] * rs, e[3] * rs));
-  }
+  combine_rows((row_tiles - 1) * kSrRows, S);
 
   // Thread -> (16-byte piece c of a weights row, rows s = sr, sr + rpp, ...).
   const int lchunks = N / 8, rpp = kSrThreads / lchunks;
@@ -405,6 +432,7 @@ __global__ __launch_bounds__(kSrThreads) void soft_route_bf16_kernel(
     const bool act = rg < RG;
     float mx = -INFINITY;
     if (act)
+#pragma unroll 8
       for (int s = rg; s < S; s += RG) mx = fmaxf(mx, bf2f(lg[(size_t)s * LDW + n]));
     red[tid] = mx;
     __syncthreads();
@@ -416,6 +444,7 @@ __global__ __launch_bounds__(kSrThreads) void soft_route_bf16_kernel(
     const float mb = mx * kLog2e;
     float sum = 0.f;
     if (act)
+#pragma unroll 8
       for (int s = rg; s < S; s += RG)
         sum += __builtin_amdgcn_exp2f(fmaf(bf2f(lg[(size_t)s * LDW + n]), kLog2e, -mb));
     red[tid] = sum;
@@ -434,6 +463,7 @@ __global__ __launch_bounds__(kSrThreads) void soft_route_bf16_kernel(
         cm[u] = cmx[pc * 8 + u];
         cr[u] = csum[pc * 8 + u];
       }
+#pragma unroll 4
       for (int s = sr; s < S; s += rpp) {
         const uint4 rawl = *reinterpret_cast<const uint4*>(lg + (size_t)s * LDW + pc * 8);
         const uint32_t w4[4] = {rawl.x, rawl.y, rawl.z, rawl.w};
@@ -564,12 +594,15 @@ extern "C" int vmoe_soft_route(const VmoeSoftRouteParams* p, vmoe_stream_t strea
   // router.py:79-82: the scale multiplies whichever of the two operands is smaller.
   const int scale_x = ((int64_t)p->G * p->S * p->D < (int64_t)p->D * p->N) ? 1 : 0;
   const SoftLds L = soft_lds_layout(p->D, SP, NP);
-  if (p->dtype == VMOE_BF16 && p->N <= 128 && p->N % 8 == 0 && p->D % 16 == 0 && p->D <= 1024 &&
-      L.total <= 160 * 1024 && aligned16(p->dispatch_w) && aligned16(p->combine_w) &&
+  if (p->dtype == VMOE_BF16 && p->N <= 128 && p->N % 8 == 0 && soft_fast_width(p->D) && L.total <= 160 * 1024 && aligned16(p->dispatch_w) && aligned16(p->combine_w) &&
       (p->logits == nullptr || aligned16(p->logits))) {
     hipLaunchKernelGGL(soft_prep_mu_kernel<bf16_t>, dim3(p->N), dim3(256), 0, stream,
                        (const bf16_t*)p->mu, (bf16_t*)p->workspace, p->scale, !scale_x, p->D, p->N);
-    auto kern = p->D <= 768 ? soft_route_bf16_kernel<24> : soft_route_bf16_kernel<32>;
+    auto kern = p->D == 1024 ? soft_route_bf16_kernel<32>
+                : p->D == 768 ? soft_route_bf16_kernel<24>
+                : p->D == 512 ? soft_route_bf16_kernel<16>
+                : p->D == 384 ? soft_route_bf16_kernel<12>
+                              : soft_route_bf16_kernel<8>;
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)L.total);
     if (e != hipSuccess) return (int)e;
