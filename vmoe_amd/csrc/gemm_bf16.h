@@ -33,6 +33,7 @@
 #ifndef VMOE_GEMM_BF16_H_
 #define VMOE_GEMM_BF16_H_
 
+#include <type_traits>
 #include "vmoe_common.h"
 
 namespace vmoe {
@@ -209,12 +210,18 @@ __global__ __launch_bounds__(Cfg::kThreads, Cfg::kBlocksPerCu) void gemm_bf16_ke
     int r = (i * Cfg::kWaves + wave) * RPL + lrow;
     b_goff[i] = (uint32_t)min(col0 + r, N - 1) * (uint32_t)Kd * 2u + chunk * 16;
   }
-  auto load_tile = [&](int stage, int k0) {
+  // The DMA loads of a k tile are issued in two halves (A rows, then B rows), one
+  // under the MFMAs of each k slice: a wave sustains about one 1 KB DMA load per
+  // 80 clocks, so they must be spread out or the wave stalls behind them.
+  auto load_a = [&](int stage, int k0) {
     unsigned char* s = smem + stage * Cfg::kStageBytes;
 #pragma unroll
     for (int i = 0; i < Cfg::kAIssues; ++i)
       __builtin_amdgcn_global_load_lds((global_ptr_t)(Ab + a_goff[i] + (size_t)k0 * 2),
                                        (lds_ptr_t)(s + (i * Cfg::kWaves + wave) * RPL * RB), 16, 0, 0);
+  };
+  auto load_b = [&](int stage, int k0) {
+    unsigned char* s = smem + stage * Cfg::kStageBytes;
 #pragma unroll
     for (int i = 0; i < Cfg::kBIssues; ++i)
       __builtin_amdgcn_global_load_lds((global_ptr_t)(Bb + b_goff[i] + (size_t)k0 * 2),
@@ -266,7 +273,8 @@ __global__ __launch_bounds__(Cfg::kThreads, Cfg::kBlocksPerCu) void gemm_bf16_ke
   // of the next slice go out behind the first MFMAs (an MFMA leads, so the wait
   // for the previous slice's reads never covers a new read); the DMA loads
   // (first slice only) are spread over the remaining MFMAs.
-  auto slice_schedule = [&](bool with_vmem) {
+  auto slice_schedule = [&](auto vmem_c) {
+    constexpr int vmem = decltype(vmem_c)::value;
     constexpr int kLead = kReads < kMfmas ? kReads : kMfmas;
     constexpr int kReadsPer = (kReads + kLead - 1) / kLead;
     constexpr int kRest = kMfmas - kLead;
@@ -275,58 +283,55 @@ __global__ __launch_bounds__(Cfg::kThreads, Cfg::kBlocksPerCu) void gemm_bf16_ke
       __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
       __builtin_amdgcn_sched_group_barrier(0x100, kReadsPer, 0);
     }
-    if (with_vmem) {
+    if constexpr (vmem > 0) {
       if constexpr (kRest > 0) {
-        constexpr int kPer = (L + kRest - 1) / kRest;
+        // one load in front of every (kRest / vmem)-th remaining MFMA
 #pragma unroll
         for (int g = 0; g < kRest; ++g) {
-          __builtin_amdgcn_sched_group_barrier(0x020, kPer, 0);
+          if (g * vmem / kRest != (g + 1) * vmem / kRest)
+            __builtin_amdgcn_sched_group_barrier(0x020, (vmem + kRest - 1) / kRest, 0);
           __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
         }
       } else {
-        __builtin_amdgcn_sched_group_barrier(0x020, L, 0);
+        __builtin_amdgcn_sched_group_barrier(0x020, vmem, 0);
       }
     }
     __builtin_amdgcn_sched_barrier(0);
   };
-  // Waits until k tile `next` has landed: only the tiles issued after it
-  // (at most PD-1, fewer at the end of the K loop) may stay in flight.
-  auto wait_tile = [&](int younger) {
-    if (younger >= PD - 1) wait_vmcnt<(PD - 1) * L>();
-    else if (PD >= 3 && younger == PD - 2) wait_vmcnt<(PD >= 3 ? PD - 2 : 0) * L>();
-    else if (PD >= 4 && younger == PD - 3) wait_vmcnt<(PD >= 4 ? PD - 3 : 0) * L>();
-    else wait_vmcnt<0>();
-  };
-  static_assert(PD <= 4, "wait_tile covers up to 4 tiles of prefetch");
-
+  // The loop body is one basic block (no branches), so that the scheduling hints
+  // hold and the fragment reads / DMA loads really are issued under the MFMAs:
+  // past the end of K the loads re-fetch the last k tile into a stage nobody
+  // reads any more, and the last iteration pre-reads fragments nobody uses.
+  // A k tile has landed when at most the PD-1 tiles issued after it are in flight.
+  static_assert((PD - 1) * L < 64, "vmcnt");
+  static_assert(KS == 2, "the two halves of a tile's loads go with its two k slices");
   const int nk = Kd / BK;
 #pragma unroll
-  for (int t = 0; t < PD; ++t)
-    if (t < nk) load_tile(t, t * BK);
-  wait_tile(min(PD, nk) - 1);
+  for (int t = 0; t < PD; ++t) {
+    load_a(t, min(t, nk - 1) * BK);
+    load_b(t, min(t, nk - 1) * BK);
+  }
+  wait_vmcnt<(PD - 1) * L>();
   raw_barrier();
   load_frags(0, 0, 0);
   int stage = 0;
   for (int kt = 0; kt < nk; ++kt) {
     const int next_stage = stage + 1 == NS ? 0 : stage + 1;
     const int load_stage = stage == 0 ? NS - 1 : stage - 1;   // (kt + PD) % NS
-    const bool do_load = kt + PD < nk;
-    const bool has_next = kt + 1 < nk;
-#pragma unroll
-    for (int ks = 0; ks < KS; ++ks) {
-      if (ks + 1 < KS) {
-        load_frags((ks + 1) & 1, stage, ks + 1);
-        if (ks == 0 && do_load) load_tile(load_stage, (kt + PD) * BK);
-      } else if (has_next) {
-        // Tiles kt+2 .. min(kt+PD, nk-1) were issued after tile kt+1.
-        wait_tile(min(kt + PD, nk - 1) - (kt + 1));
-        wait_lgkmcnt0();
-        raw_barrier();
-        load_frags(0, next_stage, 0);
-      }
-      mfma_slice(ks & 1);
-      slice_schedule(ks == 0);
-    }
+    const int load_k0 = min(kt + PD, nk - 1) * BK;
+    // slice 0: fragments of slice 1, A half of tile kt + PD
+    load_frags(1, stage, 1);
+    load_a(load_stage, load_k0);
+    mfma_slice(0);
+    slice_schedule(std::integral_constant<int, Cfg::kAIssues>{});
+    // slice 1: tile kt + 1 has landed when only the younger loads are in flight
+    wait_vmcnt<(PD - 2) * L + Cfg::kAIssues>();
+    wait_lgkmcnt0();
+    raw_barrier();
+    load_frags(0, next_stage, 0);
+    load_b(load_stage, load_k0);
+    mfma_slice(1);
+    slice_schedule(std::integral_constant<int, Cfg::kBIssues>{});
     stage = next_stage;
   }
   wait_lgkmcnt0();
