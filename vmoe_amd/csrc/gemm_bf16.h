@@ -61,6 +61,18 @@ __device__ __forceinline__ float apply_epilogue(float acc, float bias, bool has_
   return o;
 }
 
+// The same epilogue for two neighbouring outputs at once, as one bfloat16 pair:
+// every rounding step is a single packed conversion (v_cvt_pk_bf16_f32) followed
+// by a shift and a mask, instead of a conversion and a shift per element.
+template <int EPI, bool HAS_BIAS>
+__device__ __forceinline__ uint32_t epilogue_pair(float a0, float a1, float b0, float b1) {
+  uint32_t p = pack_bf16x2(a0, a1);
+  if (HAS_BIAS) p = pack_bf16x2(bf_lo(p) + b0, bf_hi(p) + b1);
+  if (EPI == kEpiBiasGeluTanh) p = pack_bf16x2(gelu_tanh_fast(bf_lo(p)), gelu_tanh_fast(bf_hi(p)));
+  if (EPI == kEpiBiasGeluErf) p = pack_bf16x2(gelu_erf(bf_lo(p)), gelu_erf(bf_hi(p)));
+  return p;
+}
+
 template <int BM_, int BN_, int WM_, int WN_, int BK_ = 32, int NSTAGE_ = 4, int BLOCKS_PER_CU_ = 1>
 struct GemmCfg {
   static constexpr int BM = BM_, BN = BN_, BK = BK_, WM = WM_, WN = WN_, NSTAGE = NSTAGE_;
@@ -109,30 +121,30 @@ __device__ __forceinline__ void store_tile(floatx16 (&acc)[TM / 32][TN / 32], un
   const bf16_t* biasb = bias != nullptr ? bias + (size_t)b * N : nullptr;
   bf16_t* Cb = C + (size_t)b * R * N;
   bf16_t* so = reinterpret_cast<bf16_t*>(smem) + (size_t)wave * TM * OLD;
+  auto stage = [&](auto has_bias_c) {
+    constexpr bool kHasBias = decltype(has_bias_c)::value;
 #pragma unroll
-  for (int j = 0; j < FN; ++j) {
+    for (int j = 0; j < FN; ++j) {
 #pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      const int cl = j * 32 + q * 8 + h * 4;          // column inside the wave tile
-      const int col = wcol0 + cl;
-      float bv[4] = {0.f, 0.f, 0.f, 0.f};
-      if (biasb != nullptr) {
+      for (int q = 0; q < 4; ++q) {
+        const int cl = j * 32 + q * 8 + h * 4;          // column inside the wave tile
+        const int col = wcol0 + cl;
+        float bv[4] = {0.f, 0.f, 0.f, 0.f};
+        if (kHasBias) {
 #pragma unroll
-        for (int t = 0; t < 4; ++t) bv[t] = bf2f(biasb[min(col + t, N - 1)]);
-      }
-#pragma unroll
-      for (int i = 0; i < FM; ++i) {
-        uint32_t p[2];
-#pragma unroll
-        for (int t = 0; t < 2; ++t) {
-          float o0 = apply_epilogue<EPI>(acc[i][j][q * 4 + 2 * t], bv[2 * t], biasb != nullptr);
-          float o1 = apply_epilogue<EPI>(acc[i][j][q * 4 + 2 * t + 1], bv[2 * t + 1], biasb != nullptr);
-          p[t] = (uint32_t)f2bf(o0) | ((uint32_t)f2bf(o1) << 16);
+          for (int t = 0; t < 4; ++t) bv[t] = bf2f(biasb[min(col + t, N - 1)]);
         }
-        *reinterpret_cast<uint2*>(so + (i * 32 + m) * OLD + cl) = make_uint2(p[0], p[1]);
+#pragma unroll
+        for (int i = 0; i < FM; ++i) {
+          const uint32_t p0 = epilogue_pair<EPI, kHasBias>(acc[i][j][q * 4], acc[i][j][q * 4 + 1], bv[0], bv[1]);
+          const uint32_t p1 = epilogue_pair<EPI, kHasBias>(acc[i][j][q * 4 + 2], acc[i][j][q * 4 + 3], bv[2], bv[3]);
+          *reinterpret_cast<uint2*>(so + (i * 32 + m) * OLD + cl) = make_uint2(p0, p1);
+        }
       }
     }
-  }
+  };
+  if (biasb != nullptr) stage(std::true_type{});
+  else stage(std::false_type{});
   // Each wave reads back only what it wrote (LDS operations of a wave complete in order).
   constexpr int kChunksOut = TN / 8;                  // 16-byte chunks per staged row
   constexpr int kRowsPerPass = 64 / kChunksOut;
