@@ -111,14 +111,38 @@ typedef __attribute__((address_space(3))) void* lds_ptr_t;
 // consecutive columns of one row).  Bias, rounding, GELU and the bf16 pack happen
 // in registers; the wave tile is staged in a wave-private LDS region and leaves
 // as 16-byte, row-contiguous global stores.
+// Bias of the wave tile's columns for one lane: four consecutive bfloat16 per
+// (column tile j, quad q), fetched before the main loop so that the epilogue does
+// not start with a round trip to memory.
+template <int TN>
+__device__ __forceinline__ void load_bias(uint2 (&bias_pk)[TN / 8], const bf16_t* __restrict__ bias,
+                                          int b, int N, int wcol0, int lane) {
+  const int h = lane >> 5;
+#pragma unroll
+  for (int jq = 0; jq < TN / 8; ++jq) {
+    bias_pk[jq] = make_uint2(0, 0);
+    if (bias != nullptr) {
+      const int col = wcol0 + jq * 8 + h * 4;
+      const bf16_t* src = bias + (size_t)b * N;
+      if ((N & 3) == 0) {
+        bias_pk[jq] = *reinterpret_cast<const uint2*>(src + min(col, N - 4));
+      } else {
+        uint32_t v[4];
+#pragma unroll
+        for (int t = 0; t < 4; ++t) v[t] = src[min(col + t, N - 1)];
+        bias_pk[jq] = make_uint2(v[0] | (v[1] << 16), v[2] | (v[3] << 16));
+      }
+    }
+  }
+}
+
 template <int EPI, int TM, int TN>
 __device__ __forceinline__ void store_tile(floatx16 (&acc)[TM / 32][TN / 32], unsigned char* smem,
-                                           int wave, int lane, const bf16_t* __restrict__ bias,
-                                           bf16_t* __restrict__ C, int b, int R, int N, int wrow0,
-                                           int wcol0) {
+                                           int wave, int lane, const uint2 (&bias_pk)[TN / 8],
+                                           bool has_bias, bf16_t* __restrict__ C, int b, int R, int N,
+                                           int wrow0, int wcol0) {
   constexpr int FM = TM / 32, FN = TN / 32, OLD = TN + 8;
   const int m = lane & 31, h = lane >> 5;
-  const bf16_t* biasb = bias != nullptr ? bias + (size_t)b * N : nullptr;
   bf16_t* Cb = C + (size_t)b * R * N;
   bf16_t* so = reinterpret_cast<bf16_t*>(smem) + (size_t)wave * TM * OLD;
   auto stage = [&](auto has_bias_c) {
@@ -128,12 +152,8 @@ __device__ __forceinline__ void store_tile(floatx16 (&acc)[TM / 32][TN / 32], un
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
         const int cl = j * 32 + q * 8 + h * 4;          // column inside the wave tile
-        const int col = wcol0 + cl;
-        float bv[4] = {0.f, 0.f, 0.f, 0.f};
-        if (kHasBias) {
-#pragma unroll
-          for (int t = 0; t < 4; ++t) bv[t] = bf2f(biasb[min(col + t, N - 1)]);
-        }
+        const uint2 bp = bias_pk[j * 4 + q];
+        const float bv[4] = {bf_lo(bp.x), bf_hi(bp.x), bf_lo(bp.y), bf_hi(bp.y)};
 #pragma unroll
         for (int i = 0; i < FM; ++i) {
           const uint32_t p0 = epilogue_pair<EPI, kHasBias>(acc[i][j][q * 4], acc[i][j][q * 4 + 1], bv[0], bv[1]);
@@ -143,7 +163,7 @@ __device__ __forceinline__ void store_tile(floatx16 (&acc)[TM / 32][TN / 32], un
       }
     }
   };
-  if (biasb != nullptr) stage(std::true_type{});
+  if (has_bias) stage(std::true_type{});
   else stage(std::false_type{});
   // Each wave reads back only what it wrote (LDS operations of a wave complete in order).
   constexpr int kChunksOut = TN / 8;                  // 16-byte chunks per staged row
@@ -310,33 +330,43 @@ __global__ __launch_bounds__(Cfg::kThreads, Cfg::kBlocksPerCu) void gemm_bf16_ke
     }
     __builtin_amdgcn_sched_barrier(0);
   };
-  // The loop body is one basic block (no branches), so that the scheduling hints
-  // hold and the fragment reads / DMA loads really are issued under the MFMAs:
-  // past the end of K the loads re-fetch the last k tile into a stage nobody
-  // reads any more, and the last iteration pre-reads fragments nobody uses.
-  // A k tile has landed when at most the PD-1 tiles issued after it are in flight.
-  static_assert((PD - 1) * L < 64, "vmcnt");
+  // Waits until a k tile has landed, given how many tiles were issued after it.
+  auto wait_tile = [&](int younger) {
+    if (younger >= PD - 1) wait_vmcnt<(PD - 1) * L>();
+    else if (PD >= 3 && younger == PD - 2) wait_vmcnt<(PD >= 3 ? PD - 2 : 0) * L>();
+    else if (PD >= 4 && younger == PD - 3) wait_vmcnt<(PD >= 4 ? PD - 3 : 0) * L>();
+    else wait_vmcnt<0>();
+  };
+  static_assert(PD <= 4, "wait_tile covers up to 4 tiles of prefetch");
   static_assert(KS == 2, "the two halves of a tile's loads go with its two k slices");
+  uint2 bias_pk[Cfg::TN / 8];
+  load_bias<Cfg::TN>(bias_pk, bias, b, N, col0 + wn * Cfg::TN, lane);
+
   const int nk = Kd / BK;
+  const int pro = min(PD, nk);
 #pragma unroll
-  for (int t = 0; t < PD; ++t) {
-    load_a(t, min(t, nk - 1) * BK);
-    load_b(t, min(t, nk - 1) * BK);
-  }
-  wait_vmcnt<(PD - 1) * L>();
+  for (int t = 0; t < PD; ++t)
+    if (t < pro) {
+      load_a(t, t * BK);
+      load_b(t, t * BK);
+    }
+  wait_tile(pro - 1);
   raw_barrier();
   load_frags(0, 0, 0);
   int stage = 0;
-  for (int kt = 0; kt < nk; ++kt) {
+  // Steady state: the body is one basic block (no branches), so that the
+  // scheduling hints hold and the fragment reads / DMA loads really are issued
+  // under the MFMAs.  Tile kt + 1 has landed when only the younger loads (PD - 2
+  // whole tiles and the A half of tile kt + PD) are still in flight.
+  const int steady = nk - PD;
+  for (int kt = 0; kt < steady; ++kt) {
     const int next_stage = stage + 1 == NS ? 0 : stage + 1;
     const int load_stage = stage == 0 ? NS - 1 : stage - 1;   // (kt + PD) % NS
-    const int load_k0 = min(kt + PD, nk - 1) * BK;
-    // slice 0: fragments of slice 1, A half of tile kt + PD
+    const int load_k0 = (kt + PD) * BK;
     load_frags(1, stage, 1);
     load_a(load_stage, load_k0);
     mfma_slice(0);
     slice_schedule(std::integral_constant<int, Cfg::kAIssues>{});
-    // slice 1: tile kt + 1 has landed when only the younger loads are in flight
     wait_vmcnt<(PD - 2) * L + Cfg::kAIssues>();
     wait_lgkmcnt0();
     raw_barrier();
@@ -346,11 +376,27 @@ __global__ __launch_bounds__(Cfg::kThreads, Cfg::kBlocksPerCu) void gemm_bf16_ke
     slice_schedule(std::integral_constant<int, Cfg::kBIssues>{});
     stage = next_stage;
   }
+  // Drain: the last min(PD, nk) tiles, nothing left to load.
+  for (int kt = steady > 0 ? steady : 0; kt < nk; ++kt) {
+    const int next_stage = stage + 1 == NS ? 0 : stage + 1;
+    load_frags(1, stage, 1);
+    mfma_slice(0);
+    slice_schedule(std::integral_constant<int, 0>{});
+    if (kt + 1 < nk) {
+      wait_tile(nk - 2 - kt);
+      wait_lgkmcnt0();
+      raw_barrier();
+      load_frags(0, next_stage, 0);
+    }
+    mfma_slice(1);
+    slice_schedule(std::integral_constant<int, 0>{});
+    stage = next_stage;
+  }
   wait_lgkmcnt0();
   __syncthreads();   // all waves are done with the operand tiles: LDS is reused below
 
-  store_tile<EPI, Cfg::TM, Cfg::TN>(acc, smem, wave, lane, bias, C, b, R, N, row0 + wm * Cfg::TM,
-                                    col0 + wn * Cfg::TN);
+  store_tile<EPI, Cfg::TM, Cfg::TN>(acc, smem, wave, lane, bias_pk, bias != nullptr, C, b, R, N,
+                                    row0 + wm * Cfg::TM, col0 + wn * Cfg::TN);
 }
 
 // Generic path (any Kd % 8 == 0): 128x128 tile, operands staged through
