@@ -96,7 +96,7 @@ struct GemmCfg {
   static constexpr int kBIssues = BN / kRowsPerLoad / kWaves;
   static constexpr int kLoads = kAIssues + kBIssues;  // DMA instructions per wave per k tile
   static_assert(BK == 32 || BK == 64, "BK");
-  static_assert(NSTAGE >= 2 && (NSTAGE - 1) * kLoads < 64, "vmcnt is a 6-bit counter");
+  static_assert(NSTAGE >= 2 && NSTAGE * kLoads < 64, "vmcnt is a 6-bit counter");
   static_assert(BM % (WM * 32) == 0 && BN % (WN * 32) == 0, "wave tile must be 32-aligned");
   static_assert(BM % (kRowsPerLoad * kWaves) == 0 && BN % (kRowsPerLoad * kWaves) == 0,
                 "tile loads must divide evenly");
@@ -338,14 +338,17 @@ __global__ __launch_bounds__(Cfg::kThreads, Cfg::kBlocksPerCu) void gemm_bf16_ke
     else wait_vmcnt<0>();
   };
   static_assert(PD <= 4, "wait_tile covers up to 4 tiles of prefetch");
-  static_assert(KS == 2, "the two halves of a tile's loads go with its two k slices");
+  static_assert(KS == 2, "slice schedule");
   uint2 bias_pk[Cfg::TN / 8];
   load_bias<Cfg::TN>(bias_pk, bias, b, N, col0 + wn * Cfg::TN, lane);
 
+  // All NS stages are in use: the barrier inside iteration kt (every wave has read
+  // the last fragments of tile kt) frees stage kt % NS, and the loads of tile
+  // kt + NS go out right behind it, under the MFMAs of the second k slice.
   const int nk = Kd / BK;
-  const int pro = min(PD, nk);
+  const int pro = min(NS, nk);
 #pragma unroll
-  for (int t = 0; t < PD; ++t)
+  for (int t = 0; t < NS; ++t)
     if (t < pro) {
       load_a(t, t * BK);
       load_b(t, t * BK);
@@ -356,27 +359,26 @@ __global__ __launch_bounds__(Cfg::kThreads, Cfg::kBlocksPerCu) void gemm_bf16_ke
   int stage = 0;
   // Steady state: the body is one basic block (no branches), so that the
   // scheduling hints hold and the fragment reads / DMA loads really are issued
-  // under the MFMAs.  Tile kt + 1 has landed when only the younger loads (PD - 2
-  // whole tiles and the A half of tile kt + PD) are still in flight.
-  const int steady = nk - PD;
+  // under the MFMAs.  Tile kt + 1 has landed when only the PD - 1 tiles issued
+  // after it are still in flight.
+  const int steady = nk - NS;
   for (int kt = 0; kt < steady; ++kt) {
     const int next_stage = stage + 1 == NS ? 0 : stage + 1;
-    const int load_stage = stage == 0 ? NS - 1 : stage - 1;   // (kt + PD) % NS
-    const int load_k0 = (kt + PD) * BK;
+    const int load_k0 = (kt + NS) * BK;
     load_frags(1, stage, 1);
-    load_a(load_stage, load_k0);
     mfma_slice(0);
-    slice_schedule(std::integral_constant<int, Cfg::kAIssues>{});
-    wait_vmcnt<(PD - 2) * L + Cfg::kAIssues>();
+    slice_schedule(std::integral_constant<int, 0>{});
+    wait_vmcnt<(PD - 1) * L>();
     wait_lgkmcnt0();
     raw_barrier();
     load_frags(0, next_stage, 0);
-    load_b(load_stage, load_k0);
+    load_a(stage, load_k0);
+    load_b(stage, load_k0);
     mfma_slice(1);
-    slice_schedule(std::integral_constant<int, Cfg::kBIssues>{});
+    slice_schedule(std::integral_constant<int, L>{});
     stage = next_stage;
   }
-  // Drain: the last min(PD, nk) tiles, nothing left to load.
+  // Drain: the last min(NS, nk) tiles, nothing left to load.
   for (int kt = steady > 0 ? steady : 0; kt < nk; ++kt) {
     const int next_stage = stage + 1 == NS ? 0 : stage + 1;
     load_frags(1, stage, 1);
