@@ -206,6 +206,7 @@ __global__ __launch_bounds__(kThreads, 2) void einsum_dispatch_bf16_kernel(
         acc[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f1, wf[ks], acc[1], 0, 0, 0);
       }
     }
+    mfma_result_fence();
     stage_tile(acc, so, m, h);
     store_staged(so, out, orow, lane, t * kTileD, D);
     wait_lgkmcnt0();
@@ -295,6 +296,7 @@ __global__ __launch_bounds__(kThreads, 2) void einsum_combine_bf16_kernel(
             acc[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f1, wf[i][ks], acc[1], 0, 0, 0);
           }
         }
+        mfma_result_fence();
         stage_tile(acc, so, m, h);
         store_staged(so, out, orow[i], lane, t * kTileD, D);
       }

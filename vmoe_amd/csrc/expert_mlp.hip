@@ -57,6 +57,7 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(
       acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a, bb, acc, 0, 0, 0);
     }
   }
+  mfma_result_fence();
   const int col = col0 + wn * 32 + m;
   const bool col_ok = col < N;
   const float bv = (bias != nullptr && col_ok) ? bias[(size_t)b * N + col] : 0.f;

@@ -7,9 +7,9 @@
 // staged once per workgroup in LDS (bf16: transposed to [expert][k] so that a
 // lane's MFMA B fragment is one 16-byte read; f32: kept [k][expert]).  Item rows
 // stream from HBM with 16-byte loads, 64 contiguous bytes per lane per step.
-// After the K loop a 32x32 accumulator tile holds, per lane, one expert column
-// for 16 item rows; the softmax and the top-K run across the 32 lanes of a
-// half-wave with xor shuffles, 16 rows at a time.
+// After the K loop the logits tile passes through a wave-private LDS tile, so
+// that each lane holds half of one item's row: softmax and top-K are serial per
+// lane, with one xor-32 shuffle per reduction to join the two halves.
 #include "vmoe_common.h"
 
 namespace vmoe {
@@ -64,7 +64,7 @@ template <typename T, int NT>
 __global__ __launch_bounds__(kGateThreads) void gate_topk_kernel(
     const T* __restrict__ x, const T* __restrict__ w, const float* __restrict__ bias,
     T* __restrict__ gates, float* __restrict__ topk_val, int32_t* __restrict__ topk_idx,
-    int num_items, int D, int E, int K, int KC, int num_chunks, int num_tiles) {
+    int num_items, int D, int E, int K, int KC, int num_chunks, int num_tiles, int stage_off) {
   extern __shared__ __align__(16) unsigned char smem[];
   T* wl = reinterpret_cast<T*>(smem);
   constexpr int EP = NT * 32;
@@ -153,6 +153,7 @@ __global__ __launch_bounds__(kGateThreads) void gate_topk_kernel(
               }
             }
           }
+          mfma_result_fence();
         }
       } else {
         const int nkb = KC / 16;
@@ -174,64 +175,95 @@ __global__ __launch_bounds__(kGateThreads) void gate_topk_kernel(
               acc[nt] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], b, acc[nt], 0, 0, 0);
             }
           }
+          mfma_result_fence();
         }
       }
     }
     if (!active) continue;
 
-    // Epilogue: 16 accumulator registers = 16 item rows per half-wave.
-    float bn[NT];
+    // Epilogue.  The 32 x EP tile of (rounded, biased) logits goes through a
+    // wave-private LDS tile so that a lane ends up with half of one item's row in
+    // registers (lane = item r, half h of the experts): softmax and top-K are then
+    // serial per lane, and the two halves of a row meet with a single xor-32
+    // shuffle per reduction instead of a five-step butterfly per row.
+    float* st = reinterpret_cast<float*>(smem + stage_off) + (size_t)wave * 32 * (EP + 1);
+    {
+      float bn[NT];
 #pragma unroll
-    for (int nt = 0; nt < NT; ++nt) {
-      int n = nt * 32 + m;
-      bn[nt] = (bias != nullptr && n < E) ? bias[n] : 0.f;
+      for (int nt = 0; nt < NT; ++nt) {
+        int n = nt * 32 + m;
+        bn[nt] = (bias != nullptr && n < E) ? bias[n] : 0.f;
+      }
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          const int rl = (i >> 2) * 8 + h * 4 + (i & 3);
+          float v = Elt<T>::round(acc[nt][i]);
+          if (bias != nullptr) v = Elt<T>::round(v + bn[nt]);
+          st[rl * (EP + 1) + nt * 32 + m] = v;
+        }
     }
+    constexpr int CNT = EP / 2;          // experts per lane
+    const int row = row0 + m;
+    const int n0 = h * CNT;
+    float g[CNT];
+    float mx = -INFINITY;
 #pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      const int row = row0 + (i >> 2) * 8 + h * 4 + (i & 3);
-      float g[NT];
-      float mx = -INFINITY;
+    for (int j = 0; j < CNT; ++j) {
+      const float v = st[m * (EP + 1) + n0 + j];
+      g[j] = (n0 + j < E) ? v : -INFINITY;
+      mx = fmaxf(mx, g[j]);
+    }
+    mx = fmaxf(mx, __shfl_xor(mx, 32, kWave));
+    float sum = 0.f;
 #pragma unroll
-      for (int nt = 0; nt < NT; ++nt) {
-        float v = Elt<T>::round(acc[nt][i]);
-        if (bias != nullptr) v = Elt<T>::round(v + bn[nt]);
-        g[nt] = (nt * 32 + m < E) ? v : -INFINITY;
-        mx = fmaxf(mx, g[nt]);
-      }
-      mx = half_wave_max(mx);
-      float sum = 0.f;
+    for (int j = 0; j < CNT; ++j) {
+      g[j] = (n0 + j < E) ? expf(g[j] - mx) : 0.f;
+      sum += g[j];
+    }
+    sum += __shfl_xor(sum, 32, kWave);
 #pragma unroll
-      for (int nt = 0; nt < NT; ++nt) {
-        g[nt] = (nt * 32 + m < E) ? expf(g[nt] - mx) : 0.f;
-        sum += g[nt];
-      }
-      sum = half_wave_sum(sum);
+    for (int j = 0; j < CNT; ++j) g[j] = Elt<T>::round(g[j] / sum);
+    const bool row_ok = row < num_items;
+    if (gates != nullptr && row_ok) {
+      T* grow = gates + (size_t)row * E + n0;
+      if (kBf16 && (E & 7) == 0 && (reinterpret_cast<uintptr_t>(gates) & 15u) == 0) {
 #pragma unroll
-      for (int nt = 0; nt < NT; ++nt) g[nt] = Elt<T>::round(g[nt] / sum);
-      const bool row_ok = row < num_items;
-      if (gates != nullptr && row_ok) {
+        for (int j = 0; j < CNT; j += 8) {
+          if (n0 + j < E) {
+            uint32_t pk[4];
 #pragma unroll
-        for (int nt = 0; nt < NT; ++nt)
-          if (nt * 32 + m < E) Elt<T>::store(gates + (size_t)row * E + nt * 32 + m, g[nt]);
-      }
-      uint32_t taken = 0;
-      for (int kk = 0; kk < K; ++kk) {
-        uint64_t best = 0;
-#pragma unroll
-        for (int nt = 0; nt < NT; ++nt) {
-          int n = nt * 32 + m;
-          if (n < E && !(taken >> nt & 1u)) {
-            uint64_t key = ((uint64_t)orderable(g[nt]) << 32) | (uint32_t)(0xFFFFFFFFu - (uint32_t)n);
-            best = key > best ? key : best;
+            for (int t = 0; t < 4; ++t) pk[t] = pack_bf16x2(g[j + 2 * t], g[j + 2 * t + 1]);
+            *reinterpret_cast<uint4*>(grow + j) = make_uint4(pk[0], pk[1], pk[2], pk[3]);
           }
         }
-        best = half_wave_max_u64(best);
-        const int n_star = (int)(0xFFFFFFFFu - (uint32_t)best);
-        if ((n_star & 31) == m) taken |= 1u << (n_star >> 5);
-        if (m == 0 && row_ok) {
-          topk_val[(size_t)row * K + kk] = inv_orderable((uint32_t)(best >> 32));
-          topk_idx[(size_t)row * K + kk] = n_star;
+      } else {
+#pragma unroll
+        for (int j = 0; j < CNT; ++j)
+          if (n0 + j < E) Elt<T>::store(grow + j, g[j]);
+      }
+    }
+    uint64_t taken = 0;
+    for (int kk = 0; kk < K; ++kk) {
+      uint64_t best = 0;
+#pragma unroll
+      for (int j = 0; j < CNT; ++j) {
+        const int n = n0 + j;
+        if (n < E && !(taken >> j & 1ull)) {
+          uint64_t key = ((uint64_t)orderable(g[j]) << 32) | (uint32_t)(0xFFFFFFFFu - (uint32_t)n);
+          best = key > best ? key : best;
         }
+      }
+      const uint32_t olo = __shfl_xor((uint32_t)best, 32, kWave);
+      const uint32_t ohi = __shfl_xor((uint32_t)(best >> 32), 32, kWave);
+      const uint64_t other = ((uint64_t)ohi << 32) | olo;
+      best = other > best ? other : best;
+      const int n_star = (int)(0xFFFFFFFFu - (uint32_t)best);
+      if (n_star >= n0 && n_star < n0 + CNT) taken |= 1ull << (n_star - n0);
+      if (h == 0 && row_ok) {
+        topk_val[(size_t)row * K + kk] = inv_orderable((uint32_t)(best >> 32));
+        topk_idx[(size_t)row * K + kk] = n_star;
       }
     }
   }
@@ -369,13 +401,16 @@ int launch_gate(const VmoeGateTopkParams* p, hipStream_t stream) {
   const int ep = (nt == 3 ? 4 : nt) * 32;
   const int gran = sizeof(T) == 2 ? 64 : 16;
   const int dpad = (p->D + gran - 1) / gran * gran;
-  // Keep the staged router kernel within 96 KiB of LDS; split D otherwise.
-  const size_t budget = 96 * 1024;
+  // LDS: the staged router kernel (split along D when it would not fit) and,
+  // behind it, a 32 x (ep + 1) float32 logits tile per wave for the epilogue.
+  const size_t stage_bytes = (size_t)kGateWaves * 32 * (ep + 1) * sizeof(float);
+  const size_t budget = 88 * 1024;
   int kc = dpad;
   while ((size_t)(sizeof(T) == 2 ? ep * (kc + 8) : kc * ep) * sizeof(T) > budget && kc > gran)
     kc = ((kc / 2) + gran - 1) / gran * gran;
   const int num_chunks = (dpad + kc - 1) / kc;
-  const size_t lds = (size_t)(sizeof(T) == 2 ? ep * (kc + 8) : kc * ep) * sizeof(T);
+  const size_t w_bytes = ((size_t)(sizeof(T) == 2 ? ep * (kc + 8) : kc * ep) * sizeof(T) + 15) / 16 * 16;
+  const size_t lds = w_bytes + stage_bytes;
   const int num_tiles = (p->num_items + 31) / 32;
   int blocks = (num_tiles + kGateWaves - 1) / kGateWaves;
   if (blocks > 1024) blocks = 1024;
@@ -385,7 +420,8 @@ int launch_gate(const VmoeGateTopkParams* p, hipStream_t stream) {
     if (e != hipSuccess) return (int)e;
     hipLaunchKernelGGL(kern, dim3(blocks), dim3(kGateThreads), lds, stream,
                        (const T*)p->x, (const T*)p->w, p->logit_bias, (T*)p->gates, p->topk_val,
-                       p->topk_idx, p->num_items, p->D, p->E, p->K, kc, num_chunks, num_tiles);
+                       p->topk_idx, p->num_items, p->D, p->E, p->K, kc, num_chunks, num_tiles,
+                       (int)w_bytes);
     return launch_status();
   };
   switch (nt) {

@@ -396,6 +396,7 @@ __global__ __launch_bounds__(Cfg::kThreads, Cfg::kBlocksPerCu) void gemm_bf16_ke
   }
   wait_lgkmcnt0();
   __syncthreads();   // all waves are done with the operand tiles: LDS is reused below
+  mfma_result_fence();
 
   store_tile<EPI, Cfg::TM, Cfg::TN>(acc, smem, wave, lane, bias_pk, bias != nullptr, C, b, R, N,
                                     row0 + wm * Cfg::TM, col0 + wn * Cfg::TN);
@@ -463,6 +464,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_generic_kernel(
           acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[j], fa[i], acc[i][j], 0, 0, 0);
     }
   }
+  mfma_result_fence();
   const bf16_t* biasb = bias != nullptr ? bias + (size_t)b * N : nullptr;
   bf16_t* Cb = C + (size_t)b * R * N;
 #pragma unroll

@@ -154,6 +154,7 @@ __global__ __launch_bounds__(256) void soft_route_kernel(
           }
         }
       }
+      mfma_result_fence();
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         if (ct0 + j >= col_tiles) continue;
@@ -392,6 +393,7 @@ __global__ __launch_bounds__(kSrThreads) void soft_route_bf16_kernel(
         // bound how many fragment reads the scheduler hoists (register pressure)
         if ((i & 3) == 3) __builtin_amdgcn_sched_barrier(0);
       }
+      mfma_result_fence();
       const int col = wave * 16 + r16;
 #pragma unroll
       for (int rh = 0; rh < 2; ++rh)
@@ -540,6 +542,7 @@ __global__ __launch_bounds__(256) void einsum_kernel(const void* __restrict__ w,
       acc = __builtin_amdgcn_mfma_f32_32x32x2f32(sa[wm * 32 + m][ks * 2 + h],
                                                  sb[ks * 2 + h][wn * 32 + m], acc, 0, 0, 0);
   }
+  mfma_result_fence();
   const int col = col0 + wn * 32 + m;
 #pragma unroll
   for (int v = 0; v < 16; ++v) {

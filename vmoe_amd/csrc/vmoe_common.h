@@ -98,6 +98,19 @@ __device__ __forceinline__ void raw_barrier() {
   __builtin_amdgcn_sched_barrier(0);
 }
 
+// Gap between the last MFMA of a loop and the first read of its accumulators.
+// The matrix cores write a result over many cycles and a reader must leave
+// enough wait states.  The compiler counts them within straight-line code, but
+// a v_mfma_f32_32x32x16_bf16 result read a few instructions behind a loop
+// back-edge came back with its last register stale (rows 27 and 31 of every
+// tile wrong), so every kernel states the gap explicitly before it touches
+// accumulators that a loop has just written.
+__device__ __forceinline__ void mfma_result_fence() {
+  __builtin_amdgcn_sched_barrier(0);
+  asm volatile("s_nop 15\n\ts_nop 15\n\ts_nop 15\n\ts_nop 15" ::: "memory");
+  __builtin_amdgcn_sched_barrier(0);
+}
+
 inline hipStream_t as_stream(vmoe_stream_t s) { return reinterpret_cast<hipStream_t>(s); }
 
 inline int launch_status() {
