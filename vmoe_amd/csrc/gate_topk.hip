@@ -103,15 +103,27 @@ __global__ __launch_bounds__(kGateThreads) void gate_topk_kernel(
         constexpr int VW = 16 / (int)sizeof(T);
         if (E % VW == 0 && (reinterpret_cast<uintptr_t>(w) & 15u) == 0) {
           const int vec_per_row = EP / VW;
-          for (int idx = tid; idx < KC * vec_per_row; idx += kGateThreads) {
-            const int k = idx / vec_per_row, n0 = (idx - k * vec_per_row) * VW;
-            uint4 raw = make_uint4(0, 0, 0, 0);
-            if (k0 + k < D && n0 < E)
-              raw = *reinterpret_cast<const uint4*>(w + (size_t)(k0 + k) * E + n0);
-            const T* v = reinterpret_cast<const T*>(&raw);
+          constexpr int kBatch = 6;   // independent loads in flight per thread
+          for (int idx0 = tid; idx0 < KC * vec_per_row; idx0 += kBatch * kGateThreads) {
+            uint4 raw[kBatch];
 #pragma unroll
-            for (int t = 0; t < VW; ++t) {
-              if (kBf16) wl[(n0 + t) * stride + k] = v[t]; else wl[k * stride + n0 + t] = v[t];
+            for (int u = 0; u < kBatch; ++u) {
+              const int idx = idx0 + u * kGateThreads;
+              const int k = idx / vec_per_row, n0 = (idx - k * vec_per_row) * VW;
+              raw[u] = make_uint4(0, 0, 0, 0);
+              if (idx < KC * vec_per_row && k0 + k < D && n0 < E)
+                raw[u] = *reinterpret_cast<const uint4*>(w + (size_t)(k0 + k) * E + n0);
+            }
+#pragma unroll
+            for (int u = 0; u < kBatch; ++u) {
+              const int idx = idx0 + u * kGateThreads;
+              if (idx >= KC * vec_per_row) continue;
+              const int k = idx / vec_per_row, n0 = (idx - k * vec_per_row) * VW;
+              const T* v = reinterpret_cast<const T*>(&raw[u]);
+#pragma unroll
+              for (int t = 0; t < VW; ++t) {
+                if (kBf16) wl[(n0 + t) * stride + k] = v[t]; else wl[k * stride + n0 + t] = v[t];
+              }
             }
           }
         } else {
@@ -127,7 +139,7 @@ __global__ __launch_bounds__(kGateThreads) void gate_topk_kernel(
       if (!active) continue;
       if constexpr (kBf16) {
         const int nkb = KC / 64;
-        constexpr int UB = 3;   // 64-k blocks in flight per step (12 x 16-byte loads per lane)
+        constexpr int UB = 6;   // 64-k blocks in flight per step (24 x 16-byte loads per lane)
         for (int kb0 = 0; kb0 < nkb; kb0 += UB) {
           uint4 a[UB][4];
 #pragma unroll
