@@ -206,6 +206,7 @@ __global__ __launch_bounds__(Cfg::kThreads, Cfg::kBlocksPerCu) void gemm_bf16_ke
     const bf16_t* __restrict__ A, const bf16_t* __restrict__ Bt, const bf16_t* __restrict__ bias,
     bf16_t* __restrict__ C, int R, int N, int Kd, int tiles_m, int tiles_n, int num_tiles,
     int tiles_per_xcd) {
+#if defined(__HIP_DEVICE_COMPILE__)   // buffer-resource builtins exist in the device pass only
   extern __shared__ __align__(1024) unsigned char smem[];
   constexpr int BM = Cfg::BM, BN = Cfg::BN, BK = Cfg::BK;
   constexpr int FM = Cfg::FM, FN = Cfg::FN;
@@ -245,20 +246,28 @@ __global__ __launch_bounds__(Cfg::kThreads, Cfg::kBlocksPerCu) void gemm_bf16_ke
   // The DMA loads of a k tile are issued in two halves (A rows, then B rows), one
   // under the MFMAs of each k slice: a wave sustains about one 1 KB DMA load per
   // 80 clocks, so they must be spread out or the wave stalls behind them.
+  // Buffer addressing: the descriptor carries the operand's base, the lane's byte
+  // offset is loop-invariant and the advance along k is a scalar, so a DMA load
+  // needs no per-iteration address arithmetic and moves one address dword per
+  // lane instead of two.
+  const __amdgpu_buffer_rsrc_t a_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<unsigned char*>(Ab), 0, -1, 0x00020000);
+  const __amdgpu_buffer_rsrc_t b_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<unsigned char*>(Bb), 0, -1, 0x00020000);
   auto load_a = [&](int stage, int k0) {
     unsigned char* s = smem + stage * Cfg::kStageBytes;
 #pragma unroll
     for (int i = 0; i < Cfg::kAIssues; ++i)
-      __builtin_amdgcn_global_load_lds((global_ptr_t)(Ab + a_goff[i] + (size_t)k0 * 2),
-                                       (lds_ptr_t)(s + (i * Cfg::kWaves + wave) * RPL * RB), 16, 0, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(a_rsrc, (lds_ptr_t)(s + (i * Cfg::kWaves + wave) * RPL * RB),
+                                               16, a_goff[i], k0 * 2, 0, 0);
   };
   auto load_b = [&](int stage, int k0) {
     unsigned char* s = smem + stage * Cfg::kStageBytes;
 #pragma unroll
     for (int i = 0; i < Cfg::kBIssues; ++i)
-      __builtin_amdgcn_global_load_lds((global_ptr_t)(Bb + b_goff[i] + (size_t)k0 * 2),
-                                       (lds_ptr_t)(s + BM * RB + (i * Cfg::kWaves + wave) * RPL * RB),
-                                       16, 0, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(
+          b_rsrc, (lds_ptr_t)(s + BM * RB + (i * Cfg::kWaves + wave) * RPL * RB), 16, b_goff[i],
+          k0 * 2, 0, 0);
   };
 
   floatx16 acc[FM][FN];
@@ -400,6 +409,7 @@ __global__ __launch_bounds__(Cfg::kThreads, Cfg::kBlocksPerCu) void gemm_bf16_ke
 
   store_tile<EPI, Cfg::TM, Cfg::TN>(acc, smem, wave, lane, bias_pk, bias != nullptr, C, b, R, N,
                                     row0 + wm * Cfg::TM, col0 + wn * Cfg::TN);
+#endif
 }
 
 // Generic path (any Kd % 8 == 0): 128x128 tile, operands staged through
