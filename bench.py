@@ -30,7 +30,7 @@ PEAK_HBM_GBS = 8000.0
 MEASURED_TRAFFIC_BYTES = {
     # mean of the two GEMM launches of a layer: (885 + 600 + 1159 + 151) / 2 MiB;
     # FETCH_SIZE x 2.0, WRITE_SIZE x 1.0 (copy-kernel calibration).
-    "vmoe_b16_layer_E32_k2_bpr": 1.466e9,
+    "vmoe_b16_layer_E32_k2_bpr": 1.607e9,
 }
 
 
@@ -257,6 +257,17 @@ def main():
   torch.cuda.synchronize()
   copy_gbs = 2 * n * 5 / (e0.elapsed_time(e1) * 1e-3) / 1e9
   del src, dst
+  # Measured arithmetic ceiling of the same device: a register-resident MFMA loop
+  # on operand fragments taken from the layer's own hidden activations.
+  if b == 2:
+    seed = out.reshape(-1)[: 1 << 20].contiguous()
+    kernels.mfma_probe(seed, 256, 500)
+    e0.record()
+    probe_flops = kernels.mfma_probe(seed, 256, 4000)
+    e1.record()
+    torch.cuda.synchronize()
+    roofline["measured_mfma_loop_TFLOPs"] = probe_flops / (e0.elapsed_time(e1) * 1e-3) / 1e12
+    roofline["frac_of_measured_loop"] = achieved_tflops / roofline["measured_mfma_loop_TFLOPs"]
   hbm = {
       "dispatch_GBps": bytes_dispatch / (stage_ms["vmoe_dispatch"] * 1e-3) / 1e9,
       "combine_GBps": bytes_combine / (stage_ms["vmoe_combine"] * 1e-3) / 1e9,

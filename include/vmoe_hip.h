@@ -278,6 +278,14 @@ int vmoe_cast(const VmoeCastParams* p, vmoe_stream_t stream);
  * that bandwidth figures are compared with. */
 int vmoe_copy_bytes(const void* in, void* out, size_t n, vmoe_stream_t stream);
 
+/* Register-resident v_mfma_f32_32x32x16_bf16 loop: the measured arithmetic
+ * ceiling that the expert GEMM figures are compared with (no counterpart in the
+ * reference; measurement aid like vmoe_copy_bytes).  Operand fragments are read
+ * once from `seed` (seed_bytes >= 16, 16-byte aligned); `sink` receives
+ * blocks * 256 floats; *flops is set to the floating-point operations issued. */
+int vmoe_mfma_probe(const void* seed, size_t seed_bytes, void* sink, int32_t blocks,
+                    int32_t iters, double* flops, vmoe_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -24,7 +24,7 @@ EXPORTS = [
     "vmoe_route_assign", "vmoe_indices_to_slots", "vmoe_dispatch", "vmoe_combine", "vmoe_densify",
     "vmoe_expert_mlp_workspace_bytes", "vmoe_expert_mlp", "vmoe_pack_expert_weights",
     "vmoe_soft_route_workspace_bytes", "vmoe_soft_route", "vmoe_einsum_dispatch",
-    "vmoe_einsum_combine", "vmoe_cast", "vmoe_copy_bytes",
+    "vmoe_einsum_combine", "vmoe_cast", "vmoe_copy_bytes", "vmoe_mfma_probe",
 ]
 
 

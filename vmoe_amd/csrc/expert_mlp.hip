@@ -122,6 +122,51 @@ int transpose(const void* in, void* out, int batch, int rows, int cols, int dtyp
 using CfgUp = GemmCfg<128, 256, 2, 2, 32, 3, 2>;
 using CfgDown = GemmCfg<256, 256, 2, 2, 32, 4, 1>;
 
+// Register-resident MFMA loop: the arithmetic ceiling that the expert GEMMs are
+// compared with.  Every wave keeps a 128 x 128 accumulator tile (16 MFMA tiles,
+// as in the 256 x 256 GEMM) and multiplies operand fragments that it read once
+// from `seed` (real data, so that operand toggling, and with it the clock the
+// power management settles on, resembles the GEMM's); nothing moves but
+// registers.
+__global__ __launch_bounds__(256) void mfma_probe_kernel(const uint4* __restrict__ seed,
+                                                         float* __restrict__ sink, int iters,
+                                                         size_t seed_vecs) {
+  bf16x8 fa[2][4], fb[2][4];
+#pragma unroll
+  for (int u = 0; u < 2; ++u)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const size_t base = ((size_t)blockIdx.x * 256 + threadIdx.x) * 16 + u * 8 + i * 2;
+      fa[u][i] = __builtin_bit_cast(bf16x8, seed[base % seed_vecs]);
+      fb[u][i] = __builtin_bit_cast(bf16x8, seed[(base + 1) % seed_vecs]);
+    }
+  floatx16 acc[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+  for (int it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int u = 0; u < 2; ++u)
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[u][j], fa[u][i], acc[i][j], 0, 0, 0);
+  }
+  mfma_result_fence();
+  float t = 0.f;
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) t += acc[i][j][v];
+  sink[(size_t)blockIdx.x * 256 + threadIdx.x] = t;
+}
+
 size_t align256(size_t v) { return (v + 255) / 256 * 256; }
 
 }  // namespace
@@ -215,4 +260,15 @@ extern "C" int vmoe_pack_expert_weights(const VmoeTransposeParams* p, vmoe_strea
   if (p->batch < 1 || p->rows < 1 || p->cols < 1 || p->batch > 65535) return VMOE_E_SHAPE;
   if (p->dtype != VMOE_F32 && p->dtype != VMOE_BF16) return VMOE_E_DTYPE;
   return transpose(p->in, p->out, p->batch, p->rows, p->cols, p->dtype, as_stream(stream));
+}
+
+extern "C" int vmoe_mfma_probe(const void* seed, size_t seed_bytes, void* sink, int32_t blocks,
+                               int32_t iters, double* flops, vmoe_stream_t stream) {
+  if (seed == nullptr || sink == nullptr || flops == nullptr) return VMOE_E_NULL;
+  if (seed_bytes < 16 || !aligned16(seed) || blocks < 1 || iters < 1) return VMOE_E_SHAPE;
+  hipLaunchKernelGGL(mfma_probe_kernel, dim3((unsigned)blocks), dim3(256), 0, as_stream(stream),
+                     (const uint4*)seed, (float*)sink, iters, seed_bytes / 16);
+  // 4 waves x 32 MFMAs of 32 x 32 x 16 per iteration
+  *flops = (double)blocks * 4.0 * iters * 32.0 * (2.0 * 32 * 32 * 16);
+  return launch_status();
 }

@@ -33,6 +33,7 @@
 #ifndef VMOE_GEMM_BF16_H_
 #define VMOE_GEMM_BF16_H_
 
+#include <cmath>
 #include <type_traits>
 #include "vmoe_common.h"
 
@@ -40,7 +41,6 @@ namespace vmoe {
 
 enum { kEpiBias = 0, kEpiBiasGeluTanh = 1, kEpiBiasGeluErf = 2 };
 
-constexpr int kPanelRows = 8;   // row tiles per panel in the tile order
 
 // 0.5 x (1 + tanh(c (x + 0.044715 x^3))) = x * sigmoid(2 c (x + 0.044715 x^3)),
 // with the hardware exp2 and reciprocal (relative error ~1e-7, far inside bf16).
@@ -183,17 +183,17 @@ __device__ __forceinline__ void store_tile(floatx16 (&acc)[TM / 32][TN / 32], un
 
 // XCD-aware workgroup -> (batch, tile_m, tile_n); returns false for padding workgroups.
 __device__ __forceinline__ bool map_tile(int tiles_m, int tiles_n, int num_tiles, int tiles_per_xcd,
-                                         int& b, int& tile_m, int& tile_n) {
+                                         int panel_rows, int& b, int& tile_m, int& tile_n) {
   const int logical = (blockIdx.x % kNumXcd) * tiles_per_xcd + blockIdx.x / kNumXcd;
   if (blockIdx.x / kNumXcd >= tiles_per_xcd || logical >= num_tiles) return false;
   const int per_batch = tiles_m * tiles_n;
   b = logical / per_batch;
   const int rem = logical - b * per_batch;
-  const int panel = rem / (kPanelRows * tiles_n);
-  const int in_panel = rem - panel * kPanelRows * tiles_n;
-  const int rows_here = min(kPanelRows, tiles_m - panel * kPanelRows);
+  const int panel = rem / (panel_rows * tiles_n);
+  const int in_panel = rem - panel * panel_rows * tiles_n;
+  const int rows_here = min(panel_rows, tiles_m - panel * panel_rows);
   tile_n = in_panel / rows_here;
-  tile_m = panel * kPanelRows + in_panel - tile_n * rows_here;
+  tile_m = panel * panel_rows + in_panel - tile_n * rows_here;
   return true;
 }
 
@@ -205,7 +205,7 @@ template <typename Cfg, int EPI>
 __global__ __launch_bounds__(Cfg::kThreads, Cfg::kBlocksPerCu) void gemm_bf16_kernel(
     const bf16_t* __restrict__ A, const bf16_t* __restrict__ Bt, const bf16_t* __restrict__ bias,
     bf16_t* __restrict__ C, int R, int N, int Kd, int tiles_m, int tiles_n, int num_tiles,
-    int tiles_per_xcd) {
+    int tiles_per_xcd, int panel_rows) {
 #if defined(__HIP_DEVICE_COMPILE__)   // buffer-resource builtins exist in the device pass only
   extern __shared__ __align__(1024) unsigned char smem[];
   constexpr int BM = Cfg::BM, BN = Cfg::BN, BK = Cfg::BK;
@@ -218,7 +218,7 @@ __global__ __launch_bounds__(Cfg::kThreads, Cfg::kBlocksPerCu) void gemm_bf16_ke
   const int m = lane & 31, h = lane >> 5;
 
   int b, tile_m, tile_n;
-  if (!map_tile(tiles_m, tiles_n, num_tiles, tiles_per_xcd, b, tile_m, tile_n)) return;
+  if (!map_tile(tiles_m, tiles_n, num_tiles, tiles_per_xcd, panel_rows, b, tile_m, tile_n)) return;
   const int row0 = tile_m * BM, col0 = tile_n * BN;
   const unsigned char* Ab = reinterpret_cast<const unsigned char*>(A + (size_t)b * R * Kd);
   const unsigned char* Bb = reinterpret_cast<const unsigned char*>(Bt + (size_t)b * N * Kd);
@@ -510,13 +510,23 @@ int launch_gemm_bf16(const bf16_t* A, const bf16_t* Bt, const bf16_t* bias, bf16
   if (tiles > 0x7ffffff0LL) return VMOE_E_OVERFLOW;
   const int tiles_per_xcd = (int)((tiles + kNumXcd - 1) / kNumXcd);
   const unsigned blocks = (unsigned)tiles_per_xcd * kNumXcd;
+  // Tile order inside a batch: panels of `panel_rows` row tiles, swept column tile
+  // by column tile.  The tiles that run together on one die (32 compute units)
+  // then form a block of about panel_rows x (concurrent / panel_rows) tiles, whose
+  // operand footprint per tile is smallest when the block's A and B bytes match.
+  const double concurrent = 32.0 * Cfg::kBlocksPerCu;
+  int panel_rows = (int)(std::sqrt(concurrent * Cfg::BN / Cfg::BM) + 0.5);
+  if (panel_rows < 1) panel_rows = 1;
+  if (panel_rows > tiles_m) panel_rows = tiles_m;
+  const int panels = (tiles_m + panel_rows / 2) / panel_rows > 0 ? (tiles_m + panel_rows / 2) / panel_rows : 1;
+  panel_rows = (tiles_m + panels - 1) / panels;
   auto kern = gemm_bf16_kernel<Cfg, EPI>;
   hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                      hipFuncAttributeMaxDynamicSharedMemorySize,
                                      (int)Cfg::kLdsBytes);
   if (e != hipSuccess) return (int)e;
   hipLaunchKernelGGL(kern, dim3(blocks), dim3(Cfg::kThreads), Cfg::kLdsBytes, stream, A, Bt, bias,
-                     C, R, N, Kd, tiles_m, tiles_n, (int)tiles, tiles_per_xcd);
+                     C, R, N, Kd, tiles_m, tiles_n, (int)tiles, tiles_per_xcd, panel_rows);
   return launch_status();
 }
 

@@ -251,3 +251,14 @@ def copy_bytes(src: torch.Tensor, dst: torch.Tensor) -> None:
   n = src.numel() * src.element_size()
   H.check(H.lib().vmoe_copy_bytes(H.ptr(src), H.ptr(dst), H.c_size_t(n), H.stream()),
           "vmoe_copy_bytes")
+
+
+def mfma_probe(seed: torch.Tensor, blocks: int = 256, iters: int = 2000) -> float:
+  """Launches the register-resident MFMA loop on operands read from `seed`;
+  returns the floating-point operations it issues (time it with events)."""
+  sink = torch.empty(blocks * 256, dtype=torch.float32, device=seed.device)
+  flops = H.ctypes.c_double(0.0)
+  n = seed.numel() * seed.element_size()
+  H.check(H.lib().vmoe_mfma_probe(H.ptr(seed), H.c_size_t(n), H.ptr(sink), blocks, iters,
+                                  H.ctypes.byref(flops), H.stream()), "vmoe_mfma_probe")
+  return float(flops.value)
