@@ -126,6 +126,28 @@ typedef struct {
 } VmoeRouteAssignParams;
 int vmoe_route_assign(const VmoeRouteAssignParams* p, vmoe_stream_t stream);
 
+/* Experts-choice ("top items per expert") routing, replacing
+ * _get_top_items_per_expert_einsum_dispatcher (vmoe/moe.py:655-694): each expert
+ * keeps the C items with its largest gates (jax.lax.top_k of the transposed
+ * gates: descending, equal gates -> lower item index first).  The result has the
+ * shape of vmoe_route_assign's with one choice per expert (K = E):
+ * indices[g,s,e] = (e, rank of item s in expert e's order), kept iff rank < C;
+ * weights[g,s,e] = gates[g,s,e] as float32.  The dense (G,S,E,C) one-hot
+ * dispatch_weights / combine_weights of the reference follow with vmoe_densify.
+ * sel_minmax (optional): per (g, e) the smallest and largest selected gate.
+ * Limit: 8*pow2ceil(S) bytes of LDS <= 160 KiB. */
+typedef struct {
+  const void* gates;      /* (G, S, E), dtype */
+  int32_t* indices;       /* out (G, S, E, 2) */
+  int32_t* token_slot;    /* out (G, S, E): slot row, -1 if not selected */
+  int32_t* slot_token;    /* out (E*G*C,): g*S+s, -1 for slots beyond S */
+  float* weights;         /* out (G, S, E) */
+  float* sel_minmax;      /* optional out (G, E, 2) */
+  int32_t G, S, E, C;
+  int32_t dtype;
+} VmoeTopItemsParams;
+int vmoe_top_items_per_expert(const VmoeTopItemsParams* p, vmoe_stream_t stream);
+
 /* Builds the two slot maps from hand-made (expert, position) indices, as
  * vmoe/moe.py:190-197 and :202-206 interpret them: entries with expert >= E or
  * position >= C are dropped.  Negative entries are counted in

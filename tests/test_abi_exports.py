@@ -61,7 +61,8 @@ def test_struct_layouts_match_header():
         "VmoeDispatchParams": _hip.DispatchParams, "VmoeCombineParams": _hip.CombineParams,
         "VmoeDensifyParams": _hip.DensifyParams, "VmoeExpertMlpParams": _hip.ExpertMlpParams,
         "VmoeTransposeParams": _hip.TransposeParams, "VmoeSoftRouteParams": _hip.SoftRouteParams,
-        "VmoeEinsumParams": _hip.EinsumParams, "VmoeCastParams": _hip.CastParams}
+        "VmoeEinsumParams": _hip.EinsumParams, "VmoeCastParams": _hip.CastParams,
+        "VmoeTopItemsParams": _hip.TopItemsParams}
   assert set(py) == set(structs)
   for name, body in structs.items():
     want = []

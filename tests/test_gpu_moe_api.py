@@ -142,6 +142,122 @@ def test_top_items_per_expert_argument_errors(moe):
     moe.get_top_items_per_expert_dispatcher(gates, name="foo", capacity=None, capacity_factor=None)
 
 
+# ------------------------------------------------------------------ GetTopItemsPerExpertDispatcherTest
+def test_top_items_per_expert_einsum_golden(moe, goldens):
+  """vmoe/moe_test.py:275-308."""
+  g = goldens["top_items_per_expert"]
+  gates = to_dev(np.asarray(g["gates"], np.float32))
+  d, metrics = moe.get_top_items_per_expert_dispatcher(gates, name="einsum", capacity=g["capacity"])
+  assert isinstance(d, moe.EinsumDispatcher)
+  np.testing.assert_array_equal(to_np(d.dispatch_weights).astype(bool),
+                                np.asarray(g["dispatch_weights"], bool))
+  np.testing.assert_array_almost_equal(to_np(d.combine_weights),
+                                       np.asarray(g["combine_weights"], np.float32))
+  assert set(metrics) == set(g["metrics"])
+  for k, v in g["metrics"].items():
+    assert float(metrics[k]) == pytest.approx(v, rel=1e-6), k
+
+
+def _experts_choice_gates(rng, G, S, E, dtype, ties):
+  logits = rng.standard_normal((G, S, E)).astype(np.float32)
+  gates = O.softmax(logits)
+  if ties:   # few distinct values: every expert column holds many equal gates
+    gates = np.round(gates * 8) / 8
+  return O.cast(gates, dtype)
+
+
+@pytest.mark.parametrize("G,S,E,C,dtype,ties", [
+    (1, 3, 3, 3, O.F32, False),       # capacity == group size: everything is taken
+    (3, 50, 8, 7, O.F32, False),
+    (3, 50, 8, 7, O.F32, True),
+    (2, 197, 6, 40, O.BF16, False),   # non power-of-two group and expert count
+    (2, 256, 32, 12, O.BF16, True),
+    (1, 1000, 4, 260, O.F32, False),
+])
+def test_top_items_per_expert_vs_oracle(moe, G, S, E, C, dtype, ties):
+  rng = np.random.default_rng(G * 1000 + S + E + C)
+  gates = _experts_choice_gates(rng, G, S, E, dtype, ties)
+  d, metrics = moe.get_top_items_per_expert_dispatcher(to_dev(gates, dtype), name="einsum",
+                                                       capacity=C)
+  cw = to_np(d.combine_weights)
+  dw = to_np(d.dispatch_weights).astype(bool)
+  data = O.cast(rng.standard_normal((G, S, 24)).astype(np.float32), dtype)
+  got_disp = d.dispatch(to_dev(data, dtype))
+  expert_out = O.cast(rng.standard_normal((E, G * C, 24)).astype(np.float32), dtype)
+  got_comb = d.combine(to_dev(expert_out, dtype))
+  want_cw, want_dw = [], []
+  for g in range(G):
+    cw_g, dw_g, m_g = O.top_items_per_expert_einsum(gates[g], C)
+    want_cw.append(cw_g)
+    want_dw.append(dw_g)
+    for k, v in m_g.items():
+      assert float(metrics[k][g]) == pytest.approx(float(v), rel=1e-6), (k, g)
+  want_cw, want_dw = np.stack(want_cw), np.stack(want_dw)
+  np.testing.assert_array_equal(dw, want_dw)        # bit-exact selection, ties included
+  np.testing.assert_array_equal(cw, want_cw)
+  assert dw.sum(axis=(1, 3)).min() == C and dw.sum(axis=(1, 3)).max() == C   # balanced load
+  ref = O.EinsumDispatcher(want_cw, want_dw)
+  np.testing.assert_array_equal(to_np(got_disp), ref.dispatch(data))         # pure row moves
+  rtol = 8e-3 if dtype == O.BF16 else 1e-5
+  assert_close(to_np(got_comb), ref.combine(expert_out), rtol, "combine")
+
+
+def test_top_items_per_expert_capacity_factor_and_errors(moe):
+  gates = torch.softmax(torch.randn((2, 64, 8), device=dev()), -1)
+  d, _ = moe.get_top_items_per_expert_dispatcher(gates, name="einsum", capacity_factor=1.0)
+  assert tuple(d.combine_weights.shape) == (2, 64, 8, 8)   # ceil(64 / 8) is a multiple of 4
+  with pytest.raises(ValueError, match="exceeds the group size"):
+    moe.get_top_items_per_expert_dispatcher(gates, name="einsum", capacity=65)
+
+
+@pytest.mark.parametrize("dtype", [O.F32, O.BF16])
+def test_dense_einsum_dispatcher(moe, dtype):
+  """vmoe/moe.py:93-124 against the einsum statement of the same class."""
+  rng = np.random.default_rng(7)
+  G, S, E, D = 2, 20, 4, 32
+  cw = O.cast(O.softmax(rng.standard_normal((G, S, E)).astype(np.float32)), dtype)
+  data = O.cast(rng.standard_normal((G, S, D)).astype(np.float32), dtype)
+  d = moe.DenseEinsumDispatcher(combine_weights=to_dev(cw, dtype))
+  ref = O.DenseEinsumDispatcher(cw)
+  out = d.dispatch(to_dev(data, dtype))
+  want = ref.dispatch(data)
+  assert tuple(out.shape) == want.shape == (E, G * S, D)
+  np.testing.assert_array_equal(to_np(out), want)
+  expert_out = O.cast(rng.standard_normal((E, G * S, D)).astype(np.float32), dtype)
+  got = d.combine(to_dev(expert_out, dtype))
+  assert_close(to_np(got), ref.combine(expert_out), 8e-3 if dtype == O.BF16 else 1e-5, "combine")
+
+
+@pytest.mark.parametrize("dtype", [O.F32, O.BF16])
+def test_top_items_per_expert_router(dtype):
+  """vmoe/nn/routing_test.py:117-137 (shapes) plus the selection against the oracle."""
+  from vmoe_amd.nn import routing
+  rng = np.random.default_rng(11)
+  G, S, D, E, C = 4, 16, 32, 8, 4
+  x = O.cast(rng.standard_normal((G, S, D)).astype(np.float32), dtype)
+  kernel = O.cast(rng.standard_normal((D, E)).astype(np.float32) / np.sqrt(D), dtype)
+  layer = routing.NoisyTopItemsPerExpertRouter(
+      num_experts=E, noise_std=0.0, dispatcher=dict(name="einsum", capacity=C))
+  variables = {"params": {"dense": {"kernel": to_dev(kernel, dtype)}}}
+  dispatcher, metrics = layer.apply(variables, to_dev(x, dtype))
+  assert metrics["auxiliary_loss"] == 0.
+  assert tuple(dispatcher.combine_weights.shape) == (G, S, E, C)
+  gates = O.router_gates(x, kernel, dtype)
+  for g in range(G):
+    cw_g, dw_g, _ = O.top_items_per_expert_einsum(gates[g], C)
+    got_cw = to_np(dispatcher.combine_weights[g])
+    got_dw = to_np(dispatcher.dispatch_weights[g]).astype(bool)
+    # Gates of the two sides may differ in the last place, which can swap two
+    # items whose gates are nearly equal: compare what was selected by value.
+    assert_close(got_cw.sum(axis=(0, 2)), cw_g.sum(axis=(0, 2)), 8e-3 if dtype == O.BF16 else 1e-5,
+                 "selected gate mass per expert")
+    assert got_dw.sum() == dw_g.sum() == E * C
+  noisy = routing.NoisyTopItemsPerExpertRouter(num_experts=E, noise_std=1.0,
+                                               dispatcher=dict(name="einsum", capacity=C))
+  with pytest.raises(NotImplementedError):
+    noisy.apply(variables, to_dev(x, dtype))
+
+
 # ------------------------------------------------------------------ SparseMoeSpmdLayerTest
 class DummyExpert:
   """Expert with a single scalar parameter that is added to the input (moe_test.py:331-337)."""

@@ -21,7 +21,7 @@ W_F32, W_BF16, W_BOOL = 0, 1, 2
 
 EXPORTS = [
     "vmoe_abi_version", "vmoe_error_string", "vmoe_gate_topk", "vmoe_topk", "vmoe_router_metrics",
-    "vmoe_route_assign", "vmoe_indices_to_slots", "vmoe_dispatch", "vmoe_combine", "vmoe_densify",
+    "vmoe_route_assign", "vmoe_top_items_per_expert", "vmoe_indices_to_slots", "vmoe_dispatch", "vmoe_combine", "vmoe_densify",
     "vmoe_expert_mlp_workspace_bytes", "vmoe_expert_mlp", "vmoe_pack_expert_weights",
     "vmoe_soft_route_workspace_bytes", "vmoe_soft_route", "vmoe_einsum_dispatch",
     "vmoe_einsum_combine", "vmoe_cast", "vmoe_copy_bytes", "vmoe_mfma_probe",
@@ -105,6 +105,12 @@ class RouteAssignParams(ctypes.Structure):
               ("token_slot", c_void_p), ("slot_token", c_void_p), ("fill", c_void_p),
               ("G", c_int32), ("S", c_int32), ("E", c_int32), ("K", c_int32), ("C", c_int32),
               ("batch_priority", c_int32)]
+
+
+class TopItemsParams(ctypes.Structure):
+  _fields_ = [("gates", c_void_p), ("indices", c_void_p), ("token_slot", c_void_p),
+              ("slot_token", c_void_p), ("weights", c_void_p), ("sel_minmax", c_void_p),
+              ("G", c_int32), ("S", c_int32), ("E", c_int32), ("C", c_int32), ("dtype", c_int32)]
 
 
 class IndicesToSlotsParams(ctypes.Structure):

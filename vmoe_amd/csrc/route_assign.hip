@@ -130,6 +130,62 @@ __global__ __launch_bounds__(kRouteThreads) void route_assign_kernel(
     for (int e = tid; e < E; e += kRouteThreads) fill[(size_t)g * E + e] = total[e] < C ? total[e] : C;
 }
 
+// Experts-choice routing (vmoe/moe.py:655-694): every expert takes the C items
+// with its largest gates (jax.lax.top_k over the transposed gates: descending,
+// equal gates -> lower item index first).  One workgroup per (expert, group)
+// sorts the S keys (descending-gate order bits << 32 | item) of that column in
+// LDS; the rank of an item is its position, kept when rank < C.  The outputs are
+// those of the slot-assignment kernel with one "choice" per expert (K = E), so
+// the same dispatch / combine kernels serve both routing schemes.
+template <typename T>
+__global__ __launch_bounds__(kRouteThreads) void top_items_kernel(
+    const T* __restrict__ gates, int32_t* __restrict__ indices, int32_t* __restrict__ token_slot,
+    int32_t* __restrict__ slot_token, float* __restrict__ weights, float* __restrict__ sel_minmax,
+    int G, int S, int E, int C, int SP) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  uint64_t* keys = reinterpret_cast<uint64_t*>(smem);
+  const int tid = threadIdx.x;
+  const int e = blockIdx.x, g = blockIdx.y;
+  const T* col = gates + (size_t)g * S * E + e;
+  for (int s = tid; s < SP; s += kRouteThreads) {
+    uint64_t key = ~0ull;
+    if (s < S) key = ((uint64_t)(~orderable(Elt<T>::load(col + (size_t)s * E))) << 32) | (uint32_t)s;
+    keys[s] = key;
+  }
+  __syncthreads();
+  for (int size = 2; size <= SP; size <<= 1) {
+    for (int stride = size >> 1; stride > 0; stride >>= 1) {
+      for (int t = tid; t < (SP >> 1); t += kRouteThreads) {
+        int lo = 2 * t - (t & (stride - 1));
+        int hi = lo + stride;
+        bool up = (lo & size) == 0;
+        uint64_t a = keys[lo], b = keys[hi];
+        if ((a > b) == up) { keys[lo] = b; keys[hi] = a; }
+      }
+      __syncthreads();
+    }
+  }
+  for (int r = tid; r < S; r += kRouteThreads) {
+    const int s = (int)(uint32_t)keys[r];
+    const size_t o = ((size_t)g * S + s) * E + e;
+    int slot = -1;
+    if (r < C) {
+      slot = slot_row(e, g, r, G, E, C);
+      slot_token[slot] = g * S + s;
+    }
+    indices[2 * o] = e;
+    indices[2 * o + 1] = r;
+    token_slot[o] = slot;
+    weights[o] = Elt<T>::load(col + (size_t)s * E);
+  }
+  for (int c = S + tid; c < C; c += kRouteThreads) slot_token[slot_row(e, g, c, G, E, C)] = -1;
+  if (tid == 0 && sel_minmax != nullptr) {
+    const int last = (C < S ? C : S) - 1;
+    sel_minmax[((size_t)g * E + e) * 2] = Elt<T>::load(col + (size_t)(uint32_t)keys[last] * E);
+    sel_minmax[((size_t)g * E + e) * 2 + 1] = Elt<T>::load(col + (size_t)(uint32_t)keys[0] * E);
+  }
+}
+
 __global__ __launch_bounds__(256) void fill_i32_kernel(int32_t* p, size_t n, int32_t v) {
   size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (i < n) p[i] = v;
@@ -227,5 +283,38 @@ extern "C" int vmoe_densify(const VmoeDensifyParams* p, vmoe_stream_t stream) {
   hipLaunchKernelGGL(densify_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0,
                      as_stream(stream), p->indices, p->weights, p->combine, p->dispatch, p->G,
                      p->S, p->E, p->K, p->C);
+  return launch_status();
+}
+
+extern "C" int vmoe_top_items_per_expert(const VmoeTopItemsParams* p, vmoe_stream_t stream) {
+  if (p == nullptr || p->gates == nullptr || p->indices == nullptr || p->token_slot == nullptr ||
+      p->slot_token == nullptr || p->weights == nullptr)
+    return VMOE_E_NULL;
+  if (p->G < 1 || p->S < 1 || p->E < 1 || p->C < 1) return VMOE_E_SHAPE;
+  if (p->dtype != VMOE_F32 && p->dtype != VMOE_BF16) return VMOE_E_DTYPE;
+  if (p->G > 65535) return VMOE_E_UNSUPPORTED;
+  if ((int64_t)p->E * p->G * p->C >= INT32_MAX || (int64_t)p->G * p->S * p->E >= INT32_MAX)
+    return VMOE_E_OVERFLOW;
+  const int SP = pow2ceil(p->S < 2 ? 2 : p->S);
+  const size_t lds = (size_t)SP * 8;
+  if (lds > 160 * 1024) return VMOE_E_UNSUPPORTED;
+  dim3 grid(p->E, p->G);
+  if (p->dtype == VMOE_BF16) {
+    auto kern = top_items_kernel<bf16_t>;
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return (int)e;
+    hipLaunchKernelGGL(kern, grid, dim3(kRouteThreads), lds, as_stream(stream),
+                       (const bf16_t*)p->gates, p->indices, p->token_slot, p->slot_token, p->weights,
+                       p->sel_minmax, p->G, p->S, p->E, p->C, SP);
+  } else {
+    auto kern = top_items_kernel<float>;
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return (int)e;
+    hipLaunchKernelGGL(kern, grid, dim3(kRouteThreads), lds, as_stream(stream),
+                       (const float*)p->gates, p->indices, p->token_slot, p->slot_token, p->weights,
+                       p->sel_minmax, p->G, p->S, p->E, p->C, SP);
+  }
   return launch_status();
 }

@@ -83,6 +83,23 @@ def route_assign(topk_val: Optional[torch.Tensor], topk_idx: torch.Tensor, num_e
   return indices, token_slot, slot_token, fill
 
 
+def top_items_per_expert(gates: torch.Tensor, capacity: int):
+  """gates (G,S,E) -> indices (G,S,E,2), token_slot (G,S,E), slot_token (E*G*C,),
+  weights (G,S,E) float32, sel_minmax (G,E,2) float32."""
+  G, S, E = gates.shape
+  dev = gates.device
+  gates = gates.contiguous()
+  indices = _i32(G, S, E, 2, device=dev)
+  token_slot = _i32(G, S, E, device=dev)
+  slot_token = _i32(E * G * capacity, device=dev)
+  weights = torch.empty((G, S, E), dtype=torch.float32, device=dev)
+  sel = torch.empty((G, E, 2), dtype=torch.float32, device=dev)
+  p = H.TopItemsParams(H.ptr(gates), H.ptr(indices), H.ptr(token_slot), H.ptr(slot_token),
+                       H.ptr(weights), H.ptr(sel), G, S, E, capacity, H.dtype_code(gates.dtype))
+  H.call("vmoe_top_items_per_expert", p)
+  return indices, token_slot, slot_token, weights, sel
+
+
 def indices_to_slots(indices: torch.Tensor, num_experts: int, capacity: int):
   """indices (G,S,K,2) -> token_slot (G,S,K), slot_token (E*G*C,), counters (2,) [dups, invalid]."""
   G, S, K, _ = indices.shape

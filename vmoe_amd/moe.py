@@ -143,6 +143,39 @@ class EinsumDispatcher(BaseDispatcher):
     return _from_rows(out.view(G * S, -1), (G, S), item_shape, width)
 
 
+class DenseEinsumDispatcher(BaseDispatcher):
+  """Dispatcher sending every item to every expert (C = S); vmoe/moe.py:93-124.
+
+  Attributes:
+    combine_weights: (G, S, E).
+  """
+
+  def __init__(self, combine_weights: Array, partition_spec=None, einsum_precision=None):
+    self.combine_weights = combine_weights
+    self.partition_spec = partition_spec
+    self.einsum_precision = einsum_precision
+
+  def dispatch(self, data: Array) -> Array:
+    # every expert receives a copy of every item: (E, G*S, ...) in the buffer row order
+    G, S, E = self.combine_weights.shape
+    dev = data.device
+    slot = torch.arange(S, dtype=torch.int32, device=dev)
+    indices = torch.stack(torch.meshgrid(torch.arange(E, dtype=torch.int32, device=dev), slot,
+                                         indexing="ij"), dim=-1)      # (E, S, 2): (e, s)
+    indices = indices.permute(1, 0, 2)[None].expand(G, S, E, 2).contiguous()
+    ones = torch.ones((G, S, E), dtype=torch.float32, device=dev)
+    return ExpertIndicesDispatcher(indices, ones, E, S).dispatch(data)
+
+  def combine(self, data: Array) -> Array:
+    G, S, E = self.combine_weights.shape
+    dev = data.device
+    slot = torch.arange(S, dtype=torch.int32, device=dev)
+    indices = torch.stack(torch.meshgrid(torch.arange(E, dtype=torch.int32, device=dev), slot,
+                                         indexing="ij"), dim=-1).permute(1, 0, 2)
+    indices = indices[None].expand(G, S, E, 2).contiguous()
+    return ExpertIndicesDispatcher(indices, self.combine_weights, E, S).combine(data)
+
+
 class _SparseEinsumDispatcher(EinsumDispatcher):
   """EinsumDispatcher produced by top-experts-per-item routing.
 
@@ -332,8 +365,9 @@ def get_top_items_per_expert_dispatcher(gates: Array, name: str, capacity: Optio
                                         **dispatcher_kwargs):
   """Top-Items-Per-Expert ("experts choice") routing; vmoe/moe.py:330-385.
 
-  Argument validation and capacity computation follow the reference; the
-  routing itself is not part of the inference path built here.
+  gates is (S, E) as in the reference, or (G, S, E) for all groups at once (what
+  the reference obtains with jax.vmap, vmoe/nn/routing.py:236-241; the metrics
+  then have a leading group axis, as under vmap).  Returns (dispatcher, metrics).
   """
   if (capacity is None) == (capacity_factor is None):
     raise ValueError(
@@ -345,9 +379,48 @@ def get_top_items_per_expert_dispatcher(gates: Array, name: str, capacity: Optio
     capacity = compute_capacity(
         num_tokens=group_size, num_experts=num_experts, capacity_factor=capacity_factor,
         ceil_or_round=capacity_ceil_or_round, multiple_of=capacity_multiple_of)
-  if name != "einsum":
+  fn_map = {"einsum": _get_top_items_per_expert_einsum_dispatcher}
+  if name not in fn_map:
     raise ValueError(f"Unknown dispatcher type: {name!r}")
-  raise NotImplementedError("Top-items-per-expert routing has no HIP kernel yet.")
+  return fn_map[name](gates, capacity, **dispatcher_kwargs)
+
+
+def _get_top_items_per_expert_einsum_dispatcher(gates: Array, capacity: int, **dispatcher_kwargs):
+  """vmoe/moe.py:655-694: every expert takes the `capacity` items with its largest gates.
+
+  The dispatcher is an EinsumDispatcher whose (G, S, E, C) one-hot weights are
+  only materialised when read; dispatch and combine move rows through the
+  item <-> slot maps (every slot has exactly one contributor), which gives the
+  results of the reference's einsums.
+  """
+  if gates.ndim not in (2, 3):
+    raise ValueError(f"gates must be (S, E) or (G, S, E), got {tuple(gates.shape)}")
+  batched = gates.ndim == 3
+  g3 = gates if batched else gates[None]
+  G, S, E = g3.shape
+  if capacity > S:   # jax.lax.top_k(operand, k) requires k <= the operand's last dimension
+    raise ValueError(f"capacity = {capacity} exceeds the group size {S}")
+  indices, token_slot, slot_token, weights, sel = K.top_items_per_expert(g3, capacity)
+  inner = ExpertIndicesDispatcher(
+      indices=indices, combine_weights=weights, num_experts=E, capacity=capacity,
+      _slots=(token_slot, slot_token))
+  inner._weights_f32 = weights
+  dispatcher = _SparseEinsumDispatcher(inner, gates.dtype, **dispatcher_kwargs)
+  # Metrics useful for monitoring training (moe.py:681-692).
+  per_item = (token_slot >= 0).sum(dim=2, dtype=torch.int32)            # (G, S)
+  metrics = {
+      "num_experts_per_item_min": per_item.amin(dim=1),
+      "num_experts_per_item_max": per_item.amax(dim=1),
+      "min_selected_gate": sel[:, :, 0].amin(dim=1).to(gates.dtype),
+      "max_selected_gate": sel[:, :, 1].amax(dim=1).to(gates.dtype),
+  }
+  log2_num_experts = int(math.log2(E))
+  for t in [2**i for i in range(log2_num_experts + 1)] + [E]:
+    metrics[f"ratio_processed_items_by_at_least_{t}_experts"] = (
+        (per_item >= t).sum(dim=1).to(torch.float32) / S)
+  if not batched:
+    return _SingleGroupView(dispatcher), {k: v[0] for k, v in metrics.items()}
+  return dispatcher, metrics
 
 
 def sparse_moe_spmd(target, variable_axes: Optional[Mapping[str, Any]] = None,

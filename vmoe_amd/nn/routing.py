@@ -97,10 +97,46 @@ class NoisyTopExpertsPerItemRouter(module.Module):
 
 
 class NoisyTopItemsPerExpertRouter(module.Module):
-  """Experts-choice router, vmoe/nn/routing.py:186-244.  Not part of the
-  inference path built here: constructing it works, calling it raises."""
+  """Experts-choice router: every expert picks its top-C items; vmoe/nn/routing.py:186-244.
+
+  Parameters: ``{'dense': {'kernel': (D, E)}}``.  Only the inference branch
+  (``deterministic=True`` or ``noise_std == 0``) is implemented.
+  """
   _fields = dict(num_experts=module._REQUIRED, noise_std=1.0, dispatcher=None,
                  deterministic=False, dtype=None)
 
-  def apply(self, variables, inputs):
-    raise NotImplementedError("Top-items-per-expert routing has no HIP kernel yet.")
+  def init(self, rng, inputs: Array):
+    gen = module.generator(rng)
+    D = inputs.shape[-1]
+    kernel = module.lecun_normal(gen, (D, self.num_experts), fan_in=D, device=inputs.device)
+    return {"params": {"dense": {"kernel": kernel}}}
+
+  def apply(self, variables, inputs: Array) -> Tuple[BaseDispatcher, Metrics]:
+    kernel = variables["params"]["dense"]["kernel"]
+    gates_softmax = self._compute_gates_softmax(inputs, kernel)
+    dispatcher, metrics = self._create_dispatcher_and_metrics(gates_softmax)
+    metrics["auxiliary_loss"] = 0.
+    return dispatcher, metrics
+
+  def _compute_gates_softmax(self, inputs: Array, kernel: Array) -> Array:
+    if inputs.ndim != 3:
+      raise ValueError(f"inputs.ndim must be 3, but it is {inputs.ndim}")
+    if kernel.shape != (inputs.shape[-1], self.num_experts):
+      raise ValueError(f"Router kernel has shape {tuple(kernel.shape)}, expected "
+                       f"{(inputs.shape[-1], self.num_experts)}")
+    if not (self.deterministic or self.noise_std == 0.0):
+      raise NotImplementedError(
+          "The noisy (training-time) branch of the router is not implemented; "
+          "use deterministic=True or noise_std=0.")
+    dtype = self.dtype or inputs.dtype
+    gates, _, _ = K.gate_topk(K.cast(inputs, dtype), K.cast(kernel, dtype), 1)
+    return gates
+
+  def _create_dispatcher_and_metrics(self, gates_dispatch: Array):
+    dispatcher_kwargs = dict(**(self.dispatcher or {}))
+    use_bfloat16 = dispatcher_kwargs.pop("bfloat16", False)
+    dispatcher, metrics = vmoe_amd.moe.get_top_items_per_expert_dispatcher(
+        gates_dispatch, **dispatcher_kwargs)
+    if use_bfloat16:
+      dispatcher = vmoe_amd.moe.Bfloat16Dispatcher(dispatcher)
+    return dispatcher, metrics
