@@ -498,7 +498,8 @@ def sparse_moe(dispatcher, expert_fn, x):
 
 def mlp_moe_block(inputs, params, *, group_size, num_selected_experts,
                   dispatcher_kwargs, dtype=F32, logit_bias=None,
-                  approximate_gelu=True):
+                  approximate_gelu=True, gshard_loss_weight=0.0,
+                  importance_loss_weight=1.0):
   """vmoe/nn/vit_moe.py:101-124 with NoisyTopExpertsPerItemRouter (deterministic).
 
   params = {"Router": {"dense": {"kernel"}}, "Mlp": {"Dense_0": {"kernel","bias"},
@@ -510,7 +511,8 @@ def mlp_moe_block(inputs, params, *, group_size, num_selected_experts,
   x = cast(inputs, dtype).reshape(-1, group_size, shape[-1])             # :107
   dispatcher, metrics, _ = noisy_top_experts_per_item_router(
       x, params["Router"]["dense"]["kernel"], num_selected_experts,
-      dispatcher_kwargs, dtype, logit_bias=logit_bias)
+      dispatcher_kwargs, dtype, gshard_loss_weight=gshard_loss_weight,
+      importance_loss_weight=importance_loss_weight, logit_bias=logit_bias)
   mlp = params["Mlp"]
   fn = lambda buf: mlp_block(buf, mlp["Dense_0"]["kernel"], mlp["Dense_0"]["bias"],
                              mlp["Dense_1"]["kernel"], mlp["Dense_1"]["bias"], dtype,

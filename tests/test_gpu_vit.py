@@ -1,0 +1,225 @@
+"""The vision transformer around the MoE layer (vmoe_amd.nn.vit_moe) against its
+CPU restatement (oracle/vit_oracle.py) and the reference's own tests for it
+(vmoe/nn/vit_moe_test.py)."""
+import copy
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import moe_oracle as O
+from oracle import vit_oracle as V
+from tests.test_vit_oracle import DEFAULT_TEST_CONFIG, _SINCOS_ROWS, _shapes
+from tests.util import assert_close, dev, to_np
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def vit_moe():
+  from vmoe_amd.nn import vit_moe
+  return vit_moe
+
+
+def tree_to_dev(tree):
+  if isinstance(tree, dict):
+    return {k: tree_to_dev(v) for k, v in tree.items()}
+  return torch.from_numpy(np.ascontiguousarray(tree, dtype=np.float32)).to(dev())
+
+
+def product_config(config, dtype):
+  """The oracle's config with torch dtypes and deterministic=True."""
+  config = copy.deepcopy(config)
+  config["deterministic"] = True
+  config["encoder"]["dtype"] = None if dtype == O.F32 else torch.bfloat16
+  return config
+
+
+def oracle_config(config, dtype):
+  config = copy.deepcopy(config)
+  config["encoder"]["dtype"] = None if dtype == O.F32 else O.BF16
+  return config
+
+
+# ------------------------------------------------------------------ EncoderMoeTest
+def test_position_embedding_learned(vit_moe):
+  """vmoe/nn/vit_moe_test.py:78-91."""
+  encoder = vit_moe.EncoderMoe(num_layers=0, mlp_dim=4, num_heads=1)
+  x = torch.zeros((2, 4, 8), device=dev())
+  pos = torch.arange(32, dtype=torch.float32, device=dev()).reshape(1, 4, 8)
+  y, _ = encoder.apply({"params": {
+      "posembed_input": {"pos_embedding": pos},
+      "encoder_norm": {"bias": torch.zeros(8, device=dev()), "scale": torch.ones(8, device=dev())},
+  }}, x)
+  p = to_np(torch.cat([pos, pos])).astype(np.float64)
+  want = (p - p.mean(-1, keepdims=True)) / np.sqrt(p.var(-1, keepdims=True) + 1e-6)
+  np.testing.assert_allclose(to_np(y), want, rtol=1e-5, atol=1e-5)
+
+
+@pytest.mark.parametrize("seq_len,rows", [(4, _SINCOS_ROWS), (5, [[0] * 8] + _SINCOS_ROWS)])
+def test_position_embedding_sincos2d(vit_moe, seq_len, rows):
+  """vmoe/nn/vit_moe_test.py:93-127."""
+  encoder = vit_moe.EncoderMoe(num_layers=0, mlp_dim=4, num_heads=1,
+                               position_emb={"name": "sincos2d", "h": 2, "w": 2, "temperature": 1.})
+  x = torch.zeros((2, seq_len, 8), device=dev())
+  y, _ = encoder.apply({"params": {"encoder_norm": {
+      "bias": torch.zeros(8, device=dev()), "scale": torch.ones(8, device=dev())}}}, x)
+  pos = np.asarray([rows], np.float64)
+  want = (pos - pos.mean(-1, keepdims=True)) / np.sqrt(pos.var(-1, keepdims=True) + 1e-6)
+  np.testing.assert_allclose(to_np(y), np.concatenate([want, want]), rtol=1e-3, atol=1e-3)
+
+
+def test_position_embedding_sincos2d_raises(vit_moe):
+  """vmoe/nn/vit_moe_test.py:129-135."""
+  encoder = vit_moe.EncoderMoe(num_layers=0, mlp_dim=4, num_heads=1,
+                               position_emb={"name": "sincos2d", "h": 2, "w": 2, "temperature": 1.})
+  with pytest.raises(ValueError, match="Unsupported sequence length"):
+    encoder.init(0, torch.zeros((2, 6, 8), device=dev()))
+
+
+# ------------------------------------------------------------------ VitMoeTest
+@pytest.mark.parametrize("position_emb", [{}, {"name": "sincos2d"}])
+def test_initialize_shapes(vit_moe, position_emb):
+  """vmoe/nn/vit_moe_test.py:142-187: same tree as the oracle's (which that test pins)."""
+  config = product_config(DEFAULT_TEST_CONFIG, O.F32)
+  config["encoder"]["position_emb"] = position_emb
+  model = vit_moe.VisionTransformerMoe(**config)
+  variables = model.init(0, torch.randn((16, 4, 4, 3), device=dev()))
+  ocfg = copy.deepcopy(DEFAULT_TEST_CONFIG)
+  ocfg["encoder"]["position_emb"] = position_emb
+  want = _shapes(V.init_params(np.random.default_rng(0), (16, 4, 4, 3), **ocfg))
+  assert _shapes(variables["params"]) == want
+
+
+def test_forward(vit_moe):
+  """vmoe/nn/vit_moe_test.py:189-199."""
+  model = vit_moe.VisionTransformerMoe(**product_config(DEFAULT_TEST_CONFIG, O.F32))
+  x = torch.randn((16, 4, 4, 3), device=dev())
+  variables = model.init(0, x)
+  output = model.apply(variables, x)
+  assert isinstance(output, tuple)
+  output, metrics = output
+  assert "auxiliary_loss" in metrics
+  assert tuple(output.shape) == (16, 4)
+
+
+def test_training_mode_raises(vit_moe):
+  config = product_config(DEFAULT_TEST_CONFIG, O.F32)
+  config["deterministic"] = False
+  config["encoder"]["moe"]["router"]["noise_std"] = 1e-3
+  model = vit_moe.VisionTransformerMoe(**config)
+  x = torch.randn((16, 4, 4, 3), device=dev())
+  with pytest.raises(NotImplementedError):
+    model.apply(model.init(0, x), x)
+
+
+# ------------------------------------------------------------------ parity with the CPU restatement
+@pytest.mark.parametrize("dtype", [O.F32, O.BF16])
+@pytest.mark.parametrize("cross,qk_norm", [(False, False), (True, False), (False, True)])
+def test_attention_vs_oracle(vit_moe, dtype, cross, qk_norm):
+  from tests.test_vit_oracle import _attention_params
+  rng = np.random.default_rng(3)
+  B, Sq, Sk, D, H = 4, 1 if cross else 50, 50, 128, 4
+  p = _attention_params(rng, D, H, qk_norm=qk_norm)
+  xq = O.cast(rng.standard_normal((B, Sq, D)).astype(np.float32), dtype)
+  xkv = O.cast(rng.standard_normal((B, Sk, D)).astype(np.float32), dtype) if cross else xq
+  odt = None if dtype == O.F32 else O.BF16
+  tdt = None if dtype == O.F32 else torch.bfloat16
+  want = V.multi_head_attention(xq, xkv, p, H, odt, qk_norm)
+  layer = vit_moe.MultiHeadDotProductAttention(num_heads=H, dtype=tdt, normalize_qk=qk_norm)
+  tq = tree_to_dev(xq)
+  got = layer.apply({"params": tree_to_dev(p)}, tq, tree_to_dev(xkv) if cross else None)
+  assert got.dtype == (torch.float32 if dtype == O.F32 else torch.bfloat16)
+  if dtype == O.F32:
+    assert_close(to_np(got), want, 1e-4, "attention")
+    return
+  # bfloat16: flax holds logits and probabilities in bfloat16, the fused library
+  # attention keeps them in float32 until the second product, so single elements
+  # differ by a few bfloat16 steps of the output sum.  Bound that, and require the
+  # GPU result to be at least as close to the float32 answer as the restatement is.
+  assert_close(to_np(got), want, 5e-2, "attention")
+  exact = V.multi_head_attention(xq, xkv, p, H, None, qk_norm)
+  rms = lambda a: float(np.sqrt(np.mean(np.square(a, dtype=np.float64))))
+  assert rms(to_np(got) - exact) <= 1.1 * rms(want - exact)
+
+
+SMALL = {
+    "num_classes": 10,
+    "patch_size": (4, 4),
+    "hidden_size": 64,
+    "encoder": {
+        "num_layers": 3,
+        "mlp_dim": 128,
+        "num_heads": 4,
+        "moe": {
+            "layers": (1,),
+            "num_experts": 4,
+            "group_size": 32,
+            "router": {"num_selected_experts": 2,
+                       "dispatcher": {"name": "indices", "capacity_factor": 1.5,
+                                      "batch_priority": True}},
+        },
+    },
+    "classifier": "gap",
+    "representation_size": None,
+}
+
+
+def _variant(**changes):
+  cfg = copy.deepcopy(SMALL)
+  for k, v in changes.items():
+    if k in cfg:
+      cfg[k] = v
+    else:
+      cfg["encoder"][k] = v
+  return cfg
+
+
+VARIANTS = {
+    "gap": _variant(),
+    "token": _variant(classifier="token", moe=dict(SMALL["encoder"]["moe"], group_size=34)),
+    "map_qknorm": _variant(classifier="map", attention_qk_norm=True, representation_size=48),
+    "sincos2d_einsum": _variant(
+        position_emb={"name": "sincos2d"},
+        moe=dict(SMALL["encoder"]["moe"], router={
+            "num_selected_experts": 1,
+            "dispatcher": {"name": "einsum", "capacity": 12, "batch_priority": False}})),
+    "all_moe": _variant(moe=dict(SMALL["encoder"]["moe"], layers=(0, 1, 2))),
+}
+
+
+@pytest.mark.parametrize("name", sorted(VARIANTS))
+def test_model_fp32_vs_oracle(vit_moe, name):
+  cfg = VARIANTS[name]
+  rng = np.random.default_rng(11)
+  images = rng.uniform(-1, 1, (8, 16, 16, 3)).astype(np.float32)     # 16 patches per image
+  params = V.init_params(rng, images.shape, **cfg)
+  want, want_metrics = V.vision_transformer_moe(images, params, **oracle_config(cfg, O.F32))
+  model = vit_moe.VisionTransformerMoe(**product_config(cfg, O.F32))
+  got, metrics = model.apply({"params": tree_to_dev(params)}, tree_to_dev(images))
+  assert got.dtype == torch.float32 and tuple(got.shape) == want.shape
+  assert_close(to_np(got), want, 2e-4, f"{name} logits")
+  assert set(metrics) == set(want_metrics)
+  np.testing.assert_allclose(to_np(metrics["auxiliary_loss"]),
+                             np.asarray(want_metrics["auxiliary_loss"]), rtol=1e-3, atol=1e-6)
+
+
+def test_model_bf16_vs_oracle(vit_moe):
+  """bfloat16 encoder (the residual stream stays float32, as under jnp promotion).
+  Rounding differs inside attention, and an item whose two best gates are nearly
+  equal can be routed differently: compared at the 2e-2 of bfloat16 parity on the
+  scale of the logits, for all but a few images."""
+  cfg = VARIANTS["gap"]
+  rng = np.random.default_rng(12)
+  images = rng.uniform(-1, 1, (16, 16, 16, 3)).astype(np.float32)
+  params = V.init_params(rng, images.shape, **cfg)
+  want, _ = V.vision_transformer_moe(images, params, **oracle_config(cfg, O.BF16))
+  model = vit_moe.VisionTransformerMoe(**product_config(cfg, O.BF16))
+  got, metrics = model.apply({"params": tree_to_dev(params)}, tree_to_dev(images))
+  assert got.dtype == torch.float32
+  err = np.abs(to_np(got) - want)
+  scale = float(np.sqrt(np.mean(want ** 2)))
+  bad_images = (err.max(axis=1) > 2e-2 * (scale + np.abs(want).max(axis=1))).sum()
+  assert bad_images <= 1, f"{bad_images} of {len(want)} images outside 2e-2 (scale {scale:.3f})"
+  assert np.isfinite(to_np(metrics["auxiliary_loss"])).all()
