@@ -155,6 +155,125 @@ def soft_main(args):
   print(json.dumps(result))
 
 
+def vit_main(args):
+  """Full V-MoE B/16 forward at 224 px, batch 512: images/s, time per module kind
+  broken out with events around the modules' apply methods."""
+  import copy
+  import torch
+  from vmoe_amd import _hip, configs
+  from vmoe_amd.nn import vit_moe
+
+  dev = torch.device("cuda:0")
+  torch.cuda.set_device(dev)
+  B = configs.VIT_B16_MOE_BATCH
+  model_cfg = configs.vit_b16_moe_model(dtype=torch.bfloat16)
+  model = vit_moe.VisionTransformerMoe(**model_cfg)
+  gen = torch.Generator(device=dev)
+  gen.manual_seed(0)
+  images = [torch.rand((B, 224, 224, 3), generator=gen, device=dev) * 2 - 1 for _ in range(2)]
+  variables = model.init(0, images[0])
+
+  spans = {}
+
+  def timed(cls, method, label):
+    fn = getattr(cls, method)
+
+    def wrapper(self, *a, **kw):
+      e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+      e0.record()
+      out = fn(self, *a, **kw)
+      e1.record()
+      if spans.get("on"):
+        spans.setdefault(label, []).append((e0, e1))
+      return out
+    setattr(cls, method, wrapper)
+
+  timed(vit_moe.MlpMoeBlock, "apply", "moe_layers")
+  timed(vit_moe.MlpBlock, "apply", "dense_mlps")
+  timed(vit_moe.MultiHeadDotProductAttention, "apply", "attention")
+
+  def step(i):
+    return model.apply(variables, images[i % 2])
+
+  for i in range(args.warmup):
+    step(i)
+  torch.cuda.synchronize()
+  sink = {}
+  _hip.set_timing_sink(sink)
+  spans["on"] = True
+  t0 = time.perf_counter()
+  for i in range(args.steps):
+    logits, metrics = step(i)
+  torch.cuda.synchronize()
+  t1 = time.perf_counter()
+  _hip.set_timing_sink(None)
+  spans.pop("on")
+  ms = (t1 - t0) * 1e3 / args.steps
+  module_ms = {k: float(sum(a.elapsed_time(b) for a, b in v)) / args.steps for k, v in spans.items()}
+  module_ms["other (patch embedding, layer norms, residuals, head)"] = ms - sum(module_ms.values())
+  stage_ms = {name: float(np.mean([a.elapsed_time(b) for a, b in pairs])) * (len(pairs) / args.steps)
+              for name, pairs in sink.items()}
+
+  # Dominant kernel: the bf16 GEMM behind the dense and the expert MLPs
+  # (two launches per MLP).  Flops: dense 2*T*D*M per launch; experts 2*A*D*M.
+  enc = model_cfg["encoder"]
+  D, M = model_cfg["hidden_size"], enc["mlp_dim"]
+  T = B * 196
+  moe_cfg = enc["moe"]
+  n_moe = len(moe_cfg["layers"])
+  n_dense = enc["num_layers"] - n_moe
+  kept = T * moe_cfg["router"]["num_selected_experts"]       # upper bound: nothing dropped
+  flops_mlp = 2 * 2.0 * D * M * (n_dense * T + n_moe * kept)
+  mlp_ms = stage_ms["vmoe_expert_mlp"]
+  achieved = flops_mlp / (mlp_ms * 1e-3) / 1e12
+  # Whole-model matrix flops per image (projections, attention, MLPs), for scale.
+  H, hd, S = enc["num_heads"], D // enc["num_heads"], 196
+  flops_attn = enc["num_layers"] * T * (2.0 * D * 3 * D + 2.0 * D * D + 2 * 2.0 * S * D)
+  flops_total = flops_mlp + flops_attn + 2.0 * T * (16 * 16 * 3) * D
+  result = {
+      "metric": "V-MoE B/16 (E=8, top-2 BPR, every odd block) forward images/sec at 224 px",
+      "value": B / (ms * 1e-3), "unit": "images/s", "n_gpus": 1, "steps": args.steps,
+      "warmup": args.warmup, "ms_per_step": ms, "higher_is_better": True, "scaling": "weak",
+      "vs_baseline": None, "dtype": "bf16",
+      "data": "synthetic (seeded U(-1,1) images, random-init parameters)",
+      "config": {"workload": configs.VIT_B16_MOE_NAME, "batch": B, "image": [224, 224, 3],
+                 "tokens": T, "blocks": enc["num_layers"], "moe_blocks": list(moe_cfg["layers"]),
+                 "experts": moe_cfg["num_experts"], "selected": 2, "group_size": moe_cfg["group_size"],
+                 "capacity_factor": 1.05},
+      "roofline": {"bound": "mfma", "kernel": "gemm_bf16_kernel", "achieved": achieved,
+                   "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": achieved / PEAK_BF16_TFLOPS,
+                   "traffic": None, "launch_ms": mlp_ms / (2 * enc["num_layers"]),
+                   "flops_all_mlps": flops_mlp},
+      "model_TFLOPs_per_step": flops_total / 1e12,
+      "model_TFLOPs_per_s": flops_total / (ms * 1e-3) / 1e12,
+      "moe_ms": module_ms.get("moe_layers"), "module_ms": module_ms, "stage_ms": stage_ms,
+  }
+  if not args.no_cpu_baseline:
+    from oracle import moe_oracle as O
+    from oracle import vit_oracle as V
+    n_img = 8                                  # one routing group
+    ocfg = copy.deepcopy(configs.vit_b16_moe_model(dtype=O.BF16))
+    to_np = lambda t: t.detach().float().cpu().numpy()
+
+    def tree(t):
+      return {k: tree(v) for k, v in t.items()} if isinstance(t, dict) else to_np(t)
+    params_np = tree(variables["params"])
+    imgs_np = to_np(images[0][:n_img])
+    t0 = time.perf_counter()
+    V.vision_transformer_moe(imgs_np, params_np, **ocfg)
+    t = time.perf_counter() - t0
+    result["cpu_baseline"] = {
+        "value": n_img / t, "unit": "images/s", "cores": int(torch.get_num_threads()),
+        "kind": "port",
+        "sample": (f"oracle/vit_oracle.py vision_transformer_moe (bfloat16 rounding modelled) on "
+                   f"{n_img} of {B} images (one routing group), one run of {t:.2f} s; NumPy BLAS + "
+                   "torch CPU threads"),
+        "host_cpus": os.cpu_count()}
+  else:
+    result["cpu_baseline"] = None
+  print(json.dumps(result))
+
+
 def main():
   args = parse_args()
   if args.gpus != 1:
@@ -163,6 +282,8 @@ def main():
     sys.exit(2)
   if args.config == "soft_moe_b16_128x1":
     return soft_main(args)
+  if args.config == "vmoe_b16_model_E8_k2_224":
+    return vit_main(args)
   import torch
   from vmoe_amd import _hip, configs, kernels
   from vmoe_amd.nn import vit_moe

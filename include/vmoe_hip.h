@@ -296,6 +296,51 @@ typedef struct {
 } VmoeCastParams;
 int vmoe_cast(const VmoeCastParams* p, vmoe_stream_t stream);
 
+/* Residual add fused with the layer norm that follows it, the pattern of every
+ * encoder block (vmoe/nn/vit_moe.py:162-179: `x = x + inputs; y = nn.LayerNorm(dtype)(x)`)
+ * with flax.linen.LayerNorm's arithmetic (float32 statistics, var = E[x^2] - E[x]^2):
+ *   x = residual (+ branch);  residual_out = x;
+ *   norm_out = (x - mean) * rsqrt(var + eps) * scale + bias   in out_dtype.
+ * residual (rows, D) float32; branch (rows, D) of branch_dtype or null (no add);
+ * scale, bias (D,) float32 or null; residual_out float32 or null (may be the
+ * residual itself); norm_out or null (add only).  One of the outputs is required. */
+typedef struct {
+  const float* residual;
+  const void* branch;
+  const float* scale;
+  const float* bias;
+  float* residual_out;
+  void* norm_out;
+  size_t rows;
+  int32_t D;
+  float eps;
+  int32_t branch_dtype, out_dtype;
+} VmoeAddLayerNormParams;
+int vmoe_add_layer_norm(const VmoeAddLayerNormParams* p, vmoe_stream_t stream);
+
+/* Multi-head softmax attention without mask or dropout, softmax(q k^T * scale) v per
+ * (image, head): flax.linen.dot_product_attention as MultiHeadDotProductAttention
+ * calls it for vmoe/nn/vit_moe.py:166-174 (float32 logits and statistics; the
+ * probabilities enter the second product as bfloat16).
+ * q (B, Sq, H, head_dim), k, v (B, Sk, H, head_dim) given by a base pointer and
+ * element strides per image and per token (heads are contiguous: head h starts at
+ * element h * head_dim), so the packed output of a fused q/k/v projection can be
+ * passed without copies; out (B, Sq, H * head_dim) contiguous.  Strides are
+ * multiples of 8 elements, pointers 16-byte aligned.
+ * VMOE_E_UNSUPPORTED unless dtype is bfloat16, head_dim is 64 and the keys and
+ * values of one head fit in LDS (Sk up to about 560). */
+typedef struct {
+  const void* q;
+  const void* k;
+  const void* v;
+  void* out;
+  int64_t q_stride_b, q_stride_s, k_stride_b, k_stride_s, v_stride_b, v_stride_s;
+  int32_t B, H, Sq, Sk, head_dim;
+  float scale;
+  int32_t dtype;
+} VmoeAttentionParams;
+int vmoe_attention(const VmoeAttentionParams* p, vmoe_stream_t stream);
+
 /* Plain device copy kernel of n bytes (n % 16 == 0); the measured HBM ceiling
  * that bandwidth figures are compared with. */
 int vmoe_copy_bytes(const void* in, void* out, size_t n, vmoe_stream_t stream);

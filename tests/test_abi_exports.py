@@ -53,7 +53,8 @@ def test_struct_layouts_match_header():
   text = open(HEADER).read()
   text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
   structs = {n: b for b, n in re.findall(r"typedef struct \{(.*?)\}\s*(\w+);", text, flags=re.S)}
-  cmap = {"int32_t": ctypes.c_int32, "float": ctypes.c_float, "size_t": ctypes.c_size_t}
+  cmap = {"int32_t": ctypes.c_int32, "float": ctypes.c_float, "size_t": ctypes.c_size_t,
+          "int64_t": ctypes.c_int64}
   py = {"VmoeGateTopkParams": _hip.GateTopkParams, "VmoeTopkParams": _hip.TopkParams,
         "VmoeRouterMetricsParams": _hip.RouterMetricsParams,
         "VmoeRouteAssignParams": _hip.RouteAssignParams,
@@ -62,7 +63,9 @@ def test_struct_layouts_match_header():
         "VmoeDensifyParams": _hip.DensifyParams, "VmoeExpertMlpParams": _hip.ExpertMlpParams,
         "VmoeTransposeParams": _hip.TransposeParams, "VmoeSoftRouteParams": _hip.SoftRouteParams,
         "VmoeEinsumParams": _hip.EinsumParams, "VmoeCastParams": _hip.CastParams,
-        "VmoeTopItemsParams": _hip.TopItemsParams}
+        "VmoeTopItemsParams": _hip.TopItemsParams,
+        "VmoeAddLayerNormParams": _hip.AddLayerNormParams,
+        "VmoeAttentionParams": _hip.AttentionParams}
   assert set(py) == set(structs)
   for name, body in structs.items():
     want = []

@@ -115,12 +115,78 @@ def test_training_mode_raises(vit_moe):
 
 
 # ------------------------------------------------------------------ parity with the CPU restatement
+@pytest.mark.parametrize("rows,D", [(5, 8), (33, 64), (1000, 768), (7, 1000), (9, 2048), (6, 2052),
+                                    (11, 770), (4099, 256)])
+@pytest.mark.parametrize("branch_dtype", [None, O.F32, O.BF16])
+@pytest.mark.parametrize("out_dtype", [O.F32, O.BF16])
+def test_add_layer_norm_kernel(rows, D, branch_dtype, out_dtype):
+  from vmoe_amd import kernels as K
+  rng = np.random.default_rng(rows * D)
+  resid = (rng.standard_normal((rows, D)) * 2 + 0.5).astype(np.float32)
+  scale = (1 + 0.2 * rng.standard_normal(D)).astype(np.float32)
+  bias = (0.2 * rng.standard_normal(D)).astype(np.float32)
+  branch = None
+  x = resid
+  if branch_dtype is not None:
+    branch = O.cast(rng.standard_normal((rows, D)).astype(np.float32), branch_dtype)
+    x = resid + branch
+  tb = None if branch is None else tree_to_dev(branch).to(
+      torch.bfloat16 if branch_dtype == O.BF16 else torch.float32)
+  got_x, got_y = K.add_layer_norm(tree_to_dev(resid), tb, tree_to_dev(scale), tree_to_dev(bias),
+                                  1e-6, torch.bfloat16 if out_dtype == O.BF16 else torch.float32)
+  np.testing.assert_array_equal(to_np(got_x), x)           # one float32 add: exact
+  exact = V.layer_norm(x, scale, bias, None)
+  if out_dtype == O.F32:
+    np.testing.assert_allclose(to_np(got_y), exact, rtol=2e-5, atol=2e-5)
+  else:   # within one bfloat16 step of the rounded float32 result
+    assert got_y.dtype == torch.bfloat16
+    np.testing.assert_allclose(to_np(got_y), exact, rtol=2 ** -7, atol=1e-5)
+  # add only, and norm only without parameters
+  if branch is not None:
+    only_x, none_y = K.add_layer_norm(tree_to_dev(resid), tb, None, None, 1e-6, None)
+    assert none_y is None
+    np.testing.assert_array_equal(to_np(only_x), x)
+  _, plain = K.add_layer_norm(tree_to_dev(resid), None, None, None, 1e-6, torch.float32)
+  np.testing.assert_allclose(to_np(plain), V.layer_norm(resid, None, None, None), rtol=2e-5,
+                             atol=2e-5)
+
+
+@pytest.mark.parametrize("B,H,Sq,Sk,packed", [
+    (2, 3, 196, 196, True), (2, 2, 197, 197, True), (3, 2, 1, 50, False), (1, 4, 33, 33, True),
+    (2, 2, 300, 300, True), (1, 2, 64, 512, False), (1, 1, 40, 7, False)])
+def test_attention_kernel(B, H, Sq, Sk, packed):
+  """softmax(q k^T / 8) v against float64 on the same bfloat16 operands; operands are
+  slices of a packed (B, S, 3, H, 64) projection output or separate tensors."""
+  from vmoe_amd import kernels as K
+  rng = np.random.default_rng(B * 1000 + Sq + Sk)
+  hd = 64
+  if packed:
+    qkv = torch.from_numpy(rng.standard_normal((B, Sq, 3, H, hd)).astype(np.float32) * 1.5).to(
+        dev()).to(torch.bfloat16)
+    q, k, v = qkv[:, :, 0], qkv[:, :, 1], qkv[:, :, 2]
+  else:
+    mk = lambda S: torch.from_numpy(rng.standard_normal((B, S, H, hd)).astype(np.float32) * 1.5).to(
+        dev()).to(torch.bfloat16)
+    q, k, v = mk(Sq), mk(Sk), mk(Sk)
+  assert K.attention_supported(q, k)
+  got = K.attention(q, k, v, hd ** -0.5)
+  assert tuple(got.shape) == (B, Sq, H * hd) and got.dtype == torch.bfloat16
+  qn, kn, vn = (to_np(t).astype(np.float64) for t in (q, k, v))
+  logits = np.einsum("bqhd,bkhd->bhqk", qn, kn) / 8.0
+  w = np.exp(logits - logits.max(-1, keepdims=True))
+  w /= w.sum(-1, keepdims=True)
+  want = np.einsum("bhqk,bkhd->bqhd", w, vn).reshape(B, Sq, H * hd)
+  assert_close(to_np(got), want, 1e-2, "attention kernel")
+
+
 @pytest.mark.parametrize("dtype", [O.F32, O.BF16])
-@pytest.mark.parametrize("cross,qk_norm", [(False, False), (True, False), (False, True)])
-def test_attention_vs_oracle(vit_moe, dtype, cross, qk_norm):
+@pytest.mark.parametrize("cross,qk_norm,D", [(False, False, 128), (True, False, 128),
+                                             (False, True, 128), (False, False, 256),
+                                             (False, True, 256)])
+def test_attention_vs_oracle(vit_moe, dtype, cross, qk_norm, D):
   from tests.test_vit_oracle import _attention_params
   rng = np.random.default_rng(3)
-  B, Sq, Sk, D, H = 4, 1 if cross else 50, 50, 128, 4
+  B, Sq, Sk, H = 4, 1 if cross else 50, 50, 4
   p = _attention_params(rng, D, H, qk_norm=qk_norm)
   xq = O.cast(rng.standard_normal((B, Sq, D)).astype(np.float32), dtype)
   xkv = O.cast(rng.standard_normal((B, Sk, D)).astype(np.float32), dtype) if cross else xq

@@ -25,6 +25,7 @@ EXPORTS = [
     "vmoe_expert_mlp_workspace_bytes", "vmoe_expert_mlp", "vmoe_pack_expert_weights",
     "vmoe_soft_route_workspace_bytes", "vmoe_soft_route", "vmoe_einsum_dispatch",
     "vmoe_einsum_combine", "vmoe_cast", "vmoe_copy_bytes", "vmoe_mfma_probe",
+    "vmoe_add_layer_norm", "vmoe_attention",
 ]
 
 
@@ -166,6 +167,22 @@ class EinsumParams(ctypes.Structure):
 class CastParams(ctypes.Structure):
   _fields_ = [("in_", c_void_p), ("out", c_void_p), ("n", c_size_t),
               ("in_dtype", c_int32), ("out_dtype", c_int32)]
+
+
+class AddLayerNormParams(ctypes.Structure):
+  _fields_ = [("residual", c_void_p), ("branch", c_void_p), ("scale", c_void_p),
+              ("bias", c_void_p), ("residual_out", c_void_p), ("norm_out", c_void_p),
+              ("rows", c_size_t), ("D", c_int32), ("eps", ctypes.c_float),
+              ("branch_dtype", c_int32), ("out_dtype", c_int32)]
+
+
+class AttentionParams(ctypes.Structure):
+  _fields_ = [("q", c_void_p), ("k", c_void_p), ("v", c_void_p), ("out", c_void_p),
+              ("q_stride_b", ctypes.c_int64), ("q_stride_s", ctypes.c_int64),
+              ("k_stride_b", ctypes.c_int64), ("k_stride_s", ctypes.c_int64),
+              ("v_stride_b", ctypes.c_int64), ("v_stride_s", ctypes.c_int64),
+              ("B", c_int32), ("H", c_int32), ("Sq", c_int32), ("Sk", c_int32),
+              ("head_dim", c_int32), ("scale", ctypes.c_float), ("dtype", c_int32)]
 
 
 _timing_sink = None

@@ -74,6 +74,25 @@ class SoftConfig:
 SOFT_B16 = SoftConfig("soft_moe_b16_128x1", 768, 3072, 128, 1, 256, 196, "bfloat16")
 
 
+def vit_b16_moe_model(dtype=None, num_classes: int = 1000) -> Dict:
+  """Constructor arguments of the full V-MoE B/16 at 224 px: 12 blocks, 12 heads,
+  d = 768, mlp 3072, experts (E = 8, top-2, batch priority routing, capacity factor
+  1.05, groups of 8 images) on every odd block, global-average-pool head."""
+  return dict(
+      num_classes=num_classes, patch_size=(16, 16), hidden_size=768, classifier="gap",
+      representation_size=None, deterministic=True, head_kernel_zero_init=False,
+      encoder=dict(
+          num_layers=12, mlp_dim=3072, num_heads=12, dtype=dtype,
+          moe=dict(layers=(1, 3, 5, 7, 9, 11), num_experts=8, group_size=8 * 196,
+                   router=dict(num_selected_experts=2,
+                               dispatcher=dict(name="indices", batch_priority=True,
+                                               capacity_factor=1.05)))))
+
+
+VIT_B16_MOE_NAME = "vmoe_b16_model_E8_k2_224"
+VIT_B16_MOE_BATCH = 512
+
+
 def make_layer_inputs(cfg: LayerConfig, seed: int = 0, num_images: Optional[int] = None):
   """float32 NumPy arrays: x (N, L, D), router kernel (D, E), optional logit bias
   (E,), expert kernels (E, D, M) / (E, M, D) LeCun-normal, zero biases."""

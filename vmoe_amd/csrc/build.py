@@ -11,7 +11,7 @@ ROOT = os.path.dirname(os.path.dirname(HERE))
 OUT_DIR = os.path.join(os.path.dirname(HERE), "_lib")
 LIB = os.path.join(OUT_DIR, "libvmoe_hip.so")
 SOURCES = ["capi.hip", "gate_topk.hip", "route_assign.hip", "dispatch_combine.hip",
-           "expert_mlp.hip", "soft_moe.hip"]
+           "expert_mlp.hip", "soft_moe.hip", "vit_ops.hip"]
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
          "-Wno-unknown-warning-option", "-Wno-unused-command-line-argument",

@@ -5,6 +5,7 @@ on a ROCm device and are used as raw device pointers on torch's current stream.
 """
 from __future__ import annotations
 
+import ctypes
 from typing import Optional, Tuple
 
 import torch
@@ -261,6 +262,72 @@ def cast(x: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
   if x.numel():
     p = H.CastParams(H.ptr(x), H.ptr(out), x.numel(), H.dtype_code(x.dtype), H.dtype_code(dtype))
     H.call("vmoe_cast", p)
+  return out
+
+
+def add_layer_norm(residual: torch.Tensor, branch: Optional[torch.Tensor],
+                   scale: Optional[torch.Tensor], bias: Optional[torch.Tensor], eps: float,
+                   out_dtype: Optional[torch.dtype], write_residual: bool = True):
+  """x = residual (+ branch); returns (x as float32 or None, layer_norm(x) in out_dtype or None).
+
+  residual (..., D) float32; branch the same shape, float32 or bfloat16, or None;
+  out_dtype None skips the norm (add only).  Without a branch the residual itself
+  is returned as x.
+  """
+  if residual.dtype != torch.float32:
+    raise TypeError(f"residual must be float32, got {residual.dtype}")
+  residual = residual.contiguous()
+  D = residual.shape[-1]
+  rows = residual.numel() // D
+  dev = residual.device
+  if branch is not None:
+    if branch.shape != residual.shape:
+      raise ValueError(f"branch {tuple(branch.shape)} != residual {tuple(residual.shape)}")
+    branch = branch.contiguous()
+  f32 = lambda t: None if t is None else t.to(torch.float32).contiguous()
+  scale, bias = f32(scale), f32(bias)
+  res_out = torch.empty_like(residual) if (branch is not None and write_residual) else None
+  norm_out = None if out_dtype is None else torch.empty(residual.shape, dtype=out_dtype, device=dev)
+  if res_out is None and norm_out is None:
+    return residual, None
+  optr = lambda t: None if t is None else H.ptr(t)
+  p = H.AddLayerNormParams(
+      H.ptr(residual), optr(branch), optr(scale), optr(bias), optr(res_out), optr(norm_out),
+      rows, D, float(eps), H.dtype_code(branch.dtype) if branch is not None else 0,
+      H.dtype_code(out_dtype) if out_dtype is not None else 0)
+  H.call("vmoe_add_layer_norm", p)
+  return (res_out if res_out is not None else residual), norm_out
+
+
+ATTENTION_HEAD_DIM = 64
+
+
+def attention_supported(q: torch.Tensor, k: torch.Tensor) -> bool:
+  """Shapes the attention kernel covers: bfloat16, head size 64, keys and values
+  of one head resident in LDS; (B, S, H, hd) views whose last two axes are contiguous."""
+  if q.dtype != torch.bfloat16 or q.shape[-1] != ATTENTION_HEAD_DIM:
+    return False
+  sk_pad = (k.shape[1] + 31) // 32 * 32
+  waves = min(8, (q.shape[1] + 31) // 32)
+  lds = sk_pad * 144 + 64 * (sk_pad + 8) * 2 + waves * 32 * 80
+  return lds <= 160 * 1024
+
+
+def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: float) -> torch.Tensor:
+  """softmax(q k^T * scale) v per (image, head).  q (B, Sq, H, hd), k, v (B, Sk, H, hd):
+  views are fine as long as heads and head columns are contiguous (e.g. slices of a
+  packed projection output).  Returns (B, Sq, H * hd)."""
+  B, Sq, heads, hd = q.shape
+  Sk = k.shape[1]
+  for t in (q, k, v):
+    if t.stride(3) != 1 or t.stride(2) != hd:
+      raise H.VmoeError("attention operands need contiguous (H, hd) trailing axes")
+  out = torch.empty((B, Sq, heads * hd), dtype=q.dtype, device=q.device)
+  p = H.AttentionParams(
+      ctypes.c_void_p(q.data_ptr()), ctypes.c_void_p(k.data_ptr()), ctypes.c_void_p(v.data_ptr()),
+      H.ptr(out), q.stride(0), q.stride(1), k.stride(0), k.stride(1), v.stride(0), v.stride(1),
+      B, heads, Sq, Sk, hd, float(scale), H.dtype_code(q.dtype))
+  H.call("vmoe_attention", p)
   return out
 
 

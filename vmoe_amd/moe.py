@@ -12,6 +12,7 @@ order of the reference's _dispatch (vmoe/moe.py:488-500); combine takes
 from __future__ import annotations
 
 import abc
+import functools
 import logging
 import math
 from typing import Any, Callable, Dict, Mapping, Optional, Tuple
@@ -238,6 +239,7 @@ def _cast_to_bfloat16(x: Array) -> Array:
   return K.cast(x, torch.bfloat16) if x.is_floating_point() else x
 
 
+@functools.lru_cache(maxsize=256)   # a layer asks on every call; compute (and warn) once per shape
 def compute_capacity(num_tokens: int, num_experts: int, capacity_factor: float,
                      ceil_or_round: str = "ceil", multiple_of: Optional[int] = 4) -> int:
   """Capacity per expert needed to distribute num_tokens among num_experts; vmoe/moe.py:230-257."""

@@ -161,6 +161,19 @@ def _layer_norm(x: Array, p: Mapping[str, Array], dtype: Optional[torch.dtype],
   return y if dtype in (None, torch.float32) else y.to(dtype)
 
 
+def _add_layer_norm(residual: Array, branch: Optional[Array], p: Mapping[str, Array],
+                    dtype: Optional[torch.dtype], eps: float = 1e-6):
+  """``x = residual + branch; y = LayerNorm(dtype)(x)`` (vmoe/nn/vit_moe.py:162-179) ->
+  (x, y).  A float32 residual takes the fused kernel; anything else keeps the
+  promotion rules of the separate operations."""
+  if residual.dtype == torch.float32 and (
+      branch is None or branch.dtype in (torch.float32, torch.bfloat16)):
+    return K.add_layer_norm(residual, branch, p.get("scale"), p.get("bias"), eps,
+                            dtype or torch.float32)
+  x = residual if branch is None else residual + branch
+  return x, _layer_norm(x, p, dtype, eps)
+
+
 class IdentityLayer(module.Module):
   """vit_jax.models_vit.IdentityLayer (exists to name the pre-logits activation)."""
 
@@ -258,9 +271,12 @@ class MultiHeadDotProductAttention(module.Module):
     if self.normalize_qk:
       q = _layer_norm(q, p["query_ln"], dtype)
       k = _layer_norm(k, p["key_ln"], dtype)
-    ctx = torch.nn.functional.scaled_dot_product_attention(
-        q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2))       # (B, H, Sq, hd)
-    ctx = ctx.transpose(1, 2).reshape(B, Sq, H * hd)
+    if q.is_cuda and K.attention_supported(q, k):
+      ctx = K.attention(q, k, v, hd ** -0.5)                            # (B, Sq, H * hd)
+    else:
+      ctx = torch.nn.functional.scaled_dot_product_attention(
+          q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2))     # (B, H, Sq, hd)
+      ctx = ctx.transpose(1, 2).reshape(B, Sq, H * hd)
     key = (p["out"]["kernel"].data_ptr(), p["out"]["kernel"]._version,
            p["out"]["bias"].data_ptr(), p["out"]["bias"]._version, dtype, "out")
     wo, bo = self._cached(key, lambda: (
@@ -342,18 +358,23 @@ class EncoderBlock(module.Module):
                        mlp.name: mlp.init(fold(rng, 2), x)["params"]}}
 
   def apply(self, variables, inputs: Array):
+    x, y, metrics = self._forward(variables["params"], inputs, None)
+    return x + y if metrics is None else (x + y, metrics)
+
+  def _forward(self, p, residual: Array, pending: Optional[Array]):
+    """The block on ``residual + pending``, the last add left to the caller:
+    returns (residual, mlp output not yet added, metrics or None).  Leaving the
+    add pending lets it run inside the kernel of the layer norm that follows."""
     self._check_inference()
     attn, mlp = self._modules()
-    p = variables["params"]
-    x = _layer_norm(inputs, p["LayerNorm_0"], self.dtype)
-    x = attn.apply({"params": p["SelfAttention"]}, x)
-    x = x + inputs
-    y = _layer_norm(x, p["LayerNorm_1"], self.dtype)
+    x, a = _add_layer_norm(residual, pending, p["LayerNorm_0"], self.dtype)
+    h = attn.apply({"params": p["SelfAttention"]}, a)
+    x, y = _add_layer_norm(x, h, p["LayerNorm_1"], self.dtype)
     y = mlp.apply({"params": p[mlp.name]}, y)
     if isinstance(y, torch.Tensor):
-      return x + y
+      return x, y, None
     y, metrics = y
-    return x + y, metrics
+    return x, y, metrics
 
 
 class EncoderMoe(module.Module):
@@ -405,13 +426,12 @@ class EncoderMoe(module.Module):
     params = variables["params"]
     x = self.add_position_emb(variables, inputs)
     metrics = {}
+    pending = None          # output of the previous block's MLP, added by the next layer norm
     for b, block in enumerate(self._blocks()):
-      out = block.apply({"params": params[block.name]}, x)
+      x, pending, m = block._forward(params[block.name], x, pending)
       if b in self._moe_layers:
-        x, metrics[block.name] = out
-      else:
-        x = out
-    encoded = _layer_norm(x, params["encoder_norm"], None)
+        metrics[block.name] = m
+    _, encoded = _add_layer_norm(x, pending, params["encoder_norm"], None)
     metrics["auxiliary_loss"] = sum(m["auxiliary_loss"] for m in metrics.values())
     return encoded, metrics
 
