@@ -327,7 +327,7 @@ int vmoe_add_layer_norm(const VmoeAddLayerNormParams* p, vmoe_stream_t stream);
  * element h * head_dim), so the packed output of a fused q/k/v projection can be
  * passed without copies; out (B, Sq, H * head_dim) contiguous.  Strides are
  * multiples of 8 elements, pointers 16-byte aligned.
- * VMOE_E_UNSUPPORTED unless dtype is bfloat16, head_dim is 64 and the keys and
+ * VMOE_E_UNSUPPORTED unless dtype is bfloat16, head_dim is 64, scale > 0 and the keys and
  * values of one head fit in LDS (Sk up to about 560). */
 typedef struct {
   const void* q;

@@ -213,41 +213,79 @@ __global__ __launch_bounds__(kAttnMaxWaves * 64) void attention_bf16_kernel(
   const bf16_t* Vb = Vp + (size_t)b * v_sb + (size_t)head * kHd;
   const bf16_t* Qb = Q + (size_t)b * q_sb + (size_t)head * kHd;
 
-  // Stage K (row-major) and V (transposed); keys past Sk are zero.
-  for (int c = tid; c < sk_pad * 8; c += nthreads) {
-    const int key = c >> 3, part = c & 7;
-    uint4 kv = make_uint4(0, 0, 0, 0), vv = make_uint4(0, 0, 0, 0);
-    if (key < Sk) {
-      kv = *reinterpret_cast<const uint4*>(Kb + (size_t)key * k_ss + part * 8);
-      vv = *reinterpret_cast<const uint4*>(Vb + (size_t)key * v_ss + part * 8);
-    }
-    *reinterpret_cast<uint4*>(Ks + key * kKRow + part * 8) = kv;
-    const uint32_t w[4] = {vv.x, vv.y, vv.z, vv.w};
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      Vt[(part * 8 + 2 * i) * vt_row + key] = (bf16_t)(w[i] & 0xffffu);
-      Vt[(part * 8 + 2 * i + 1) * vt_row + key] = (bf16_t)(w[i] >> 16);
-    }
-  }
-  __syncthreads();
-
   const int ql = lane & 31, hh = lane >> 5;
-  bf16_t* stage = stage_all + (size_t)wave * 32 * kStageRow;
   const int q_tiles = (Sq + 31) >> 5, k_tiles = sk_pad >> 5;
-  for (int qt = wave; qt < q_tiles; qt += nwaves) {
-    const int q = qt * 32 + ql;
+  // The first query tile's fragments are requested before anything else.
+  bf16x8 qf[4];
+  {
+    const int q = wave * 32 + ql;
     const int qc = q < Sq ? q : Sq - 1;
-    bf16x8 qf[4];
 #pragma unroll
     for (int c = 0; c < 4; ++c)
       qf[c] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(
           Qb + (size_t)qc * q_ss + 16 * c + 8 * hh));
+  }
+  // Stage K row-major; keys past Sk are zero.  Four chunks in flight per thread.
+  for (int c0 = tid; c0 < sk_pad * 8; c0 += 4 * nthreads) {
+    uint4 kv[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int c = c0 + u * nthreads;
+      const int key = c >> 3, part = c & 7;
+      kv[u] = make_uint4(0, 0, 0, 0);
+      if (key < Sk) kv[u] = *reinterpret_cast<const uint4*>(Kb + (size_t)key * k_ss + part * 8);
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int c = c0 + u * nthreads;
+      if (c < sk_pad * 8)
+        *reinterpret_cast<uint4*>(Ks + (c >> 3) * kKRow + (c & 7) * 8) = kv[u];
+    }
+  }
+  // Stage V transposed: a thread takes 8 keys x 8 head columns, transposes the
+  // block in registers and writes each head column's 8 keys as one 16-byte chunk.
+  // Consecutive lanes take consecutive key blocks of one column group, so 16 lanes
+  // write 2 x 128 contiguous bytes that fall in disjoint banks.
+  const int kblocks = sk_pad >> 3;
+  for (int id = tid; id < kblocks * 8; id += nthreads) {
+    const int part = id / kblocks, kb = id - part * kblocks;
+    uint32_t w[8][4];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int key = kb * 8 + i;
+      uint4 r = make_uint4(0, 0, 0, 0);
+      if (key < Sk) r = *reinterpret_cast<const uint4*>(Vb + (size_t)key * v_ss + part * 8);
+      w[i][0] = r.x; w[i][1] = r.y; w[i][2] = r.z; w[i][3] = r.w;
+    }
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const uint32_t sel = (j & 1) ? 0x07060302u : 0x05040100u;
+      uint4 o4;
+      o4.x = __builtin_amdgcn_perm(w[1][j >> 1], w[0][j >> 1], sel);
+      o4.y = __builtin_amdgcn_perm(w[3][j >> 1], w[2][j >> 1], sel);
+      o4.z = __builtin_amdgcn_perm(w[5][j >> 1], w[4][j >> 1], sel);
+      o4.w = __builtin_amdgcn_perm(w[7][j >> 1], w[6][j >> 1], sel);
+      *reinterpret_cast<uint4*>(Vt + (part * 8 + j) * vt_row + kb * 8) = o4;
+    }
+  }
+  __syncthreads();
+
+  bf16_t* stage = stage_all + (size_t)wave * 32 * kStageRow;
+  for (int qt = wave; qt < q_tiles; qt += nwaves) {
+    if (qt != wave) {
+      const int q = qt * 32 + ql;
+      const int qc = q < Sq ? q : Sq - 1;
+#pragma unroll
+      for (int c = 0; c < 4; ++c)
+        qf[c] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(
+            Qb + (size_t)qc * q_ss + 16 * c + 8 * hh));
+    }
     floatx16 o[2];
 #pragma unroll
     for (int i = 0; i < 2; ++i)
 #pragma unroll
       for (int j = 0; j < 16; ++j) o[i][j] = 0.f;
-    float m = -INFINITY, l = 0.f;
+    float m = 0.f, l = 0.f;
     for (int kt = 0; kt < k_tiles; ++kt) {
       floatx16 sacc;
 #pragma unroll
@@ -260,32 +298,45 @@ __global__ __launch_bounds__(kAttnMaxWaves * 64) void attention_bf16_kernel(
       }
       // sacc[4 * g + t] is the logit of key kt * 32 + 8 * g + 4 * hh + t for query ql.
       float p[16];
-      float tmax = -INFINITY;
-      const int key0 = kt * 32 + 4 * hh;
 #pragma unroll
-      for (int g = 0; g < 4; ++g)
+      for (int j = 0; j < 16; ++j) p[j] = sacc[j];
+      if (kt == k_tiles - 1 && Sk < sk_pad) {      // only the last tile holds padding keys
+        const int key0 = kt * 32 + 4 * hh;
 #pragma unroll
-        for (int t = 0; t < 4; ++t) {
-          float v = sacc[4 * g + t] * scale_log2e;
-          if (key0 + 8 * g + t >= Sk) v = -INFINITY;
-          p[4 * g + t] = v;
-          tmax = fmaxf(tmax, v);
+        for (int g = 0; g < 4; ++g)
+#pragma unroll
+          for (int t = 0; t < 4; ++t)
+            if (key0 + 8 * g + t >= Sk) p[4 * g + t] = -INFINITY;
+      }
+      float tmax = p[0];
+#pragma unroll
+      for (int j = 1; j < 16; ++j) tmax = fmaxf(tmax, p[j]);
+      tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64)) * scale_log2e;   // scale > 0
+      // The running maximum only has to bound the exponents: it is raised when a
+      // tile exceeds it by more than 2^8, which keeps every term below 2^8 and
+      // makes the rescaling of the accumulators rare (wave-uniform branch).
+      if (kt == 0) {
+        m = tmax;
+      } else {
+        const bool raise = tmax > m + 8.0f;
+        if (__any(raise)) {
+          const float m_new = raise ? tmax : m;
+          const float alpha = __builtin_amdgcn_exp2f(m - m_new);
+          l *= alpha;
+          m = m_new;
+#pragma unroll
+          for (int i = 0; i < 2; ++i)
+#pragma unroll
+            for (int j = 0; j < 16; ++j) o[i][j] *= alpha;
         }
-      tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
-      const float m_new = fmaxf(m, tmax);        // finite: every tile holds at least one key
-      const float alpha = __builtin_amdgcn_exp2f(m - m_new);
+      }
       float lsum = 0.f;
 #pragma unroll
       for (int j = 0; j < 16; ++j) {
-        p[j] = __builtin_amdgcn_exp2f(p[j] - m_new);
+        p[j] = __builtin_amdgcn_exp2f(__builtin_fmaf(p[j], scale_log2e, -m));
         lsum += p[j];
       }
-      l = l * alpha + lsum;
-      m = m_new;
-#pragma unroll
-      for (int i = 0; i < 2; ++i)
-#pragma unroll
-        for (int j = 0; j < 16; ++j) o[i][j] *= alpha;
+      l += lsum;
 #pragma unroll
       for (int c2 = 0; c2 < 2; ++c2) {
         uint4 pk;
@@ -358,7 +409,7 @@ extern "C" int vmoe_attention(const VmoeAttentionParams* p, vmoe_stream_t stream
   if (p == nullptr || p->q == nullptr || p->k == nullptr || p->v == nullptr || p->out == nullptr)
     return VMOE_E_NULL;
   if (p->B < 1 || p->H < 1 || p->Sq < 1 || p->Sk < 1) return VMOE_E_SHAPE;
-  if (p->dtype != VMOE_BF16 || p->head_dim != kHd) return VMOE_E_UNSUPPORTED;
+  if (p->dtype != VMOE_BF16 || p->head_dim != kHd || !(p->scale > 0.f)) return VMOE_E_UNSUPPORTED;
   if ((int64_t)p->B * p->H >= INT32_MAX) return VMOE_E_OVERFLOW;
   const int64_t strides[6] = {p->q_stride_b, p->q_stride_s, p->k_stride_b,
                               p->k_stride_s, p->v_stride_b, p->v_stride_s};
