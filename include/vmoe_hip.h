@@ -72,8 +72,27 @@ typedef struct {
   int32_t num_items;       /* T = G*S */
   int32_t D, E, K;
   int32_t dtype;
+  float* logits;           /* optional out (G*S, E) float32: the logits (exact dtype values,
+                              bias included), what the noisy branch of the router adds to */
 } VmoeGateTopkParams;
 int vmoe_gate_topk(const VmoeGateTopkParams* p, vmoe_stream_t stream);
+
+/* Noisy branch of the routers, vmoe/nn/routing.py:92-114 (and :226-232):
+ *   logits_noisy = logits + noise_std * noise;  gates_noisy = softmax(logits_noisy)
+ * and, per group, the load loss of vmoe/nn/routing.py:159-183: with t the K-th
+ * largest noisy logit of an item, p = 1 - Phi((t - logits) / noise_std) averaged
+ * over the group's items per expert, loss = (std(p_mean) / mean(p_mean))^2.
+ * noise is standard normal (the caller draws it); noise_std is the effective
+ * standard deviation, (1 / E) * the router's noise_std.  E <= 128, 1 <= K <= E. */
+typedef struct {
+  const float* logits;     /* (G*S, E) float32 */
+  const float* noise;      /* (G*S, E) float32, standard normal */
+  float* gates_noisy;      /* out (G*S, E) float32 */
+  float* load_loss;        /* optional out (G,) float32 */
+  int32_t G, S, E, K;
+  float noise_std;
+} VmoeNoisyGatesParams;
+int vmoe_noisy_gates(const VmoeNoisyGatesParams* p, vmoe_stream_t stream);
 
 /* Top-k alone on given gates (G*S, E) float32: the jax.lax.top_k of
  * vmoe/moe.py:567.  Bit-exact selection; E <= 1024. */

@@ -447,8 +447,11 @@ def router_metrics(gates: np.ndarray, gshard_loss_weight: float = 0.0,
 
 def noisy_top_experts_per_item_router(
     x, kernel, num_selected_experts, dispatcher_kwargs, dtype=F32,
-    gshard_loss_weight=0.0, importance_loss_weight=1.0, logit_bias=None):
-  """vmoe/nn/routing.py:55-60 + :116-131, deterministic branch."""
+    gshard_loss_weight=0.0, importance_loss_weight=1.0, logit_bias=None,
+    noise=None, noise_std=1.0, load_loss_weight=1.0):
+  """vmoe/nn/routing.py:55-60 + :62-131.  With ``noise`` None the deterministic
+  branch; otherwise ``noise`` is the standard normal sample (G,S,E) that
+  ``jax.random.normal`` would supply and the noisy branch (:92-114) runs."""
   if x.ndim != 3:
     raise ValueError(f"inputs.ndim must be 3, but it is {x.ndim}")
   num_experts = kernel.shape[-1]
@@ -456,10 +459,27 @@ def noisy_top_experts_per_item_router(
     raise ValueError(f"num_experts >= num_selected_experts >= 1, but got "
                      f"num_experts = {num_experts} and "
                      f"num_selected_experts = {num_selected_experts}.")
-  gates = router_gates(x, kernel, dtype, logit_bias)
-  metrics = router_metrics(gates, gshard_loss_weight, importance_loss_weight)
   kw = dict(dispatcher_kwargs or {})
   use_bfloat16 = kw.pop("bfloat16", False)
+  if noise is None:
+    gates = router_gates(x, kernel, dtype, logit_bias)
+    metrics = router_metrics(gates, gshard_loss_weight, importance_loss_weight)
+  else:
+    logits = dense(x, kernel, None, dtype)                                    # :73-74
+    if logit_bias is not None:
+      logits = cast(logits + np.asarray(logit_bias, np.float32), dtype)
+    gates_clean = cast(softmax(logits), dtype)                                # :80
+    imp = np.stack([importance_auxiliary_loss(g) for g in gates_clean])       # :81
+    std = np.float32((1.0 / num_experts) * noise_std)                         # :93
+    logits_noisy = (logits + std * np.asarray(noise, np.float32)).astype(np.float32)   # :94-96
+    gates = softmax(logits_noisy)                                             # :97
+    load = np.stack([load_auxiliary_loss(l, ln, std, num_selected_experts)
+                     for l, ln in zip(logits, logits_noisy)]).astype(np.float32)  # :98-102
+    gsh = np.stack([gshard_auxiliary_loss(g) for g in gates])                 # :103
+    aux = sum(v * w for w, v in ((gshard_loss_weight, gsh), (importance_loss_weight, imp),
+                                 (load_loss_weight, load)) if w > 0)
+    metrics = {"auxiliary_loss": aux, "gshard_loss": gsh, "importance_loss": imp,
+               "load_loss": load}
   dispatcher = get_top_experts_per_item_dispatcher(
       gates, num_selected_experts=num_selected_experts, **kw)
   if use_bfloat16:

@@ -65,7 +65,8 @@ def test_struct_layouts_match_header():
         "VmoeEinsumParams": _hip.EinsumParams, "VmoeCastParams": _hip.CastParams,
         "VmoeTopItemsParams": _hip.TopItemsParams,
         "VmoeAddLayerNormParams": _hip.AddLayerNormParams,
-        "VmoeAttentionParams": _hip.AttentionParams}
+        "VmoeAttentionParams": _hip.AttentionParams,
+        "VmoeNoisyGatesParams": _hip.NoisyGatesParams}
   assert set(py) == set(structs)
   for name, body in structs.items():
     want = []

@@ -254,8 +254,93 @@ def test_top_items_per_expert_router(dtype):
     assert got_dw.sum() == dw_g.sum() == E * C
   noisy = routing.NoisyTopItemsPerExpertRouter(num_experts=E, noise_std=1.0,
                                                dispatcher=dict(name="einsum", capacity=C))
-  with pytest.raises(NotImplementedError):
+  with pytest.raises(ValueError, match="rngs"):
     noisy.apply(variables, to_dev(x, dtype))
+  # vmoe/nn/routing.py:226-232: softmax of logits + (noise_std / E) * normal noise.
+  d1, _ = noisy.apply(variables, to_dev(x, dtype), rngs={"gating": 5})
+  noise = torch.randn((G, S, E), generator=torch.Generator(device=dev()).manual_seed(5),
+                      device=dev(), dtype=torch.float32)
+  logits = O.dense(x, kernel, None, dtype)
+  gates_noisy = O.softmax(logits + np.float32(1.0 / E) * to_np(noise))
+  for g in range(G):
+    cw_g, dw_g, _ = O.top_items_per_expert_einsum(gates_noisy[g], C)
+    assert_close(to_np(d1.combine_weights[g]).sum(axis=(0, 2)), cw_g.sum(axis=(0, 2)), 1e-5,
+                 "noisy selected gate mass per expert")
+
+
+def test_load_auxiliary_loss_golden(goldens):
+  """vmoe/nn/routing_test.py:62-80 through the kernel: logits, noise and the expected loss."""
+  from vmoe_amd import kernels as K
+  ld = goldens["router_aux_losses"]["load"]
+  logits = np.asarray(ld["logits"], np.float32)[None]
+  # the kernel takes standard normal noise and the standard deviation separately
+  noise = np.asarray(ld["noise"], np.float32)[None] / np.float32(ld["noise_std"])
+  gates, loss = K.noisy_gates(to_dev(logits), to_dev(noise), ld["noise_std"],
+                              ld["num_selected_experts"])
+  assert float(loss[0]) == pytest.approx(ld["expected"], abs=2e-6)
+  np.testing.assert_allclose(to_np(gates), O.softmax(logits + np.asarray(ld["noise"], np.float32)),
+                             rtol=1e-6, atol=1e-7)
+
+
+@pytest.mark.parametrize("G,S,E,K", [(3, 50, 8, 2), (2, 197, 32, 1), (1, 64, 100, 5), (2, 33, 128, 3)])
+def test_noisy_gates_kernel_vs_oracle(G, S, E, K):
+  from vmoe_amd import kernels as K_
+  rng = np.random.default_rng(G + S + E + K)
+  logits = rng.standard_normal((G, S, E)).astype(np.float32)
+  logits[0, 0, :] = 0.25                       # a row of equal logits
+  noise = rng.standard_normal((G, S, E)).astype(np.float32)
+  std = np.float32(0.7 / E)
+  gates, loss = K_.noisy_gates(to_dev(logits), to_dev(noise), float(std), K)
+  noisy = logits + std * noise
+  np.testing.assert_allclose(to_np(gates), O.softmax(noisy), rtol=2e-6, atol=1e-8)
+  want = [float(O.load_auxiliary_loss(logits[g], noisy[g], std, K)) for g in range(G)]
+  np.testing.assert_allclose(to_np(loss), want, rtol=2e-4, atol=1e-7)
+
+
+@pytest.mark.parametrize("dtype", [O.F32, O.BF16])
+def test_router_noisy_branch_vs_oracle(dtype):
+  """vmoe/nn/routing.py:92-114 with the noise the router drew handed to the oracle."""
+  from vmoe_amd.nn import routing
+  rng = np.random.default_rng(21)
+  G, S, D, E, K = 3, 64, 32, 8, 2
+  x = O.cast(rng.standard_normal((G, S, D)).astype(np.float32), dtype)
+  kernel = O.cast(rng.standard_normal((D, E)).astype(np.float32) / np.sqrt(D), dtype)
+  kw = dict(num_experts=E, num_selected_experts=K, noise_std=2.0, gshard_loss_weight=0.5,
+            importance_loss_weight=0.25, load_loss_weight=2.0,
+            dispatcher=dict(name="indices", capacity=20, batch_priority=True))
+  layer = routing.NoisyTopExpertsPerItemRouter(**kw)
+  variables = {"params": {"dense": {"kernel": to_dev(kernel, dtype)}}}
+  dispatcher, metrics = layer.apply(variables, to_dev(x, dtype), rngs={"gating": 9})
+  noise = torch.randn((G, S, E), generator=torch.Generator(device=dev()).manual_seed(9),
+                      device=dev(), dtype=torch.float32)
+  want_d, want_m, want_gates = O.noisy_top_experts_per_item_router(
+      x, kernel, K, dict(name="indices", capacity=20, batch_priority=True), dtype,
+      gshard_loss_weight=0.5, importance_loss_weight=0.25, noise=to_np(noise), noise_std=2.0,
+      load_loss_weight=2.0)
+  assert set(metrics) == {"auxiliary_loss", "gshard_loss", "importance_loss", "load_loss"}
+  tol = 2e-2 if dtype == O.BF16 else 2e-4
+  for k in metrics:
+    np.testing.assert_allclose(to_np(metrics[k]), want_m[k], rtol=tol, atol=1e-6, err_msg=k)
+  agree = (to_np(dispatcher.indices) == want_d.indices).all(axis=(2, 3)).mean()
+  assert agree >= (0.97 if dtype == O.BF16 else 0.999), agree
+
+
+def test_router_forward_not_deterministic():
+  """vmoe/nn/routing_test.py:102-122."""
+  from vmoe_amd.nn import routing
+  x = torch.arange(5 * 4, dtype=torch.float32, device=dev()).reshape(1, 5, 4)
+  variables = {"params": {"dense": {"kernel": torch.eye(4, device=dev())}}}
+  layer = routing.NoisyTopExpertsPerItemRouter(
+      num_experts=4, num_selected_experts=2, noise_std=2.0, deterministic=False,
+      dispatcher=dict(name="einsum", capacity=2, batch_priority=False))
+  d1, m1 = layer.apply(variables, x, rngs={"gating": 0})
+  d2, m2 = layer.apply(variables, x, rngs={"gating": 1})
+  assert (d1.combine_weights - d2.combine_weights).abs().sum() > 0.01
+  np.testing.assert_allclose(to_np(m1["importance_loss"]), to_np(m2["importance_loss"]))
+  for k in ("auxiliary_loss", "gshard_loss", "load_loss"):
+    assert (m1[k] - m2[k]).abs().sum() > 0.01, k
+  d3, m3 = layer.apply(variables, x, rngs={"gating": 0})   # same seed, same result
+  np.testing.assert_array_equal(to_np(d1.combine_weights), to_np(d3.combine_weights))
 
 
 # ------------------------------------------------------------------ SparseMoeSpmdLayerTest
@@ -364,7 +449,7 @@ def test_router_argument_errors():
   with pytest.raises(ValueError, match="inputs.ndim must be 3"):
     layer.apply(variables, torch.zeros((5, 4), device=dev()))
   noisy = routing.NoisyTopExpertsPerItemRouter(num_experts=4, num_selected_experts=2, noise_std=1.0)
-  with pytest.raises(NotImplementedError):
+  with pytest.raises(ValueError, match="rngs"):
     noisy.apply(variables, torch.zeros((1, 5, 4), device=dev()))
 
 

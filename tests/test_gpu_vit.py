@@ -104,14 +104,23 @@ def test_forward(vit_moe):
   assert tuple(output.shape) == (16, 4)
 
 
-def test_training_mode_raises(vit_moe):
+def test_forward_noisy_router(vit_moe):
+  """The reference's default test config (vmoe/nn/vit_moe_test.py:28-55) has a noisy
+  router: the forward pass needs a 'gating' rng and reports the load loss."""
   config = product_config(DEFAULT_TEST_CONFIG, O.F32)
   config["deterministic"] = False
-  config["encoder"]["moe"]["router"]["noise_std"] = 1e-3
+  config["encoder"]["moe"]["router"].update(noise_std=1e-3, load_loss_weight=0.02)
   model = vit_moe.VisionTransformerMoe(**config)
   x = torch.randn((16, 4, 4, 3), device=dev())
+  variables = model.init(0, x)
+  with pytest.raises(ValueError, match="rngs"):
+    model.apply(variables, x)
+  out, metrics = model.apply(variables, x, rngs={"gating": 1})
+  assert tuple(out.shape) == (16, 4)
+  assert "load_loss" in metrics["encoderblock_1"]
+  config["encoder"]["dropout_rate"] = 0.1
   with pytest.raises(NotImplementedError):
-    model.apply(model.init(0, x), x)
+    vit_moe.VisionTransformerMoe(**config).apply(variables, x, rngs={"gating": 1})
 
 
 # ------------------------------------------------------------------ parity with the CPU restatement

@@ -25,7 +25,7 @@ EXPORTS = [
     "vmoe_expert_mlp_workspace_bytes", "vmoe_expert_mlp", "vmoe_pack_expert_weights",
     "vmoe_soft_route_workspace_bytes", "vmoe_soft_route", "vmoe_einsum_dispatch",
     "vmoe_einsum_combine", "vmoe_cast", "vmoe_copy_bytes", "vmoe_mfma_probe",
-    "vmoe_add_layer_norm", "vmoe_attention",
+    "vmoe_add_layer_norm", "vmoe_attention", "vmoe_noisy_gates",
 ]
 
 
@@ -85,7 +85,14 @@ def stream() -> c_void_p:
 class GateTopkParams(ctypes.Structure):
   _fields_ = [("x", c_void_p), ("w", c_void_p), ("logit_bias", c_void_p), ("gates", c_void_p),
               ("topk_val", c_void_p), ("topk_idx", c_void_p), ("num_items", c_int32),
-              ("D", c_int32), ("E", c_int32), ("K", c_int32), ("dtype", c_int32)]
+              ("D", c_int32), ("E", c_int32), ("K", c_int32), ("dtype", c_int32),
+              ("logits", c_void_p)]
+
+
+class NoisyGatesParams(ctypes.Structure):
+  _fields_ = [("logits", c_void_p), ("noise", c_void_p), ("gates_noisy", c_void_p),
+              ("load_loss", c_void_p), ("G", c_int32), ("S", c_int32), ("E", c_int32),
+              ("K", c_int32), ("noise_std", ctypes.c_float)]
 
 
 class TopkParams(ctypes.Structure):

@@ -63,7 +63,8 @@ template <typename T> __host__ __device__ constexpr int w_stride(int kc, int epa
 template <typename T, int NT>
 __global__ __launch_bounds__(kGateThreads) void gate_topk_kernel(
     const T* __restrict__ x, const T* __restrict__ w, const float* __restrict__ bias,
-    T* __restrict__ gates, float* __restrict__ topk_val, int32_t* __restrict__ topk_idx,
+    T* __restrict__ gates, float* __restrict__ logits, float* __restrict__ topk_val,
+    int32_t* __restrict__ topk_idx,
     int num_items, int D, int E, int K, int KC, int num_chunks, int num_tiles, int stage_off) {
   extern __shared__ __align__(16) unsigned char smem[];
   T* wl = reinterpret_cast<T*>(smem);
@@ -226,6 +227,11 @@ __global__ __launch_bounds__(kGateThreads) void gate_topk_kernel(
       const float v = st[m * (EP + 1) + n0 + j];
       g[j] = (n0 + j < E) ? v : -INFINITY;
       mx = fmaxf(mx, g[j]);
+    }
+    if (logits != nullptr && row < num_items) {
+#pragma unroll
+      for (int j = 0; j < CNT; ++j)
+        if (n0 + j < E) logits[(size_t)row * E + n0 + j] = g[j];
     }
     mx = fmaxf(mx, __shfl_xor(mx, 32, kWave));
     float sum = 0.f;
@@ -431,8 +437,8 @@ int launch_gate(const VmoeGateTopkParams* p, hipStream_t stream) {
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return (int)e;
     hipLaunchKernelGGL(kern, dim3(blocks), dim3(kGateThreads), lds, stream,
-                       (const T*)p->x, (const T*)p->w, p->logit_bias, (T*)p->gates, p->topk_val,
-                       p->topk_idx, p->num_items, p->D, p->E, p->K, kc, num_chunks, num_tiles,
+                       (const T*)p->x, (const T*)p->w, p->logit_bias, (T*)p->gates, p->logits,
+                       p->topk_val, p->topk_idx, p->num_items, p->D, p->E, p->K, kc, num_chunks, num_tiles,
                        (int)w_bytes);
     return launch_status();
   };
@@ -440,6 +446,90 @@ int launch_gate(const VmoeGateTopkParams* p, hipStream_t stream) {
     case 1: return run(gate_topk_kernel<T, 1>);
     case 2: return run(gate_topk_kernel<T, 2>);
     default: return run(gate_topk_kernel<T, 4>);
+  }
+}
+
+
+// Noisy branch of the routers (vmoe/nn/routing.py:92-114): softmax of the noisy
+// logits and, per group, the load loss (vmoe/nn/routing.py:159-183).  One
+// workgroup per group, a wave per item, a lane per expert (two for E > 64).
+constexpr int kNoisyWaves = 8;
+
+__device__ __forceinline__ float wave_max_f(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, kWave));
+  return v;
+}
+__device__ __forceinline__ float wave_sum_f(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, kWave);
+  return v;
+}
+__device__ __forceinline__ uint64_t wave_max_u64(uint64_t v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    const uint32_t lo = __shfl_xor((uint32_t)v, o, kWave);
+    const uint32_t hi = __shfl_xor((uint32_t)(v >> 32), o, kWave);
+    const uint64_t other = ((uint64_t)hi << 32) | lo;
+    v = other > v ? other : v;
+  }
+  return v;
+}
+
+__global__ __launch_bounds__(kNoisyWaves * 64) void noisy_gates_kernel(
+    const float* __restrict__ logits, const float* __restrict__ noise,
+    float* __restrict__ gates, float* __restrict__ load_loss, int S, int E, int K,
+    float noise_std) {
+  __shared__ float psum[kNoisyWaves][128];
+  const int g = blockIdx.x;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const bool has0 = lane < E, has1 = lane + 64 < E;
+  const float inv = 1.0f / (noise_std * 1.41421356237309515f);
+  float acc0 = 0.f, acc1 = 0.f;
+  for (int s = wave; s < S; s += kNoisyWaves) {
+    const size_t base = ((size_t)g * S + s) * E;
+    const float l0 = has0 ? logits[base + lane] : 0.f;
+    const float l1 = has1 ? logits[base + lane + 64] : 0.f;
+    const float v0 = has0 ? l0 + noise_std * noise[base + lane] : -INFINITY;
+    const float v1 = has1 ? l1 + noise_std * noise[base + lane + 64] : -INFINITY;
+    const float mx = wave_max_f(fmaxf(v0, v1));
+    const float e0 = has0 ? expf(v0 - mx) : 0.f;
+    const float e1 = has1 ? expf(v1 - mx) : 0.f;
+    const float sum = wave_sum_f(e0 + e1);
+    if (has0) gates[base + lane] = e0 / sum;
+    if (has1) gates[base + lane + 64] = e1 / sum;
+    if (load_loss == nullptr) continue;
+    // Value of the K-th largest noisy logit (lax.top_k order: equal values, lower index first).
+    uint64_t k0 = has0 ? (((uint64_t)orderable(v0) << 32) | (0xFFFFFFFFu - (uint32_t)lane)) : 0;
+    uint64_t k1 = has1 ? (((uint64_t)orderable(v1) << 32) | (0xFFFFFFFFu - (uint32_t)(lane + 64))) : 0;
+    uint64_t best = 0;
+    for (int kk = 0; kk < K; ++kk) {
+      best = wave_max_u64(k0 > k1 ? k0 : k1);
+      if (best == k0) k0 = 0;
+      else if (best == k1) k1 = 0;
+    }
+    const float thr = inv_orderable((uint32_t)(best >> 32));
+    // p = 1 - Phi(z) = erfc(z / sqrt(2)) / 2,  z = (thr - logit) / noise_std.
+    if (has0) acc0 += 0.5f * erfcf((thr - l0) * inv);
+    if (has1) acc1 += 0.5f * erfcf((thr - l1) * inv);
+  }
+  if (load_loss == nullptr) return;
+  psum[wave][lane] = acc0;
+  psum[wave][lane + 64] = acc1;
+  __syncthreads();
+  if (wave == 0) {
+    float p0 = 0.f, p1 = 0.f;
+#pragma unroll
+    for (int w = 0; w < kNoisyWaves; ++w) {
+      p0 += psum[w][lane];
+      p1 += psum[w][lane + 64];
+    }
+    p0 = has0 ? p0 / (float)S : 0.f;
+    p1 = has1 ? p1 / (float)S : 0.f;
+    const float mean = wave_sum_f(p0 + p1) / (float)E;
+    const float d0 = has0 ? p0 - mean : 0.f, d1 = has1 ? p1 - mean : 0.f;
+    const float var = wave_sum_f(d0 * d0 + d1 * d1) / (float)E;
+    if (lane == 0) load_loss[g] = var / (mean * mean);
   }
 }
 
@@ -499,5 +589,17 @@ extern "C" int vmoe_router_metrics(const VmoeRouterMetricsParams* p, vmoe_stream
                        as_stream(stream), (const float*)p->gates, p->top1_idx, p->importance_loss,
                        p->gshard_loss, p->auxiliary_loss, p->gshard_loss_weight,
                        p->importance_loss_weight, p->S, p->E, p->top1_stride, V);
+  return launch_status();
+}
+
+extern "C" int vmoe_noisy_gates(const VmoeNoisyGatesParams* p, vmoe_stream_t stream) {
+  if (p == nullptr || p->logits == nullptr || p->noise == nullptr || p->gates_noisy == nullptr)
+    return VMOE_E_NULL;
+  if (p->G < 1 || p->S < 1 || p->E < 1 || p->K < 1 || p->K > p->E || !(p->noise_std > 0.f))
+    return VMOE_E_SHAPE;
+  if (p->E > 128) return VMOE_E_UNSUPPORTED;
+  hipLaunchKernelGGL(noisy_gates_kernel, dim3(p->G), dim3(kNoisyWaves * 64), 0, as_stream(stream),
+                     p->logits, p->noise, p->gates_noisy, p->load_loss, p->S, p->E, p->K,
+                     p->noise_std);
   return launch_status();
 }

@@ -22,8 +22,10 @@ def _f32(*shape, device):
 
 
 def gate_topk(x: torch.Tensor, w: torch.Tensor, num_selected_experts: int,
-              logit_bias: Optional[torch.Tensor] = None, return_gates: bool = True):
-  """x (G,S,D), w (D,E) -> gates (G,S,E) or None, topk_val (G,S,K) f32, topk_idx (G,S,K) i32."""
+              logit_bias: Optional[torch.Tensor] = None, return_gates: bool = True,
+              return_logits: bool = False):
+  """x (G,S,D), w (D,E) -> gates (G,S,E) or None, topk_val (G,S,K) f32, topk_idx (G,S,K) i32
+  [, logits (G,S,E) f32 with return_logits]."""
   G, S, D = x.shape
   E = w.shape[1]
   K = num_selected_experts
@@ -34,10 +36,30 @@ def gate_topk(x: torch.Tensor, w: torch.Tensor, num_selected_experts: int,
   idx = _i32(G, S, K, device=x.device)
   if logit_bias is not None:
     logit_bias = logit_bias.to(torch.float32).contiguous()
+  logits = _f32(G, S, E, device=x.device) if return_logits else None
   p = H.GateTopkParams(H.ptr(x), H.ptr(w), H.ptr(logit_bias), H.ptr(gates), H.ptr(val), H.ptr(idx),
-                       G * S, D, E, K, H.dtype_code(x.dtype))
+                       G * S, D, E, K, H.dtype_code(x.dtype), H.ptr(logits))
   H.call("vmoe_gate_topk", p)
+  if return_logits:
+    return gates, val, idx, logits
   return gates, val, idx
+
+
+def noisy_gates(logits: torch.Tensor, noise: torch.Tensor, noise_std: float,
+                num_selected_experts: int, return_load_loss: bool = True):
+  """logits, noise (G,S,E) f32 -> softmax(logits + noise_std * noise) (G,S,E) f32 and the
+  load loss per group (G,) f32 (None if not asked for)."""
+  G, S, E = logits.shape
+  logits = logits.to(torch.float32).contiguous()
+  noise = noise.to(torch.float32).contiguous()
+  if noise.shape != logits.shape:
+    raise ValueError(f"noise {tuple(noise.shape)} != logits {tuple(logits.shape)}")
+  gates = torch.empty_like(logits)
+  loss = _f32(G, device=logits.device) if return_load_loss else None
+  p = H.NoisyGatesParams(H.ptr(logits), H.ptr(noise), H.ptr(gates), H.ptr(loss), G, S, E,
+                         num_selected_experts, float(noise_std))
+  H.call("vmoe_noisy_gates", p)
+  return gates, loss
 
 
 def topk(gates: torch.Tensor, k: int):

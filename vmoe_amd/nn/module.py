@@ -58,3 +58,15 @@ def lecun_normal(gen: torch.Generator, shape, fan_in: int, dtype=torch.float32, 
   torch.nn.init.trunc_normal_(t, mean=0.0, std=1.0, a=-2.0, b=2.0, generator=gen)
   t = t * (1.0 / 0.87962566103423978) / (fan_in ** 0.5)
   return t.to(dtype).to(device) if device is not None else t.to(dtype)
+
+
+def make_rngs(rngs, device):
+  """``rngs={'gating': seed or torch.Generator}`` (flax's ``rngs=`` argument of apply)
+  with every seed turned into a generator on ``device``, so that modules that draw
+  one after the other get different numbers.  None stays None."""
+  if rngs is None:
+    return None
+  out = {}
+  for name, rng in rngs.items():
+    out[name] = rng if isinstance(rng, torch.Generator) else generator(rng, device=device)
+  return out

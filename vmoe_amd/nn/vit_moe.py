@@ -123,23 +123,33 @@ class MlpMoeBlock(module.Module):
               deterministic=self.deterministic, name="Mlp")
     return self._router, self._mlp
 
+  @staticmethod
+  def _route(router, variables, x: Array, rngs):
+    """Routers that draw random numbers take them as ``rngs=``; the others are
+    called without (their apply has no such argument)."""
+    if isinstance(router, (routing.NoisyTopExpertsPerItemRouter,
+                           routing.NoisyTopItemsPerExpertRouter)):
+      return router.apply(variables, x, rngs=module.make_rngs(rngs, x.device))
+    return router.apply(variables, x)
+
   def init(self, rng, inputs: Array):
     assert inputs.ndim == 3, f"Expected ndim = 3, but got shape {inputs.shape}"
     router, mlp = self._modules()
     x = inputs.reshape(-1, self.group_size, inputs.shape[-1])
     seed = vmoe_amd.moe._fold_seed(rng, 17)
     router_vars = router.init(seed, x)
-    dispatcher, _ = router.apply(router_vars, x)
+    dispatcher, _ = self._route(router, router_vars, x,
+                                {"gating": vmoe_amd.moe._fold_seed(rng, 29)})
     mlp_vars = mlp.init(vmoe_amd.moe._fold_seed(rng, 23), dispatcher, x)
     return {"params": {"Router": router_vars["params"], "Mlp": mlp_vars["params"]}}
 
-  def apply(self, variables, inputs: Array):
+  def apply(self, variables, inputs: Array, rngs=None):
     assert inputs.ndim == 3, f"Expected ndim = 3, but got shape {inputs.shape}"
     router, mlp = self._modules()
     inputs_shape = inputs.shape
     x = inputs.reshape(-1, self.group_size, inputs.shape[-1])
     params = variables["params"]
-    dispatcher, metrics = router.apply({"params": params["Router"]}, x)
+    dispatcher, metrics = self._route(router, {"params": params["Router"]}, x, rngs)
     outputs = mlp.apply({"params": params["Mlp"]}, dispatcher, x)
     outputs = outputs.reshape(*inputs_shape[:-1], outputs.shape[-1])
     return outputs, metrics
@@ -357,11 +367,12 @@ class EncoderBlock(module.Module):
                        "SelfAttention": attn.init(fold(rng, 1), x)["params"],
                        mlp.name: mlp.init(fold(rng, 2), x)["params"]}}
 
-  def apply(self, variables, inputs: Array):
-    x, y, metrics = self._forward(variables["params"], inputs, None)
+  def apply(self, variables, inputs: Array, rngs=None):
+    x, y, metrics = self._forward(variables["params"], inputs, None,
+                                  module.make_rngs(rngs, inputs.device))
     return x + y if metrics is None else (x + y, metrics)
 
-  def _forward(self, p, residual: Array, pending: Optional[Array]):
+  def _forward(self, p, residual: Array, pending: Optional[Array], rngs=None):
     """The block on ``residual + pending``, the last add left to the caller:
     returns (residual, mlp output not yet added, metrics or None).  Leaving the
     add pending lets it run inside the kernel of the layer norm that follows."""
@@ -370,6 +381,9 @@ class EncoderBlock(module.Module):
     x, a = _add_layer_norm(residual, pending, p["LayerNorm_0"], self.dtype)
     h = attn.apply({"params": p["SelfAttention"]}, a)
     x, y = _add_layer_norm(x, h, p["LayerNorm_1"], self.dtype)
+    if isinstance(mlp, MlpMoeBlock):
+      y, metrics = mlp.apply({"params": p[mlp.name]}, y, rngs=rngs)
+      return x, y, metrics
     y = mlp.apply({"params": p[mlp.name]}, y)
     if isinstance(y, torch.Tensor):
       return x, y, None
@@ -419,8 +433,9 @@ class EncoderMoe(module.Module):
       params[block.name] = block.init(fold(rng, b), x)["params"]
     return {"params": params}
 
-  def apply(self, variables, inputs: Array):
+  def apply(self, variables, inputs: Array, rngs=None):
     assert inputs.ndim == 3, f"Expected ndim = 3, but got shape {inputs.shape}"
+    rngs = module.make_rngs(rngs, inputs.device)
     if not self.deterministic and self.dropout_rate > 0:
       raise NotImplementedError("Dropout (training) is not implemented; use deterministic=True.")
     params = variables["params"]
@@ -428,7 +443,7 @@ class EncoderMoe(module.Module):
     metrics = {}
     pending = None          # output of the previous block's MLP, added by the next layer norm
     for b, block in enumerate(self._blocks()):
-      x, pending, m = block._forward(params[block.name], x, pending)
+      x, pending, m = block._forward(params[block.name], x, pending, rngs)
       if b in self._moe_layers:
         metrics[block.name] = m
     _, encoded = _add_layer_norm(x, pending, params["encoder_norm"], None)
@@ -547,14 +562,14 @@ class VisionTransformerMoe(module.Module):
     return torch.addmm(p["bias"].float(), rows.reshape(-1, rows.shape[-1]),
                        k.float().reshape(-1, k.shape[-1])).view(*rows.shape[:3], k.shape[-1])
 
-  def apply(self, variables, inputs: Array):
+  def apply(self, variables, inputs: Array, rngs=None):
     params = variables["params"]
     x = self._embed(params, inputs)
     grid = x.shape[1:3]
     x = x.reshape(x.shape[0], -1, x.shape[-1])
     if self.classifier == "token":
       x = torch.cat([params["cls"].to(x.dtype).expand(x.shape[0], 1, x.shape[-1]), x], dim=1)
-    x, metrics = self._encoder(grid).apply({"params": params["Encoder"]}, x)
+    x, metrics = self._encoder(grid).apply({"params": params["Encoder"]}, x, rngs=rngs)
     if self.classifier in ("token", "0"):
       x = x[:, 0]
     elif self.classifier == "gap":
