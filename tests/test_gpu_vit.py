@@ -298,3 +298,22 @@ def test_model_bf16_vs_oracle(vit_moe):
   bad_images = (err.max(axis=1) > 2e-2 * (scale + np.abs(want).max(axis=1))).sum()
   assert bad_images <= 1, f"{bad_images} of {len(want)} images outside 2e-2 (scale {scale:.3f})"
   assert np.isfinite(to_np(metrics["auxiliary_loss"])).all()
+
+
+def test_model_from_checkpoint_files(vit_moe, tmp_path):
+  """A dense model's parameters written in the reference's sharded checkpoint format,
+  read back, upcycled (every expert a copy of the dense MLP) and run on the GPU."""
+  from vmoe_amd import checkpoints as C
+  dense_cfg = copy.deepcopy(SMALL)
+  dense_cfg["encoder"].pop("moe")
+  rng = np.random.default_rng(31)
+  images = rng.uniform(-1, 1, (8, 16, 16, 3)).astype(np.float32)
+  dense = V.init_params(rng, images.shape, **dense_cfg)
+  prefix = str(tmp_path / "ckpt_1")
+  C.save_checkpoint(prefix, {"params": dense}, num_shards=3, max_chunk_bytes=4096)
+  restored = C.restore_checkpoint(prefix)["params"]
+  sparse = C.dense_to_moe_params(restored, moe_layers=(1,), num_experts=4)
+  want, _ = V.vision_transformer_moe(images, sparse, **oracle_config(SMALL, O.F32))
+  model = vit_moe.VisionTransformerMoe(**product_config(SMALL, O.F32))
+  got, _ = model.apply({"params": C.to_device(sparse, dev())}, tree_to_dev(images))
+  assert_close(to_np(got), want, 2e-4, "logits from restored parameters")
