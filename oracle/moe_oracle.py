@@ -487,6 +487,46 @@ def noisy_top_experts_per_item_router(
   return dispatcher, metrics, gates
 
 
+def ensemble_router(x, kernel, ensemble_size, num_selected_experts, dispatcher_kwargs,
+                    dtype=F32, gshard_loss_weight=0.0, importance_loss_weight=1.0,
+                    noises=None, noise_std=1.0, load_loss_weight=1.0):
+  """vmoe/nn/ensemble_routing.py:73-134: x (G,S,D) with items ordered (S/M, M), kernel
+  (D, M, E/M).  Member m routes items i*M+m inside experts m*E/M .. (m+1)*E/M - 1; the
+  gating matrix is block diagonal and the losses have shape (G, M).  ``noises`` is a
+  list of M standard normal samples (G, S/M, E/M) for the noisy branch."""
+  if x.ndim != 3:
+    raise ValueError(f"inputs.ndim must be 3, but it is {x.ndim}")
+  G, S, D = x.shape
+  M = ensemble_size
+  _, m2, e_m = kernel.shape
+  E = M * e_m
+  if m2 != M or S % M != 0:
+    raise ValueError("kernel / group size do not match the ensemble size")
+  x4 = x.reshape(G, S // M, M, D)
+  full = None
+  per_member = []
+  for m in range(M):
+    _, metrics_m, gates_m = noisy_top_experts_per_item_router(
+        x4[:, :, m, :], kernel[:, m, :], min(num_selected_experts, e_m),
+        dict(name="indices", capacity=1, batch_priority=False), dtype, gshard_loss_weight,
+        importance_loss_weight,
+        noise=None if noises is None else noises[m], noise_std=noise_std,
+        load_loss_weight=load_loss_weight)
+    if full is None:
+      full = np.zeros((G, S // M, M, M, e_m), gates_m.dtype)
+    full[:, :, m, m, :] = gates_m
+    per_member.append(metrics_m)
+  gates = full.reshape(G, S, E)
+  metrics = {k: np.stack([pm[k] for pm in per_member], axis=1) for k in per_member[0]}
+  kw = dict(dispatcher_kwargs or {})
+  use_bfloat16 = kw.pop("bfloat16", False)
+  dispatcher = get_top_experts_per_item_dispatcher(
+      gates, num_selected_experts=num_selected_experts, **kw)
+  if use_bfloat16:
+    dispatcher = Bfloat16Dispatcher(dispatcher, inner_result_dtype=dtype)
+  return dispatcher, metrics, gates
+
+
 # --------------------------------------------------------------------------- experts
 def gelu(x: np.ndarray, approximate: bool = True) -> np.ndarray:
   """``flax.linen.gelu``: tanh form by default, erf form otherwise (float32)."""

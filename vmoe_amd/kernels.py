@@ -31,6 +31,12 @@ def gate_topk(x: torch.Tensor, w: torch.Tensor, num_selected_experts: int,
   K = num_selected_experts
   x = x.contiguous()
   w = w.to(x.dtype).contiguous()
+  vec = 8 if x.dtype == torch.bfloat16 else 4
+  if D % vec != 0:   # the kernel reads rows in 16-byte pieces: zero columns change nothing
+    pad = vec - D % vec
+    x = torch.nn.functional.pad(x, (0, pad))
+    w = torch.nn.functional.pad(w, (0, 0, 0, pad))
+    D += pad
   gates = torch.empty((G, S, E), dtype=x.dtype, device=x.device) if return_gates else None
   val = _f32(G, S, K, device=x.device)
   idx = _i32(G, S, K, device=x.device)

@@ -6,6 +6,8 @@ from __future__ import annotations
 
 from typing import Any, Dict
 
+import weakref
+
 import torch
 
 
@@ -70,3 +72,38 @@ def make_rngs(rngs, device):
   for name, rng in rngs.items():
     out[name] = rng if isinstance(rng, torch.Generator) else generator(rng, device=device)
   return out
+
+
+class ParamCache:
+  """Derived copies of parameter tensors (casts, packed layouts).
+
+  An entry is valid while the very tensors it was built from are alive and
+  unmodified: they are identified by object (views by their base tensor, offset,
+  shape and strides), held weakly, and their version counters are compared.  An
+  address alone does not identify a tensor: the allocator hands a freed block
+  to the next tensor of that size."""
+
+  def __init__(self, limit: int = 16):
+    self._entries = {}
+    self._limit = limit
+
+  @staticmethod
+  def _ident(t: torch.Tensor):
+    base = t._base if t._base is not None else t
+    return base, (id(base), t.storage_offset(), tuple(t.shape), tuple(t.stride()), t.dtype)
+
+  def get(self, tensors, tag, build):
+    tensors = tuple(tensors)
+    idents = [self._ident(t) for t in tensors]
+    key = (tuple(i[1] for i in idents), tag)
+    versions = tuple(t._version for t in tensors)
+    hit = self._entries.get(key)
+    if hit is not None:
+      refs, vers, value = hit
+      if vers == versions and all(r() is i[0] for r, i in zip(refs, idents)):
+        return value
+    value = build()
+    if len(self._entries) >= self._limit:
+      self._entries.clear()
+    self._entries[key] = (tuple(weakref.ref(i[0]) for i in idents), versions, value)
+    return value

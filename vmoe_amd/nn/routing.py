@@ -47,8 +47,9 @@ class NoisyTopExpertsPerItemRouter(module.Module):
     dispatcher = self._create_dispatcher(gates, topk)
     return dispatcher, metrics
 
-  def _compute_gates_softmax_and_metrics(self, inputs: Array, kernel: Array, rngs=None):
-    num_experts = self.num_experts
+  def _compute_gates_softmax_and_metrics(self, inputs: Array, kernel: Array, rngs=None,
+                                         num_experts: Optional[int] = None):
+    num_experts = self.num_experts if num_experts is None else num_experts
     if inputs.ndim != 3:
       raise ValueError(f"inputs.ndim must be 3, but it is {inputs.ndim}")
     if not num_experts >= self.num_selected_experts >= 1:
@@ -95,12 +96,8 @@ class NoisyTopExpertsPerItemRouter(module.Module):
     done once and reused until the tensor changes."""
     if kernel.dtype == dtype:
       return kernel
-    key = (kernel.data_ptr(), kernel._version, dtype)
-    cached = getattr(self, "_kernel_cache", None)
-    if cached is None or cached[0] != key:
-      cached = (key, K.cast(kernel, dtype))
-      self._kernel_cache = cached
-    return cached[1]
+    cache = self.__dict__.setdefault("_kernel_cache", module.ParamCache())
+    return cache.get((kernel,), dtype, lambda: K.cast(kernel, dtype))
 
   def _create_dispatcher(self, gates_dispatch: Array, topk=None):
     dispatcher_kwargs = dict(**(self.dispatcher or {}))

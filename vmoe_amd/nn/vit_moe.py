@@ -32,7 +32,7 @@ class MlpBlock(module.Module):
 
   def __init__(self, **kwargs):
     super().__init__(**kwargs)
-    self._packed = {}
+    self._packed = module.ParamCache()
 
   def init(self, rng, inputs: Array):
     gen = module.generator(rng)
@@ -50,14 +50,7 @@ class MlpBlock(module.Module):
                        "Dense_1": {"kernel": k1.to(dev), "bias": b1.to(dev)}}}
 
   def _pack(self, w: Array, dtype) -> Array:
-    key = (w.data_ptr(), w._version, tuple(w.shape), dtype)
-    hit = self._packed.get(key)
-    if hit is None:
-      if len(self._packed) > 8:
-        self._packed.clear()
-      hit = K.pack_expert_weights(K.cast(w, dtype))
-      self._packed[key] = hit
-    return hit
+    return self._packed.get((w,), dtype, lambda: K.pack_expert_weights(K.cast(w, dtype)))
 
   def apply_experts(self, variables, inputs: Array) -> Array:
     """inputs (E, R, D) with parameters stacked on axis 0 -> (E, R, D)."""
@@ -220,7 +213,7 @@ class MultiHeadDotProductAttention(module.Module):
 
   def __init__(self, **kwargs):
     super().__init__(**kwargs)
-    self._packed = {}
+    self._packed = module.ParamCache()
 
   def init(self, rng, inputs_q: Array, inputs_kv: Optional[Array] = None):
     gen = module.generator(rng)
@@ -238,24 +231,14 @@ class MultiHeadDotProductAttention(module.Module):
       p["key_ln"] = {"scale": torch.ones((hd,), device=dev)}
     return {"params": p}
 
-  def _cached(self, key, build):
-    hit = self._packed.get(key)
-    if hit is None:
-      if len(self._packed) > 8:
-        self._packed.clear()
-      hit = build()
-      self._packed[key] = hit
-    return hit
-
   def _proj_weights(self, p, names, dtype):
-    key = tuple((p[n]["kernel"].data_ptr(), p[n]["kernel"]._version,
-                 p[n]["bias"].data_ptr(), p[n]["bias"]._version) for n in names) + (dtype,)
-
+    """(sum of H * hd, D) weight and bias of the named input projections, packed once."""
     def build():
       w = torch.cat([p[n]["kernel"].reshape(p[n]["kernel"].shape[0], -1).t() for n in names])
       b = torch.cat([p[n]["bias"].reshape(-1) for n in names])
       return w.to(dtype).contiguous(), b.to(dtype).contiguous()
-    return self._cached(key, build)
+    tensors = [p[n][leaf] for n in names for leaf in ("kernel", "bias")]
+    return self._packed.get(tensors, (dtype, names), build)
 
   def apply(self, variables, inputs_q: Array, inputs_kv: Optional[Array] = None) -> Array:
     p = variables["params"]
@@ -287,11 +270,10 @@ class MultiHeadDotProductAttention(module.Module):
       ctx = torch.nn.functional.scaled_dot_product_attention(
           q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2))     # (B, H, Sq, hd)
       ctx = ctx.transpose(1, 2).reshape(B, Sq, H * hd)
-    key = (p["out"]["kernel"].data_ptr(), p["out"]["kernel"]._version,
-           p["out"]["bias"].data_ptr(), p["out"]["bias"]._version, dtype, "out")
-    wo, bo = self._cached(key, lambda: (
-        p["out"]["kernel"].reshape(H * hd, -1).t().to(dtype).contiguous(),
-        p["out"]["bias"].to(dtype)))
+    wo, bo = self._packed.get(
+        (p["out"]["kernel"], p["out"]["bias"]), (dtype, "out"),
+        lambda: (p["out"]["kernel"].reshape(H * hd, -1).t().to(dtype).contiguous(),
+                 p["out"]["bias"].to(dtype)))
     return linear(ctx, wo, bo)
 
 
