@@ -288,10 +288,16 @@ def test_expert_mlp_erf_gelu_and_no_bias(K):
 # ------------------------------------------------------------------ error handling
 def test_bad_arguments_return_error_codes(K):
   from vmoe_amd import _hip as H
-  x = torch.zeros((1, 4, 12), dtype=torch.bfloat16, device=dev())    # D % 8 != 0
-  w = torch.zeros((12, 4), dtype=torch.bfloat16, device=dev())
-  with pytest.raises(H.VmoeError, match="aligned"):
-    K.gate_topk(x, w, 2)
+  x = torch.randn((1, 4, 12), device=dev()).to(torch.bfloat16)       # D % 8 != 0
+  w = torch.randn((12, 4), device=dev()).to(torch.bfloat16)
+  val = torch.empty((4, 2), dtype=torch.float32, device=dev())
+  idx = torch.empty((4, 2), dtype=torch.int32, device=dev())
+  with pytest.raises(H.VmoeError, match="aligned"):                  # the C ABI refuses the width
+    H.call("vmoe_gate_topk", H.GateTopkParams(H.ptr(x), H.ptr(w), None, None, H.ptr(val),
+                                              H.ptr(idx), 4, 12, 4, 2, H.BF16, None))
+  gates, _, _ = K.gate_topk(x, w, 2)                                 # the wrapper pads with zeros
+  want = torch.softmax((x.float() @ w.float()).to(torch.bfloat16).float(), -1)
+  np.testing.assert_allclose(to_np(gates), to_np(want), rtol=1e-2, atol=1e-3)
   x = torch.zeros((1, 4, 16), dtype=torch.float32, device=dev())
   w = torch.zeros((16, 4), dtype=torch.float32, device=dev())
   with pytest.raises(H.VmoeError, match="invalid sizes"):

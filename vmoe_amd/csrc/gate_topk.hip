@@ -60,7 +60,7 @@ template <typename T> __host__ __device__ constexpr int w_stride(int kc, int epa
   return sizeof(T) == 2 ? kc + 8 : epad;
 }
 
-template <typename T, int NT>
+template <typename T, int NT, bool LOGITS>
 __global__ __launch_bounds__(kGateThreads) void gate_topk_kernel(
     const T* __restrict__ x, const T* __restrict__ w, const float* __restrict__ bias,
     T* __restrict__ gates, float* __restrict__ logits, float* __restrict__ topk_val,
@@ -228,7 +228,7 @@ __global__ __launch_bounds__(kGateThreads) void gate_topk_kernel(
       g[j] = (n0 + j < E) ? v : -INFINITY;
       mx = fmaxf(mx, g[j]);
     }
-    if (logits != nullptr && row < num_items) {
+    if (LOGITS && row < num_items) {
 #pragma unroll
       for (int j = 0; j < CNT; ++j)
         if (n0 + j < E) logits[(size_t)row * E + n0 + j] = g[j];
@@ -442,10 +442,19 @@ int launch_gate(const VmoeGateTopkParams* p, hipStream_t stream) {
                        (int)w_bytes);
     return launch_status();
   };
+  // The logits output is a separate instantiation: its extra live pointer costs
+  // the common one a wave of occupancy.
+  if (p->logits != nullptr) {
+    switch (nt) {
+      case 1: return run(gate_topk_kernel<T, 1, true>);
+      case 2: return run(gate_topk_kernel<T, 2, true>);
+      default: return run(gate_topk_kernel<T, 4, true>);
+    }
+  }
   switch (nt) {
-    case 1: return run(gate_topk_kernel<T, 1>);
-    case 2: return run(gate_topk_kernel<T, 2>);
-    default: return run(gate_topk_kernel<T, 4>);
+    case 1: return run(gate_topk_kernel<T, 1, false>);
+    case 2: return run(gate_topk_kernel<T, 2, false>);
+    default: return run(gate_topk_kernel<T, 4, false>);
   }
 }
 
