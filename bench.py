@@ -20,6 +20,13 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 if ROOT not in sys.path:
   sys.path.insert(0, ROOT)
 
+# Steps run before the warm-up so that no one-time initialisation (first launches,
+# memory pools, event objects) falls into the warm-up or the timed steps.
+INIT_STEPS = 10
+# Entry-point calls of one layer step, rounded up: their timing events are created
+# before the timed region, which then only records them.
+CALLS_PER_STEP = 12
+
 # Published MI355X peaks used as roofline denominators.
 PEAK_BF16_TFLOPS = 2500.0
 PEAK_FP32_MATRIX_TFLOPS = 157.3
@@ -119,10 +126,11 @@ def soft_main(args):
     dispatcher, metrics = layer.apply(rvars, xs[i % 4])
     return mlp.apply(mvars, dispatcher, xs[i % 4])
 
-  for i in range(args.warmup):
+  _hip.set_timing_sink({})
+  for i in range(INIT_STEPS + args.warmup):
     step(i)
   torch.cuda.synchronize()
-  sink = {}
+  sink = _hip.TimingSink(pairs=args.steps * CALLS_PER_STEP)
   _hip.set_timing_sink(sink)
   t0 = time.perf_counter()
   for i in range(args.steps):
@@ -179,12 +187,13 @@ def vit_main(args):
     fn = getattr(cls, method)
 
     def wrapper(self, *a, **kw):
-      e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+      if not spans.get("on"):
+        return fn(self, *a, **kw)
+      e0, e1 = spans["pool"].take()
       e0.record()
       out = fn(self, *a, **kw)
       e1.record()
-      if spans.get("on"):
-        spans.setdefault(label, []).append((e0, e1))
+      spans.setdefault(label, []).append((e0, e1))
       return out
     setattr(cls, method, wrapper)
 
@@ -195,10 +204,12 @@ def vit_main(args):
   def step(i):
     return model.apply(variables, images[i % 2])
 
-  for i in range(args.warmup):
+  _hip.set_timing_sink({})
+  for i in range(3 + args.warmup):
     step(i)
   torch.cuda.synchronize()
-  sink = {}
+  sink = _hip.TimingSink(pairs=args.steps * 120)     # about 110 entry-point calls per pass
+  spans["pool"] = _hip.TimingSink(pairs=args.steps * 24)
   _hip.set_timing_sink(sink)
   spans["on"] = True
   t0 = time.perf_counter()
@@ -208,6 +219,7 @@ def vit_main(args):
   t1 = time.perf_counter()
   _hip.set_timing_sink(None)
   spans.pop("on")
+  spans.pop("pool")
   ms = (t1 - t0) * 1e3 / args.steps
   module_ms = {k: float(sum(a.elapsed_time(b) for a, b in v)) / args.steps for k, v in spans.items()}
   module_ms["other (patch embedding, layer norms, residuals, head)"] = ms - sum(module_ms.values())
@@ -222,8 +234,23 @@ def vit_main(args):
   moe_cfg = enc["moe"]
   n_moe = len(moe_cfg["layers"])
   n_dense = enc["num_layers"] - n_moe
-  kept = T * moe_cfg["router"]["num_selected_experts"]       # upper bound: nothing dropped
-  flops_mlp = 2 * 2.0 * D * M * (n_dense * T + n_moe * kept)
+  # Rows the expert MLPs really compute: the kept assignments of every MoE block
+  # (dropped ones are skipped), read from one more, untimed, pass.
+  from vmoe_amd import moe as moe_lib
+  live_rows = []
+  packed = moe_lib.ExpertIndicesDispatcher.dispatch_packed
+
+  def recording(self, data):
+    out, rows = packed(self, data)
+    live_rows.append(rows)
+    return out, rows
+  moe_lib.ExpertIndicesDispatcher.dispatch_packed = recording
+  step(0)
+  torch.cuda.synchronize()
+  moe_lib.ExpertIndicesDispatcher.dispatch_packed = packed
+  kept_per_block = [int(r.sum()) for r in live_rows]
+  assert len(kept_per_block) == n_moe
+  flops_mlp = 2 * 2.0 * D * M * (n_dense * T + sum(kept_per_block))
   mlp_ms = stage_ms["vmoe_expert_mlp"]
   achieved = flops_mlp / (mlp_ms * 1e-3) / 1e12
   # Whole-model matrix flops per image (projections, attention, MLPs), for scale.
@@ -243,7 +270,8 @@ def vit_main(args):
       "roofline": {"bound": "mfma", "kernel": "gemm_bf16_kernel", "achieved": achieved,
                    "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": achieved / PEAK_BF16_TFLOPS,
                    "traffic": None, "launch_ms": mlp_ms / (2 * enc["num_layers"]),
-                   "flops_all_mlps": flops_mlp},
+                   "flops_all_mlps": flops_mlp, "kept_rows_per_moe_block": kept_per_block,
+                   "assignments_per_moe_block": T * moe_cfg["router"]["num_selected_experts"]},
       "model_TFLOPs_per_step": flops_total / 1e12,
       "model_TFLOPs_per_s": flops_total / (ms * 1e-3) / 1e12,
       "moe_ms": module_ms.get("moe_layers"), "module_ms": module_ms, "stage_ms": stage_ms,
@@ -322,11 +350,17 @@ def main():
   def step(i):
     return layer.apply(variables, xs[i % n_rot])
 
+  # Untimed: one-time costs (code objects, allocator pools, timing events) and
+  # then the W warm-up steps, run exactly as the timed steps are.
+  _hip.set_timing_sink({})
+  for i in range(INIT_STEPS):
+    out, metrics = step(i)
+  torch.cuda.synchronize()
   for i in range(args.warmup):
     out, metrics = step(i)
   torch.cuda.synchronize()
 
-  sink = {}
+  sink = _hip.TimingSink(pairs=args.steps * CALLS_PER_STEP)
   _hip.set_timing_sink(sink)
   torch.cuda.synchronize()
   t0 = time.perf_counter()

@@ -184,6 +184,23 @@ typedef struct {
 } VmoeIndicesToSlotsParams;
 int vmoe_indices_to_slots(const VmoeIndicesToSlotsParams* p, vmoe_stream_t stream);
 
+/* Packed ("ragged") expert buffers.  The reference's buffer gives every (group, expert)
+ * pair C rows whether or not items fill them (vmoe/moe.py:190-197); the expert MLP then
+ * also runs over the empty rows.  This call renumbers the kept assignments so that
+ * expert e's items occupy rows 0 .. rows_per_expert[e]-1 of its (G*C)-row block, groups
+ * in order: token_row = e*G*C + sum_{g' < g} fill[g'][e] + position.  dispatch (with
+ * slot_token null), the expert MLP (rows_per_expert) and combine take token_row in
+ * place of token_slot; the layer's output is unchanged. */
+typedef struct {
+  const int32_t* fill;        /* (G, E) from vmoe_route_assign */
+  const int32_t* token_slot;  /* (G, S, K) from vmoe_route_assign */
+  int32_t* token_row;         /* out (G, S, K), -1 for dropped assignments */
+  int32_t* rows_per_expert;   /* out (E,) */
+  int32_t* prefix;            /* scratch (G, E): rows of expert e taken by the groups before g */
+  int32_t G, S, E, K, C;
+} VmoeCompactRowsParams;
+int vmoe_compact_rows(const VmoeCompactRowsParams* p, vmoe_stream_t stream);
+
 /* ------------------------------------------------------------------ dispatch / combine
  * dispatch replaces ExpertIndicesDispatcher.dispatch (vmoe/moe.py:190-197:
  * repeat + scatter_nd into zeros + _dispatch layout): out[slot] = x[item] for
@@ -192,11 +209,13 @@ int vmoe_indices_to_slots(const VmoeIndicesToSlotsParams* p, vmoe_stream_t strea
  * out[item] = sum_k weights[item,k] * (slot >= 0 ? y[slot] : 0), products and
  * sums in float32 in k order, rounded once to dtype.
  * Row width D*sizeof(dtype) must be a multiple of 16 bytes.
+ * With slot_token null, dispatch leaves unclaimed slot rows untouched instead of
+ * zeroing them (for the packed layout of vmoe_compact_rows, where no one reads them).
  */
 typedef struct {
   const void* x;             /* (num_items, D) dtype */
   const int32_t* token_slot; /* (num_items, K) */
-  const int32_t* slot_token; /* (num_slots,) */
+  const int32_t* slot_token; /* (num_slots,) or null */
   void* out;                 /* (num_slots, D) dtype */
   int32_t num_items, num_slots, K, D;
   int32_t dtype;
@@ -251,6 +270,9 @@ typedef struct {
   int32_t E, R, D, M;
   int32_t dtype;
   int32_t gelu;     /* VMOE_GELU_TANH (flax default) or VMOE_GELU_ERF */
+  const int32_t* rows_per_expert; /* optional (E,): only the first rows_per_expert[e] rows of
+                                     expert e hold data; the other rows of x are not read
+                                     for results and their rows of out are left untouched */
 } VmoeExpertMlpParams;
 size_t vmoe_expert_mlp_workspace_bytes(const VmoeExpertMlpParams* p);
 int vmoe_expert_mlp(const VmoeExpertMlpParams* p, vmoe_stream_t stream);

@@ -66,7 +66,8 @@ def test_struct_layouts_match_header():
         "VmoeTopItemsParams": _hip.TopItemsParams,
         "VmoeAddLayerNormParams": _hip.AddLayerNormParams,
         "VmoeAttentionParams": _hip.AttentionParams,
-        "VmoeNoisyGatesParams": _hip.NoisyGatesParams}
+        "VmoeNoisyGatesParams": _hip.NoisyGatesParams,
+        "VmoeCompactRowsParams": _hip.CompactRowsParams}
   assert set(py) == set(structs)
   for name, body in structs.items():
     want = []

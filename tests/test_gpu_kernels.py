@@ -394,3 +394,53 @@ def test_einsum_golden_and_bool_weights(K, goldens):
     np.testing.assert_array_almost_equal(to_np(buf).reshape(E, 2 * C, 4), np.asarray(g["expected_dispatch"]))
     out = K.einsum_combine(to_dev(cw), buf, torch.float32)
     np.testing.assert_array_almost_equal(to_np(out), np.asarray(g["expected_combine"]))
+
+
+# ------------------------------------------------------------------ packed expert rows
+@pytest.mark.parametrize("G,S,E,Kk,C,bpr", [(4, 64, 4, 2, 20, True), (8, 50, 8, 2, 16, False),
+                                            (3, 33, 5, 1, 8, True), (300, 16, 4, 2, 6, False)])
+def test_compact_rows(K, G, S, E, Kk, C, bpr):
+  """token_row = e*G*C + (kept items of expert e in the groups before g) + position."""
+  rng = np.random.default_rng(G * S + E)
+  gates = O.softmax(rng.standard_normal((G, S, E)).astype(np.float32) * 2)
+  val, idx = K.topk(to_dev(gates), Kk)
+  indices, token_slot, slot_token, fill = K.route_assign(val, idx, E, C, bpr)
+  token_row, rows = K.compact_rows(fill, token_slot, C)
+  f = to_np(fill)
+  np.testing.assert_array_equal(to_np(rows), f.sum(0))
+  ind = to_np(indices)
+  prefix = np.cumsum(f, axis=0) - f                         # (G, E)
+  e, pos = ind[..., 0], ind[..., 1]
+  kept = pos < C
+  want = np.where(kept, e * (G * C) + np.take_along_axis(
+      prefix[:, None, :].repeat(S, 1), e, axis=2) + pos, -1)
+  np.testing.assert_array_equal(to_np(token_row), want)
+  # a bijection onto the first rows of every expert
+  r = to_np(token_row)[kept]
+  assert len(np.unique(r)) == r.size
+  for ee in range(E):
+    mine = r[(r // (G * C)) == ee] - ee * G * C
+    assert sorted(mine) == list(range(f.sum(0)[ee]))
+
+
+@pytest.mark.parametrize("dtype", [O.F32, O.BF16])
+@pytest.mark.parametrize("E", [5, 20])      # planned launch (few experts per die) / static order
+def test_expert_mlp_rows_per_expert(K, dtype, E):
+  """Leading rows equal the full computation bit for bit; the other rows are not written."""
+  rng = np.random.default_rng(3)
+  R, D, M = 300, 64, 128
+  x = to_dev(O.cast(rng.standard_normal((E, R, D)).astype(np.float32), dtype), dtype)
+  w0 = to_dev(O.cast(rng.standard_normal((E, D, M)).astype(np.float32) / 8, dtype), dtype)
+  w1 = to_dev(O.cast(rng.standard_normal((E, M, D)).astype(np.float32) / 11, dtype), dtype)
+  b0 = to_dev(O.cast(rng.standard_normal((E, M)).astype(np.float32) * 0.1, dtype), dtype)
+  b1 = to_dev(O.cast(rng.standard_normal((E, D)).astype(np.float32) * 0.1, dtype), dtype)
+  full = K.expert_mlp(x, w0, b0, w1, b1)
+  rows = np.asarray(([300, 0, 1, 129, 256] * 4)[:E], np.int32)
+  out = torch.full_like(full, 7.0)
+  x_bad = x.clone()
+  for e, n in enumerate(rows):
+    x_bad[e, n:] = float("nan")                      # rows past the count must not matter
+  K.expert_mlp(x_bad, w0, b0, w1, b1, out=out, rows_per_expert=to_dev(rows))
+  for e, n in enumerate(rows):
+    np.testing.assert_array_equal(to_np(out[e, :n]), to_np(full[e, :n]))
+    assert (to_np(out[e, n:]) == 7.0).all()

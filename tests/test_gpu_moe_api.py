@@ -647,3 +647,37 @@ def test_layer_configs_vs_oracle(name):
   if name.startswith("vmoe_l16"):
     # capacity factor 0.5: at least half of the assignments are dropped -> many all-zero rows
     assert (np.abs(got).max(-1) == 0).mean() > 0.1
+
+
+@pytest.mark.parametrize("dtype,bf16_dispatcher", [(O.F32, False), (O.BF16, False), (O.F32, True)])
+@pytest.mark.parametrize("name", ["indices", "einsum"])
+def test_packed_rows_path_equals_reference_layout(moe, dtype, bf16_dispatcher, name):
+  """sparse_moe_spmd packs each expert's items into its first rows and lets the MLP skip
+  the rest; the result equals dispatch -> experts over all rows -> combine bit for bit."""
+  from vmoe_amd.nn import routing, vit_moe
+  rng = np.random.default_rng(17)
+  G, S, D, M, E, K = 4, 96, 64, 128, 8, 2
+  x = to_dev(O.cast(rng.standard_normal((G, S, D)).astype(np.float32), dtype), dtype)
+  router = routing.NoisyTopExpertsPerItemRouter(
+      num_experts=E, num_selected_experts=K, deterministic=True,
+      dispatcher=dict(name=name, capacity_factor=0.75, batch_priority=True,
+                      bfloat16=bf16_dispatcher))
+  rvars = {"params": {"dense": {"kernel": to_dev(
+      rng.standard_normal((D, E)).astype(np.float32) / 8)}}}
+  dispatcher, _ = router.apply(rvars, x)
+  assert dispatcher.supports_packed()
+  mlp = moe.sparse_moe_spmd(vit_moe.MlpBlock, variable_axes={"params": 0})(
+      mlp_dim=M, dtype=tdtype(dtype))
+  mvars = {"params": {
+      "Dense_0": {"kernel": to_dev(rng.standard_normal((E, D, M)).astype(np.float32) / 8),
+                  "bias": to_dev(rng.standard_normal((E, M)).astype(np.float32) * 0.1)},
+      "Dense_1": {"kernel": to_dev(rng.standard_normal((E, M, D)).astype(np.float32) / 11),
+                  "bias": to_dev(rng.standard_normal((E, D)).astype(np.float32) * 0.1)}}}
+  got = mlp.apply(mvars, dispatcher, x)
+  want = dispatcher.combine(mlp.expert.apply_experts(mvars, dispatcher.dispatch(x)))
+  np.testing.assert_array_equal(to_np(got), to_np(want))
+  buf, rows = dispatcher.dispatch_packed(x)
+  inner = dispatcher.dispatcher if bf16_dispatcher else dispatcher
+  fill = getattr(inner, "_inner", inner).fill
+  np.testing.assert_array_equal(to_np(rows), to_np(fill).sum(0))
+  assert int(rows.sum()) < E * G * buf.shape[1] // G          # capacity 0.75: some slots stay empty

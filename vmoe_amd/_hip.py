@@ -25,7 +25,7 @@ EXPORTS = [
     "vmoe_expert_mlp_workspace_bytes", "vmoe_expert_mlp", "vmoe_pack_expert_weights",
     "vmoe_soft_route_workspace_bytes", "vmoe_soft_route", "vmoe_einsum_dispatch",
     "vmoe_einsum_combine", "vmoe_cast", "vmoe_copy_bytes", "vmoe_mfma_probe",
-    "vmoe_add_layer_norm", "vmoe_attention", "vmoe_noisy_gates",
+    "vmoe_add_layer_norm", "vmoe_attention", "vmoe_noisy_gates", "vmoe_compact_rows",
 ]
 
 
@@ -150,7 +150,13 @@ class ExpertMlpParams(ctypes.Structure):
               ("b1", c_void_p), ("w0t", c_void_p), ("w1t", c_void_p), ("out", c_void_p),
               ("workspace", c_void_p), ("workspace_bytes", c_size_t),
               ("E", c_int32), ("R", c_int32), ("D", c_int32), ("M", c_int32),
-              ("dtype", c_int32), ("gelu", c_int32)]
+              ("dtype", c_int32), ("gelu", c_int32), ("rows_per_expert", c_void_p)]
+
+
+class CompactRowsParams(ctypes.Structure):
+  _fields_ = [("fill", c_void_p), ("token_slot", c_void_p), ("token_row", c_void_p),
+              ("rows_per_expert", c_void_p), ("prefix", c_void_p), ("G", c_int32), ("S", c_int32),
+              ("E", c_int32), ("K", c_int32), ("C", c_int32)]
 
 
 class TransposeParams(ctypes.Structure):
@@ -195,9 +201,32 @@ class AttentionParams(ctypes.Structure):
 _timing_sink = None
 
 
+class TimingSink(dict):
+  """``sink[name]`` -> list of (start, stop) event pairs, one per call of entry point
+  ``name``.  Creating a timing event costs the host far more than recording one, so
+  ``pairs`` of them are created (and recorded once, which is when the runtime really
+  allocates them) up front; a measured loop then only records."""
+
+  def __init__(self, pairs: int = 0):
+    super().__init__()
+    self._pool = []
+    for _ in range(pairs):
+      pair = (torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
+      pair[0].record()
+      pair[1].record()
+      self._pool.append(pair)
+    if pairs:
+      torch.cuda.synchronize()
+
+  def take(self):
+    if self._pool:
+      return self._pool.pop()
+    return torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+
+
 def set_timing_sink(sink) -> None:
-  """With a dict as sink, every entry point is bracketed by a pair of timing
-  events on the stream it is launched on; the pairs are appended to
+  """With a dict (or a TimingSink) as sink, every entry point is bracketed by a pair
+  of timing events on the stream it is launched on; the pairs are appended to
   ``sink[name]`` for the caller to read after synchronising.  None disables."""
   global _timing_sink
   _timing_sink = sink
@@ -209,8 +238,9 @@ def call(name: str, params: ctypes.Structure) -> None:
   if sink is None:
     check(fn(ctypes.byref(params), stream()), name)
     return
-  start = torch.cuda.Event(enable_timing=True)
-  stop = torch.cuda.Event(enable_timing=True)
+  take = getattr(sink, "take", None)
+  start, stop = take() if take is not None else (
+      torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
   start.record()
   code = fn(ctypes.byref(params), stream())
   stop.record()

@@ -279,19 +279,20 @@ static uint32_t chunk_magic(int cpr) {
 }
 
 extern "C" int vmoe_dispatch(const VmoeDispatchParams* p, vmoe_stream_t stream) {
-  if (p == nullptr || p->token_slot == nullptr || p->slot_token == nullptr) return VMOE_E_NULL;
+  if (p == nullptr || p->token_slot == nullptr) return VMOE_E_NULL;
   int rc = check_move(p->x, p->token_slot, p->out, p->num_items, p->num_slots, p->K, p->D, p->dtype);
   if (rc != VMOE_OK) return rc;
   const int cpr = (int)((size_t)p->D * (p->dtype == VMOE_BF16 ? 2 : 4) / 16);
+  const bool zero_fill = p->slot_token != nullptr;
   if (p->K <= kMaxK && kRowsPerBlock * cpr < 65536) {
     const int item_blocks = (p->num_items + kRowsPerBlock - 1) / kRowsPerBlock;
-    const int zero_blocks = (p->num_slots + kRowsPerBlock - 1) / kRowsPerBlock;
+    const int zero_blocks = zero_fill ? (p->num_slots + kRowsPerBlock - 1) / kRowsPerBlock : 0;
     hipLaunchKernelGGL(dispatch_kernel, dim3(item_blocks + zero_blocks), dim3(kMoveThreads), 0,
                        as_stream(stream), (const uint4*)p->x, p->token_slot, p->slot_token,
                        (uint4*)p->out, p->num_items, p->num_slots, p->K, cpr, chunk_magic(cpr),
                        item_blocks);
   } else {
-    const long long waves = (long long)p->num_items + p->num_slots;
+    const long long waves = (long long)p->num_items + (zero_fill ? p->num_slots : 0);
     const long long blocks = (waves + 3) / 4;
     if (blocks > 0x7fffffffLL) return VMOE_E_OVERFLOW;
     hipLaunchKernelGGL(dispatch_generic_kernel, dim3((unsigned)blocks), dim3(kMoveThreads), 0,

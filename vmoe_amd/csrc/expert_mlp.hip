@@ -19,7 +19,8 @@ constexpr int kF32Tile = 64, kF32BK = 16;
 template <int EPI>
 __global__ __launch_bounds__(256) void gemm_f32_kernel(
     const float* __restrict__ A, const float* __restrict__ B, const float* __restrict__ bias,
-    float* __restrict__ C, int R, int N, int Kd, int tiles_m, int tiles_n) {
+    float* __restrict__ C, int R, int N, int Kd, int tiles_m, int tiles_n,
+    const int32_t* __restrict__ rows) {
   __shared__ float sa[kF32Tile][kF32BK + 1];
   __shared__ float sb[kF32BK][kF32Tile + 4];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -30,6 +31,11 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(
   const int rem = blockIdx.x - b * per_batch;
   const int tile_n = rem / tiles_m, tile_m = rem - tile_n * tiles_m;
   const int row0 = tile_m * kF32Tile, col0 = tile_n * kF32Tile;
+  int live = R;               // ragged batches: only rows[b] rows of batch b hold data
+  if (rows != nullptr) {
+    live = min(rows[b], R);
+    if (row0 >= live) return;
+  }
   const float* Ab = A + (size_t)b * R * Kd;
   const float* Bb = B + (size_t)b * Kd * N;
   floatx16 acc;
@@ -68,18 +74,18 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(
     float o = acc[v] + bv;
     if (EPI == kEpiBiasGeluTanh) o = gelu_tanh(o);
     if (EPI == kEpiBiasGeluErf) o = gelu_erf(o);
-    if (row < R && col_ok) Cb[(size_t)row * N + col] = o;
+    if (row < live && col_ok) Cb[(size_t)row * N + col] = o;
   }
 }
 
 template <int EPI>
 int launch_gemm_f32(const float* A, const float* B, const float* bias, float* C, int batch, int R,
-                    int N, int Kd, hipStream_t stream) {
+                    int N, int Kd, hipStream_t stream, const int32_t* rows = nullptr) {
   const int tiles_m = (R + kF32Tile - 1) / kF32Tile, tiles_n = (N + kF32Tile - 1) / kF32Tile;
   const long long blocks = (long long)batch * tiles_m * tiles_n;
   if (blocks > 0x7fffffffLL) return VMOE_E_OVERFLOW;
   hipLaunchKernelGGL(gemm_f32_kernel<EPI>, dim3((unsigned)blocks), dim3(256), 0, stream, A, B, bias,
-                     C, R, N, Kd, tiles_m, tiles_n);
+                     C, R, N, Kd, tiles_m, tiles_n, rows);
   return launch_status();
 }
 
@@ -169,6 +175,33 @@ __global__ __launch_bounds__(256) void mfma_probe_kernel(const uint4* __restrict
 
 size_t align256(size_t v) { return (v + 255) / 256 * 256; }
 
+// Launch plans of the two ragged products of an MLP: geometry, bytes, one planning launch.
+struct MlpPlans {
+  GemmGeom up, down;
+  size_t up_bytes = 0, down_bytes = 0;   // 0: that product keeps the static tile order
+};
+
+MlpPlans mlp_plans(int E, int R, int D, int M) {
+  MlpPlans m;
+  m.up = gemm_geometry<CfgUp>(E, R, M, D);
+  m.down = gemm_geometry<CfgDown>(E, R, D, M);
+  // With many experts per die the static order (whole experts per die, tiles past an
+  // expert's rows leaving at once) is already balanced and measured 2 % faster than a
+  // planned launch, whose workgroups start with a dependent load; with one or two
+  // experts per die the fullest expert would set the time, and the plan wins by far
+  // (a third off the MoE blocks of the B/16 model with 8 experts).
+  const bool few_per_die = E <= 2 * kNumXcd;
+  auto bytes = [&](const GemmGeom& g) -> size_t {
+    if (!few_per_die || !g.fast || g.ragged_slots * kNumXcd > 0x7ffffff0LL ||
+        (size_t)(E + 1) * 8 > 60000)
+      return 0;
+    return align256((size_t)g.ragged_slots * kNumXcd * sizeof(int4));
+  };
+  m.up_bytes = bytes(m.up);
+  m.down_bytes = bytes(m.down);
+  return m;
+}
+
 }  // namespace
 }  // namespace vmoe
 
@@ -196,6 +229,10 @@ extern "C" size_t vmoe_expert_mlp_workspace_bytes(const VmoeExpertMlpParams* p) 
   if (p == nullptr || p->E < 1 || p->R < 1 || p->D < 1 || p->M < 1) return 0;
   const size_t b = p->dtype == VMOE_BF16 ? 2 : 4;
   size_t bytes = align256((size_t)p->E * p->R * p->M * b);  // hidden activations
+  if (p->dtype == VMOE_BF16 && p->rows_per_expert != nullptr) {   // launch plans of the ragged products
+    const MlpPlans m = mlp_plans(p->E, p->R, p->D, p->M);
+    bytes += m.up_bytes + m.down_bytes;
+  }
   if (p->dtype == VMOE_BF16) {
     if (p->w0t == nullptr) bytes += align256((size_t)p->E * p->D * p->M * b);
     if (p->w1t == nullptr) bytes += align256((size_t)p->E * p->D * p->M * b);
@@ -214,6 +251,24 @@ extern "C" int vmoe_expert_mlp(const VmoeExpertMlpParams* p, vmoe_stream_t strea
   const size_t b = p->dtype == VMOE_BF16 ? 2 : 4;
   void* hidden = ws;
   ws += align256((size_t)p->E * p->R * p->M * b);
+  int4* plan_up = nullptr;
+  int4* plan_down = nullptr;
+  if (p->dtype == VMOE_BF16 && p->rows_per_expert != nullptr) {
+    const MlpPlans m = mlp_plans(p->E, p->R, p->D, p->M);
+    if (m.up_bytes) plan_up = reinterpret_cast<int4*>(ws);
+    ws += m.up_bytes;
+    if (m.down_bytes) plan_down = reinterpret_cast<int4*>(ws);
+    ws += m.down_bytes;
+    if (plan_up != nullptr || plan_down != nullptr) {
+      const RaggedGeom ga{CfgUp::BM, m.up.tiles_n, m.up.panel_rows,
+                          plan_up ? (int)(m.up.ragged_slots * kNumXcd) : 0, plan_up};
+      const RaggedGeom gb{CfgDown::BM, m.down.tiles_n, m.down.panel_rows,
+                          plan_down ? (int)(m.down.ragged_slots * kNumXcd) : 0, plan_down};
+      const int n = ga.num_blocks > gb.num_blocks ? ga.num_blocks : gb.num_blocks;
+      hipLaunchKernelGGL(plan_ragged_tiles_kernel, dim3((n + 255) / 256), dim3(256),
+                         (size_t)(p->E + 1) * 8, stream, p->rows_per_expert, p->E, p->R, ga, gb);
+    }
+  }
   const bool tanh_gelu = p->gelu == VMOE_GELU_TANH;
   if (p->dtype == VMOE_BF16) {
     const void* w0t = p->w0t;
@@ -232,27 +287,30 @@ extern "C" int vmoe_expert_mlp(const VmoeExpertMlpParams* p, vmoe_stream_t strea
     if (tanh_gelu)
       rc = launch_gemm_bf16<CfgUp, kEpiBiasGeluTanh>((const bf16_t*)p->x, (const bf16_t*)w0t,
                                                       (const bf16_t*)p->b0, (bf16_t*)hidden, p->E,
-                                                      p->R, p->M, p->D, stream);
+                                                      p->R, p->M, p->D, stream, p->rows_per_expert,
+                                                      plan_up);
     else
       rc = launch_gemm_bf16<CfgUp, kEpiBiasGeluErf>((const bf16_t*)p->x, (const bf16_t*)w0t,
                                                      (const bf16_t*)p->b0, (bf16_t*)hidden, p->E,
-                                                     p->R, p->M, p->D, stream);
+                                                     p->R, p->M, p->D, stream, p->rows_per_expert,
+                                                     plan_up);
     if (rc != VMOE_OK) return rc;
     return launch_gemm_bf16<CfgDown, kEpiBias>((const bf16_t*)hidden, (const bf16_t*)w1t,
                                               (const bf16_t*)p->b1, (bf16_t*)p->out, p->E, p->R,
-                                              p->D, p->M, stream);
+                                              p->D, p->M, stream, p->rows_per_expert, plan_down);
   }
   if (tanh_gelu)
     rc = launch_gemm_f32<kEpiBiasGeluTanh>((const float*)p->x, (const float*)p->w0,
                                            (const float*)p->b0, (float*)hidden, p->E, p->R, p->M,
-                                           p->D, stream);
+                                           p->D, stream, p->rows_per_expert);
   else
     rc = launch_gemm_f32<kEpiBiasGeluErf>((const float*)p->x, (const float*)p->w0,
                                           (const float*)p->b0, (float*)hidden, p->E, p->R, p->M,
-                                          p->D, stream);
+                                          p->D, stream, p->rows_per_expert);
   if (rc != VMOE_OK) return rc;
   return launch_gemm_f32<kEpiBias>((const float*)hidden, (const float*)p->w1, (const float*)p->b1,
-                                   (float*)p->out, p->E, p->R, p->D, p->M, stream);
+                                   (float*)p->out, p->E, p->R, p->D, p->M, stream,
+                                   p->rows_per_expert);
 }
 
 extern "C" int vmoe_pack_expert_weights(const VmoeTransposeParams* p, vmoe_stream_t stream) {

@@ -139,8 +139,8 @@ __device__ __forceinline__ void load_bias(uint2 (&bias_pk)[TN / 8], const bf16_t
 template <int EPI, int TM, int TN>
 __device__ __forceinline__ void store_tile(floatx16 (&acc)[TM / 32][TN / 32], unsigned char* smem,
                                            int wave, int lane, const uint2 (&bias_pk)[TN / 8],
-                                           bool has_bias, bf16_t* __restrict__ C, int b, int R, int N,
-                                           int wrow0, int wcol0) {
+                                           bool has_bias, bf16_t* __restrict__ C, int b, int R,
+                                           int live, int N, int wrow0, int wcol0) {
   constexpr int FM = TM / 32, FN = TN / 32, OLD = TN + 8;
   const int m = lane & 31, h = lane >> 5;
   bf16_t* Cb = C + (size_t)b * R * N;
@@ -177,7 +177,7 @@ __device__ __forceinline__ void store_tile(floatx16 (&acc)[TM / 32][TN / 32], un
     const int row = wrow0 + rl;
     const int col = wcol0 + oc;
     uint4 v = *reinterpret_cast<const uint4*>(so + rl * OLD + oc);
-    if (row < R && col + 8 <= N) *reinterpret_cast<uint4*>(Cb + (size_t)row * N + col) = v;
+    if (row < live && col + 8 <= N) *reinterpret_cast<uint4*>(Cb + (size_t)row * N + col) = v;
   }
 }
 
@@ -197,6 +197,106 @@ __device__ __forceinline__ bool map_tile(int tiles_m, int tiles_n, int num_tiles
   return true;
 }
 
+// Ragged batches (only rows[b] leading rows of batch b are live).  A small kernel plans
+// the launch first: the live row tiles of all batches, batch-major, form one list that
+// is cut into kNumXcd equal runs, one per die, so that every die gets the same amount
+// of work whatever the batches' sizes while a batch's weights are still read by one die
+// (two, where a cut falls inside it).  Inside a die's run the tiles are ordered in
+// panels as in map_tile.  plan[blockIdx] = (batch, tile_m, tile_n, live rows of the
+// batch), batch -1 for a workgroup without work.  One launch plans up to two products
+// (the two of an MLP differ in tile height and width).
+struct RaggedGeom {
+  int bm, tiles_n, panel_rows, num_blocks;
+  int4* plan;
+};
+
+__device__ __forceinline__ void plan_one(const RaggedGeom& g, const int32_t* tile_prefix,
+                                         const int32_t* __restrict__ rows, int batch, int R,
+                                         int i) {
+  if (g.plan == nullptr || i >= g.num_blocks) return;
+  const int total = tile_prefix[batch];
+  const int share = (total + kNumXcd - 1) / kNumXcd;
+  const int xcd = i % kNumXcd;
+  int slot = i / kNumXcd;
+  const int first = xcd * share;
+  const int last = min(first + share, total);      // this die's run of the tile list
+  int4 out = make_int4(-1, 0, 0, 0);
+  if (first < last && slot < (last - first) * g.tiles_n) {
+    int lo = 0, hi = batch;                        // tile_prefix[lo] <= first < tile_prefix[hi]
+    while (hi - lo > 1) {
+      const int mid = (lo + hi) >> 1;
+      if (tile_prefix[mid] <= first) lo = mid;
+      else hi = mid;
+    }
+    // Walk the run batch by batch; the tiles of one batch are cut into panels of about
+    // panel_rows row tiles (never across batches: a panel shares one batch's B operand),
+    // each swept column tile by column tile.
+    int pos = first;
+    for (int b = lo; b < batch && pos < last; ++b) {
+      const int seg_end = min(tile_prefix[b + 1], last);
+      const int seg = seg_end - pos;
+      if (seg <= 0) continue;
+      const int panels = max(1, (seg + g.panel_rows / 2) / g.panel_rows);
+      const int per_panel = (seg + panels - 1) / panels;
+      if (slot < seg * g.tiles_n) {
+        int q = slot / (per_panel * g.tiles_n);      // panels before the last are full
+        if (q > panels - 1) q = panels - 1;
+        const int rows_here = min(per_panel, seg - q * per_panel);
+        const int in_panel = slot - q * per_panel * g.tiles_n;
+        const int tile_n = in_panel / rows_here;
+        const int entry = pos + q * per_panel + (in_panel - tile_n * rows_here);
+        out = make_int4(b, entry - tile_prefix[b], tile_n, min(max(rows[b], 0), R));
+        break;
+      }
+      slot -= seg * g.tiles_n;
+      pos = seg_end;
+    }
+  }
+  g.plan[i] = out;
+}
+
+__global__ __launch_bounds__(256) void plan_ragged_tiles_kernel(
+    const int32_t* __restrict__ rows, int batch, int R, RaggedGeom ga, RaggedGeom gb) {
+  extern __shared__ int32_t tile_prefix[];      // 2 x (batch + 1): live row tiles before batch b
+  __shared__ int32_t wsum[2][4];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  int32_t* pa = tile_prefix;
+  int32_t* pb = tile_prefix + batch + 1;
+  int carry_a = 0, carry_b = 0;
+  for (int b0 = 0; b0 < batch; b0 += 256) {     // every workgroup scans all batches (few)
+    const int bb = b0 + tid;
+    const int n = bb < batch ? min(max(rows[bb], 0), R) : 0;
+    const int ta = (n + ga.bm - 1) / ga.bm, tb = (n + gb.bm - 1) / gb.bm;
+    int xa = ta, xb = tb;
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+      const int ya = __shfl_up(xa, o, kWave), yb = __shfl_up(xb, o, kWave);
+      if (lane >= o) { xa += ya; xb += yb; }
+    }
+    if (lane == 63) { wsum[0][wave] = xa; wsum[1][wave] = xb; }
+    __syncthreads();
+    int woff_a = 0, woff_b = 0, total_a = 0, total_b = 0;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      if (w < wave) { woff_a += wsum[0][w]; woff_b += wsum[1][w]; }
+      total_a += wsum[0][w];
+      total_b += wsum[1][w];
+    }
+    if (bb < batch) {
+      pa[bb] = carry_a + woff_a + xa - ta;
+      pb[bb] = carry_b + woff_b + xb - tb;
+    }
+    carry_a += total_a;
+    carry_b += total_b;
+    __syncthreads();
+  }
+  if (tid == 0) { pa[batch] = carry_a; pb[batch] = carry_b; }
+  __syncthreads();
+  const int i = blockIdx.x * 256 + tid;
+  plan_one(ga, pa, rows, batch, R, i);
+  plan_one(gb, pb, rows, batch, R, i);
+}
+
 // Fast path: Kd % BK == 0.  Global tiles go straight into LDS
 // (global_load_lds_dwordx4: lane L of a wave lands at base + 16*L), so lane L
 // fetches the global chunk that the XOR swizzle assigns to LDS slot L:
@@ -205,7 +305,8 @@ template <typename Cfg, int EPI>
 __global__ __launch_bounds__(Cfg::kThreads, Cfg::kBlocksPerCu) void gemm_bf16_kernel(
     const bf16_t* __restrict__ A, const bf16_t* __restrict__ Bt, const bf16_t* __restrict__ bias,
     bf16_t* __restrict__ C, int R, int N, int Kd, int tiles_m, int tiles_n, int num_tiles,
-    int tiles_per_xcd, int panel_rows) {
+    int tiles_per_xcd, int panel_rows, const int32_t* __restrict__ rows,
+    const int4* __restrict__ plan) {
 #if defined(__HIP_DEVICE_COMPILE__)   // buffer-resource builtins exist in the device pass only
   extern __shared__ __align__(1024) unsigned char smem[];
   constexpr int BM = Cfg::BM, BN = Cfg::BN, BK = Cfg::BK;
@@ -218,7 +319,23 @@ __global__ __launch_bounds__(Cfg::kThreads, Cfg::kBlocksPerCu) void gemm_bf16_ke
   const int m = lane & 31, h = lane >> 5;
 
   int b, tile_m, tile_n;
-  if (!map_tile(tiles_m, tiles_n, num_tiles, tiles_per_xcd, panel_rows, b, tile_m, tile_n)) return;
+  // Ragged batches: only the first `live` rows of batch b hold data; tiles past them
+  // have nothing to do, and the last tile stores only its live rows.
+  int live = R;
+  if (plan != nullptr) {
+    const int4 mine = plan[blockIdx.x];
+    if (mine.x < 0) return;
+    b = mine.x;
+    tile_m = mine.y;
+    tile_n = mine.z;
+    live = mine.w;
+  } else {
+    if (!map_tile(tiles_m, tiles_n, num_tiles, tiles_per_xcd, panel_rows, b, tile_m, tile_n)) return;
+    if (rows != nullptr) {
+      live = min(rows[b], R);
+      if (tile_m * BM >= live) return;
+    }
+  }
   const int row0 = tile_m * BM, col0 = tile_n * BN;
   const unsigned char* Ab = reinterpret_cast<const unsigned char*>(A + (size_t)b * R * Kd);
   const unsigned char* Bb = reinterpret_cast<const unsigned char*>(Bt + (size_t)b * N * Kd);
@@ -407,8 +524,8 @@ __global__ __launch_bounds__(Cfg::kThreads, Cfg::kBlocksPerCu) void gemm_bf16_ke
   __syncthreads();   // all waves are done with the operand tiles: LDS is reused below
   mfma_result_fence();
 
-  store_tile<EPI, Cfg::TM, Cfg::TN>(acc, smem, wave, lane, bias_pk, bias != nullptr, C, b, R, N,
-                                    row0 + wm * Cfg::TM, col0 + wn * Cfg::TN);
+  store_tile<EPI, Cfg::TM, Cfg::TN>(acc, smem, wave, lane, bias_pk, bias != nullptr, C, b, R, live,
+                                    N, row0 + wm * Cfg::TM, col0 + wn * Cfg::TN);
 #endif
 }
 
@@ -417,7 +534,8 @@ __global__ __launch_bounds__(Cfg::kThreads, Cfg::kBlocksPerCu) void gemm_bf16_ke
 template <int EPI>
 __global__ __launch_bounds__(256) void gemm_bf16_generic_kernel(
     const bf16_t* __restrict__ A, const bf16_t* __restrict__ Bt, const bf16_t* __restrict__ bias,
-    bf16_t* __restrict__ C, int R, int N, int Kd, int tiles_m, int tiles_n) {
+    bf16_t* __restrict__ C, int R, int N, int Kd, int tiles_m, int tiles_n,
+    const int32_t* __restrict__ rows) {
   constexpr int BM = 128, BN = 128, BK = 64, LD = BK + 8, NCH = 4;
   __shared__ __align__(16) bf16_t lds[(BM + BN) * LD];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -428,6 +546,11 @@ __global__ __launch_bounds__(256) void gemm_bf16_generic_kernel(
   const int rem = blockIdx.x - b * per_batch;
   const int tile_n = rem / tiles_m, tile_m = rem - tile_n * tiles_m;
   const int row0 = tile_m * BM, col0 = tile_n * BN;
+  int live = R;
+  if (rows != nullptr) {
+    live = min(rows[b], R);
+    if (row0 >= live) return;     // uniform over the workgroup: no barrier is skipped by a part of it
+  }
   const bf16_t* Ab = A + (size_t)b * R * Kd;
   const bf16_t* Bb = Bt + (size_t)b * N * Kd;
   const int kc8 = (tid & 7) * 8;
@@ -485,7 +608,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_generic_kernel(
 #pragma unroll
       for (int v = 0; v < 16; ++v) {
         const int col = col0 + wn * 64 + j * 32 + (v >> 2) * 8 + h * 4 + (v & 3);
-        if (row < R && col < N) {
+        if (row < live && col < N) {
           float bv = biasb != nullptr ? bf2f(biasb[col]) : 0.f;
           Cb[(size_t)row * N + col] = f2bf(apply_epilogue<EPI>(acc[i][j][v], bv, biasb != nullptr));
         }
@@ -493,23 +616,22 @@ __global__ __launch_bounds__(256) void gemm_bf16_generic_kernel(
   }
 }
 
-template <typename Cfg, int EPI>
-int launch_gemm_bf16(const bf16_t* A, const bf16_t* Bt, const bf16_t* bias, bf16_t* C, int batch,
-                     int R, int N, int Kd, hipStream_t stream) {
-  if (Kd % Cfg::BK != 0 || (uint64_t)(R > N ? R : N) * Kd * 2 >= (1ull << 32)) {
-    const int tiles_m = (R + 127) / 128, tiles_n = (N + 127) / 128;
-    const long long blocks = (long long)batch * tiles_m * tiles_n;
-    if (blocks > 0x7fffffffLL) return VMOE_E_OVERFLOW;
-    hipLaunchKernelGGL(gemm_bf16_generic_kernel<EPI>, dim3((unsigned)blocks), dim3(256), 0, stream,
-                       A, Bt, bias, C, R, N, Kd, tiles_m, tiles_n);
-    return launch_status();
-  }
-  const int tiles_m = (R + Cfg::BM - 1) / Cfg::BM;
-  const int tiles_n = (N + Cfg::BN - 1) / Cfg::BN;
-  const long long tiles = (long long)batch * tiles_m * tiles_n;
-  if (tiles > 0x7ffffff0LL) return VMOE_E_OVERFLOW;
-  const int tiles_per_xcd = (int)((tiles + kNumXcd - 1) / kNumXcd);
-  const unsigned blocks = (unsigned)tiles_per_xcd * kNumXcd;
+struct GemmGeom {
+  bool fast;             // the LDS-DMA kernel applies (else the generic one)
+  int tiles_m, tiles_n, panel_rows, tiles_per_xcd;
+  long long tiles;
+  long long ragged_slots;   // workgroups per die of a planned (ragged) launch
+};
+
+template <typename Cfg>
+GemmGeom gemm_geometry(int batch, int R, int N, int Kd) {
+  GemmGeom g{};
+  g.fast = !(Kd % Cfg::BK != 0 || (uint64_t)(R > N ? R : N) * Kd * 2 >= (1ull << 32));
+  if (!g.fast) return g;
+  g.tiles_m = (R + Cfg::BM - 1) / Cfg::BM;
+  g.tiles_n = (N + Cfg::BN - 1) / Cfg::BN;
+  g.tiles = (long long)batch * g.tiles_m * g.tiles_n;
+  g.tiles_per_xcd = (int)((g.tiles + kNumXcd - 1) / kNumXcd);
   // Tile order inside a batch: panels of `panel_rows` row tiles, swept column tile
   // by column tile.  The tiles that run together on one die (32 compute units)
   // then form a block of about panel_rows x (concurrent / panel_rows) tiles, whose
@@ -517,16 +639,39 @@ int launch_gemm_bf16(const bf16_t* A, const bf16_t* Bt, const bf16_t* bias, bf16
   const double concurrent = 32.0 * Cfg::kBlocksPerCu;
   int panel_rows = (int)(std::sqrt(concurrent * Cfg::BN / Cfg::BM) + 0.5);
   if (panel_rows < 1) panel_rows = 1;
-  if (panel_rows > tiles_m) panel_rows = tiles_m;
-  const int panels = (tiles_m + panel_rows / 2) / panel_rows > 0 ? (tiles_m + panel_rows / 2) / panel_rows : 1;
-  panel_rows = (tiles_m + panels - 1) / panels;
+  if (panel_rows > g.tiles_m) panel_rows = g.tiles_m;
+  const int panels = (g.tiles_m + panel_rows / 2) / panel_rows > 0 ? (g.tiles_m + panel_rows / 2) / panel_rows : 1;
+  g.panel_rows = (g.tiles_m + panels - 1) / panels;
+  // Slots per die for the largest possible run (every row tile live).
+  const long long share_max = ((long long)batch * g.tiles_m + kNumXcd - 1) / kNumXcd;
+  g.ragged_slots = share_max * g.tiles_n;
+  return g;
+}
+
+// `plan`, if given, was filled by plan_ragged_tiles_kernel for this product's geometry.
+template <typename Cfg, int EPI>
+int launch_gemm_bf16(const bf16_t* A, const bf16_t* Bt, const bf16_t* bias, bf16_t* C, int batch,
+                     int R, int N, int Kd, hipStream_t stream, const int32_t* rows = nullptr,
+                     const int4* plan = nullptr) {
+  const GemmGeom g = gemm_geometry<Cfg>(batch, R, N, Kd);
+  if (!g.fast) {
+    const int tiles_m = (R + 127) / 128, tiles_n = (N + 127) / 128;
+    const long long blocks = (long long)batch * tiles_m * tiles_n;
+    if (blocks > 0x7fffffffLL) return VMOE_E_OVERFLOW;
+    hipLaunchKernelGGL(gemm_bf16_generic_kernel<EPI>, dim3((unsigned)blocks), dim3(256), 0, stream,
+                       A, Bt, bias, C, R, N, Kd, tiles_m, tiles_n, rows);
+    return launch_status();
+  }
+  if (g.tiles > 0x7ffffff0LL) return VMOE_E_OVERFLOW;
+  const unsigned blocks = (unsigned)(plan != nullptr ? g.ragged_slots : g.tiles_per_xcd) * kNumXcd;
   auto kern = gemm_bf16_kernel<Cfg, EPI>;
   hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                      hipFuncAttributeMaxDynamicSharedMemorySize,
                                      (int)Cfg::kLdsBytes);
   if (e != hipSuccess) return (int)e;
   hipLaunchKernelGGL(kern, dim3(blocks), dim3(Cfg::kThreads), Cfg::kLdsBytes, stream, A, Bt, bias,
-                     C, R, N, Kd, tiles_m, tiles_n, (int)tiles, tiles_per_xcd, panel_rows);
+                     C, R, N, Kd, g.tiles_m, g.tiles_n, (int)g.tiles, g.tiles_per_xcd, g.panel_rows,
+                     rows, plan);
   return launch_status();
 }
 

@@ -226,6 +226,58 @@ __global__ __launch_bounds__(256) void densify_kernel(
   if (dispatch != nullptr) dispatch[o] = 1;
 }
 
+
+// Packed expert rows, step 1: exclusive prefix over the groups of fill[:, e], one
+// workgroup per expert; the total is the expert's row count.
+__global__ __launch_bounds__(256) void fill_prefix_kernel(
+    const int32_t* __restrict__ fill, int32_t* __restrict__ prefix,
+    int32_t* __restrict__ rows_per_expert, int G, int E) {
+  __shared__ int32_t wsum[4];
+  const int e = blockIdx.x;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  int carry = 0;
+  for (int g0 = 0; g0 < G; g0 += 256) {
+    const int g = g0 + tid;
+    const int v = g < G ? fill[(size_t)g * E + e] : 0;
+    int x = v;
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+      const int y = __shfl_up(x, o, kWave);
+      if (lane >= o) x += y;
+    }
+    if (lane == 63) wsum[wave] = x;
+    __syncthreads();
+    int woff = 0, total = 0;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      if (w < wave) woff += wsum[w];
+      total += wsum[w];
+    }
+    if (g < G) prefix[(size_t)g * E + e] = carry + woff + x - v;
+    carry += total;
+    __syncthreads();
+  }
+  if (tid == 0) rows_per_expert[e] = carry;
+}
+
+// Step 2: token_slot = e*G*C + r(g, c)  ->  token_row = e*G*C + prefix[g][e] + c.
+__global__ __launch_bounds__(256) void compact_rows_kernel(
+    const int32_t* __restrict__ prefix, const int32_t* __restrict__ token_slot,
+    int32_t* __restrict__ token_row, int G, int E, int C, int per_group, size_t n) {
+  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= n) return;
+  const int slot = token_slot[i];
+  int row = -1;
+  if (slot >= 0) {
+    const int per_expert = G * C;
+    const int g = (int)(i / per_group);
+    const int e = slot / per_expert;
+    const int c = (slot - e * per_expert) % C;
+    row = e * per_expert + prefix[(size_t)g * E + e] + c;
+  }
+  token_row[i] = row;
+}
+
 }  // namespace
 }  // namespace vmoe
 
@@ -316,5 +368,20 @@ extern "C" int vmoe_top_items_per_expert(const VmoeTopItemsParams* p, vmoe_strea
                        (const float*)p->gates, p->indices, p->token_slot, p->slot_token, p->weights,
                        p->sel_minmax, p->G, p->S, p->E, p->C, SP);
   }
+  return launch_status();
+}
+
+extern "C" int vmoe_compact_rows(const VmoeCompactRowsParams* p, vmoe_stream_t stream) {
+  if (p == nullptr || p->fill == nullptr || p->token_slot == nullptr || p->token_row == nullptr ||
+      p->rows_per_expert == nullptr || p->prefix == nullptr)
+    return VMOE_E_NULL;
+  int rc = check_route_shapes(p->G, p->S, p->E, p->K, p->C);
+  if (rc != VMOE_OK) return rc;
+  hipLaunchKernelGGL(fill_prefix_kernel, dim3(p->E), dim3(256), 0, as_stream(stream), p->fill,
+                     p->prefix, p->rows_per_expert, p->G, p->E);
+  const size_t n = (size_t)p->G * p->S * p->K;
+  hipLaunchKernelGGL(compact_rows_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0,
+                     as_stream(stream), p->prefix, p->token_slot, p->token_row, p->G, p->E, p->C,
+                     p->S * p->K, n);
   return launch_status();
 }

@@ -144,12 +144,27 @@ def indices_to_slots(indices: torch.Tensor, num_experts: int, capacity: int):
   return token_slot, slot_token, counters
 
 
-def dispatch(x: torch.Tensor, token_slot: torch.Tensor, slot_token: torch.Tensor,
-             out: Optional[torch.Tensor] = None) -> torch.Tensor:
-  """x (T,D), token_slot (T,K), slot_token (NS,) -> (NS, D)."""
+def compact_rows(fill: torch.Tensor, token_slot: torch.Tensor, capacity: int):
+  """fill (G,E), token_slot (G,S,K) -> token_row (G,S,K): the kept assignments of every
+  expert renumbered into the first rows of its block; rows_per_expert (E,)."""
+  G, E = fill.shape
+  _, S, K = token_slot.shape
+  token_row = _i32(G, S, K, device=fill.device)
+  rows = _i32(E, device=fill.device)
+  prefix = _i32(G, E, device=fill.device)
+  p = H.CompactRowsParams(H.ptr(fill), H.ptr(token_slot), H.ptr(token_row), H.ptr(rows),
+                          H.ptr(prefix), G, S, E, K, capacity)
+  H.call("vmoe_compact_rows", p)
+  return token_row, rows
+
+
+def dispatch(x: torch.Tensor, token_slot: torch.Tensor, slot_token: Optional[torch.Tensor],
+             out: Optional[torch.Tensor] = None, num_slots: Optional[int] = None) -> torch.Tensor:
+  """x (T,D), token_slot (T,K), slot_token (NS,) -> (NS, D).  With slot_token None (and
+  num_slots given) unclaimed rows are left as allocated instead of zeroed."""
   T, D = x.shape
   K = token_slot.shape[-1]
-  NS = slot_token.numel()
+  NS = slot_token.numel() if slot_token is not None else int(num_slots)
   x = x.contiguous()
   if out is None:
     out = torch.empty((NS, D), dtype=x.dtype, device=x.device)
@@ -198,8 +213,10 @@ def pack_expert_weights(w: torch.Tensor) -> torch.Tensor:
 
 
 def expert_mlp(x: torch.Tensor, w0, b0, w1, b1, w0t=None, w1t=None, approximate_gelu: bool = True,
-               workspace: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None):
-  """x (E,R,D) -> (E,R,D): gelu(x @ w0 + b0) @ w1 + b1 per expert."""
+               workspace: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None,
+               rows_per_expert: Optional[torch.Tensor] = None):
+  """x (E,R,D) -> (E,R,D): gelu(x @ w0 + b0) @ w1 + b1 per expert; with rows_per_expert (E,)
+  int32 only that many leading rows of every expert are computed."""
   E, R, D = x.shape
   M = (w0.shape[2] if w0 is not None else w0t.shape[1])
   x = x.contiguous()
@@ -207,7 +224,7 @@ def expert_mlp(x: torch.Tensor, w0, b0, w1, b1, w0t=None, w1t=None, approximate_
     out = torch.empty_like(x)
   p = H.ExpertMlpParams(H.ptr(x), H.ptr(w0), H.ptr(b0), H.ptr(w1), H.ptr(b1), H.ptr(w0t),
                         H.ptr(w1t), H.ptr(out), None, 0, E, R, D, M, H.dtype_code(x.dtype),
-                        H.GELU_TANH if approximate_gelu else H.GELU_ERF)
+                        H.GELU_TANH if approximate_gelu else H.GELU_ERF, H.ptr(rows_per_expert))
   need = H.lib().vmoe_expert_mlp_workspace_bytes(H.ctypes.byref(p))
   if workspace is None or workspace.numel() * workspace.element_size() < need:
     workspace = torch.empty(need, dtype=torch.uint8, device=x.device)

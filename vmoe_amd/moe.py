@@ -80,6 +80,8 @@ class ExpertIndicesDispatcher(BaseDispatcher):
     self.einsum_precision = einsum_precision      # combine always accumulates in float32
     self._slots = _slots                          # (token_slot (G,S,K), slot_token (E*G*C,))
     self._weights_f32 = None                      # float32 copy of combine_weights, if on hand
+    self.fill = None                              # (G, E) kept items per (group, expert), if known
+    self._packed_maps = None                      # (token_row (G,S,K), rows_per_expert (E,))
 
   def _maps(self):
     if self._slots is None:
@@ -110,6 +112,42 @@ class ExpertIndicesDispatcher(BaseDispatcher):
     w = self._weights_f32 if self._weights_f32 is not None else K.cast(
         self.combine_weights.contiguous(), torch.float32)
     out = K.combine(rows, token_slot.view(G * S, Kk), w.view(G * S, Kk))
+    return _from_rows(out, (G, S), item_shape, width)
+
+
+  # Packed rows.  The reference's buffer gives every (group, expert) pair `capacity`
+  # rows, filled or not, and the experts run over all of them.  When the fill counts
+  # are known (dispatchers made by the routers), the same buffer can hold each
+  # expert's items in its first rows instead; experts that accept a row count per
+  # expert then skip the rest.  dispatch_packed / combine_packed are the pair used
+  # by sparse_moe_spmd for that; dispatch / combine keep the reference layout.
+  def supports_packed(self) -> bool:
+    return self.fill is not None
+
+  def _packed(self):
+    if self._packed_maps is None:
+      token_slot, _ = self._maps()
+      self._packed_maps = K.compact_rows(self.fill, token_slot, self.capacity)
+    return self._packed_maps
+
+  def dispatch_packed(self, data: Array):
+    """-> (buffer (E, G * capacity, ...) whose expert e holds items in rows
+    0 .. rows_per_expert[e] - 1 and arbitrary values after them, rows_per_expert (E,) int32)."""
+    G, S, Kk, _ = self.indices.shape
+    token_row, rows_per_expert = self._packed()
+    rows, item_shape, width = _as_rows(data, 2)
+    out = K.dispatch(rows, token_row.view(G * S, Kk), None,
+                     num_slots=self.num_experts * G * self.capacity)
+    return (_from_rows(out, (self.num_experts, G * self.capacity), item_shape, width),
+            rows_per_expert)
+
+  def combine_packed(self, data: Array) -> Array:
+    G, S, Kk, _ = self.indices.shape
+    token_row, _ = self._packed()
+    rows, item_shape, width = _as_rows(data, 2)
+    w = self._weights_f32 if self._weights_f32 is not None else K.cast(
+        self.combine_weights.contiguous(), torch.float32)
+    out = K.combine(rows, token_row.view(G * S, Kk), w.view(G * S, Kk))
     return _from_rows(out, (G, S), item_shape, width)
 
 
@@ -214,6 +252,15 @@ class _SparseEinsumDispatcher(EinsumDispatcher):
   def combine(self, data: Array) -> Array:
     return self._inner.combine(data)
 
+  def supports_packed(self) -> bool:
+    return self._inner.supports_packed()
+
+  def dispatch_packed(self, data: Array):
+    return self._inner.dispatch_packed(data)
+
+  def combine_packed(self, data: Array) -> Array:
+    return self._inner.combine_packed(data)
+
 
 class Bfloat16Dispatcher(BaseDispatcher):
   """Wrapper converting data to bfloat16 around the inner dispatcher; vmoe/moe.py:212-227."""
@@ -232,6 +279,20 @@ class Bfloat16Dispatcher(BaseDispatcher):
     data = _cast_to_bfloat16(data)
     data = self.dispatcher.combine(data)
     return K.cast(data, dtype) if data.is_floating_point() else data
+
+  def supports_packed(self) -> bool:
+    fn = getattr(self.dispatcher, "supports_packed", None)
+    return bool(fn and fn())
+
+  def dispatch_packed(self, data: Array):
+    dtype = data.dtype
+    out, rows = self.dispatcher.dispatch_packed(_cast_to_bfloat16(data))
+    return (K.cast(out, dtype) if out.is_floating_point() else out), rows
+
+  def combine_packed(self, data: Array) -> Array:
+    dtype = data.dtype
+    out = self.dispatcher.combine_packed(_cast_to_bfloat16(data))
+    return K.cast(out, dtype) if out.is_floating_point() else out
 
 
 def _cast_to_bfloat16(x: Array) -> Array:
@@ -462,6 +523,14 @@ def sparse_moe_spmd(target, variable_axes: Optional[Mapping[str, Any]] = None,
       return _tree_stack(per_expert)
 
     def apply(self, variables, dispatcher: BaseDispatcher, *inputs):
+      supports = getattr(dispatcher, "supports_packed", None)
+      if (not has_aux and len(inputs) == 1 and supports is not None and supports()
+          and getattr(self.expert, "supports_packed_rows", False)):
+        # Each expert's items in its first rows; the expert skips the empty ones.
+        dispatched, rows_per_expert = dispatcher.dispatch_packed(inputs[0])
+        outputs = self.expert.apply_experts(variables, dispatched,
+                                            rows_per_expert=rows_per_expert)
+        return _tree_map(dispatcher.combine_packed, outputs)
       dispatched = [dispatcher.dispatch(x) for x in inputs]
       if hasattr(self.expert, "apply_experts"):
         outputs = self.expert.apply_experts(variables, *dispatched)

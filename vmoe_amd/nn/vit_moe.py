@@ -52,8 +52,12 @@ class MlpBlock(module.Module):
   def _pack(self, w: Array, dtype) -> Array:
     return self._packed.get((w,), dtype, lambda: K.pack_expert_weights(K.cast(w, dtype)))
 
-  def apply_experts(self, variables, inputs: Array) -> Array:
-    """inputs (E, R, D) with parameters stacked on axis 0 -> (E, R, D)."""
+  supports_packed_rows = True
+
+  def apply_experts(self, variables, inputs: Array, rows_per_expert: Optional[Array] = None) -> Array:
+    """inputs (E, R, D) with parameters stacked on axis 0 -> (E, R, D).  With
+    rows_per_expert (E,) int32 only that many leading rows of each expert are
+    computed; the other rows of the result are not written."""
     p = variables["params"]
     dtype = self.dtype or inputs.dtype
     x = K.cast(inputs, dtype)
@@ -62,9 +66,10 @@ class MlpBlock(module.Module):
     cast = lambda t: None if t is None else K.cast(t, dtype)
     if dtype == torch.bfloat16:
       return K.expert_mlp(x, None, cast(b0), None, cast(b1), w0t=self._pack(w0, dtype),
-                          w1t=self._pack(w1, dtype), approximate_gelu=self.approximate_gelu)
+                          w1t=self._pack(w1, dtype), approximate_gelu=self.approximate_gelu,
+                          rows_per_expert=rows_per_expert)
     return K.expert_mlp(x, cast(w0), cast(b0), cast(w1), cast(b1),
-                        approximate_gelu=self.approximate_gelu)
+                        approximate_gelu=self.approximate_gelu, rows_per_expert=rows_per_expert)
 
   def apply(self, variables, inputs: Array) -> Array:
     """Single MLP: inputs (..., D)."""
