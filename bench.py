@@ -395,7 +395,8 @@ def main():
               "buffer_rows": E * G * C}
 
   # HBM-bound stages, algorithmic bytes (each item row read once, whole buffer written).
-  bytes_dispatch = T * D * b + E * G * C * D * b + 8 * T * K
+  # dispatch writes only the kept rows (packed layout: no zero fill of empty slots)
+  bytes_dispatch = T * D * b + kept * D * b + 8 * T * K
   bytes_combine = kept * D * b + 12 * T * K + T * D * b
   bytes_gate = T * D * b + D * E * b + 12 * T * K + T * E * b
   # Measured copy ceiling of the same device (read + write of 512 MiB).
@@ -423,6 +424,27 @@ def main():
     torch.cuda.synchronize()
     roofline["measured_mfma_loop_TFLOPs"] = probe_flops / (e0.elapsed_time(e1) * 1e-3) / 1e12
     roofline["frac_of_measured_loop"] = achieved_tflops / roofline["measured_mfma_loop_TFLOPs"]
+  # The vendor library's GEMM on the same two products as dense matrices of the kept
+  # rows (torch.nn.functional.linear -> hipBLASLt, no GELU), same run: a reference
+  # point for what this part sustains on these shapes.
+  if b == 2:
+    a_up = xs[0].reshape(-1, D)[:1].expand(kept, D).contiguous()
+    w_up = torch.randn((M, D), device=dev).to(tdt) * D ** -0.5
+    a_dn = torch.randn((kept, M), device=dev).to(tdt)
+    w_dn = torch.randn((D, M), device=dev).to(tdt) * M ** -0.5
+    a_up.copy_(torch.randn((kept, D), device=dev).to(tdt))
+    lib = {}
+    for name, a_, w_ in (("up", a_up, w_up), ("down", a_dn, w_dn)):
+      for _ in range(3):
+        torch.nn.functional.linear(a_, w_)
+      e0.record()
+      for _ in range(10):
+        torch.nn.functional.linear(a_, w_)
+      e1.record()
+      torch.cuda.synchronize()
+      lib[name] = 2.0 * kept * D * M * 10 / (e0.elapsed_time(e1) * 1e-3) / 1e12
+    roofline["library_gemm_same_shapes_TFLOPs"] = lib
+    del a_up, a_dn, w_up, w_dn
   hbm = {
       "dispatch_GBps": bytes_dispatch / (stage_ms["vmoe_dispatch"] * 1e-3) / 1e9,
       "combine_GBps": bytes_combine / (stage_ms["vmoe_combine"] * 1e-3) / 1e9,

@@ -73,7 +73,7 @@ class ExpertIndicesDispatcher(BaseDispatcher):
   def __init__(self, indices: Array, combine_weights: Array, num_experts: int, capacity: int,
                partition_spec=None, einsum_precision=None, _slots=None):
     self.indices = indices
-    self.combine_weights = combine_weights
+    self._combine_weights = combine_weights       # a tensor, or (float32 tensor, dtype) cast on first read
     self.num_experts = int(num_experts)
     self.capacity = int(capacity)
     self.partition_spec = partition_spec          # accepted for API parity; one GPU, no mesh
@@ -82,6 +82,17 @@ class ExpertIndicesDispatcher(BaseDispatcher):
     self._weights_f32 = None                      # float32 copy of combine_weights, if on hand
     self.fill = None                              # (G, E) kept items per (group, expert), if known
     self._packed_maps = None                      # (token_row (G,S,K), rows_per_expert (E,))
+
+  @property
+  def combine_weights(self) -> Array:
+    cw = self._combine_weights
+    if isinstance(cw, tuple):                     # made by a router: the cast is only for readers
+      cw = self._combine_weights = K.cast(cw[0], cw[1])
+    return cw
+
+  @combine_weights.setter
+  def combine_weights(self, value: Array):
+    self._combine_weights = value
 
   def _maps(self):
     if self._slots is None:
@@ -374,7 +385,7 @@ def _route(gates: Array, num_selected_experts: int, capacity: int, batch_priorit
   indices, token_slot, slot_token, fill = K.route_assign(
       val, idx, num_experts, capacity, batch_priority)
   inner = ExpertIndicesDispatcher(
-      indices=indices, combine_weights=K.cast(val, gates.dtype) if gates.dtype != val.dtype else val,
+      indices=indices, combine_weights=(val, gates.dtype) if gates.dtype != val.dtype else val,
       num_experts=num_experts, capacity=capacity, _slots=(token_slot, slot_token),
       **dispatcher_kwargs)
   inner.fill = fill
