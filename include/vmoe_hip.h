@@ -232,6 +232,28 @@ typedef struct {
 } VmoeCombineParams;
 int vmoe_combine(const VmoeCombineParams* p, vmoe_stream_t stream);
 
+/* Gradients of dispatch / combine (the gather <-> scatter duals; the reference gets them
+ * from JAX's autodiff of vmoe/moe.py:190-209).  With combine  out[t] = sum_k w[t,k] *
+ * y[slot(t,k)]:
+ *   vmoe_combine_backward_data:     dy[slot(t,k)] = w[t,k] * dout[t]; slots no item claims
+ *                                   get 0 (slot_token given) or stay untouched (null);
+ *   vmoe_combine_backward_weights:  dweights[t,k] = <dout[t], y[slot(t,k)]>, 0 if dropped.
+ * The gradient of dispatch with respect to its input, dx[t] = sum_k dbuf[slot(t,k)], is
+ * vmoe_combine with unit weights.  Row width as for dispatch / combine. */
+typedef struct {
+  const void* dout;           /* (num_items, D) dtype: gradient of combine's output */
+  const void* y;              /* (num_slots, D) dtype: combine's input (weights gradient only) */
+  const int32_t* token_slot;  /* (num_items, K) */
+  const float* weights;       /* (num_items, K) float32 (data gradient only) */
+  const int32_t* slot_token;  /* (num_slots,) or null (data gradient only) */
+  void* dy;                   /* out (num_slots, D) dtype */
+  float* dweights;            /* out (num_items, K) float32 */
+  int32_t num_items, num_slots, K, D;
+  int32_t dtype;
+} VmoeCombineBackwardParams;
+int vmoe_combine_backward_data(const VmoeCombineBackwardParams* p, vmoe_stream_t stream);
+int vmoe_combine_backward_weights(const VmoeCombineBackwardParams* p, vmoe_stream_t stream);
+
 /* Dense (G,S,E,C) view of a sparse assignment, for callers that read
  * EinsumDispatcher.combine_weights / dispatch_weights (vmoe/moe.py:609-619):
  * combine[g,s,e,c] = weight of the kept assignment (s -> e,c), else 0;

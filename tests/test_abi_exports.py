@@ -67,7 +67,8 @@ def test_struct_layouts_match_header():
         "VmoeAddLayerNormParams": _hip.AddLayerNormParams,
         "VmoeAttentionParams": _hip.AttentionParams,
         "VmoeNoisyGatesParams": _hip.NoisyGatesParams,
-        "VmoeCompactRowsParams": _hip.CompactRowsParams}
+        "VmoeCompactRowsParams": _hip.CompactRowsParams,
+        "VmoeCombineBackwardParams": _hip.CombineBackwardParams}
   assert set(py) == set(structs)
   for name, body in structs.items():
     want = []

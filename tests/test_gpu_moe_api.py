@@ -681,3 +681,63 @@ def test_packed_rows_path_equals_reference_layout(moe, dtype, bf16_dispatcher, n
   fill = getattr(inner, "_inner", inner).fill
   np.testing.assert_array_equal(to_np(rows), to_np(fill).sum(0))
   assert int(rows.sum()) < E * G * buf.shape[1] // G          # capacity 0.75: some slots stay empty
+
+
+# ------------------------------------------------------------------ gradients of dispatch / combine
+@pytest.mark.parametrize("dtype", [O.F32, O.BF16])
+def test_dispatch_combine_gradients(moe, dtype):
+  """The gather <-> scatter duals against torch autograd on the same maps written with
+  index ops in float64."""
+  rng = np.random.default_rng(41)
+  G, S, D, E, K, C = 3, 40, 32, 4, 2, 12
+  gates = O.softmax(rng.standard_normal((G, S, E)).astype(np.float32) * 2)
+  d0 = moe.get_top_experts_per_item_dispatcher(to_dev(gates), "indices", num_selected_experts=K,
+                                               capacity=C, batch_priority=True)
+  token_slot, slot_token = d0._maps()
+  ts = token_slot.view(G * S, K).long()
+  kept = ts >= 0
+  NS = slot_token.numel()
+  tdt = tdtype(dtype)
+  x = to_dev(O.cast(rng.standard_normal((G, S, D)).astype(np.float32), dtype), dtype).requires_grad_()
+  w = to_dev(rng.uniform(0.1, 1.0, (G, S, K)).astype(np.float32)).requires_grad_()
+  d = moe.ExpertIndicesDispatcher(d0.indices, w, E, C)
+  buf = d.dispatch(x)                                    # (E, G*C, D)
+  assert buf.requires_grad
+  y = (buf.float() * 1.5 + 0.25).to(tdt)                 # any differentiable "expert"
+  out = d.combine(y)
+  gout = to_dev(O.cast(rng.standard_normal((G, S, D)).astype(np.float32), dtype), dtype)
+  out.backward(gout)
+  # float64 statement with torch index ops
+  x64 = x.detach().double().view(G * S, D).requires_grad_()
+  w64 = w.detach().double().view(G * S, K).requires_grad_()
+  buf64 = torch.zeros((NS + 1, D), dtype=torch.float64, device=dev())
+  idx = torch.where(kept, ts, torch.full_like(ts, NS))   # dropped -> a dump row
+  buf64 = buf64.index_add(0, idx.reshape(-1), x64.repeat_interleave(K, dim=0))[:NS]
+  y64 = buf64 * 1.5 + 0.25
+  picked = y64[ts.clamp(min=0)] * kept[..., None]         # (T, K, D)
+  out64 = (picked * w64[..., None]).sum(1)
+  out64.backward(gout.double().view(G * S, D))
+  tol = 2e-2 if dtype == O.BF16 else 1e-5
+  assert_close(to_np(out), out64.detach().cpu().numpy().reshape(G, S, D), tol, "forward")
+  assert_close(to_np(x.grad), x64.grad.cpu().numpy().reshape(G, S, D), tol, "dx")
+  assert_close(to_np(w.grad), w64.grad.cpu().numpy().reshape(G, S, K), tol, "dw")
+  assert (to_np(w.grad).reshape(G * S, K)[~kept.cpu().numpy()] == 0).all()
+
+
+def test_combine_backward_data_zero_fills_unclaimed_slots(moe):
+  from vmoe_amd import kernels as K
+  rng = np.random.default_rng(42)
+  G, S, D, E, Kk, C = 2, 16, 16, 4, 1, 8
+  gates = O.softmax(rng.standard_normal((G, S, E)).astype(np.float32))
+  d0 = moe.get_top_experts_per_item_dispatcher(to_dev(gates), "indices", num_selected_experts=Kk,
+                                               capacity=C, batch_priority=False)
+  token_slot, slot_token = d0._maps()
+  g = to_dev(rng.standard_normal((G * S, D)).astype(np.float32))
+  w = to_dev(rng.uniform(0.5, 1, (G * S, Kk)).astype(np.float32))
+  dy = K.combine_backward_data(g, token_slot.view(G * S, Kk), w, slot_token, slot_token.numel())
+  st = to_np(slot_token)
+  dyn = to_np(dy)
+  assert (dyn[st < 0] == 0).all() and (st < 0).any()
+  for slot in np.nonzero(st >= 0)[0][:10]:
+    t = st[slot]
+    np.testing.assert_allclose(dyn[slot], to_np(g)[t] * to_np(w)[t, 0], rtol=1e-6)

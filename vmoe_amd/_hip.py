@@ -26,6 +26,7 @@ EXPORTS = [
     "vmoe_soft_route_workspace_bytes", "vmoe_soft_route", "vmoe_einsum_dispatch",
     "vmoe_einsum_combine", "vmoe_cast", "vmoe_copy_bytes", "vmoe_mfma_probe",
     "vmoe_add_layer_norm", "vmoe_attention", "vmoe_noisy_gates", "vmoe_compact_rows",
+    "vmoe_combine_backward_data", "vmoe_combine_backward_weights",
 ]
 
 
@@ -180,6 +181,13 @@ class EinsumParams(ctypes.Structure):
 class CastParams(ctypes.Structure):
   _fields_ = [("in_", c_void_p), ("out", c_void_p), ("n", c_size_t),
               ("in_dtype", c_int32), ("out_dtype", c_int32)]
+
+
+class CombineBackwardParams(ctypes.Structure):
+  _fields_ = [("dout", c_void_p), ("y", c_void_p), ("token_slot", c_void_p), ("weights", c_void_p),
+              ("slot_token", c_void_p), ("dy", c_void_p), ("dweights", c_void_p),
+              ("num_items", c_int32), ("num_slots", c_int32), ("K", c_int32), ("D", c_int32),
+              ("dtype", c_int32)]
 
 
 class AddLayerNormParams(ctypes.Structure):

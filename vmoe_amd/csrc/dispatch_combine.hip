@@ -258,6 +258,70 @@ __global__ __launch_bounds__(256) void cast_bf16_to_f32_kernel(const bf16_t* __r
   }
 }
 
+
+// ---------------------------------------------------------------- gradients
+// combine is  out[t] = sum_k w[t,k] * y[slot(t,k)].  Its duals:
+//   dy[slot(t,k)] = w[t,k] * dout[t]   (a dispatch that scales; unclaimed slots get 0)
+//   dw[t,k]       = <dout[t], y[slot(t,k)]>
+// (dispatch's own dual, dx[t] = sum_k dbuf[slot(t,k)], is combine with unit weights.)
+template <typename T>
+__global__ __launch_bounds__(kMoveThreads) void scatter_scaled_kernel(
+    const uint4* __restrict__ g, const int32_t* __restrict__ token_slot,
+    const float* __restrict__ weights, const int32_t* __restrict__ slot_token,
+    uint4* __restrict__ out, int num_items, int num_slots, int K, int cpr, int item_waves) {
+  constexpr int N = Chunk<T>::n;
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(
+      (int)((blockIdx.x * (unsigned)kMoveThreads + threadIdx.x) >> 6));
+  if (wave < item_waves) {
+    for (int ch = lane; ch < cpr; ch += kWave) {
+      float a[N];
+      Chunk<T>::unpack(g[(size_t)wave * cpr + ch], a);
+      for (int k = 0; k < K; ++k) {
+        const int slot = token_slot[(size_t)wave * K + k];
+        if (slot < 0) continue;
+        const float w = weights[(size_t)wave * K + k];
+        float b[N];
+#pragma unroll
+        for (int j = 0; j < N; ++j) b[j] = __fmul_rn(w, a[j]);
+        out[(size_t)slot * cpr + ch] = Chunk<T>::pack(b);
+      }
+    }
+  } else {
+    const int s = wave - item_waves;
+    if (slot_token != nullptr && s < num_slots && slot_token[s] < 0)
+      for (int ch = lane; ch < cpr; ch += kWave) out[(size_t)s * cpr + ch] = make_uint4(0, 0, 0, 0);
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(kMoveThreads) void row_dots_kernel(
+    const uint4* __restrict__ g, const uint4* __restrict__ y,
+    const int32_t* __restrict__ token_slot, float* __restrict__ dw, int num_items, int K,
+    int cpr) {
+  constexpr int N = Chunk<T>::n;
+  const int lane = threadIdx.x & 63;
+  const int t = __builtin_amdgcn_readfirstlane(
+      (int)((blockIdx.x * (unsigned)kMoveThreads + threadIdx.x) >> 6));
+  if (t >= num_items) return;
+  for (int k = 0; k < K; ++k) {
+    const int slot = token_slot[(size_t)t * K + k];
+    float acc = 0.f;
+    if (slot >= 0) {
+      for (int ch = lane; ch < cpr; ch += kWave) {
+        float a[N], b[N];
+        Chunk<T>::unpack(g[(size_t)t * cpr + ch], a);
+        Chunk<T>::unpack(y[(size_t)slot * cpr + ch], b);
+#pragma unroll
+        for (int j = 0; j < N; ++j) acc += a[j] * b[j];
+      }
+#pragma unroll
+      for (int o = 32; o > 0; o >>= 1) acc += __shfl_xor(acc, o, kWave);
+    }
+    if (lane == 0) dw[(size_t)t * K + k] = acc;
+  }
+}
+
 int check_move(const void* a, const void* b, const void* c, int num_items, int num_slots, int K,
                int D, int dtype) {
   if (a == nullptr || b == nullptr || c == nullptr) return VMOE_E_NULL;
@@ -357,5 +421,44 @@ extern "C" int vmoe_cast(const VmoeCastParams* p, vmoe_stream_t stream) {
                        as_stream(stream), (const bf16_t*)p->in, (float*)p->out, p->n);
   else
     return VMOE_E_DTYPE;
+  return launch_status();
+}
+
+extern "C" int vmoe_combine_backward_data(const VmoeCombineBackwardParams* p, vmoe_stream_t stream) {
+  if (p == nullptr || p->weights == nullptr || p->dy == nullptr) return VMOE_E_NULL;
+  int rc = check_move(p->dout, p->token_slot, p->dy, p->num_items, p->num_slots, p->K, p->D, p->dtype);
+  if (rc != VMOE_OK) return rc;
+  const int cpr = (int)((size_t)p->D * (p->dtype == VMOE_BF16 ? 2 : 4) / 16);
+  const long long waves = (long long)p->num_items + (p->slot_token != nullptr ? p->num_slots : 0);
+  const long long blocks = (waves + 3) / 4;
+  if (blocks > 0x7fffffffLL) return VMOE_E_OVERFLOW;
+  if (p->dtype == VMOE_BF16)
+    hipLaunchKernelGGL(scatter_scaled_kernel<bf16_t>, dim3((unsigned)blocks), dim3(kMoveThreads), 0,
+                       as_stream(stream), (const uint4*)p->dout, p->token_slot, p->weights,
+                       p->slot_token, (uint4*)p->dy, p->num_items, p->num_slots, p->K, cpr,
+                       p->num_items);
+  else
+    hipLaunchKernelGGL(scatter_scaled_kernel<float>, dim3((unsigned)blocks), dim3(kMoveThreads), 0,
+                       as_stream(stream), (const uint4*)p->dout, p->token_slot, p->weights,
+                       p->slot_token, (uint4*)p->dy, p->num_items, p->num_slots, p->K, cpr,
+                       p->num_items);
+  return launch_status();
+}
+
+extern "C" int vmoe_combine_backward_weights(const VmoeCombineBackwardParams* p,
+                                             vmoe_stream_t stream) {
+  if (p == nullptr || p->y == nullptr || p->dweights == nullptr) return VMOE_E_NULL;
+  int rc = check_move(p->dout, p->token_slot, p->y, p->num_items, p->num_slots, p->K, p->D, p->dtype);
+  if (rc != VMOE_OK) return rc;
+  const int cpr = (int)((size_t)p->D * (p->dtype == VMOE_BF16 ? 2 : 4) / 16);
+  const int blocks = (p->num_items + 3) / 4;
+  if (p->dtype == VMOE_BF16)
+    hipLaunchKernelGGL(row_dots_kernel<bf16_t>, dim3(blocks), dim3(kMoveThreads), 0,
+                       as_stream(stream), (const uint4*)p->dout, (const uint4*)p->y, p->token_slot,
+                       p->dweights, p->num_items, p->K, cpr);
+  else
+    hipLaunchKernelGGL(row_dots_kernel<float>, dim3(blocks), dim3(kMoveThreads), 0,
+                       as_stream(stream), (const uint4*)p->dout, (const uint4*)p->y, p->token_slot,
+                       p->dweights, p->num_items, p->K, cpr);
   return launch_status();
 }

@@ -189,6 +189,35 @@ def combine(y: torch.Tensor, token_slot: torch.Tensor, weights: torch.Tensor,
   return out
 
 
+def combine_backward_data(dout: torch.Tensor, token_slot: torch.Tensor, weights: torch.Tensor,
+                          slot_token: Optional[torch.Tensor], num_slots: int) -> torch.Tensor:
+  """dout (T,D) -> dy (NS,D): dy[slot(t,k)] = w[t,k] * dout[t]; unclaimed slots are zero when
+  slot_token is given, unwritten otherwise."""
+  T, D = dout.shape
+  Kk = token_slot.shape[-1]
+  dout = dout.contiguous()
+  weights = weights.to(torch.float32).contiguous()
+  dy = torch.empty((num_slots, D), dtype=dout.dtype, device=dout.device)
+  p = H.CombineBackwardParams(H.ptr(dout), None, H.ptr(token_slot), H.ptr(weights),
+                              H.ptr(slot_token), H.ptr(dy), None, T, num_slots, Kk, D,
+                              H.dtype_code(dout.dtype))
+  H.call("vmoe_combine_backward_data", p)
+  return dy
+
+
+def combine_backward_weights(dout: torch.Tensor, y: torch.Tensor,
+                             token_slot: torch.Tensor) -> torch.Tensor:
+  """dout (T,D), y (NS,D) -> dweights (T,K) f32: <dout[t], y[slot(t,k)]>, 0 where dropped."""
+  T, D = dout.shape
+  Kk = token_slot.shape[-1]
+  dout, y = dout.contiguous(), y.contiguous()
+  dw = _f32(T, Kk, device=dout.device)
+  p = H.CombineBackwardParams(H.ptr(dout), H.ptr(y), H.ptr(token_slot), None, None, None,
+                              H.ptr(dw), T, y.shape[0], Kk, D, H.dtype_code(dout.dtype))
+  H.call("vmoe_combine_backward_weights", p)
+  return dw
+
+
 def densify(indices: torch.Tensor, weights: torch.Tensor, num_experts: int, capacity: int):
   """indices (G,S,K,2), weights (G,S,K) -> combine (G,S,E,C) f32, dispatch (G,S,E,C) bool."""
   G, S, K, _ = indices.shape

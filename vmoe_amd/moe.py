@@ -57,6 +57,46 @@ def _from_rows(rows: Array, lead_shape, item_shape, width: int) -> Array:
   return rows.reshape(*lead_shape, *item_shape)
 
 
+class _DispatchFn(torch.autograd.Function):
+  """dispatch with its gradient: dx[t] = sum_k dbuf[slot(t, k)] (combine with unit weights)."""
+
+  @staticmethod
+  def forward(ctx, rows, token_slot, slot_token, num_slots):
+    ctx.save_for_backward(token_slot)
+    return K.dispatch(rows, token_slot, slot_token, num_slots=num_slots)
+
+  @staticmethod
+  def backward(ctx, grad):
+    (token_slot,) = ctx.saved_tensors
+    ones = torch.ones(token_slot.shape, dtype=torch.float32, device=grad.device)
+    return K.combine(grad.contiguous(), token_slot, ones), None, None, None
+
+
+class _CombineFn(torch.autograd.Function):
+  """combine with its gradients: dy[slot(t, k)] = w[t, k] * dout[t] and
+  dw[t, k] = <dout[t], y[slot(t, k)]>."""
+
+  @staticmethod
+  def forward(ctx, rows, token_slot, weights, slot_token):
+    ctx.save_for_backward(rows, token_slot, weights, slot_token)
+    return K.combine(rows, token_slot, weights)
+
+  @staticmethod
+  def backward(ctx, grad):
+    rows, token_slot, weights, slot_token = ctx.saved_tensors
+    grad = grad.contiguous()
+    d_rows = d_w = None
+    if ctx.needs_input_grad[0]:
+      d_rows = K.combine_backward_data(grad, token_slot, weights, slot_token, rows.shape[0])
+    if ctx.needs_input_grad[2]:
+      d_w = K.combine_backward_weights(grad, rows, token_slot).to(weights.dtype)
+    return d_rows, None, d_w, None
+
+
+def _wants_grad(*tensors) -> bool:
+  return torch.is_grad_enabled() and any(t is not None and t.requires_grad for t in tensors)
+
+
 class ExpertIndicesDispatcher(BaseDispatcher):
   """Dispatcher using (expert, buffer position) indices; vmoe/moe.py:164-209.
 
@@ -113,18 +153,26 @@ class ExpertIndicesDispatcher(BaseDispatcher):
     G, S, Kk, _ = self.indices.shape
     token_slot, slot_token = self._maps()
     rows, item_shape, width = _as_rows(data, 2)
-    out = K.dispatch(rows, token_slot.view(G * S, Kk), slot_token)
+    if _wants_grad(rows):
+      out = _DispatchFn.apply(rows, token_slot.view(G * S, Kk), slot_token, slot_token.numel())
+    else:
+      out = K.dispatch(rows, token_slot.view(G * S, Kk), slot_token)
     return _from_rows(out, (self.num_experts, G * self.capacity), item_shape, width)
 
   def combine(self, data: Array) -> Array:
     G, S, Kk, _ = self.indices.shape
-    token_slot, _ = self._maps()
+    token_slot, slot_token = self._maps()
     rows, item_shape, width = _as_rows(data, 2)
+    cw = self._combine_weights
+    if _wants_grad(rows, cw if isinstance(cw, torch.Tensor) else None):
+      # differentiable in the data and in combine_weights
+      w = self.combine_weights.to(torch.float32)
+      out = _CombineFn.apply(rows, token_slot.view(G * S, Kk), w.reshape(G * S, Kk), slot_token)
+      return _from_rows(out, (G, S), item_shape, width)
     w = self._weights_f32 if self._weights_f32 is not None else K.cast(
         self.combine_weights.contiguous(), torch.float32)
     out = K.combine(rows, token_slot.view(G * S, Kk), w.view(G * S, Kk))
     return _from_rows(out, (G, S), item_shape, width)
-
 
   # Packed rows.  The reference's buffer gives every (group, expert) pair `capacity`
   # rows, filled or not, and the experts run over all of them.  When the fill counts
@@ -536,7 +584,8 @@ def sparse_moe_spmd(target, variable_axes: Optional[Mapping[str, Any]] = None,
     def apply(self, variables, dispatcher: BaseDispatcher, *inputs):
       supports = getattr(dispatcher, "supports_packed", None)
       if (not has_aux and len(inputs) == 1 and supports is not None and supports()
-          and getattr(self.expert, "supports_packed_rows", False)):
+          and getattr(self.expert, "supports_packed_rows", False)
+          and not _wants_grad(inputs[0])):
         # Each expert's items in its first rows; the expert skips the empty ones.
         dispatched, rows_per_expert = dispatcher.dispatch_packed(inputs[0])
         outputs = self.expert.apply_experts(variables, dispatched,
