@@ -130,17 +130,26 @@ def soft_main(args):
   for i in range(INIT_STEPS + args.warmup):
     step(i)
   torch.cuda.synchronize()
-  sink = _hip.TimingSink(pairs=args.steps * CALLS_PER_STEP)
+  # As in main(): events only around the dominant entry point inside the timed region,
+  # the other stages from a second, fully instrumented pass.
+  sink = _hip.TimingSink(pairs=args.steps * 2, only=("vmoe_expert_mlp",))
   _hip.set_timing_sink(sink)
   t0 = time.perf_counter()
   for i in range(args.steps):
     step(i)
   torch.cuda.synchronize()
   t1 = time.perf_counter()
-  _hip.set_timing_sink(None)
   ms = (t1 - t0) * 1e3 / args.steps
-  stage_ms = {name: float(np.mean([a.elapsed_time(b) for a, b in pairs])) * (len(pairs) / args.steps)
-              for name, pairs in sink.items()}
+  full = _hip.TimingSink(pairs=args.steps * CALLS_PER_STEP)
+  _hip.set_timing_sink(full)
+  for i in range(args.steps):
+    step(i)
+  torch.cuda.synchronize()
+  _hip.set_timing_sink(None)
+  per_step = lambda d: {name: float(np.mean([a.elapsed_time(b) for a, b in pairs])) *
+                        (len(pairs) / args.steps) for name, pairs in d.items()}
+  stage_ms = per_step(full)
+  stage_ms.update(per_step(sink))
   T = G * m
   # Dominant kernel: the expert GEMM, weight-bandwidth bound here (1.2 GB of weights
   # for 309 GFLOP): algorithmic bytes = weights + slot activations in and out + hidden.
@@ -208,23 +217,37 @@ def vit_main(args):
   for i in range(3 + args.warmup):
     step(i)
   torch.cuda.synchronize()
-  sink = _hip.TimingSink(pairs=args.steps * 120)     # about 110 entry-point calls per pass
-  spans["pool"] = _hip.TimingSink(pairs=args.steps * 24)
+  # Timed region: events only around the dominant entry point (the MLP GEMMs); module
+  # spans and the other stages come from a second, fully instrumented pass of the same
+  # steps (events between kernels serialise their hand-over and would slow the pass).
+  sink = _hip.TimingSink(pairs=args.steps * 14, only=("vmoe_expert_mlp",))
   _hip.set_timing_sink(sink)
-  spans["on"] = True
   t0 = time.perf_counter()
   for i in range(args.steps):
     logits, metrics = step(i)
   torch.cuda.synchronize()
   t1 = time.perf_counter()
+  ms = (t1 - t0) * 1e3 / args.steps
+  full = _hip.TimingSink(pairs=args.steps * 120)     # about 110 entry-point calls per pass
+  spans["pool"] = _hip.TimingSink(pairs=args.steps * 24)
+  _hip.set_timing_sink(full)
+  spans["on"] = True
+  ti0 = time.perf_counter()
+  for i in range(args.steps):
+    step(i)
+  torch.cuda.synchronize()
+  ms_instrumented = (time.perf_counter() - ti0) * 1e3 / args.steps
   _hip.set_timing_sink(None)
   spans.pop("on")
   spans.pop("pool")
-  ms = (t1 - t0) * 1e3 / args.steps
   module_ms = {k: float(sum(a.elapsed_time(b) for a, b in v)) / args.steps for k, v in spans.items()}
-  module_ms["other (patch embedding, layer norms, residuals, head)"] = ms - sum(module_ms.values())
-  stage_ms = {name: float(np.mean([a.elapsed_time(b) for a, b in pairs])) * (len(pairs) / args.steps)
-              for name, pairs in sink.items()}
+  per_step = lambda d: {name: float(np.mean([a.elapsed_time(b) for a, b in pairs])) *
+                        (len(pairs) / args.steps) for name, pairs in d.items()}
+  stage_ms = per_step(full)
+  stage_ms.update(per_step(sink))
+  module_ms["other (patch embedding, layer norms, residuals, head)"] = ms_instrumented - sum(
+      module_ms.values())
+  module_ms["instrumented_pass_ms_per_step"] = ms_instrumented
 
   # Dominant kernel: the bf16 GEMM behind the dense and the expert MLPs
   # (two launches per MLP).  Flops: dense 2*T*D*M per launch; experts 2*A*D*M.
@@ -360,7 +383,11 @@ def main():
     out, metrics = step(i)
   torch.cuda.synchronize()
 
-  sink = _hip.TimingSink(pairs=args.steps * CALLS_PER_STEP)
+  # Timed region: only the dominant entry point (the expert GEMMs) carries timing events.
+  # An event between two kernels serialises their hand-over, and eight pairs per step
+  # cost the layer about 6 % of its throughput; the other stages are timed in a second,
+  # fully instrumented pass of the same K steps right after.
+  sink = _hip.TimingSink(pairs=args.steps * 2, only=("vmoe_expert_mlp",))
   _hip.set_timing_sink(sink)
   torch.cuda.synchronize()
   t0 = time.perf_counter()
@@ -372,8 +399,18 @@ def main():
   ms_per_step = (t1 - t0) * 1e3 / args.steps
   tokens_per_s = T / (ms_per_step * 1e-3)
 
-  stage_ms = {name: float(np.mean([a.elapsed_time(b) for a, b in pairs])) * (len(pairs) / args.steps)
-              for name, pairs in sink.items()}
+  def per_step(pairs_by_name):
+    return {name: float(np.mean([a.elapsed_time(b) for a, b in pairs])) * (len(pairs) / args.steps)
+            for name, pairs in pairs_by_name.items()}
+  full = _hip.TimingSink(pairs=args.steps * CALLS_PER_STEP)
+  _hip.set_timing_sink(full)
+  for i in range(args.steps):
+    step(i)
+  torch.cuda.synchronize()
+  _hip.set_timing_sink(None)
+  stage_ms = per_step(full)
+  stage_ms_instrumented_mlp = stage_ms["vmoe_expert_mlp"]
+  stage_ms.update(per_step(sink))          # the GEMMs' time is the one of the timed region
 
   # Kept assignments (rows that carry an item) for the algorithmic flop count.
   gates, val, idx = kernels.gate_topk(xs[0].view(G, S, D), variables["params"]["Router"]["dense"]["kernel"].to(tdt), K,
@@ -465,6 +502,9 @@ def main():
                  "batch_priority": cfg.batch_priority, "capacity_factor": cfg.capacity_factor},
       "roofline": roofline,
       "stage_ms": stage_ms,
+      "stage_ms_note": ("vmoe_expert_mlp: events in the timed region; other stages: second pass of "
+                        "the same steps with events around every call (its vmoe_expert_mlp read "
+                        f"{stage_ms_instrumented_mlp:.4f} ms)"),
       "hbm": hbm,
   }
   if not args.no_cpu_baseline:

@@ -213,10 +213,13 @@ class TimingSink(dict):
   """``sink[name]`` -> list of (start, stop) event pairs, one per call of entry point
   ``name``.  Creating a timing event costs the host far more than recording one, so
   ``pairs`` of them are created (and recorded once, which is when the runtime really
-  allocates them) up front; a measured loop then only records."""
+  allocates them) up front; a measured loop then only records.  An event between two
+  kernels also keeps the second from being set up while the first still runs, so a
+  loop whose total time matters passes ``only`` = the entry points it needs timed."""
 
-  def __init__(self, pairs: int = 0):
+  def __init__(self, pairs: int = 0, only=None):
     super().__init__()
+    self.only = None if only is None else frozenset(only)   # entry points to time; None = all
     self._pool = []
     for _ in range(pairs):
       pair = (torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
@@ -243,7 +246,7 @@ def set_timing_sink(sink) -> None:
 def call(name: str, params: ctypes.Structure) -> None:
   fn = getattr(lib(), name)
   sink = _timing_sink
-  if sink is None:
+  if sink is None or (getattr(sink, "only", None) is not None and name not in sink.only):
     check(fn(ctypes.byref(params), stream()), name)
     return
   take = getattr(sink, "take", None)
