@@ -260,17 +260,20 @@ def vit_main(args):
   # Rows the expert MLPs really compute: the kept assignments of every MoE block
   # (dropped ones are skipped), read from one more, untimed, pass.
   from vmoe_amd import moe as moe_lib
-  live_rows = []
-  packed = moe_lib.ExpertIndicesDispatcher.dispatch_packed
+  live_rows = {}
+  packed = moe_lib.ExpertIndicesDispatcher._packed
 
-  def recording(self, data):
-    out, rows = packed(self, data)
-    live_rows.append(rows)
-    return out, rows
-  moe_lib.ExpertIndicesDispatcher.dispatch_packed = recording
+  def recording(self):
+    maps = packed(self)
+    live_rows[id(self)] = maps[1]          # rows_per_expert of this block's dispatcher
+    recording.keep.append(self)            # keeps ids distinct until they are read
+    return maps
+  recording.keep = []
+  moe_lib.ExpertIndicesDispatcher._packed = recording
   step(0)
   torch.cuda.synchronize()
-  moe_lib.ExpertIndicesDispatcher.dispatch_packed = packed
+  moe_lib.ExpertIndicesDispatcher._packed = packed
+  live_rows = list(live_rows.values())
   kept_per_block = [int(r.sum()) for r in live_rows]
   assert len(kept_per_block) == n_moe
   flops_mlp = 2 * 2.0 * D * M * (n_dense * T + sum(kept_per_block))
@@ -416,7 +419,7 @@ def main():
   gates, val, idx = kernels.gate_topk(xs[0].view(G, S, D), variables["params"]["Router"]["dense"]["kernel"].to(tdt), K,
                                       logit_bias=router_kwargs.get("logit_bias"))
   C = cfg_capacity(cfg)
-  _, token_slot, _, fill = kernels.route_assign(val, idx, E, C, cfg.batch_priority)
+  _, token_slot, slot_token, fill = kernels.route_assign(val, idx, E, C, cfg.batch_priority)
   kept = int(fill.sum())
   b = 2 if tdt == torch.bfloat16 else 4
   # Dominant kernel: the expert GEMM (two launches per step, 2*A*D*M flops each).
@@ -432,8 +435,34 @@ def main():
               "buffer_rows": E * G * C}
 
   # HBM-bound stages, algorithmic bytes (each item row read once, whole buffer written).
-  # dispatch writes only the kept rows (packed layout: no zero fill of empty slots)
-  bytes_dispatch = T * D * b + kept * D * b + 8 * T * K
+  # dispatch: in the bf16 layer the first expert product gathers its rows itself and no
+  # dispatch kernel runs inside the step; the kernel (what ExpertIndicesDispatcher.dispatch
+  # runs: reference layout, every slot row written, empty ones zeroed) is timed on its own.
+  bytes_dispatch = T * D * b + E * G * C * D * b + 8 * T * K
+  if "vmoe_dispatch" not in stage_ms:
+    # the layer through the dispatcher's own dispatch() / combine(), as a caller of the
+    # reference API would run it: same kernels before and after it as in the step
+    router, mlp = layer._modules()
+    p_ = variables["params"]
+
+    def reference_layout_step(i):
+      xg = xs[i % n_rot].view(G, S, D)
+      dispatcher, _ = router.apply({"params": p_["Router"]}, xg)
+      buf = dispatcher.dispatch(xg)
+      return dispatcher.combine(mlp.expert.apply_experts({"params": p_["Mlp"]}, buf))
+    for i in range(3):
+      reference_layout_step(i)
+    ref_sink = _hip.TimingSink(pairs=args.steps * CALLS_PER_STEP)
+    _hip.set_timing_sink(ref_sink)
+    for i in range(args.steps):
+      reference_layout_step(i)
+    torch.cuda.synchronize()
+    _hip.set_timing_sink(None)
+    dispatch_ms = per_step(ref_sink)["vmoe_dispatch"]
+    stage_ms["vmoe_dispatch (reference-layout pass, not in the step)"] = dispatch_ms
+  else:
+    dispatch_ms = stage_ms["vmoe_dispatch"]
+    bytes_dispatch = T * D * b + kept * D * b + 8 * T * K      # packed: kept rows only
   bytes_combine = kept * D * b + 12 * T * K + T * D * b
   bytes_gate = T * D * b + D * E * b + 12 * T * K + T * E * b
   # Measured copy ceiling of the same device (read + write of 512 MiB).
@@ -483,7 +512,7 @@ def main():
     roofline["library_gemm_same_shapes_TFLOPs"] = lib
     del a_up, a_dn, w_up, w_dn
   hbm = {
-      "dispatch_GBps": bytes_dispatch / (stage_ms["vmoe_dispatch"] * 1e-3) / 1e9,
+      "dispatch_GBps": bytes_dispatch / (dispatch_ms * 1e-3) / 1e9,
       "combine_GBps": bytes_combine / (stage_ms["vmoe_combine"] * 1e-3) / 1e9,
       "gate_topk_GBps": bytes_gate / (stage_ms["vmoe_gate_topk"] * 1e-3) / 1e9,
       "copy_kernel_GBps": copy_gbs, "peak_GBps": PEAK_HBM_GBS,

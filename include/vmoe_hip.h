@@ -197,6 +197,8 @@ typedef struct {
   int32_t* token_row;         /* out (G, S, K), -1 for dropped assignments */
   int32_t* rows_per_expert;   /* out (E,) */
   int32_t* prefix;            /* scratch (G, E): rows of expert e taken by the groups before g */
+  int32_t* row_token;         /* optional out (E*G*C,): item (g*S + s) held by each packed row;
+                                 rows past rows_per_expert[e] are not written */
   int32_t G, S, E, K, C;
 } VmoeCompactRowsParams;
 int vmoe_compact_rows(const VmoeCompactRowsParams* p, vmoe_stream_t stream);
@@ -295,6 +297,13 @@ typedef struct {
   const int32_t* rows_per_expert; /* optional (E,): only the first rows_per_expert[e] rows of
                                      expert e hold data; the other rows of x are not read
                                      for results and their rows of out are left untouched */
+  const int32_t* x_rows;          /* optional (E, R), needs rows_per_expert: x is then the
+                                     (num_items, D) matrix of items itself and x_rows[e][r] the
+                                     item in row r of expert e (row_token of vmoe_compact_rows):
+                                     the first product gathers its rows, no dispatched buffer
+                                     is needed.  bf16 with D % 32 == 0 only
+                                     (VMOE_E_UNSUPPORTED otherwise) */
+  int32_t num_items;              /* rows of x when x_rows is given */
 } VmoeExpertMlpParams;
 size_t vmoe_expert_mlp_workspace_bytes(const VmoeExpertMlpParams* p);
 int vmoe_expert_mlp(const VmoeExpertMlpParams* p, vmoe_stream_t stream);

@@ -405,7 +405,7 @@ def test_compact_rows(K, G, S, E, Kk, C, bpr):
   gates = O.softmax(rng.standard_normal((G, S, E)).astype(np.float32) * 2)
   val, idx = K.topk(to_dev(gates), Kk)
   indices, token_slot, slot_token, fill = K.route_assign(val, idx, E, C, bpr)
-  token_row, rows = K.compact_rows(fill, token_slot, C)
+  token_row, rows, row_token = K.compact_rows(fill, token_slot, C)
   f = to_np(fill)
   np.testing.assert_array_equal(to_np(rows), f.sum(0))
   ind = to_np(indices)
@@ -415,6 +415,10 @@ def test_compact_rows(K, G, S, E, Kk, C, bpr):
   want = np.where(kept, e * (G * C) + np.take_along_axis(
       prefix[:, None, :].repeat(S, 1), e, axis=2) + pos, -1)
   np.testing.assert_array_equal(to_np(token_row), want)
+  # row_token is the inverse map on the packed rows
+  tr, rt = to_np(token_row).reshape(G * S, Kk), to_np(row_token).reshape(-1)
+  items = np.repeat(np.arange(G * S), Kk).reshape(G * S, Kk)
+  np.testing.assert_array_equal(rt[tr[tr >= 0]], items[tr >= 0])
   # a bijection onto the first rows of every expert
   r = to_np(token_row)[kept]
   assert len(np.unique(r)) == r.size

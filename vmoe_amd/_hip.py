@@ -151,13 +151,14 @@ class ExpertMlpParams(ctypes.Structure):
               ("b1", c_void_p), ("w0t", c_void_p), ("w1t", c_void_p), ("out", c_void_p),
               ("workspace", c_void_p), ("workspace_bytes", c_size_t),
               ("E", c_int32), ("R", c_int32), ("D", c_int32), ("M", c_int32),
-              ("dtype", c_int32), ("gelu", c_int32), ("rows_per_expert", c_void_p)]
+              ("dtype", c_int32), ("gelu", c_int32), ("rows_per_expert", c_void_p),
+              ("x_rows", c_void_p), ("num_items", c_int32)]
 
 
 class CompactRowsParams(ctypes.Structure):
   _fields_ = [("fill", c_void_p), ("token_slot", c_void_p), ("token_row", c_void_p),
-              ("rows_per_expert", c_void_p), ("prefix", c_void_p), ("G", c_int32), ("S", c_int32),
-              ("E", c_int32), ("K", c_int32), ("C", c_int32)]
+              ("rows_per_expert", c_void_p), ("prefix", c_void_p), ("row_token", c_void_p),
+              ("G", c_int32), ("S", c_int32), ("E", c_int32), ("K", c_int32), ("C", c_int32)]
 
 
 class TransposeParams(ctypes.Structure):

@@ -211,6 +211,11 @@ static int check_mlp(const VmoeExpertMlpParams* p) {
   if (p == nullptr || p->x == nullptr || p->out == nullptr) return VMOE_E_NULL;
   if (p->E < 1 || p->R < 1 || p->D < 1 || p->M < 1) return VMOE_E_SHAPE;
   if (p->dtype != VMOE_F32 && p->dtype != VMOE_BF16) return VMOE_E_DTYPE;
+  if (p->x_rows != nullptr) {
+    if (p->rows_per_expert == nullptr) return VMOE_E_NULL;
+    if (p->num_items < 1) return VMOE_E_SHAPE;
+    if (p->dtype != VMOE_BF16) return VMOE_E_UNSUPPORTED;
+  }
   if (p->gelu != VMOE_GELU_TANH && p->gelu != VMOE_GELU_ERF) return VMOE_E_DTYPE;
   if (p->dtype == VMOE_BF16) {
     if ((p->w0 == nullptr && p->w0t == nullptr) || (p->w1 == nullptr && p->w1t == nullptr))
@@ -288,12 +293,12 @@ extern "C" int vmoe_expert_mlp(const VmoeExpertMlpParams* p, vmoe_stream_t strea
       rc = launch_gemm_bf16<CfgUp, kEpiBiasGeluTanh>((const bf16_t*)p->x, (const bf16_t*)w0t,
                                                       (const bf16_t*)p->b0, (bf16_t*)hidden, p->E,
                                                       p->R, p->M, p->D, stream, p->rows_per_expert,
-                                                      plan_up);
+                                                      plan_up, p->x_rows, p->num_items);
     else
       rc = launch_gemm_bf16<CfgUp, kEpiBiasGeluErf>((const bf16_t*)p->x, (const bf16_t*)w0t,
                                                      (const bf16_t*)p->b0, (bf16_t*)hidden, p->E,
                                                      p->R, p->M, p->D, stream, p->rows_per_expert,
-                                                     plan_up);
+                                                     plan_up, p->x_rows, p->num_items);
     if (rc != VMOE_OK) return rc;
     return launch_gemm_bf16<CfgDown, kEpiBias>((const bf16_t*)hidden, (const bf16_t*)w1t,
                                               (const bf16_t*)p->b1, (bf16_t*)p->out, p->E, p->R,

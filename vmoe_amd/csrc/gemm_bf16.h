@@ -306,7 +306,7 @@ __global__ __launch_bounds__(Cfg::kThreads, Cfg::kBlocksPerCu) void gemm_bf16_ke
     const bf16_t* __restrict__ A, const bf16_t* __restrict__ Bt, const bf16_t* __restrict__ bias,
     bf16_t* __restrict__ C, int R, int N, int Kd, int tiles_m, int tiles_n, int num_tiles,
     int tiles_per_xcd, int panel_rows, const int32_t* __restrict__ rows,
-    const int4* __restrict__ plan) {
+    const int4* __restrict__ plan, const int32_t* __restrict__ a_rows) {
 #if defined(__HIP_DEVICE_COMPILE__)   // buffer-resource builtins exist in the device pass only
   extern __shared__ __align__(1024) unsigned char smem[];
   constexpr int BM = Cfg::BM, BN = Cfg::BN, BK = Cfg::BK;
@@ -337,7 +337,11 @@ __global__ __launch_bounds__(Cfg::kThreads, Cfg::kBlocksPerCu) void gemm_bf16_ke
     }
   }
   const int row0 = tile_m * BM, col0 = tile_n * BN;
-  const unsigned char* Ab = reinterpret_cast<const unsigned char*>(A + (size_t)b * R * Kd);
+  // With a_rows, A is a matrix of items shared by all batches and a_rows[b * R + r] names
+  // the item that row r of batch b holds: the gather of the dispatch step happens here,
+  // in the operand load, and the dispatched buffer never exists.
+  const unsigned char* Ab = reinterpret_cast<const unsigned char*>(
+      a_rows != nullptr ? A : A + (size_t)b * R * Kd);
   const unsigned char* Bb = reinterpret_cast<const unsigned char*>(Bt + (size_t)b * N * Kd);
 
   // Byte offsets of this lane's chunk in each of its load instructions.  Lane L
@@ -353,7 +357,9 @@ __global__ __launch_bounds__(Cfg::kThreads, Cfg::kBlocksPerCu) void gemm_bf16_ke
 #pragma unroll
   for (int i = 0; i < Cfg::kAIssues; ++i) {
     int r = (i * Cfg::kWaves + wave) * RPL + lrow;
-    a_goff[i] = (uint32_t)min(row0 + r, R - 1) * (uint32_t)Kd * 2u + chunk * 16;
+    int arow = min(row0 + r, (a_rows != nullptr ? live : R) - 1);
+    if (a_rows != nullptr) arow = a_rows[(size_t)b * R + arow];
+    a_goff[i] = (uint32_t)arow * (uint32_t)Kd * 2u + chunk * 16;
   }
 #pragma unroll
   for (int i = 0; i < Cfg::kBIssues; ++i) {
@@ -652,8 +658,12 @@ GemmGeom gemm_geometry(int batch, int R, int N, int Kd) {
 template <typename Cfg, int EPI>
 int launch_gemm_bf16(const bf16_t* A, const bf16_t* Bt, const bf16_t* bias, bf16_t* C, int batch,
                      int R, int N, int Kd, hipStream_t stream, const int32_t* rows = nullptr,
-                     const int4* plan = nullptr) {
+                     const int4* plan = nullptr, const int32_t* a_rows = nullptr,
+                     long long a_items = 0) {
   const GemmGeom g = gemm_geometry<Cfg>(batch, R, N, Kd);
+  if (a_rows != nullptr && (!g.fast || rows == nullptr ||
+                            (unsigned long long)a_items * Kd * 2 >= (1ull << 32)))
+    return VMOE_E_UNSUPPORTED;     // the gathering load exists in the LDS-DMA kernel only
   if (!g.fast) {
     const int tiles_m = (R + 127) / 128, tiles_n = (N + 127) / 128;
     const long long blocks = (long long)batch * tiles_m * tiles_n;
@@ -671,7 +681,7 @@ int launch_gemm_bf16(const bf16_t* A, const bf16_t* Bt, const bf16_t* bias, bf16
   if (e != hipSuccess) return (int)e;
   hipLaunchKernelGGL(kern, dim3(blocks), dim3(Cfg::kThreads), Cfg::kLdsBytes, stream, A, Bt, bias,
                      C, R, N, Kd, g.tiles_m, g.tiles_n, (int)g.tiles, g.tiles_per_xcd, g.panel_rows,
-                     rows, plan);
+                     rows, plan, a_rows);
   return launch_status();
 }
 

@@ -263,7 +263,8 @@ __global__ __launch_bounds__(256) void fill_prefix_kernel(
 // Step 2: token_slot = e*G*C + r(g, c)  ->  token_row = e*G*C + prefix[g][e] + c.
 __global__ __launch_bounds__(256) void compact_rows_kernel(
     const int32_t* __restrict__ prefix, const int32_t* __restrict__ token_slot,
-    int32_t* __restrict__ token_row, int G, int E, int C, int per_group, size_t n) {
+    int32_t* __restrict__ token_row, int32_t* __restrict__ row_token, int G, int E, int C,
+    int per_group, int K, size_t n) {
   const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
   if (i >= n) return;
   const int slot = token_slot[i];
@@ -274,6 +275,7 @@ __global__ __launch_bounds__(256) void compact_rows_kernel(
     const int e = slot / per_expert;
     const int c = (slot - e * per_expert) % C;
     row = e * per_expert + prefix[(size_t)g * E + e] + c;
+    if (row_token != nullptr) row_token[row] = (int)(i / K);
   }
   token_row[i] = row;
 }
@@ -381,7 +383,7 @@ extern "C" int vmoe_compact_rows(const VmoeCompactRowsParams* p, vmoe_stream_t s
                      p->prefix, p->rows_per_expert, p->G, p->E);
   const size_t n = (size_t)p->G * p->S * p->K;
   hipLaunchKernelGGL(compact_rows_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0,
-                     as_stream(stream), p->prefix, p->token_slot, p->token_row, p->G, p->E, p->C,
-                     p->S * p->K, n);
+                     as_stream(stream), p->prefix, p->token_slot, p->token_row, p->row_token, p->G,
+                     p->E, p->C, p->S * p->K, p->K, n);
   return launch_status();
 }

@@ -146,16 +146,18 @@ def indices_to_slots(indices: torch.Tensor, num_experts: int, capacity: int):
 
 def compact_rows(fill: torch.Tensor, token_slot: torch.Tensor, capacity: int):
   """fill (G,E), token_slot (G,S,K) -> token_row (G,S,K): the kept assignments of every
-  expert renumbered into the first rows of its block; rows_per_expert (E,)."""
+  expert renumbered into the first rows of its block; rows_per_expert (E,); row_token
+  (E, G*C): the item in every packed row (rows past an expert's count are unset)."""
   G, E = fill.shape
   _, S, K = token_slot.shape
   token_row = _i32(G, S, K, device=fill.device)
   rows = _i32(E, device=fill.device)
   prefix = _i32(G, E, device=fill.device)
+  row_token = _i32(E, G * capacity, device=fill.device)
   p = H.CompactRowsParams(H.ptr(fill), H.ptr(token_slot), H.ptr(token_row), H.ptr(rows),
-                          H.ptr(prefix), G, S, E, K, capacity)
+                          H.ptr(prefix), H.ptr(row_token), G, S, E, K, capacity)
   H.call("vmoe_compact_rows", p)
-  return token_row, rows
+  return token_row, rows, row_token
 
 
 def dispatch(x: torch.Tensor, token_slot: torch.Tensor, slot_token: Optional[torch.Tensor],
@@ -243,17 +245,26 @@ def pack_expert_weights(w: torch.Tensor) -> torch.Tensor:
 
 def expert_mlp(x: torch.Tensor, w0, b0, w1, b1, w0t=None, w1t=None, approximate_gelu: bool = True,
                workspace: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None,
-               rows_per_expert: Optional[torch.Tensor] = None):
+               rows_per_expert: Optional[torch.Tensor] = None,
+               x_rows: Optional[torch.Tensor] = None):
   """x (E,R,D) -> (E,R,D): gelu(x @ w0 + b0) @ w1 + b1 per expert; with rows_per_expert (E,)
-  int32 only that many leading rows of every expert are computed."""
-  E, R, D = x.shape
+  int32 only that many leading rows of every expert are computed.  With x_rows (E,R) int32,
+  x is the (T,D) matrix of items and x_rows names the item of every row (gathered by the
+  first product; see expert_mlp_can_gather)."""
+  num_items = 0
+  if x_rows is not None:
+    E, R = x_rows.shape
+    num_items, D = x.shape
+  else:
+    E, R, D = x.shape
   M = (w0.shape[2] if w0 is not None else w0t.shape[1])
   x = x.contiguous()
   if out is None:
-    out = torch.empty_like(x)
+    out = torch.empty((E, R, D), dtype=x.dtype, device=x.device)
   p = H.ExpertMlpParams(H.ptr(x), H.ptr(w0), H.ptr(b0), H.ptr(w1), H.ptr(b1), H.ptr(w0t),
                         H.ptr(w1t), H.ptr(out), None, 0, E, R, D, M, H.dtype_code(x.dtype),
-                        H.GELU_TANH if approximate_gelu else H.GELU_ERF, H.ptr(rows_per_expert))
+                        H.GELU_TANH if approximate_gelu else H.GELU_ERF, H.ptr(rows_per_expert),
+                        H.ptr(x_rows), num_items)
   need = H.lib().vmoe_expert_mlp_workspace_bytes(H.ctypes.byref(p))
   if workspace is None or workspace.numel() * workspace.element_size() < need:
     workspace = torch.empty(need, dtype=torch.uint8, device=x.device)
@@ -261,6 +272,11 @@ def expert_mlp(x: torch.Tensor, w0, b0, w1, b1, w0t=None, w1t=None, approximate_
   p.workspace_bytes = workspace.numel() * workspace.element_size()
   H.call("vmoe_expert_mlp", p)
   return out
+
+
+def expert_mlp_can_gather(dtype: torch.dtype, D: int, num_items: int) -> bool:
+  """Whether expert_mlp can take the items themselves plus x_rows (no dispatched buffer)."""
+  return dtype == torch.bfloat16 and D % 32 == 0 and num_items * D * 2 < (1 << 32)
 
 
 def expert_mlp_workspace_bytes(E, R, D, M, dtype, prepacked: bool) -> int:

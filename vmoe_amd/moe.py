@@ -189,11 +189,17 @@ class ExpertIndicesDispatcher(BaseDispatcher):
       self._packed_maps = K.compact_rows(self.fill, token_slot, self.capacity)
     return self._packed_maps
 
+  def packed_rows(self):
+    """-> (row_token (E, G * capacity) int32: the item (g * S + s) in every packed row,
+    rows_per_expert (E,) int32): what an expert needs to gather its rows itself."""
+    _, rows_per_expert, row_token = self._packed()
+    return row_token, rows_per_expert
+
   def dispatch_packed(self, data: Array):
     """-> (buffer (E, G * capacity, ...) whose expert e holds items in rows
     0 .. rows_per_expert[e] - 1 and arbitrary values after them, rows_per_expert (E,) int32)."""
     G, S, Kk, _ = self.indices.shape
-    token_row, rows_per_expert = self._packed()
+    token_row, rows_per_expert, _ = self._packed()
     rows, item_shape, width = _as_rows(data, 2)
     out = K.dispatch(rows, token_row.view(G * S, Kk), None,
                      num_slots=self.num_experts * G * self.capacity)
@@ -202,7 +208,7 @@ class ExpertIndicesDispatcher(BaseDispatcher):
 
   def combine_packed(self, data: Array) -> Array:
     G, S, Kk, _ = self.indices.shape
-    token_row, _ = self._packed()
+    token_row = self._packed()[0]
     rows, item_shape, width = _as_rows(data, 2)
     w = self._weights_f32 if self._weights_f32 is not None else K.cast(
         self.combine_weights.contiguous(), torch.float32)
@@ -316,6 +322,9 @@ class _SparseEinsumDispatcher(EinsumDispatcher):
 
   def dispatch_packed(self, data: Array):
     return self._inner.dispatch_packed(data)
+
+  def packed_rows(self):
+    return self._inner.packed_rows()
 
   def combine_packed(self, data: Array) -> Array:
     return self._inner.combine_packed(data)
@@ -587,9 +596,18 @@ def sparse_moe_spmd(target, variable_axes: Optional[Mapping[str, Any]] = None,
           and getattr(self.expert, "supports_packed_rows", False)
           and not _wants_grad(inputs[0])):
         # Each expert's items in its first rows; the expert skips the empty ones.
-        dispatched, rows_per_expert = dispatcher.dispatch_packed(inputs[0])
-        outputs = self.expert.apply_experts(variables, dispatched,
-                                            rows_per_expert=rows_per_expert)
+        gather = getattr(self.expert, "apply_experts_gathered", None)
+        packed_rows = getattr(dispatcher, "packed_rows", None)
+        x = inputs[0]
+        if (gather is not None and packed_rows is not None and x.ndim == 3
+            and self.expert.can_gather(x)):
+          # ... and fetches them from the items itself: no dispatched buffer at all.
+          row_token, rows_per_expert = packed_rows()
+          outputs = gather(variables, x.reshape(-1, x.shape[-1]), row_token, rows_per_expert)
+        else:
+          dispatched, rows_per_expert = dispatcher.dispatch_packed(x)
+          outputs = self.expert.apply_experts(variables, dispatched,
+                                              rows_per_expert=rows_per_expert)
         return _tree_map(dispatcher.combine_packed, outputs)
       dispatched = [dispatcher.dispatch(x) for x in inputs]
       if hasattr(self.expert, "apply_experts"):

@@ -71,6 +71,27 @@ class MlpBlock(module.Module):
     return K.expert_mlp(x, cast(w0), cast(b0), cast(w1), cast(b1),
                         approximate_gelu=self.approximate_gelu, rows_per_expert=rows_per_expert)
 
+  def can_gather(self, items: Array) -> bool:
+    """Whether apply_experts_gathered covers these items (dtype and width of the kernel)."""
+    dtype = self.dtype or items.dtype
+    return (items.is_cuda and dtype == torch.bfloat16 and items.dtype == torch.bfloat16
+            and K.expert_mlp_can_gather(dtype, items.shape[-1], items.numel() // items.shape[-1]))
+
+  def apply_experts_gathered(self, variables, items: Array, row_token: Array,
+                             rows_per_expert: Array) -> Array:
+    """items (T, D); row_token (E, R) int32 names the item in row r of expert e,
+    rows_per_expert (E,) how many rows each expert has -> (E, R, D).  The first product
+    reads its rows straight from ``items``: the dispatched buffer is never built."""
+    p = variables["params"]
+    dtype = self.dtype or items.dtype
+    w0, b0 = p["Dense_0"]["kernel"], p["Dense_0"].get("bias")
+    w1, b1 = p["Dense_1"]["kernel"], p["Dense_1"].get("bias")
+    cast = lambda t: None if t is None else K.cast(t, dtype)
+    return K.expert_mlp(K.cast(items, dtype), None, cast(b0), None, cast(b1),
+                        w0t=self._pack(w0, dtype), w1t=self._pack(w1, dtype),
+                        approximate_gelu=self.approximate_gelu, rows_per_expert=rows_per_expert,
+                        x_rows=row_token)
+
   def apply(self, variables, inputs: Array) -> Array:
     """Single MLP: inputs (..., D)."""
     stacked = vmoe_amd.moe._tree_map(lambda t: t[None], variables)
