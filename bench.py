@@ -35,9 +35,9 @@ PEAK_HBM_GBS = 8000.0
 # HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc runs
 # (FETCH_SIZE + WRITE_SIZE, scaled by a copy kernel of known size); None until measured.
 MEASURED_TRAFFIC_BYTES = {
-    # mean of the two GEMM launches of a layer: (872 + 565 + 1185 + 169) / 2 MiB;
+    # mean of the two GEMM launches of a layer: (894 + 565 + 1177 + 169) / 2 MiB;
     # FETCH_SIZE x 2.0, WRITE_SIZE x 1.0 (copy-kernel calibration).
-    "vmoe_b16_layer_E32_k2_bpr": 1.463e9,
+    "vmoe_b16_layer_E32_k2_bpr": 1.470e9,
 }
 
 
@@ -48,6 +48,9 @@ def parse_args():
   ap.add_argument("--warmup", type=int, default=5)
   ap.add_argument("--config", default="vmoe_b16_layer_E32_k2_bpr")
   ap.add_argument("--no-cpu-baseline", action="store_true")
+  ap.add_argument("--no-dispatch-pass", action="store_true",
+                  help="skip the extra pass that times dispatcher.dispatch() (for counter runs "
+                       "that should see the step's kernels only)")
   ap.add_argument("--cpu-groups", type=int, default=2,
                   help="groups of the workload the CPU baseline is timed on")
   return ap.parse_args()
@@ -439,7 +442,10 @@ def main():
   # dispatch kernel runs inside the step; the kernel (what ExpertIndicesDispatcher.dispatch
   # runs: reference layout, every slot row written, empty ones zeroed) is timed on its own.
   bytes_dispatch = T * D * b + E * G * C * D * b + 8 * T * K
-  if "vmoe_dispatch" not in stage_ms:
+  dispatch_ms = None
+  if "vmoe_dispatch" not in stage_ms and args.no_dispatch_pass:
+    pass
+  elif "vmoe_dispatch" not in stage_ms:
     # the layer through the dispatcher's own dispatch() / combine(), as a caller of the
     # reference API would run it: same kernels before and after it as in the step
     router, mlp = layer._modules()
@@ -512,12 +518,12 @@ def main():
     roofline["library_gemm_same_shapes_TFLOPs"] = lib
     del a_up, a_dn, w_up, w_dn
   hbm = {
-      "dispatch_GBps": bytes_dispatch / (dispatch_ms * 1e-3) / 1e9,
+      "dispatch_GBps": bytes_dispatch / (dispatch_ms * 1e-3) / 1e9 if dispatch_ms else None,
       "combine_GBps": bytes_combine / (stage_ms["vmoe_combine"] * 1e-3) / 1e9,
       "gate_topk_GBps": bytes_gate / (stage_ms["vmoe_gate_topk"] * 1e-3) / 1e9,
       "copy_kernel_GBps": copy_gbs, "peak_GBps": PEAK_HBM_GBS,
   }
-  hbm["dispatch_frac_of_peak"] = hbm["dispatch_GBps"] / PEAK_HBM_GBS
+  hbm["dispatch_frac_of_peak"] = hbm["dispatch_GBps"] / PEAK_HBM_GBS if dispatch_ms else None
   hbm["combine_frac_of_peak"] = hbm["combine_GBps"] / PEAK_HBM_GBS
 
   result = {
