@@ -339,6 +339,19 @@ typedef struct {
 size_t vmoe_soft_route_workspace_bytes(const VmoeSoftRouteParams* p);
 int vmoe_soft_route(const VmoeSoftRouteParams* p, vmoe_stream_t stream);
 
+/* Monitoring scalars of SoftRouter.get_metrics (vmoe/projects/soft_moe/router.py:119-125):
+ * partial[g] = (sum_s min_n combine_w, sum_s max_n combine_w, sum_n min_s dispatch_w,
+ * sum_n max_s dispatch_w) for group g; the four metrics are the sums over g divided
+ * by G*S (combine) and G*N (dispatch). */
+typedef struct {
+  const void* combine_w;   /* (G, S, N) dtype */
+  const void* dispatch_w;  /* (G, S, N) dtype */
+  float* partial;          /* out (G, 4) float32 */
+  int32_t G, S, N;
+  int32_t dtype;
+} VmoeSoftStatsParams;
+int vmoe_soft_router_stats(const VmoeSoftStatsParams* p, vmoe_stream_t stream);
+
 /* EinsumDispatcher.dispatch / .combine with dense weights
  * (vmoe/moe.py:148-161): per group,
  *   dispatch: out[slot(g,n)] = sum_s w[g,s,n] * x[g,s,:]

@@ -68,7 +68,8 @@ def test_struct_layouts_match_header():
         "VmoeAttentionParams": _hip.AttentionParams,
         "VmoeNoisyGatesParams": _hip.NoisyGatesParams,
         "VmoeCompactRowsParams": _hip.CompactRowsParams,
-        "VmoeCombineBackwardParams": _hip.CombineBackwardParams}
+        "VmoeCombineBackwardParams": _hip.CombineBackwardParams,
+        "VmoeSoftStatsParams": _hip.SoftStatsParams}
   assert set(py) == set(structs)
   for name, body in structs.items():
     want = []

@@ -448,3 +448,15 @@ def test_expert_mlp_rows_per_expert(K, dtype, E):
   for e, n in enumerate(rows):
     np.testing.assert_array_equal(to_np(out[e, :n]), to_np(full[e, :n]))
     assert (to_np(out[e, n:]) == 7.0).all()
+
+
+@pytest.mark.parametrize("G,S,N,dtype", [(3, 50, 16, O.F32), (4, 196, 128, O.BF16), (2, 7, 300, O.BF16), (3, 196, 128, O.F32),
+                          (2, 9, 96, O.BF16), (5, 33, 8, O.BF16), (2, 300, 512, O.BF16)])
+def test_soft_router_stats(K, G, S, N, dtype):
+  """The four means of vmoe/projects/soft_moe/router.py:119-125 in one kernel."""
+  rng = np.random.default_rng(G + S + N)
+  cw = O.cast(O.softmax(rng.standard_normal((G, S, N)).astype(np.float32), axis=2), dtype)
+  dw = O.cast(O.softmax(rng.standard_normal((G, S, N)).astype(np.float32), axis=1), dtype)
+  got = [float(v) for v in K.soft_router_stats(to_dev(cw, dtype), to_dev(dw, dtype))]
+  want = [cw.min(axis=2).mean(), cw.max(axis=2).mean(), dw.min(axis=1).mean(), dw.max(axis=1).mean()]
+  np.testing.assert_allclose(got, want, rtol=2e-6)

@@ -26,7 +26,7 @@ EXPORTS = [
     "vmoe_soft_route_workspace_bytes", "vmoe_soft_route", "vmoe_einsum_dispatch",
     "vmoe_einsum_combine", "vmoe_cast", "vmoe_copy_bytes", "vmoe_mfma_probe",
     "vmoe_add_layer_norm", "vmoe_attention", "vmoe_noisy_gates", "vmoe_compact_rows",
-    "vmoe_combine_backward_data", "vmoe_combine_backward_weights",
+    "vmoe_combine_backward_data", "vmoe_combine_backward_weights", "vmoe_soft_router_stats",
 ]
 
 
@@ -182,6 +182,11 @@ class EinsumParams(ctypes.Structure):
 class CastParams(ctypes.Structure):
   _fields_ = [("in_", c_void_p), ("out", c_void_p), ("n", c_size_t),
               ("in_dtype", c_int32), ("out_dtype", c_int32)]
+
+
+class SoftStatsParams(ctypes.Structure):
+  _fields_ = [("combine_w", c_void_p), ("dispatch_w", c_void_p), ("partial", c_void_p),
+              ("G", c_int32), ("S", c_int32), ("N", c_int32), ("dtype", c_int32)]
 
 
 class CombineBackwardParams(ctypes.Structure):

@@ -568,6 +568,145 @@ int check_einsum(const VmoeEinsumParams* p, bool dispatch) {
   return VMOE_OK;
 }
 
+
+// Monitoring scalars of the Soft MoE router (vmoe/projects/soft_moe/router.py:119-125),
+// per group: sum over items of the min / max over slots of the combine weights, and
+// sum over slots of the min / max over items of the dispatch weights.  The caller
+// sums the (G, 4) partials and divides by the counts.
+template <typename T>
+__global__ __launch_bounds__(256) void soft_stats_kernel(const T* __restrict__ combine_w,
+                                                         const T* __restrict__ dispatch_w,
+                                                         float* __restrict__ partial, int S, int N) {
+  __shared__ float red[4][4];
+  const int g = blockIdx.x;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const T* cw = combine_w + (size_t)g * S * N;
+  const T* dw = dispatch_w + (size_t)g * S * N;
+  // combine weights: a wave per item row
+  float cmin_sum = 0.f, cmax_sum = 0.f;
+  for (int r = wave; r < S; r += 4) {
+    float mn = INFINITY, mx = -INFINITY;
+    for (int c = lane; c < N; c += 64) {
+      const float v = Elt<T>::load(cw + (size_t)r * N + c);
+      mn = fminf(mn, v);
+      mx = fmaxf(mx, v);
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+      mn = fminf(mn, __shfl_xor(mn, o, 64));
+      mx = fmaxf(mx, __shfl_xor(mx, o, 64));
+    }
+    cmin_sum += mn;
+    cmax_sum += mx;
+  }
+  // dispatch weights: a thread per slot column
+  float dmin_sum = 0.f, dmax_sum = 0.f;
+  for (int c = tid; c < N; c += 256) {
+    float mn = INFINITY, mx = -INFINITY;
+    for (int r = 0; r < S; ++r) {
+      const float v = Elt<T>::load(dw + (size_t)r * N + c);
+      mn = fminf(mn, v);
+      mx = fmaxf(mx, v);
+    }
+    dmin_sum += mn;
+    dmax_sum += mx;
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    dmin_sum += __shfl_xor(dmin_sum, o, 64);
+    dmax_sum += __shfl_xor(dmax_sum, o, 64);
+  }
+  if (lane == 0) {
+    red[wave][0] = cmin_sum; red[wave][1] = cmax_sum;
+    red[wave][2] = dmin_sum; red[wave][3] = dmax_sum;
+  }
+  __syncthreads();
+  if (tid < 4) partial[(size_t)g * 4 + tid] = red[0][tid] + red[1][tid] + red[2][tid] + red[3][tid];
+}
+
+template <typename T> __device__ __forceinline__ void unpack16(uint4 q, float* v);
+template <> __device__ __forceinline__ void unpack16<float>(uint4 q, float* v) {
+  v[0] = __builtin_bit_cast(float, q.x); v[1] = __builtin_bit_cast(float, q.y);
+  v[2] = __builtin_bit_cast(float, q.z); v[3] = __builtin_bit_cast(float, q.w);
+}
+template <> __device__ __forceinline__ void unpack16<bf16_t>(uint4 q, float* v) {
+  v[0] = bf_lo(q.x); v[1] = bf_hi(q.x); v[2] = bf_lo(q.y); v[3] = bf_hi(q.y);
+  v[4] = bf_lo(q.z); v[5] = bf_hi(q.z); v[6] = bf_lo(q.w); v[7] = bf_hi(q.w);
+}
+
+// The same sums with 16-byte loads when a row is a power-of-two number NC <= 64 of
+// 16-byte chunks.  blockIdx.y = 0 takes the combine weights (a row's chunks sit in NC
+// adjacent lanes, so the row minimum is a lane exchange), blockIdx.y = 1 the dispatch
+// weights (a thread keeps one chunk column over all its rows; the 256 / NC threads of
+// a column meet in LDS).
+template <typename T>
+__global__ __launch_bounds__(256) void soft_stats_vec_kernel(const T* __restrict__ combine_w,
+                                                             const T* __restrict__ dispatch_w,
+                                                             float* __restrict__ partial, int S, int N) {
+  constexpr int V = 16 / sizeof(T);
+  __shared__ float lds_min[256 * V];
+  __shared__ float lds_max[256 * V];
+  __shared__ float red[4][2];
+  const int g = blockIdx.x;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int NC = N / V;
+  const int total = S * NC;
+  float sum_min = 0.f, sum_max = 0.f;
+  if (blockIdx.y == 0) {
+    const uint4* src = reinterpret_cast<const uint4*>(combine_w + (size_t)g * S * N);
+    const int rounds = (total + 255) / 256;
+    for (int k = 0; k < rounds; ++k) {
+      const int i = k * 256 + tid;
+      float mn = INFINITY, mx = -INFINITY;
+      if (i < total) {
+        float v[V];
+        unpack16<T>(src[i], v);
+#pragma unroll
+        for (int j = 0; j < V; ++j) { mn = fminf(mn, v[j]); mx = fmaxf(mx, v[j]); }
+      }
+      for (int o = 1; o < NC; o <<= 1) {
+        mn = fminf(mn, __shfl_xor(mn, o, 64));
+        mx = fmaxf(mx, __shfl_xor(mx, o, 64));
+      }
+      if (i < total && (lane & (NC - 1)) == 0) { sum_min += mn; sum_max += mx; }
+    }
+  } else {
+    const uint4* src = reinterpret_cast<const uint4*>(dispatch_w + (size_t)g * S * N);
+    float mn[V], mx[V];
+#pragma unroll
+    for (int j = 0; j < V; ++j) { mn[j] = INFINITY; mx[j] = -INFINITY; }
+    for (int i = tid; i < total; i += 256) {
+      float v[V];
+      unpack16<T>(src[i], v);
+#pragma unroll
+      for (int j = 0; j < V; ++j) { mn[j] = fminf(mn[j], v[j]); mx[j] = fmaxf(mx[j], v[j]); }
+    }
+    // thread t holds chunk column t % NC; LDS as [t / NC][column * V + j]
+#pragma unroll
+    for (int j = 0; j < V; ++j) {
+      lds_min[(tid / NC) * N + (tid % NC) * V + j] = mn[j];
+      lds_max[(tid / NC) * N + (tid % NC) * V + j] = mx[j];
+    }
+    __syncthreads();
+    const int parts = 256 / NC;
+    for (int c = tid; c < N; c += 256) {
+      float a = INFINITY, b = -INFINITY;
+      for (int q = 0; q < parts; ++q) { a = fminf(a, lds_min[q * N + c]); b = fmaxf(b, lds_max[q * N + c]); }
+      sum_min += a;
+      sum_max += b;
+    }
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    sum_min += __shfl_xor(sum_min, o, 64);
+    sum_max += __shfl_xor(sum_max, o, 64);
+  }
+  if (lane == 0) { red[wave][0] = sum_min; red[wave][1] = sum_max; }
+  __syncthreads();
+  if (tid < 2)
+    partial[(size_t)g * 4 + blockIdx.y * 2 + tid] = red[0][tid] + red[1][tid] + red[2][tid] + red[3][tid];
+}
+
 }  // namespace
 }  // namespace vmoe
 
@@ -656,5 +795,34 @@ extern "C" int vmoe_einsum_combine(const VmoeEinsumParams* p, vmoe_stream_t stre
   dim3 grid((p->D + 63) / 64, (p->S + 63) / 64, p->G);
   hipLaunchKernelGGL(einsum_kernel<false>, grid, dim3(256), 0, as_stream(stream), p->w, p->data,
                      p->out, p->G, p->S, p->E, p->C, p->D, p->w_dtype, p->data_dtype, p->out_dtype);
+  return launch_status();
+}
+
+extern "C" int vmoe_soft_router_stats(const VmoeSoftStatsParams* p, vmoe_stream_t stream) {
+  if (p == nullptr || p->combine_w == nullptr || p->dispatch_w == nullptr || p->partial == nullptr)
+    return VMOE_E_NULL;
+  if (p->G < 1 || p->S < 1 || p->N < 1) return VMOE_E_SHAPE;
+  if (p->dtype != VMOE_BF16 && p->dtype != VMOE_F32) return VMOE_E_DTYPE;
+  const int vec = p->dtype == VMOE_BF16 ? 8 : 4;
+  const int nc = p->N / vec;
+  const bool wide = p->N % vec == 0 && nc <= 64 && (nc & (nc - 1)) == 0 &&
+                    aligned16(p->combine_w) && aligned16(p->dispatch_w) && p->G <= 65535 * 32;
+  hipStream_t s = as_stream(stream);
+  if (wide && p->dtype == VMOE_BF16)
+    hipLaunchKernelGGL(soft_stats_vec_kernel<bf16_t>, dim3(p->G, 2), dim3(256), 0, s,
+                       (const bf16_t*)p->combine_w, (const bf16_t*)p->dispatch_w, p->partial, p->S,
+                       p->N);
+  else if (wide)
+    hipLaunchKernelGGL(soft_stats_vec_kernel<float>, dim3(p->G, 2), dim3(256), 0, s,
+                       (const float*)p->combine_w, (const float*)p->dispatch_w, p->partial, p->S,
+                       p->N);
+  else if (p->dtype == VMOE_BF16)
+    hipLaunchKernelGGL(soft_stats_kernel<bf16_t>, dim3(p->G), dim3(256), 0, s,
+                       (const bf16_t*)p->combine_w, (const bf16_t*)p->dispatch_w, p->partial, p->S,
+                       p->N);
+  else
+    hipLaunchKernelGGL(soft_stats_kernel<float>, dim3(p->G), dim3(256), 0, s,
+                       (const float*)p->combine_w, (const float*)p->dispatch_w, p->partial, p->S,
+                       p->N);
   return launch_status();
 }

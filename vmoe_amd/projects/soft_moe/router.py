@@ -61,7 +61,7 @@ class SoftRouter(module.Module):
     if tuple(mu.shape) != (dim, self.num_experts, num_slots):
       raise ValueError(f"mu has shape {tuple(mu.shape)}, expected {(dim, self.num_experts, num_slots)}")
     n, s = self.num_experts, num_slots
-    dw, cw = K.soft_route(x, K.cast(mu, dtype).reshape(dim, n * s), float(p["scale"]))
+    dw, cw = K.soft_route(x, K.cast(mu, dtype).reshape(dim, n * s), self._scale_value(p["scale"]))
     dispatch_weights = dw.view(G, m, n, s)
     combine_weights = cw.view(G, m, n, s)
     dispatcher = EinsumDispatcher(combine_weights, dispatch_weights,
@@ -71,18 +71,33 @@ class SoftRouter(module.Module):
     metrics = self.get_metrics(combine_weights, dispatch_weights, K.cast(mu, dtype))
     return dispatcher, metrics
 
+  def _scale_value(self, scale) -> float:
+    """The scalar parameter as a host float.  Reading a device scalar waits for the
+    stream, so it is read once per parameter tensor (and again if it is modified)."""
+    if not isinstance(scale, torch.Tensor):
+      return float(scale)
+    cache = self.__dict__.setdefault("_scale_cache", module.ParamCache())
+    return cache.get((scale,), "scale", lambda: float(scale))
+
   def get_metrics(self, combine_weights: Array, dispatch_weights: Array, mu: Array):
     """router.py:112-167.  Monitoring scalars; mu is normalised inside cosine_psim."""
     g, m, n, p = combine_weights.shape
-    cwf, dwf = combine_weights.float(), dispatch_weights.float()
+    if combine_weights.is_cuda and combine_weights.dtype in (torch.float32, torch.bfloat16):
+      cmin, cmax, dmin, dmax = K.soft_router_stats(combine_weights.reshape(g, m, n * p),
+                                                   dispatch_weights.reshape(g, m, n * p))
+    else:
+      cwf, dwf = combine_weights.float(), dispatch_weights.float()
+      cmin, cmax = cwf.amin(dim=(2, 3)).mean(), cwf.amax(dim=(2, 3)).mean()
+      dmin, dmax = dwf.amin(dim=1).mean(), dwf.amax(dim=1).mean()
     metrics = {
-        "auxiliary_loss": torch.zeros((), dtype=torch.float32, device=cwf.device),
-        "combine_weights_min_mean": cwf.amin(dim=(2, 3)).mean(),
-        "combine_weights_max_mean": cwf.amax(dim=(2, 3)).mean(),
-        "dispatch_weights_min_mean": dwf.amin(dim=1).mean(),
-        "dispatch_weights_max_mean": dwf.amax(dim=1).mean(),
+        "auxiliary_loss": torch.zeros((), dtype=torch.float32, device=combine_weights.device),
+        "combine_weights_min_mean": cmin,
+        "combine_weights_max_mean": cmax,
+        "dispatch_weights_min_mean": dmin,
+        "dispatch_weights_max_mean": dmax,
     }
     if self.compute_similarity_metrics:
+      cwf, dwf = combine_weights.float(), dispatch_weights.float()
       def masked(sim, eye):
         mk = (1 - eye) * sim
         return mk + eye * mk.max()
