@@ -175,6 +175,20 @@ __global__ __launch_bounds__(256) void mfma_probe_kernel(const uint4* __restrict
 
 size_t align256(size_t v) { return (v + 255) / 256 * 256; }
 
+// The second product's 256x256 tiles run one per CU, in whole rounds of kNumCu tiles:
+// 384 tiles (128 experts x 256 rows x 768 columns) take two rounds for 1.5 rounds of
+// work.  Tiles of 128x256, two per CU, waste less then; they are a few percent slower
+// per flop, so they are taken only where the rounds say 10 % or more.
+bool down_prefers_half_tiles(int E, int R, int N) {
+  constexpr int64_t kNumCu = 256;
+  const int64_t tn = (N + 255) / 256;
+  const int64_t full = (int64_t)E * ((R + 255) / 256) * tn;
+  const int64_t half = (int64_t)E * ((R + 127) / 128) * tn;
+  const double t_full = (double)((full + kNumCu - 1) / kNumCu);
+  const double t_half = 0.5 * 1.05 * (double)((half + kNumCu - 1) / kNumCu);
+  return t_half < 0.9 * t_full;
+}
+
 // Launch plans of the two ragged products of an MLP: geometry, bytes, one planning launch.
 struct MlpPlans {
   GemmGeom up, down;
@@ -300,6 +314,10 @@ extern "C" int vmoe_expert_mlp(const VmoeExpertMlpParams* p, vmoe_stream_t strea
                                                      p->R, p->M, p->D, stream, p->rows_per_expert,
                                                      plan_up, p->x_rows, p->num_items);
     if (rc != VMOE_OK) return rc;
+    if (p->rows_per_expert == nullptr && down_prefers_half_tiles(p->E, p->R, p->D))
+      return launch_gemm_bf16<CfgUp, kEpiBias>((const bf16_t*)hidden, (const bf16_t*)w1t,
+                                              (const bf16_t*)p->b1, (bf16_t*)p->out, p->E, p->R,
+                                              p->D, p->M, stream, nullptr, nullptr);
     return launch_gemm_bf16<CfgDown, kEpiBias>((const bf16_t*)hidden, (const bf16_t*)w1t,
                                               (const bf16_t*)p->b1, (bf16_t*)p->out, p->E, p->R,
                                               p->D, p->M, stream, p->rows_per_expert, plan_down);
