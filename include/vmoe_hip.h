@@ -341,12 +341,15 @@ int vmoe_soft_route(const VmoeSoftRouteParams* p, vmoe_stream_t stream);
 
 /* Monitoring scalars of SoftRouter.get_metrics (vmoe/projects/soft_moe/router.py:119-125):
  * partial[g] = (sum_s min_n combine_w, sum_s max_n combine_w, sum_n min_s dispatch_w,
- * sum_n max_s dispatch_w) for group g; the four metrics are the sums over g divided
- * by G*S (combine) and G*N (dispatch). */
+ * sum_n max_s dispatch_w) for group g; a second launch adds them over g in index
+ * order (bit-reproducible) and writes
+ *   stats = (combine_weights_min_mean, combine_weights_max_mean,
+ *            dispatch_weights_min_mean, dispatch_weights_max_mean, auxiliary_loss = 0). */
 typedef struct {
   const void* combine_w;   /* (G, S, N) dtype */
   const void* dispatch_w;  /* (G, S, N) dtype */
-  float* partial;          /* out (G, 4) float32 */
+  float* partial;          /* scratch (G, 4) float32 */
+  float* stats;            /* out (5,) float32 */
   int32_t G, S, N;
   int32_t dtype;
 } VmoeSoftStatsParams;

@@ -186,7 +186,7 @@ class CastParams(ctypes.Structure):
 
 class SoftStatsParams(ctypes.Structure):
   _fields_ = [("combine_w", c_void_p), ("dispatch_w", c_void_p), ("partial", c_void_p),
-              ("G", c_int32), ("S", c_int32), ("N", c_int32), ("dtype", c_int32)]
+              ("stats", c_void_p), ("G", c_int32), ("S", c_int32), ("N", c_int32), ("dtype", c_int32)]
 
 
 class CombineBackwardParams(ctypes.Structure):

@@ -707,6 +707,26 @@ __global__ __launch_bounds__(256) void soft_stats_vec_kernel(const T* __restrict
     partial[(size_t)g * 4 + blockIdx.y * 2 + tid] = red[0][tid] + red[1][tid] + red[2][tid] + red[3][tid];
 }
 
+// Sums the (G, 4) partials over the groups in index order and scales them to means;
+// stats[4] is the router's auxiliary loss, which is always zero.
+__global__ __launch_bounds__(256) void soft_stats_finish_kernel(const float* __restrict__ partial,
+                                                                float* __restrict__ stats, int G,
+                                                                float inv_items, float inv_slots) {
+  __shared__ float part[64][4];
+  const int tid = threadIdx.x, col = tid & 3, seg = tid >> 2;
+  const int per = (G + 63) / 64;
+  float s = 0.f;
+  for (int g = seg * per; g < min(G, (seg + 1) * per); ++g) s += partial[(size_t)g * 4 + col];
+  part[seg][col] = s;
+  __syncthreads();
+  if (tid < 4) {
+    float t = 0.f;
+    for (int q = 0; q < 64; ++q) t += part[q][tid];
+    stats[tid] = t * (tid < 2 ? inv_items : inv_slots);
+  }
+  if (tid == 4) stats[4] = 0.f;
+}
+
 }  // namespace
 }  // namespace vmoe
 
@@ -799,7 +819,8 @@ extern "C" int vmoe_einsum_combine(const VmoeEinsumParams* p, vmoe_stream_t stre
 }
 
 extern "C" int vmoe_soft_router_stats(const VmoeSoftStatsParams* p, vmoe_stream_t stream) {
-  if (p == nullptr || p->combine_w == nullptr || p->dispatch_w == nullptr || p->partial == nullptr)
+  if (p == nullptr || p->combine_w == nullptr || p->dispatch_w == nullptr ||
+      p->partial == nullptr || p->stats == nullptr)
     return VMOE_E_NULL;
   if (p->G < 1 || p->S < 1 || p->N < 1) return VMOE_E_SHAPE;
   if (p->dtype != VMOE_BF16 && p->dtype != VMOE_F32) return VMOE_E_DTYPE;
@@ -824,5 +845,7 @@ extern "C" int vmoe_soft_router_stats(const VmoeSoftStatsParams* p, vmoe_stream_
     hipLaunchKernelGGL(soft_stats_kernel<float>, dim3(p->G), dim3(256), 0, s,
                        (const float*)p->combine_w, (const float*)p->dispatch_w, p->partial, p->S,
                        p->N);
+  hipLaunchKernelGGL(soft_stats_finish_kernel, dim3(1), dim3(256), 0, s, p->partial, p->stats, p->G,
+                     1.0f / ((float)p->G * (float)p->S), 1.0f / ((float)p->G * (float)p->N));
   return launch_status();
 }

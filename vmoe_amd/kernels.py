@@ -307,30 +307,17 @@ def soft_route(x: torch.Tensor, mu: torch.Tensor, scale: float, return_logits: b
 
 
 def soft_router_stats(combine_w: torch.Tensor, dispatch_w: torch.Tensor):
-  """combine_w, dispatch_w (G,S,N) -> the four means of SoftRouter.get_metrics as 0-dim
-  float32 tensors: (combine min-mean, combine max-mean, dispatch min-mean, dispatch max-mean)."""
+  """combine_w, dispatch_w (G,S,N) -> the scalars of SoftRouter.get_metrics as 0-dim
+  float32 tensors: (combine min-mean, combine max-mean, dispatch min-mean, dispatch
+  max-mean, auxiliary loss = 0)."""
   G, S, N = combine_w.shape
   combine_w, dispatch_w = combine_w.contiguous(), dispatch_w.contiguous()
-  partial = _f32(G, 4, device=combine_w.device)
+  buf = _f32(G * 4 + 8, device=combine_w.device)
+  stats = buf[G * 4:G * 4 + 5]
   H.call("vmoe_soft_router_stats", H.SoftStatsParams(
-      H.ptr(combine_w), H.ptr(dispatch_w), H.ptr(partial), G, S, N, H.dtype_code(combine_w.dtype)))
-  scale = torch.tensor([1.0 / (G * S), 1.0 / (G * S), 1.0 / (G * N), 1.0 / (G * N)],
-                       dtype=torch.float32)
-  sums = partial.sum(0) * _to_device_cached(scale, combine_w.device)
-  return sums[0], sums[1], sums[2], sums[3]
-
-
-_DEVICE_CONSTANTS = {}
-
-
-def _to_device_cached(t: torch.Tensor, device) -> torch.Tensor:
-  key = (tuple(t.tolist()), str(device))
-  hit = _DEVICE_CONSTANTS.get(key)
-  if hit is None:
-    if len(_DEVICE_CONSTANTS) > 64:
-      _DEVICE_CONSTANTS.clear()
-    hit = _DEVICE_CONSTANTS[key] = t.to(device)
-  return hit
+      H.ptr(combine_w), H.ptr(dispatch_w), H.ptr(buf), H.ptr(stats), G, S, N,
+      H.dtype_code(combine_w.dtype)))
+  return stats[0], stats[1], stats[2], stats[3], stats[4]
 
 
 def _w_code(w: torch.Tensor) -> int:

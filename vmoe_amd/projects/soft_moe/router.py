@@ -61,15 +61,23 @@ class SoftRouter(module.Module):
     if tuple(mu.shape) != (dim, self.num_experts, num_slots):
       raise ValueError(f"mu has shape {tuple(mu.shape)}, expected {(dim, self.num_experts, num_slots)}")
     n, s = self.num_experts, num_slots
-    dw, cw = K.soft_route(x, K.cast(mu, dtype).reshape(dim, n * s), self._scale_value(p["scale"]))
+    mu_c = self._cast_mu(mu, dtype)
+    dw, cw = K.soft_route(x, mu_c.reshape(dim, n * s), self._scale_value(p["scale"]))
     dispatch_weights = dw.view(G, m, n, s)
     combine_weights = cw.view(G, m, n, s)
     dispatcher = EinsumDispatcher(combine_weights, dispatch_weights,
                                   partition_spec=self.partition_spec,
                                   einsum_precision=self.precision)
     dispatcher = Bfloat16Dispatcher(dispatcher)
-    metrics = self.get_metrics(combine_weights, dispatch_weights, K.cast(mu, dtype))
+    metrics = self.get_metrics(combine_weights, dispatch_weights, mu_c)
     return dispatcher, metrics
+
+  def _cast_mu(self, mu: Array, dtype) -> Array:
+    """The slot parameters in the compute dtype, cast once per parameter tensor."""
+    if mu.dtype == dtype:
+      return mu
+    cache = self.__dict__.setdefault("_mu_cache", module.ParamCache())
+    return cache.get((mu,), dtype, lambda: K.cast(mu, dtype))
 
   def _scale_value(self, scale) -> float:
     """The scalar parameter as a host float.  Reading a device scalar waits for the
@@ -83,14 +91,15 @@ class SoftRouter(module.Module):
     """router.py:112-167.  Monitoring scalars; mu is normalised inside cosine_psim."""
     g, m, n, p = combine_weights.shape
     if combine_weights.is_cuda and combine_weights.dtype in (torch.float32, torch.bfloat16):
-      cmin, cmax, dmin, dmax = K.soft_router_stats(combine_weights.reshape(g, m, n * p),
-                                                   dispatch_weights.reshape(g, m, n * p))
+      cmin, cmax, dmin, dmax, aux = K.soft_router_stats(
+          combine_weights.reshape(g, m, n * p), dispatch_weights.reshape(g, m, n * p))
     else:
+      aux = torch.zeros((), dtype=torch.float32, device=combine_weights.device)
       cwf, dwf = combine_weights.float(), dispatch_weights.float()
       cmin, cmax = cwf.amin(dim=(2, 3)).mean(), cwf.amax(dim=(2, 3)).mean()
       dmin, dmax = dwf.amin(dim=1).mean(), dwf.amax(dim=1).mean()
     metrics = {
-        "auxiliary_loss": torch.zeros((), dtype=torch.float32, device=combine_weights.device),
+        "auxiliary_loss": aux,
         "combine_weights_min_mean": cmin,
         "combine_weights_max_mean": cmax,
         "dispatch_weights_min_mean": dmin,
@@ -141,5 +150,5 @@ def cosine_psim(x: Array, batch_axes, contract_axes, precision=None, eps: float 
   fshape = tuple(x.shape[a] for a in free)
   xm = xt.reshape(max(1, int(torch.tensor(bshape).prod()) if bshape else 1), -1,
                   int(torch.tensor([x.shape[a] for a in contract_axes]).prod()))
-  out = torch.matmul(xm, xm.transpose(1, 2))
+  out = torch.matmul(xm, xm.transpose(1, 2).contiguous())
   return out.reshape(*bshape, *fshape, *fshape)
