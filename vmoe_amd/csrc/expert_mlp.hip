@@ -199,14 +199,13 @@ MlpPlans mlp_plans(int E, int R, int D, int M) {
   MlpPlans m;
   m.up = gemm_geometry<CfgUp>(E, R, M, D);
   m.down = gemm_geometry<CfgDown>(E, R, D, M);
-  // With many experts per die the static order (whole experts per die, tiles past an
-  // expert's rows leaving at once) is already balanced and measured 2 % faster than a
-  // planned launch, whose workgroups start with a dependent load; with one or two
-  // experts per die the fullest expert would set the time, and the plan wins by far
-  // (a third off the MoE blocks of the B/16 model with 8 experts).
-  const bool few_per_die = E <= 2 * kNumXcd;
+  // Ragged launches are planned whenever the geometry allows: with whole experts per
+  // die in a static order the die that drew the fullest experts sets the time (a layer
+  // with capacity factor 0.5 and a skewed router: 399 -> 267 us for the two products,
+  // a third off the MoE blocks of the B/16 model with 8 experts), and on a balanced
+  // layer the planned launch costs 0.3 %.
   auto bytes = [&](const GemmGeom& g) -> size_t {
-    if (!few_per_die || !g.fast || g.ragged_slots * kNumXcd > 0x7ffffff0LL ||
+    if (!g.fast || g.ragged_slots * kNumXcd > 0x7ffffff0LL ||
         (size_t)(E + 1) * 8 > 60000)
       return 0;
     return align256((size_t)g.ragged_slots * kNumXcd * sizeof(int4));
