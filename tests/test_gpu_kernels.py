@@ -114,6 +114,10 @@ ROUTE_CASES = [
     (2, 1568, 32, 2, 100, True),
     (2, 513, 7, 1, 30, True),
     (1, 1, 2, 2, 1, False),
+    (2, 1024, 8, 2, 100, True),      # one key per thread, lane and LDS exchanges
+    (3, 1025, 4, 1, 300, False),     # two keys per thread
+    (2, 2304, 32, 2, 72, True),      # four
+    (1, 5000, 4, 2, 700, True),      # eight
 ]
 
 

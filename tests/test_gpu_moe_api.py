@@ -173,6 +173,9 @@ def _experts_choice_gates(rng, G, S, E, dtype, ties):
     (2, 197, 6, 40, O.BF16, False),   # non power-of-two group and expert count
     (2, 256, 32, 12, O.BF16, True),
     (1, 1000, 4, 260, O.F32, False),
+    (1, 3000, 3, 100, O.BF16, True),  # 4 keys per thread in the sort
+    (1, 6000, 2, 64, O.F32, True),    # 8 keys per thread
+    (1, 9000, 2, 40, O.F32, False),   # keys sorted in LDS
 ])
 def test_top_items_per_expert_vs_oracle(moe, G, S, E, C, dtype, ties):
   rng = np.random.default_rng(G * 1000 + S + E + C)

@@ -6,6 +6,9 @@
 // group and works entirely in LDS:
 //   1. 64-bit keys (descending-gate order bits << 32 | item) are bitonic-sorted;
 //      the item index in the low word makes the order stable by construction.
+//      The keys stay in registers (R consecutive keys per thread): exchanges at
+//      distances below R are register moves, below 64*R lane exchanges, and only
+//      the few stages beyond that go through LDS with barriers;
 //   2. every (item, choice) sets bit  k*S + rank(item)  in its expert's bitmap
 //      (integer LDS atomics: order-independent result);
 //   3. an exclusive prefix of per-word popcounts turns "how many set bits come
@@ -26,15 +29,93 @@ __host__ __device__ inline int pow2ceil(int v) {
   return p;
 }
 
+// One side of a compare-exchange: the smaller (take_min) or larger of two keys.
+__device__ __forceinline__ uint64_t pick(uint64_t mine, uint64_t other, bool take_min) {
+  return ((other < mine) == take_min) ? other : mine;
+}
+
+template <int R, int ST>
+__device__ __forceinline__ void bitonic_in_thread(uint64_t (&key)[R], int size, int tid) {
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    if ((r & ST) == 0 && r + ST < R) {
+      const bool up = (((tid * R + r) & size) == 0);
+      const uint64_t a = key[r], b = key[r + ST];
+      const bool swap = (b < a) == up;
+      key[r] = swap ? b : a;
+      key[r + ST] = swap ? a : b;
+    }
+  }
+}
+
+// Ascending bitonic sort of the first SP (a power of two) of 1024*R keys, element
+// tid*R + r in key[r] of thread tid.  Every thread of the workgroup calls it; `xch`
+// holds 1024*R keys.
+template <int R>
+__device__ __forceinline__ void bitonic_sort_regs(uint64_t (&key)[R], uint64_t* xch, int SP,
+                                                  int tid) {
+  for (int size = 2; size <= SP; size <<= 1) {
+    for (int stride = size >> 1; stride > 0; stride >>= 1) {
+      if (stride >= 64 * R) {
+#pragma unroll
+        for (int r = 0; r < R; ++r) xch[tid * R + r] = key[r];
+        __syncthreads();
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+          const int i = tid * R + r;
+          key[r] = pick(key[r], xch[i ^ stride], ((i & stride) == 0) == ((i & size) == 0));
+        }
+        __syncthreads();
+      } else if (stride >= R) {
+        const int lane_xor = stride / R;
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+          const int i = tid * R + r;
+          const uint64_t other = __shfl_xor((unsigned long long)key[r], lane_xor, kWave);
+          key[r] = pick(key[r], other, ((i & stride) == 0) == ((i & size) == 0));
+        }
+      } else {
+        if constexpr (R > 4) { if (stride == 4) bitonic_in_thread<R, 4>(key, size, tid); }
+        if constexpr (R > 2) { if (stride == 2) bitonic_in_thread<R, 2>(key, size, tid); }
+        if constexpr (R > 1) { if (stride == 1) bitonic_in_thread<R, 1>(key, size, tid); }
+      }
+    }
+  }
+}
+
+// Keys per thread for a sort of SP keys by 1024 threads; 0 = the keys do not fit in
+// registers and are sorted in LDS.
+inline int keys_per_thread(int SP) {
+  const int r = SP <= kRouteThreads ? 1 : SP / kRouteThreads;
+  return r <= 8 ? r : 0;
+}
+
+// The same sort with the keys resident in LDS (any SP).
+__device__ __forceinline__ void bitonic_sort_lds(uint64_t* keys, int SP, int tid) {
+  for (int size = 2; size <= SP; size <<= 1) {
+    for (int stride = size >> 1; stride > 0; stride >>= 1) {
+      for (int t = tid; t < (SP >> 1); t += kRouteThreads) {
+        int lo = 2 * t - (t & (stride - 1));
+        int hi = lo + stride;
+        bool up = (lo & size) == 0;
+        uint64_t a = keys[lo], b = keys[hi];
+        if ((a > b) == up) { keys[lo] = b; keys[hi] = a; }
+      }
+      __syncthreads();
+    }
+  }
+}
+
+template <int R>
 __global__ __launch_bounds__(kRouteThreads) void route_assign_kernel(
     const float* __restrict__ topk_val, const int32_t* __restrict__ topk_idx,
     int32_t* __restrict__ indices, int32_t* __restrict__ token_slot,
     int32_t* __restrict__ slot_token, int32_t* __restrict__ fill, int G, int S, int E, int K,
-    int C, int bpr, int SP, int W) {
+    int C, int bpr, int SP, int NK, int W) {
   extern __shared__ __align__(16) unsigned char smem[];
-  // Layout: keys[SP] (u64, only with bpr) | bitmap[E*W] | prefix[E*W] | rank[S] | total[E]
+  // Layout: keys[NK] (u64, only with bpr) | bitmap[E*W] | prefix[E*W] | rank[S] | total[E]
   uint64_t* keys = reinterpret_cast<uint64_t*>(smem);
-  uint32_t* bitmap = reinterpret_cast<uint32_t*>(smem + (bpr ? (size_t)SP * 8 : 0));
+  uint32_t* bitmap = reinterpret_cast<uint32_t*>(smem + (bpr ? (size_t)NK * 8 : 0));
   uint32_t* prefix = bitmap + (size_t)E * W;
   int32_t* rank = reinterpret_cast<int32_t*>(prefix + (size_t)E * W);
   int32_t* total = rank + S;
@@ -45,26 +126,27 @@ __global__ __launch_bounds__(kRouteThreads) void route_assign_kernel(
 
   for (int i = tid; i < E * W; i += kRouteThreads) bitmap[i] = 0u;
   if (bpr) {
-    for (int s = tid; s < SP; s += kRouteThreads) {
-      uint64_t key = ~0ull;
-      if (s < S) key = ((uint64_t)(~orderable(val[(size_t)s * K])) << 32) | (uint32_t)s;
-      keys[s] = key;
-    }
-    __syncthreads();
-    // Bitonic sort, ascending.
-    for (int size = 2; size <= SP; size <<= 1) {
-      for (int stride = size >> 1; stride > 0; stride >>= 1) {
-        for (int t = tid; t < (SP >> 1); t += kRouteThreads) {
-          int lo = 2 * t - (t & (stride - 1));
-          int hi = lo + stride;
-          bool up = (lo & size) == 0;
-          uint64_t a = keys[lo], b = keys[hi];
-          if ((a > b) == up) { keys[lo] = b; keys[hi] = a; }
-        }
-        __syncthreads();
+    if constexpr (R == 0) {
+      for (int s = tid; s < SP; s += kRouteThreads) {
+        uint64_t key = ~0ull;
+        if (s < S) key = ((uint64_t)(~orderable(val[(size_t)s * K])) << 32) | (uint32_t)s;
+        keys[s] = key;
       }
+      __syncthreads();
+      bitonic_sort_lds(keys, SP, tid);
+      for (int r = tid; r < S; r += kRouteThreads) rank[(uint32_t)keys[r]] = r;
+    } else {
+      uint64_t key[R];
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        const int s = tid * R + r;
+        key[r] = s < S ? ((uint64_t)(~orderable(val[(size_t)s * K])) << 32) | (uint32_t)s : ~0ull;
+      }
+      bitonic_sort_regs<R>(key, keys, SP, tid);
+#pragma unroll
+      for (int r = 0; r < R; ++r)
+        if (tid * R + r < S) rank[(uint32_t)key[r]] = tid * R + r;
     }
-    for (int r = tid; r < S; r += kRouteThreads) rank[(uint32_t)keys[r]] = r;
   } else {
     for (int s = tid; s < S; s += kRouteThreads) rank[s] = s;
   }
@@ -137,7 +219,7 @@ __global__ __launch_bounds__(kRouteThreads) void route_assign_kernel(
 // LDS; the rank of an item is its position, kept when rank < C.  The outputs are
 // those of the slot-assignment kernel with one "choice" per expert (K = E), so
 // the same dispatch / combine kernels serve both routing schemes.
-template <typename T>
+template <typename T, int R>
 __global__ __launch_bounds__(kRouteThreads) void top_items_kernel(
     const T* __restrict__ gates, int32_t* __restrict__ indices, int32_t* __restrict__ token_slot,
     int32_t* __restrict__ slot_token, float* __restrict__ weights, float* __restrict__ sel_minmax,
@@ -147,26 +229,9 @@ __global__ __launch_bounds__(kRouteThreads) void top_items_kernel(
   const int tid = threadIdx.x;
   const int e = blockIdx.x, g = blockIdx.y;
   const T* col = gates + (size_t)g * S * E + e;
-  for (int s = tid; s < SP; s += kRouteThreads) {
-    uint64_t key = ~0ull;
-    if (s < S) key = ((uint64_t)(~orderable(Elt<T>::load(col + (size_t)s * E))) << 32) | (uint32_t)s;
-    keys[s] = key;
-  }
-  __syncthreads();
-  for (int size = 2; size <= SP; size <<= 1) {
-    for (int stride = size >> 1; stride > 0; stride >>= 1) {
-      for (int t = tid; t < (SP >> 1); t += kRouteThreads) {
-        int lo = 2 * t - (t & (stride - 1));
-        int hi = lo + stride;
-        bool up = (lo & size) == 0;
-        uint64_t a = keys[lo], b = keys[hi];
-        if ((a > b) == up) { keys[lo] = b; keys[hi] = a; }
-      }
-      __syncthreads();
-    }
-  }
-  for (int r = tid; r < S; r += kRouteThreads) {
-    const int s = (int)(uint32_t)keys[r];
+  const int last = (C < S ? C : S) - 1;
+  // Rank r of the column holds item s: the outputs of that (item, expert) pair.
+  auto emit = [&](int r, int s) {
     const size_t o = ((size_t)g * S + s) * E + e;
     int slot = -1;
     if (r < C) {
@@ -176,14 +241,36 @@ __global__ __launch_bounds__(kRouteThreads) void top_items_kernel(
     indices[2 * o] = e;
     indices[2 * o + 1] = r;
     token_slot[o] = slot;
-    weights[o] = Elt<T>::load(col + (size_t)s * E);
+    const T gate = col[(size_t)s * E];
+    weights[o] = Elt<T>::load(&gate);
+    if (sel_minmax != nullptr) {
+      if (r == last) sel_minmax[((size_t)g * E + e) * 2] = Elt<T>::load(&gate);
+      if (r == 0) sel_minmax[((size_t)g * E + e) * 2 + 1] = Elt<T>::load(&gate);
+    }
+  };
+  if constexpr (R == 0) {
+    for (int s = tid; s < SP; s += kRouteThreads) {
+      uint64_t key = ~0ull;
+      if (s < S) key = ((uint64_t)(~orderable(Elt<T>::load(col + (size_t)s * E))) << 32) | (uint32_t)s;
+      keys[s] = key;
+    }
+    __syncthreads();
+    bitonic_sort_lds(keys, SP, tid);
+    for (int r = tid; r < S; r += kRouteThreads) emit(r, (int)(uint32_t)keys[r]);
+  } else {
+    uint64_t key[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      const int s = tid * R + r;
+      key[r] = s < S ? ((uint64_t)(~orderable(Elt<T>::load(col + (size_t)s * E))) << 32) | (uint32_t)s
+                     : ~0ull;
+    }
+    bitonic_sort_regs<R>(key, keys, SP, tid);
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+      if (tid * R + r < S) emit(tid * R + r, (int)(uint32_t)key[r]);
   }
   for (int c = S + tid; c < C; c += kRouteThreads) slot_token[slot_row(e, g, c, G, E, C)] = -1;
-  if (tid == 0 && sel_minmax != nullptr) {
-    const int last = (C < S ? C : S) - 1;
-    sel_minmax[((size_t)g * E + e) * 2] = Elt<T>::load(col + (size_t)(uint32_t)keys[last] * E);
-    sel_minmax[((size_t)g * E + e) * 2 + 1] = Elt<T>::load(col + (size_t)(uint32_t)keys[0] * E);
-  }
 }
 
 __global__ __launch_bounds__(256) void fill_i32_kernel(int32_t* p, size_t n, int32_t v) {
@@ -300,16 +387,27 @@ extern "C" int vmoe_route_assign(const VmoeRouteAssignParams* p, vmoe_stream_t s
   if (rc != VMOE_OK) return rc;
   const int SP = pow2ceil(p->S);
   const int W = (p->S * p->K + 31) / 32;
-  const size_t lds = (p->batch_priority ? (size_t)SP * 8 : 0) + (size_t)p->E * W * 8 +
+  const int R = keys_per_thread(SP);
+  const int NK = R == 0 ? SP : kRouteThreads * R;
+  const size_t lds = (p->batch_priority ? (size_t)NK * 8 : 0) + (size_t)p->E * W * 8 +
                      (size_t)p->S * 4 + (size_t)p->E * 4;
   if (lds > 160 * 1024) return VMOE_E_UNSUPPORTED;
-  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(route_assign_kernel),
-                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-  if (e != hipSuccess) return (int)e;
-  hipLaunchKernelGGL(route_assign_kernel, dim3(p->G), dim3(kRouteThreads), lds, as_stream(stream),
-                     p->topk_val, p->topk_idx, p->indices, p->token_slot, p->slot_token, p->fill,
-                     p->G, p->S, p->E, p->K, p->C, p->batch_priority ? 1 : 0, SP, W);
-  return launch_status();
+  auto launch = [&](auto kern) -> int {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return (int)e;
+    hipLaunchKernelGGL(kern, dim3(p->G), dim3(kRouteThreads), lds, as_stream(stream), p->topk_val,
+                       p->topk_idx, p->indices, p->token_slot, p->slot_token, p->fill, p->G, p->S,
+                       p->E, p->K, p->C, p->batch_priority ? 1 : 0, SP, NK, W);
+    return launch_status();
+  };
+  switch (R) {
+    case 1: return launch(route_assign_kernel<1>);
+    case 2: return launch(route_assign_kernel<2>);
+    case 4: return launch(route_assign_kernel<4>);
+    case 8: return launch(route_assign_kernel<8>);
+    default: return launch(route_assign_kernel<0>);
+  }
 }
 
 extern "C" int vmoe_indices_to_slots(const VmoeIndicesToSlotsParams* p, vmoe_stream_t stream) {
@@ -350,27 +448,37 @@ extern "C" int vmoe_top_items_per_expert(const VmoeTopItemsParams* p, vmoe_strea
   if ((int64_t)p->E * p->G * p->C >= INT32_MAX || (int64_t)p->G * p->S * p->E >= INT32_MAX)
     return VMOE_E_OVERFLOW;
   const int SP = pow2ceil(p->S < 2 ? 2 : p->S);
-  const size_t lds = (size_t)SP * 8;
+  const int R = keys_per_thread(SP);
+  const size_t lds = (size_t)(R == 0 ? SP : kRouteThreads * R) * 8;
   if (lds > 160 * 1024) return VMOE_E_UNSUPPORTED;
   dim3 grid(p->E, p->G);
+  auto launch = [&](auto kern, auto* gates) -> int {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return (int)e;
+    hipLaunchKernelGGL(kern, grid, dim3(kRouteThreads), lds, as_stream(stream), gates, p->indices,
+                       p->token_slot, p->slot_token, p->weights, p->sel_minmax, p->G, p->S, p->E,
+                       p->C, SP);
+    return launch_status();
+  };
   if (p->dtype == VMOE_BF16) {
-    auto kern = top_items_kernel<bf16_t>;
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    if (e != hipSuccess) return (int)e;
-    hipLaunchKernelGGL(kern, grid, dim3(kRouteThreads), lds, as_stream(stream),
-                       (const bf16_t*)p->gates, p->indices, p->token_slot, p->slot_token, p->weights,
-                       p->sel_minmax, p->G, p->S, p->E, p->C, SP);
-  } else {
-    auto kern = top_items_kernel<float>;
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    if (e != hipSuccess) return (int)e;
-    hipLaunchKernelGGL(kern, grid, dim3(kRouteThreads), lds, as_stream(stream),
-                       (const float*)p->gates, p->indices, p->token_slot, p->slot_token, p->weights,
-                       p->sel_minmax, p->G, p->S, p->E, p->C, SP);
+    const bf16_t* gates = (const bf16_t*)p->gates;
+    switch (R) {
+      case 1: return launch(top_items_kernel<bf16_t, 1>, gates);
+      case 2: return launch(top_items_kernel<bf16_t, 2>, gates);
+      case 4: return launch(top_items_kernel<bf16_t, 4>, gates);
+      case 8: return launch(top_items_kernel<bf16_t, 8>, gates);
+      default: return launch(top_items_kernel<bf16_t, 0>, gates);
+    }
   }
-  return launch_status();
+  const float* gates = (const float*)p->gates;
+  switch (R) {
+    case 1: return launch(top_items_kernel<float, 1>, gates);
+    case 2: return launch(top_items_kernel<float, 2>, gates);
+    case 4: return launch(top_items_kernel<float, 4>, gates);
+    case 8: return launch(top_items_kernel<float, 8>, gates);
+    default: return launch(top_items_kernel<float, 0>, gates);
+  }
 }
 
 extern "C" int vmoe_compact_rows(const VmoeCompactRowsParams* p, vmoe_stream_t stream) {
