@@ -10,13 +10,13 @@
 // After the K loop the logits tile passes through a wave-private LDS tile, so
 // that each lane holds half of one item's row: softmax and top-K are serial per
 // lane, with one xor-32 shuffle per reduction to join the two halves.
+#include <type_traits>
+
 #include "vmoe_common.h"
 
 namespace vmoe {
 namespace {
 
-constexpr int kGateThreads = 256;
-constexpr int kGateWaves = kGateThreads / kWave;
 
 __device__ __forceinline__ float inv_orderable(uint32_t u) {
   uint32_t b = (u & 0x80000000u) ? (u & 0x7fffffffu) : ~u;
@@ -60,14 +60,16 @@ template <typename T> __host__ __device__ constexpr int w_stride(int kc, int epa
   return sizeof(T) == 2 ? kc + 8 : epad;
 }
 
-template <typename T, int NT, bool LOGITS>
-__global__ __launch_bounds__(kGateThreads) void gate_topk_kernel(
+template <typename T, int NT, bool LOGITS, int WAVES>
+__global__ __launch_bounds__(WAVES * kWave) void gate_topk_kernel(
     const T* __restrict__ x, const T* __restrict__ w, const float* __restrict__ bias,
     T* __restrict__ gates, float* __restrict__ logits, float* __restrict__ topk_val,
     int32_t* __restrict__ topk_idx,
     int num_items, int D, int E, int K, int KC, int num_chunks, int num_tiles, int stage_off) {
   extern __shared__ __align__(16) unsigned char smem[];
   T* wl = reinterpret_cast<T*>(smem);
+  constexpr int kGateWaves = WAVES;
+  constexpr int kGateThreads = kGateWaves * kWave;
   constexpr int EP = NT * 32;
   constexpr bool kBf16 = sizeof(T) == 2;
   const int tid = threadIdx.x;
@@ -94,6 +96,62 @@ __global__ __launch_bounds__(kGateThreads) void gate_topk_kernel(
 #pragma unroll
       for (int i = 0; i < 16; ++i) acc[nt][i] = 0.f;
 
+    // bf16: the loads of the first round of router-kernel blocks and of the first
+    // batch of item rows go out together, before anything waits: the blocks come back
+    // first and are staged under the latency of the rows.
+    constexpr int UB = 2;   // 64-k blocks per batch; two batches (16 x 16-byte loads per lane) in flight
+    uint4 wraw[kBf16 ? 8 : 1];
+    uint4 a[kBf16 ? 2 : 1][UB][4];
+    using Buf0 = std::integral_constant<int, 0>;
+    using Buf1 = std::integral_constant<int, kBf16 ? 1 : 0>;
+    auto load_w_block = [&](int k0, int kb, int nb, bool in_range) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const int k = k0 + kb * 8 + i;
+        wraw[kBf16 ? i : 0] = (in_range && k < D && nb * 8 < E)
+                                  ? *reinterpret_cast<const uint4*>(w + (size_t)k * E + nb * 8)
+                                  : make_uint4(0, 0, 0, 0);
+      }
+    };
+    auto load_rows = [&](auto buf, int k0, int kb0, int nkb) {
+#pragma unroll
+      for (int u = 0; u < UB; ++u)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const int kg = k0 + (kb0 + u) * 64 + h * 32 + j * 8;
+          a[decltype(buf)::value][u][j] = (kb0 + u < nkb && kg + 8 <= D)
+                                              ? *reinterpret_cast<const uint4*>(xrow + kg)
+                                              : make_uint4(0, 0, 0, 0);
+        }
+    };
+    auto mma_rows = [&](auto buf, int kb0, int nkb) {
+#pragma unroll
+      for (int u = 0; u < UB; ++u) {
+        if (kb0 + u >= nkb) break;
+        const int kl = (kb0 + u) * 64 + h * 32;  // this lane's 32 k's inside the chunk
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          bf16x8 af = __builtin_bit_cast(bf16x8, a[decltype(buf)::value][u][j]);
+#pragma unroll
+          for (int nt = 0; nt < NT; ++nt) {
+            uint4 b = *reinterpret_cast<const uint4*>(wl + (nt * 32 + m) * stride + kl + j * 8);
+            acc[nt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af, __builtin_bit_cast(bf16x8, b),
+                                                              acc[nt], 0, 0, 0);
+          }
+        }
+      }
+    };
+    if constexpr (kBf16) {
+      if (it == 0 && E % 8 == 0 && (reinterpret_cast<uintptr_t>(w) & 15u) == 0) {
+        const int nbn = EP / 8;
+        load_w_block(0, tid / nbn, tid % nbn, tid < (KC / 8) * nbn);
+      }
+      if (active) {
+        load_rows(Buf0{}, 0, 0, KC / 64);
+        load_rows(Buf1{}, 0, UB, KC / 64);
+      }
+    }
+
     for (int c = 0; c < num_chunks; ++c) {
       const int k0 = c * KC;
       if (num_chunks > 1 || it == 0) {
@@ -102,7 +160,33 @@ __global__ __launch_bounds__(kGateThreads) void gate_topk_kernel(
         // a row of W is a whole number of 16-byte vectors the loads are vector
         // loads, all independent, so the staging costs one memory round trip.
         constexpr int VW = 16 / (int)sizeof(T);
-        if (E % VW == 0 && (reinterpret_cast<uintptr_t>(w) & 15u) == 0) {
+        if (kBf16 && E % VW == 0 && (reinterpret_cast<uintptr_t>(w) & 15u) == 0) {
+          // bf16: a thread loads an 8(k) x 8(expert) block with eight 16-byte loads,
+          // transposes it in registers and writes each expert's eight consecutive k
+          // as one 16-byte chunk (2-byte LDS writes made this the longest phase of
+          // the kernel).  The first round of loads was issued before the item rows.
+          const int nbn = EP / 8, nblk = (KC / 8) * nbn;
+          for (int b0 = 0; b0 < nblk; b0 += kGateThreads) {
+            const int b = b0 + tid;
+            const int kb = b / nbn, nb = b - kb * nbn;
+            if (!(b0 == 0 && c == 0 && it == 0)) load_w_block(k0, kb, nb, b < nblk);
+            if (b < nblk) {
+#pragma unroll
+              for (int j = 0; j < 8; ++j) {
+                const uint32_t sel = (j & 1) ? 0x07060302u : 0x05040100u;
+                uint32_t o[4];
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                  const uint32_t hi = reinterpret_cast<const uint32_t*>(&wraw[2 * q + 1])[j >> 1];
+                  const uint32_t lo = reinterpret_cast<const uint32_t*>(&wraw[2 * q])[j >> 1];
+                  o[q] = __builtin_amdgcn_perm(hi, lo, sel);
+                }
+                *reinterpret_cast<uint4*>(wl + (size_t)(nb * 8 + j) * stride + kb * 8) =
+                    make_uint4(o[0], o[1], o[2], o[3]);
+              }
+            }
+          }
+        } else if (E % VW == 0 && (reinterpret_cast<uintptr_t>(w) & 15u) == 0) {
           const int vec_per_row = EP / VW;
           constexpr int kBatch = 6;   // independent loads in flight per thread
           for (int idx0 = tid; idx0 < KC * vec_per_row; idx0 += kBatch * kGateThreads) {
@@ -140,32 +224,16 @@ __global__ __launch_bounds__(kGateThreads) void gate_topk_kernel(
       if (!active) continue;
       if constexpr (kBf16) {
         const int nkb = KC / 64;
-        constexpr int UB = 6;   // 64-k blocks in flight per step (24 x 16-byte loads per lane)
-        for (int kb0 = 0; kb0 < nkb; kb0 += UB) {
-          uint4 a[UB][4];
-#pragma unroll
-          for (int u = 0; u < UB; ++u)
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-              int kg = k0 + (kb0 + u) * 64 + h * 32 + j * 8;
-              a[u][j] = (kb0 + u < nkb && kg + 8 <= D) ? *reinterpret_cast<const uint4*>(xrow + kg)
-                                                       : make_uint4(0, 0, 0, 0);
-            }
-#pragma unroll
-          for (int u = 0; u < UB; ++u) {
-            if (kb0 + u >= nkb) break;
-            const int kl = (kb0 + u) * 64 + h * 32;  // this lane's 32 k's inside the chunk
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-              bf16x8 af = __builtin_bit_cast(bf16x8, a[u][j]);
-#pragma unroll
-              for (int nt = 0; nt < NT; ++nt) {
-                uint4 b = *reinterpret_cast<const uint4*>(wl + (nt * 32 + m) * stride + kl + j * 8);
-                acc[nt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af, __builtin_bit_cast(bf16x8, b),
-                                                                  acc[nt], 0, 0, 0);
-              }
-            }
-          }
+        if (c > 0) {
+          load_rows(Buf0{}, k0, 0, nkb);
+          load_rows(Buf1{}, k0, UB, nkb);
+        }
+        // A buffer is refilled as soon as its MFMAs are issued, so two batches stay in flight.
+        for (int kb0 = 0; kb0 < nkb; kb0 += 2 * UB) {
+          mma_rows(Buf0{}, kb0, nkb);
+          load_rows(Buf0{}, k0, kb0 + 2 * UB, nkb);
+          mma_rows(Buf1{}, kb0 + UB, nkb);
+          load_rows(Buf1{}, k0, kb0 + 3 * UB, nkb);
           mfma_result_fence();
         }
       } else {
@@ -421,22 +489,30 @@ int launch_gate(const VmoeGateTopkParams* p, hipStream_t stream) {
   const int dpad = (p->D + gran - 1) / gran * gran;
   // LDS: the staged router kernel (split along D when it would not fit) and,
   // behind it, a 32 x (ep + 1) float32 logits tile per wave for the epilogue.
-  const size_t stage_bytes = (size_t)kGateWaves * 32 * (ep + 1) * sizeof(float);
   const size_t budget = 88 * 1024;
   int kc = dpad;
   while ((size_t)(sizeof(T) == 2 ? ep * (kc + 8) : kc * ep) * sizeof(T) > budget && kc > gran)
     kc = ((kc / 2) + gran - 1) / gran * gran;
   const int num_chunks = (dpad + kc - 1) / kc;
   const size_t w_bytes = ((size_t)(sizeof(T) == 2 ? ep * (kc + 8) : kc * ep) * sizeof(T) + 15) / 16 * 16;
-  const size_t lds = w_bytes + stage_bytes;
+  // Two workgroups of four waves per CU, each with its own staged copy of the router
+  // kernel, where both copies fit in LDS; one workgroup of eight waves sharing a copy
+  // where they do not (D = 1024 in bf16), the registers allow it (up to 32 experts) and
+  // four-wave workgroups would not all be resident at once anyway.
+  const size_t tile_bytes = (size_t)32 * (ep + 1) * sizeof(float);
+  const size_t lds_cu = 160 * 1024;
   const int num_tiles = (p->num_items + 31) / 32;
-  int blocks = (num_tiles + kGateWaves - 1) / kGateWaves;
+  const int waves = (nt == 1 && 2 * (w_bytes + 4 * tile_bytes) > lds_cu &&
+                     w_bytes + 8 * tile_bytes <= lds_cu && num_tiles > 4 * 256) ? 8 : 4;
+  const size_t stage_bytes = waves * tile_bytes;
+  const size_t lds = w_bytes + stage_bytes;
+  int blocks = (num_tiles + waves - 1) / waves;
   if (blocks > 1024) blocks = 1024;
   auto run = [&](auto kern) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return (int)e;
-    hipLaunchKernelGGL(kern, dim3(blocks), dim3(kGateThreads), lds, stream,
+    hipLaunchKernelGGL(kern, dim3(blocks), dim3(waves * kWave), lds, stream,
                        (const T*)p->x, (const T*)p->w, p->logit_bias, (T*)p->gates, p->logits,
                        p->topk_val, p->topk_idx, p->num_items, p->D, p->E, p->K, kc, num_chunks, num_tiles,
                        (int)w_bytes);
@@ -446,15 +522,15 @@ int launch_gate(const VmoeGateTopkParams* p, hipStream_t stream) {
   // the common one a wave of occupancy.
   if (p->logits != nullptr) {
     switch (nt) {
-      case 1: return run(gate_topk_kernel<T, 1, true>);
-      case 2: return run(gate_topk_kernel<T, 2, true>);
-      default: return run(gate_topk_kernel<T, 4, true>);
+      case 1: return waves == 8 ? run(gate_topk_kernel<T, 1, true, 8>) : run(gate_topk_kernel<T, 1, true, 4>);
+      case 2: return run(gate_topk_kernel<T, 2, true, 4>);
+      default: return run(gate_topk_kernel<T, 4, true, 4>);
     }
   }
   switch (nt) {
-    case 1: return run(gate_topk_kernel<T, 1, false>);
-    case 2: return run(gate_topk_kernel<T, 2, false>);
-    default: return run(gate_topk_kernel<T, 4, false>);
+    case 1: return waves == 8 ? run(gate_topk_kernel<T, 1, false, 8>) : run(gate_topk_kernel<T, 1, false, 4>);
+    case 2: return run(gate_topk_kernel<T, 2, false, 4>);
+    default: return run(gate_topk_kernel<T, 4, false, 4>);
   }
 }
 
