@@ -517,6 +517,36 @@ def main():
       lib[name] = 2.0 * kept * D * M * 10 / (e0.elapsed_time(e1) * 1e-3) / 1e12
     roofline["library_gemm_same_shapes_TFLOPs"] = lib
     del a_up, a_dn, w_up, w_dn
+  # The same K steps replayed from HIP graphs (one per rotating input buffer), as a
+  # serving loop would run the layer; reported beside the eager figure, never as `value`.
+  graph_ms = None
+  try:
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+      for i in range(n_rot):
+        step(i)
+    torch.cuda.current_stream().wait_stream(side)
+    graphs, keep = [], []
+    for i in range(n_rot):
+      g_ = torch.cuda.CUDAGraph()
+      with torch.cuda.graph(g_):
+        keep.append(step(i))
+      graphs.append(g_)
+    for i in range(args.warmup):
+      graphs[i % n_rot].replay()
+    torch.cuda.synchronize()
+    tg0 = time.perf_counter()
+    for i in range(args.steps):
+      graphs[i % n_rot].replay()
+    torch.cuda.synchronize()
+    graph_ms = (time.perf_counter() - tg0) * 1e3 / args.steps
+    if not torch.equal(keep[(args.steps - 1) % n_rot][0], step(args.steps - 1)[0]):
+      raise RuntimeError("graph replay and eager step disagree")
+    del graphs, keep
+  except Exception as e:   # pylint: disable=broad-except
+    print(f"bench.py: HIP graph pass skipped: {e}", file=sys.stderr)
+    graph_ms = None
   hbm = {
       "dispatch_GBps": bytes_dispatch / (dispatch_ms * 1e-3) / 1e9 if dispatch_ms else None,
       "combine_GBps": bytes_combine / (stage_ms["vmoe_combine"] * 1e-3) / 1e9,
@@ -541,6 +571,7 @@ def main():
                         "the same steps with events around every call (its vmoe_expert_mlp read "
                         f"{stage_ms_instrumented_mlp:.4f} ms)"),
       "hbm": hbm,
+      "hip_graph_ms_per_step": graph_ms,
   }
   if not args.no_cpu_baseline:
     params_np = {

@@ -744,3 +744,40 @@ def test_combine_backward_data_zero_fills_unclaimed_slots(moe):
   for slot in np.nonzero(st >= 0)[0][:10]:
     t = st[slot]
     np.testing.assert_allclose(dyn[slot], to_np(g)[t] * to_np(w)[t, 0], rtol=1e-6)
+
+
+# ------------------------------------------------------------------ HIP graphs
+@pytest.mark.parametrize("dtype,dkw", [
+    (O.BF16, dict(name="indices", batch_priority=True, capacity_factor=1.0)),
+    (O.F32, dict(name="einsum", batch_priority=False, capacity_factor=1.05)),
+])
+def test_layer_replays_from_hip_graph(dtype, dkw):
+  """The layer makes no host round trip and allocates only through torch, so a serving
+  loop can capture it once and replay it: every replay, with eager work and
+  synchronisations in between, must give the bits of the eager step."""
+  from vmoe_amd.nn import vit_moe
+  N, L, D, M, E, k, gs = 8, 196, 256, 512, 8, 2, 784
+  rng = np.random.default_rng(5)
+  variables = _params_to_dev(_layer_params(rng, D, M, E, dtype, bias_scale=0.1), dtype)
+  layer = vit_moe.MlpMoeBlock(mlp_dim=M, num_experts=E, group_size=gs, deterministic=True,
+                              router=dict(num_selected_experts=k, dispatcher=dkw), dtype=tdtype(dtype))
+  xs = [to_dev(O.cast(rng.standard_normal((N, L, D)), dtype), dtype) for _ in range(3)]
+  eager = [layer.apply(variables, x) for x in xs]
+  static_x = xs[0].clone()
+  side = torch.cuda.Stream()
+  side.wait_stream(torch.cuda.current_stream())
+  with torch.cuda.stream(side):
+    layer.apply(variables, static_x)
+  torch.cuda.current_stream().wait_stream(side)
+  graph = torch.cuda.CUDAGraph()
+  with torch.cuda.graph(graph):
+    out, metrics = layer.apply(variables, static_x)
+  for rep in range(2):
+    for i, x in enumerate(xs):
+      static_x.copy_(x)
+      graph.replay()
+      torch.cuda.synchronize()
+      assert torch.equal(out, eager[i][0]), (rep, i)
+      for key in metrics:
+        assert torch.equal(metrics[key], eager[i][1][key]), (rep, i, key)
+      layer.apply(variables, xs[(i + 1) % 3])   # eager work between replays
