@@ -51,7 +51,7 @@ def parse_args():
   ap.add_argument("--no-dispatch-pass", action="store_true",
                   help="skip the extra pass that times dispatcher.dispatch() (for counter runs "
                        "that should see the step's kernels only)")
-  ap.add_argument("--cpu-groups", type=int, default=2,
+  ap.add_argument("--cpu-groups", type=int, default=32,
                   help="groups of the workload the CPU baseline is timed on")
   return ap.parse_args()
 
