@@ -92,3 +92,33 @@ def test_null_params_are_rejected_without_a_gpu():
   for fn in ("vmoe_gate_topk", "vmoe_route_assign", "vmoe_dispatch", "vmoe_combine",
              "vmoe_expert_mlp", "vmoe_soft_route", "vmoe_einsum_dispatch", "vmoe_cast"):
     assert getattr(lib, fn)(None, None) == -1
+
+
+def _params_entry_points():
+  """(function name, struct name) of every `int vmoe_x(const VmoeXParams* p, vmoe_stream_t)`."""
+  text = open(HEADER).read()
+  text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+  return sorted(set(re.findall(r"\bint\s+(vmoe_[a-z0-9_]+)\s*\(\s*const\s+(Vmoe\w+Params)\s*\*\s*\w+\s*,\s*vmoe_stream_t", text)))
+
+
+def test_entry_points_reject_null_and_empty_params():
+  """Argument checks run before any device call: a null parameter block and an all-zero
+  one (null buffers, zero sizes) come back as negative VMOE_E_* codes.  Nothing is
+  launched, so this runs without a GPU."""
+  from vmoe_amd import _hip
+  lib = _lib()
+  lib.vmoe_error_string.restype = ctypes.c_char_p
+  by_name = {"Vmoe" + cls.__name__: cls for cls in vars(_hip).values()
+             if isinstance(cls, type) and issubclass(cls, ctypes.Structure)}
+  entries = _params_entry_points()
+  assert len(entries) >= 20
+  for fn_name, struct_name in entries:
+    fn = getattr(lib, fn_name)
+    fn.restype = ctypes.c_int
+    fn.argtypes = [ctypes.c_void_p, ctypes.c_void_p]
+    rc = fn(None, None)
+    assert rc < 0, f"{fn_name}(NULL) returned {rc}"
+    assert lib.vmoe_error_string(rc) != b"unknown vmoe error"
+    zeroed = by_name[struct_name]()
+    rc = fn(ctypes.byref(zeroed), None)
+    assert rc < 0, f"{fn_name}(zeroed {struct_name}) returned {rc}"
