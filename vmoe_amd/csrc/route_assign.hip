@@ -367,6 +367,59 @@ __global__ __launch_bounds__(256) void compact_rows_kernel(
   token_row[i] = row;
 }
 
+// Both steps in one launch, for E <= 256 and at least 256 assignments per group (a
+// workgroup then touches at most two groups): the workgroup adds up the fill counts of
+// the groups before its first group itself -- 256 / E threads per expert, each a strided
+// share of the groups, joined in LDS -- instead of reading a prefix that another launch
+// wrote.  Workgroup 0 also writes the experts' row counts.
+__global__ __launch_bounds__(256) void compact_rows_fused_kernel(
+    const int32_t* __restrict__ fill, const int32_t* __restrict__ token_slot,
+    int32_t* __restrict__ token_row, int32_t* __restrict__ row_token,
+    int32_t* __restrict__ rows_per_expert, int G, int E, int C, int per_group, int K, size_t n) {
+  __shared__ int32_t part[256];
+  __shared__ int32_t before[2][256];
+  const int tid = threadIdx.x;
+  const size_t i0 = (size_t)blockIdx.x * 256;
+  const int g_lo = (int)(i0 / per_group);
+  const int parts = 256 / E;
+  const int e_t = tid % E, q = tid / E;
+  auto column_sum = [&](int g_end) {   // sum of fill[0 .. g_end) [e], valid in threads tid < E
+    int acc = 0;
+    if (q < parts)
+      for (int g = q; g < g_end; g += parts) acc += fill[(size_t)g * E + e_t];
+    part[tid] = acc;
+    __syncthreads();
+    int total = 0;
+    if (tid < E)
+      for (int j = 0; j < parts; ++j) total += part[j * E + tid];
+    __syncthreads();
+    return total;
+  };
+  const int lo = column_sum(g_lo);
+  if (tid < E) {
+    before[0][tid] = lo;
+    before[1][tid] = lo + (g_lo < G ? fill[(size_t)g_lo * E + tid] : 0);
+  }
+  if (blockIdx.x == 0) {
+    const int total = column_sum(G);
+    if (tid < E) rows_per_expert[tid] = total;
+  }
+  __syncthreads();
+  const size_t i = i0 + tid;
+  if (i >= n) return;
+  const int slot = token_slot[i];
+  int row = -1;
+  if (slot >= 0) {
+    const int per_expert = G * C;
+    const int g = (int)(i / per_group);
+    const int e = slot / per_expert;
+    const int c = (slot - e * per_expert) % C;
+    row = e * per_expert + before[g - g_lo][e] + c;
+    if (row_token != nullptr) row_token[row] = (int)(i / K);
+  }
+  token_row[i] = row;
+}
+
 }  // namespace
 }  // namespace vmoe
 
@@ -487,9 +540,16 @@ extern "C" int vmoe_compact_rows(const VmoeCompactRowsParams* p, vmoe_stream_t s
     return VMOE_E_NULL;
   int rc = check_route_shapes(p->G, p->S, p->E, p->K, p->C);
   if (rc != VMOE_OK) return rc;
+  const size_t n = (size_t)p->G * p->S * p->K;
+  const int parts = p->E <= 256 ? 256 / p->E : 1;
+  if (p->E <= 256 && (int64_t)p->S * p->K >= 256 && (p->G + parts - 1) / parts <= 16) {
+    hipLaunchKernelGGL(compact_rows_fused_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0,
+                       as_stream(stream), p->fill, p->token_slot, p->token_row, p->row_token,
+                       p->rows_per_expert, p->G, p->E, p->C, p->S * p->K, p->K, n);
+    return launch_status();
+  }
   hipLaunchKernelGGL(fill_prefix_kernel, dim3(p->E), dim3(256), 0, as_stream(stream), p->fill,
                      p->prefix, p->rows_per_expert, p->G, p->E);
-  const size_t n = (size_t)p->G * p->S * p->K;
   hipLaunchKernelGGL(compact_rows_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0,
                      as_stream(stream), p->prefix, p->token_slot, p->token_row, p->row_token, p->G,
                      p->E, p->C, p->S * p->K, p->K, n);
