@@ -146,6 +146,14 @@ typedef struct {
 } VmoeRouteAssignParams;
 int vmoe_route_assign(const VmoeRouteAssignParams* p, vmoe_stream_t stream);
 
+/* vmoe_route_assign and vmoe_router_metrics in one launch (the losses run as extra
+ * workgroups beside the slot assignment; both read the same top-k output and neither
+ * reads what the other writes).  Same results as the two calls; m->G, m->S, m->E must
+ * equal p's.  The deterministic branch of NoisyTopExpertsPerItemRouter
+ * (vmoe/nn/routing.py:76-91 followed by :116-131) is this call after vmoe_gate_topk. */
+int vmoe_route_assign_metrics(const VmoeRouteAssignParams* p, const VmoeRouterMetricsParams* m,
+                              vmoe_stream_t stream);
+
 /* Experts-choice ("top items per expert") routing, replacing
  * _get_top_items_per_expert_einsum_dispatcher (vmoe/moe.py:655-694): each expert
  * keeps the C items with its largest gates (jax.lax.top_k of the transposed

@@ -122,3 +122,13 @@ def test_entry_points_reject_null_and_empty_params():
     zeroed = by_name[struct_name]()
     rc = fn(ctypes.byref(zeroed), None)
     assert rc < 0, f"{fn_name}(zeroed {struct_name}) returned {rc}"
+
+
+def test_two_block_entry_point_rejects_null():
+  from vmoe_amd import _hip
+  lib = _lib()
+  fn = lib.vmoe_route_assign_metrics
+  fn.restype = ctypes.c_int
+  fn.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p]
+  assert fn(None, None, None) < 0
+  assert fn(ctypes.byref(_hip.RouteAssignParams()), ctypes.byref(_hip.RouterMetricsParams()), None) < 0

@@ -157,6 +157,25 @@ def test_route_assign_bit_exact(K, G, S, E, k, C, ties, bpr):
   np.testing.assert_array_equal(fill, np.minimum(demand, C))
 
 
+@pytest.mark.parametrize("bpr", [False, True])
+@pytest.mark.parametrize("G,S,E,k,C,dtype", [(4, 64, 8, 2, 4, O.F32), (32, 1568, 32, 2, 100, O.BF16),
+                                             (3, 100, 5, 3, 7, O.F32), (2, 2304, 32, 2, 72, O.BF16),
+                                             (2, 50, 100, 2, 3, O.F32)])
+def test_route_assign_with_metrics_equals_separate_calls(K, G, S, E, k, C, dtype, bpr):
+  """One launch for slot assignment and the router's losses: every output has the bits
+  of the two separate entry points."""
+  rng = np.random.default_rng(S + E)
+  gates = to_dev(O.cast(O.softmax(rng.standard_normal((G, S, E)).astype(np.float32) * 2), dtype), dtype)
+  val, idx = K.topk(gates.float(), k)
+  want = K.route_assign(val, idx, E, C, bpr)
+  want_losses = K.router_metrics(gates, idx, 0.25, 1.0)
+  got = K.route_assign(val, idx, E, C, bpr, metrics=(gates, 0.25, 1.0))
+  for a, b in zip(got[:4], want):
+    assert torch.equal(a, b)
+  for a, b in zip(got[4], want_losses):
+    assert torch.equal(a, b)
+
+
 def test_route_assign_golden(K, goldens):
   g = goldens["top_experts_per_item"]
   gates = np.asarray(g["gates"], np.float32)[None]

@@ -21,7 +21,7 @@ W_F32, W_BF16, W_BOOL = 0, 1, 2
 
 EXPORTS = [
     "vmoe_abi_version", "vmoe_error_string", "vmoe_gate_topk", "vmoe_topk", "vmoe_router_metrics",
-    "vmoe_route_assign", "vmoe_top_items_per_expert", "vmoe_indices_to_slots", "vmoe_dispatch", "vmoe_combine", "vmoe_densify",
+    "vmoe_route_assign", "vmoe_route_assign_metrics", "vmoe_top_items_per_expert", "vmoe_indices_to_slots", "vmoe_dispatch", "vmoe_combine", "vmoe_densify",
     "vmoe_expert_mlp_workspace_bytes", "vmoe_expert_mlp", "vmoe_pack_expert_weights",
     "vmoe_soft_route_workspace_bytes", "vmoe_soft_route", "vmoe_einsum_dispatch",
     "vmoe_einsum_combine", "vmoe_cast", "vmoe_copy_bytes", "vmoe_mfma_probe",
@@ -247,6 +247,23 @@ def set_timing_sink(sink) -> None:
   ``sink[name]`` for the caller to read after synchronising.  None disables."""
   global _timing_sink
   _timing_sink = sink
+
+
+def call2(name: str, first: ctypes.Structure, second: ctypes.Structure) -> None:
+  """An entry point that takes two parameter blocks; timed like call()."""
+  fn = getattr(lib(), name)
+  sink = _timing_sink
+  if sink is None or (getattr(sink, "only", None) is not None and name not in sink.only):
+    check(fn(ctypes.byref(first), ctypes.byref(second), stream()), name)
+    return
+  take = getattr(sink, "take", None)
+  start, stop = take() if take is not None else (
+      torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
+  start.record()
+  code = fn(ctypes.byref(first), ctypes.byref(second), stream())
+  stop.record()
+  sink.setdefault(name, []).append((start, stop))
+  check(code, name)
 
 
 def call(name: str, params: ctypes.Structure) -> None:

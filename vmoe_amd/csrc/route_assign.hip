@@ -17,6 +17,7 @@
 // The kernel also emits the two maps the data-movement kernels use: item ->
 // slot row (-1 when over capacity) and slot row -> item (-1 when empty).
 #include "vmoe_common.h"
+#include "router_metrics.h"
 
 namespace vmoe {
 namespace {
@@ -107,12 +108,11 @@ __device__ __forceinline__ void bitonic_sort_lds(uint64_t* keys, int SP, int tid
 }
 
 template <int R>
-__global__ __launch_bounds__(kRouteThreads) void route_assign_kernel(
+__device__ __forceinline__ void route_assign_group(
     const float* __restrict__ topk_val, const int32_t* __restrict__ topk_idx,
     int32_t* __restrict__ indices, int32_t* __restrict__ token_slot,
     int32_t* __restrict__ slot_token, int32_t* __restrict__ fill, int G, int S, int E, int K,
-    int C, int bpr, int SP, int NK, int W) {
-  extern __shared__ __align__(16) unsigned char smem[];
+    int C, int bpr, int SP, int NK, int W, int g, unsigned char* smem) {
   // Layout: keys[NK] (u64, only with bpr) | bitmap[E*W] | prefix[E*W] | rank[S] | total[E]
   uint64_t* keys = reinterpret_cast<uint64_t*>(smem);
   uint32_t* bitmap = reinterpret_cast<uint32_t*>(smem + (bpr ? (size_t)NK * 8 : 0));
@@ -120,7 +120,6 @@ __global__ __launch_bounds__(kRouteThreads) void route_assign_kernel(
   int32_t* rank = reinterpret_cast<int32_t*>(prefix + (size_t)E * W);
   int32_t* total = rank + S;
   const int tid = threadIdx.x;
-  const int g = blockIdx.x;
   const float* val = topk_val + (size_t)g * S * K;
   const int32_t* idx = topk_idx + (size_t)g * S * K;
 
@@ -210,6 +209,39 @@ __global__ __launch_bounds__(kRouteThreads) void route_assign_kernel(
   }
   if (fill != nullptr)
     for (int e = tid; e < E; e += kRouteThreads) fill[(size_t)g * E + e] = total[e] < C ? total[e] : C;
+}
+
+template <int R>
+__global__ __launch_bounds__(kRouteThreads) void route_assign_kernel(
+    const float* __restrict__ topk_val, const int32_t* __restrict__ topk_idx,
+    int32_t* __restrict__ indices, int32_t* __restrict__ token_slot,
+    int32_t* __restrict__ slot_token, int32_t* __restrict__ fill, int G, int S, int E, int K,
+    int C, int bpr, int SP, int NK, int W) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  route_assign_group<R>(topk_val, topk_idx, indices, token_slot, slot_token, fill, G, S, E, K, C,
+                        bpr, SP, NK, W, blockIdx.x, smem);
+}
+
+// Slot assignment and the router's auxiliary losses in one launch: workgroups 0 .. G-1
+// assign slots, workgroups G .. 2G-1 compute the losses of group blockIdx.x - G.  Both
+// are one workgroup per group, bound by latency, and read the same top-k output, so side
+// by side they take the time of the longer one.
+template <int R, typename T>
+__global__ __launch_bounds__(kRouteThreads) void route_assign_metrics_kernel(
+    const float* __restrict__ topk_val, const int32_t* __restrict__ topk_idx,
+    int32_t* __restrict__ indices, int32_t* __restrict__ token_slot,
+    int32_t* __restrict__ slot_token, int32_t* __restrict__ fill, int G, int S, int E, int K,
+    int C, int bpr, int SP, int NK, int W, RouterMetricsArgs m) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  static_assert(kRouteThreads == kMetricThreads, "both roles use the launch's workgroup size");
+  if ((int)blockIdx.x < G) {
+    route_assign_group<R>(topk_val, topk_idx, indices, token_slot, slot_token, fill, G, S, E, K,
+                          C, bpr, SP, NK, W, blockIdx.x, smem);
+  } else {
+    router_metrics_group<T>(static_cast<const T*>(m.gates), m.top1, m.imp_loss, m.gsh_loss,
+                            m.aux_loss, m.w_gsh, m.w_imp, m.S, m.E, m.top1_stride, m.V,
+                            (int)blockIdx.x - G, smem);
+  }
 }
 
 // Experts-choice routing (vmoe/moe.py:655-694): every expert takes the C items
@@ -431,36 +463,85 @@ static int check_route_shapes(int G, int S, int E, int K, int C) {
   return VMOE_OK;
 }
 
-extern "C" int vmoe_route_assign(const VmoeRouteAssignParams* p, vmoe_stream_t stream) {
+static int check_route_assign(const VmoeRouteAssignParams* p) {
   if (p == nullptr || p->topk_idx == nullptr || p->indices == nullptr ||
       p->token_slot == nullptr || p->slot_token == nullptr)
     return VMOE_E_NULL;
   if (p->batch_priority && p->topk_val == nullptr) return VMOE_E_NULL;
-  int rc = check_route_shapes(p->G, p->S, p->E, p->K, p->C);
-  if (rc != VMOE_OK) return rc;
+  return check_route_shapes(p->G, p->S, p->E, p->K, p->C);
+}
+
+// Launches the slot assignment, with the router's losses as extra workgroups when m is given.
+static int launch_route_assign(const VmoeRouteAssignParams* p, const VmoeRouterMetricsParams* m,
+                               vmoe_stream_t stream) {
   const int SP = pow2ceil(p->S);
   const int W = (p->S * p->K + 31) / 32;
   const int R = keys_per_thread(SP);
   const int NK = R == 0 ? SP : kRouteThreads * R;
-  const size_t lds = (p->batch_priority ? (size_t)NK * 8 : 0) + (size_t)p->E * W * 8 +
-                     (size_t)p->S * 4 + (size_t)p->E * 4;
+  size_t lds = (p->batch_priority ? (size_t)NK * 8 : 0) + (size_t)p->E * W * 8 +
+               (size_t)p->S * 4 + (size_t)p->E * 4;
+  RouterMetricsArgs ma{};
+  if (m != nullptr) {
+    size_t mlds;
+    int V;
+    if (!router_metrics_geometry(m, &V, &mlds)) return VMOE_E_UNSUPPORTED;
+    if (mlds > lds) lds = mlds;
+    ma = RouterMetricsArgs{m->gates, m->top1_idx, m->importance_loss, m->gshard_loss,
+                           m->auxiliary_loss, m->gshard_loss_weight, m->importance_loss_weight,
+                           m->S, m->E, m->top1_stride, V};
+  }
   if (lds > 160 * 1024) return VMOE_E_UNSUPPORTED;
-  auto launch = [&](auto kern) -> int {
+  auto launch = [&](auto kern, auto... extra) -> int {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return (int)e;
-    hipLaunchKernelGGL(kern, dim3(p->G), dim3(kRouteThreads), lds, as_stream(stream), p->topk_val,
-                       p->topk_idx, p->indices, p->token_slot, p->slot_token, p->fill, p->G, p->S,
-                       p->E, p->K, p->C, p->batch_priority ? 1 : 0, SP, NK, W);
+    hipLaunchKernelGGL(kern, dim3(m != nullptr ? 2 * p->G : p->G), dim3(kRouteThreads), lds,
+                       as_stream(stream), p->topk_val, p->topk_idx, p->indices, p->token_slot,
+                       p->slot_token, p->fill, p->G, p->S, p->E, p->K, p->C,
+                       p->batch_priority ? 1 : 0, SP, NK, W, extra...);
     return launch_status();
   };
-  switch (R) {
-    case 1: return launch(route_assign_kernel<1>);
-    case 2: return launch(route_assign_kernel<2>);
-    case 4: return launch(route_assign_kernel<4>);
-    case 8: return launch(route_assign_kernel<8>);
-    default: return launch(route_assign_kernel<0>);
+  if (m == nullptr) {
+    switch (R) {
+      case 1: return launch(route_assign_kernel<1>);
+      case 2: return launch(route_assign_kernel<2>);
+      case 4: return launch(route_assign_kernel<4>);
+      case 8: return launch(route_assign_kernel<8>);
+      default: return launch(route_assign_kernel<0>);
+    }
   }
+  if (m->dtype == VMOE_BF16) {
+    switch (R) {
+      case 1: return launch(route_assign_metrics_kernel<1, bf16_t>, ma);
+      case 2: return launch(route_assign_metrics_kernel<2, bf16_t>, ma);
+      case 4: return launch(route_assign_metrics_kernel<4, bf16_t>, ma);
+      case 8: return launch(route_assign_metrics_kernel<8, bf16_t>, ma);
+      default: return launch(route_assign_metrics_kernel<0, bf16_t>, ma);
+    }
+  }
+  switch (R) {
+    case 1: return launch(route_assign_metrics_kernel<1, float>, ma);
+    case 2: return launch(route_assign_metrics_kernel<2, float>, ma);
+    case 4: return launch(route_assign_metrics_kernel<4, float>, ma);
+    case 8: return launch(route_assign_metrics_kernel<8, float>, ma);
+    default: return launch(route_assign_metrics_kernel<0, float>, ma);
+  }
+}
+
+extern "C" int vmoe_route_assign(const VmoeRouteAssignParams* p, vmoe_stream_t stream) {
+  int rc = check_route_assign(p);
+  if (rc != VMOE_OK) return rc;
+  return launch_route_assign(p, nullptr, stream);
+}
+
+extern "C" int vmoe_route_assign_metrics(const VmoeRouteAssignParams* p,
+                                         const VmoeRouterMetricsParams* m, vmoe_stream_t stream) {
+  int rc = check_route_assign(p);
+  if (rc != VMOE_OK) return rc;
+  rc = check_router_metrics(m);
+  if (rc != VMOE_OK) return rc;
+  if (m->G != p->G || m->S != p->S || m->E != p->E) return VMOE_E_SHAPE;
+  return launch_route_assign(p, m, stream);
 }
 
 extern "C" int vmoe_indices_to_slots(const VmoeIndicesToSlotsParams* p, vmoe_stream_t stream) {

@@ -94,8 +94,12 @@ def router_metrics(gates: torch.Tensor, topk_idx: torch.Tensor, gshard_loss_weig
 
 
 def route_assign(topk_val: Optional[torch.Tensor], topk_idx: torch.Tensor, num_experts: int,
-                 capacity: int, batch_priority: bool):
-  """topk_idx (G,S,K) -> indices (G,S,K,2), token_slot (G,S,K), slot_token (E*G*C,), fill (G,E)."""
+                 capacity: int, batch_priority: bool, metrics=None):
+  """topk_idx (G,S,K) -> indices (G,S,K,2), token_slot (G,S,K), slot_token (E*G*C,), fill (G,E).
+
+  With ``metrics=(gates (G,S,E), gshard_loss_weight, importance_loss_weight)`` the router's
+  losses are computed in the same launch and a fifth result
+  ``(importance_loss, gshard_loss, auxiliary_loss)`` is returned (what router_metrics gives)."""
   G, S, K = topk_idx.shape
   dev = topk_idx.device
   topk_idx = topk_idx.contiguous()
@@ -108,8 +112,19 @@ def route_assign(topk_val: Optional[torch.Tensor], topk_idx: torch.Tensor, num_e
   p = H.RouteAssignParams(H.ptr(topk_val), H.ptr(topk_idx), H.ptr(indices), H.ptr(token_slot),
                           H.ptr(slot_token), H.ptr(fill), G, S, num_experts, K, capacity,
                           int(bool(batch_priority)))
-  H.call("vmoe_route_assign", p)
-  return indices, token_slot, slot_token, fill
+  if metrics is None:
+    H.call("vmoe_route_assign", p)
+    return indices, token_slot, slot_token, fill
+  gates, gshard_loss_weight, importance_loss_weight = metrics
+  if tuple(gates.shape) != (G, S, num_experts):
+    raise ValueError(f"gates have shape {tuple(gates.shape)}, expected {(G, S, num_experts)}")
+  gates = gates.contiguous()
+  imp, gsh, aux = (_f32(G, device=dev) for _ in range(3))
+  m = H.RouterMetricsParams(H.ptr(gates), H.ptr(topk_idx), H.ptr(imp), H.ptr(gsh), H.ptr(aux),
+                            float(gshard_loss_weight), float(importance_loss_weight), G, S,
+                            num_experts, K, H.dtype_code(gates.dtype))
+  H.call2("vmoe_route_assign_metrics", p, m)
+  return indices, token_slot, slot_token, fill, (imp, gsh, aux)
 
 
 def top_items_per_expert(gates: torch.Tensor, capacity: int):

@@ -428,8 +428,12 @@ def get_top_experts_per_item_dispatcher(
 
 
 def _route(gates: Array, num_selected_experts: int, capacity: int, batch_priority: bool,
-           topk: Optional[Tuple[Array, Array]] = None, **dispatcher_kwargs):
-  """Shared core of vmoe/moe.py:547-590: top-k, priority order, slot positions."""
+           topk: Optional[Tuple[Array, Array]] = None, _metrics=None, **dispatcher_kwargs):
+  """Shared core of vmoe/moe.py:547-590: top-k, priority order, slot positions.
+
+  ``_metrics=(gshard_loss_weight, importance_loss_weight, out)`` (used by the routers)
+  computes the auxiliary losses of vmoe/nn/routing.py:133-157 in the same launch and
+  stores them in the dict ``out``."""
   if gates.ndim not in (2, 3):
     raise ValueError(f"gates must be (S, E) or (G, S, E), got {tuple(gates.shape)}")
   batched = gates.ndim == 3
@@ -439,8 +443,14 @@ def _route(gates: Array, num_selected_experts: int, capacity: int, batch_priorit
     val, idx = K.topk(g3, num_selected_experts)
   else:
     val, idx = topk
-  indices, token_slot, slot_token, fill = K.route_assign(
-      val, idx, num_experts, capacity, batch_priority)
+  if _metrics is not None and batched:
+    w_gshard, w_importance, out = _metrics
+    indices, token_slot, slot_token, fill, losses = K.route_assign(
+        val, idx, num_experts, capacity, batch_priority, metrics=(g3, w_gshard, w_importance))
+    out["importance_loss"], out["gshard_loss"], out["auxiliary_loss"] = losses
+  else:
+    indices, token_slot, slot_token, fill = K.route_assign(
+        val, idx, num_experts, capacity, batch_priority)
   inner = ExpertIndicesDispatcher(
       indices=indices, combine_weights=(val, gates.dtype) if gates.dtype != val.dtype else val,
       num_experts=num_experts, capacity=capacity, _slots=(token_slot, slot_token),
@@ -452,10 +462,10 @@ def _route(gates: Array, num_selected_experts: int, capacity: int, batch_priorit
 
 def _get_top_experts_per_item_expert_indices_dispatcher(
     gates: Array, num_selected_experts: int, capacity: int, batch_priority: bool,
-    _topk=None, **dispatcher_kwargs) -> ExpertIndicesDispatcher:
+    _topk=None, _metrics=None, **dispatcher_kwargs) -> ExpertIndicesDispatcher:
   """vmoe/moe.py:626-652."""
   inner, batched = _route(gates, num_selected_experts, capacity, batch_priority, _topk,
-                          **dispatcher_kwargs)
+                          _metrics=_metrics, **dispatcher_kwargs)
   if not batched:   # reference shapes for a single group: (S, K, 2) and (S, K)
     return _SingleGroupView(inner)
   return inner
@@ -463,9 +473,10 @@ def _get_top_experts_per_item_expert_indices_dispatcher(
 
 def _get_top_experts_per_item_einsum_dispatcher(
     gates: Array, num_selected_experts: int, capacity: int, batch_priority: bool,
-    _topk=None, **dispatcher_kwargs) -> EinsumDispatcher:
+    _topk=None, _metrics=None, **dispatcher_kwargs) -> EinsumDispatcher:
   """vmoe/moe.py:593-623."""
-  inner, batched = _route(gates, num_selected_experts, capacity, batch_priority, _topk)
+  inner, batched = _route(gates, num_selected_experts, capacity, batch_priority, _topk,
+                          _metrics=_metrics)
   d = _SparseEinsumDispatcher(inner, gates.dtype, **dispatcher_kwargs)
   if not batched:
     return _SingleGroupView(d)

@@ -43,12 +43,24 @@ class NoisyTopExpertsPerItemRouter(module.Module):
 
   def apply(self, variables, inputs: Array, rngs=None) -> Tuple[BaseDispatcher, Metrics]:
     kernel = variables["params"]["dense"]["kernel"]
+    if self.deterministic or self.noise_std == 0.0:
+      # The losses run as extra workgroups of the slot-assignment launch.
+      gates, _, topk = self._compute_gates_softmax_and_metrics(inputs, kernel, rngs,
+                                                               with_metrics=False)
+      metrics = {}
+      dispatcher = self._create_dispatcher(
+          gates, topk, _metrics=(self.gshard_loss_weight, self.importance_loss_weight, metrics))
+      if not metrics:   # a dispatcher that does not come from the slot-assignment kernel
+        metrics["importance_loss"], metrics["gshard_loss"], metrics["auxiliary_loss"] = (
+            K.router_metrics(gates, topk[1], self.gshard_loss_weight, self.importance_loss_weight))
+      return dispatcher, {k: metrics[k] for k in ("auxiliary_loss", "gshard_loss", "importance_loss")}
     gates, metrics, topk = self._compute_gates_softmax_and_metrics(inputs, kernel, rngs)
     dispatcher = self._create_dispatcher(gates, topk)
     return dispatcher, metrics
 
   def _compute_gates_softmax_and_metrics(self, inputs: Array, kernel: Array, rngs=None,
-                                         num_experts: Optional[int] = None):
+                                         num_experts: Optional[int] = None,
+                                         with_metrics: bool = True):
     num_experts = self.num_experts if num_experts is None else num_experts
     if inputs.ndim != 3:
       raise ValueError(f"inputs.ndim must be 3, but it is {inputs.ndim}")
@@ -64,6 +76,8 @@ class NoisyTopExpertsPerItemRouter(module.Module):
     w = self._cast_kernel(kernel, dtype)
     if self.deterministic or self.noise_std == 0.0:
       gates, val, idx = K.gate_topk(x, w, self.num_selected_experts, logit_bias=self.logit_bias)
+      if not with_metrics:
+        return gates, None, (val, idx)
       importance_loss, gshard_loss, auxiliary_loss = K.router_metrics(
           gates, idx, self.gshard_loss_weight, self.importance_loss_weight)
       metrics = {
@@ -99,12 +113,12 @@ class NoisyTopExpertsPerItemRouter(module.Module):
     cache = self.__dict__.setdefault("_kernel_cache", module.ParamCache())
     return cache.get((kernel,), dtype, lambda: K.cast(kernel, dtype))
 
-  def _create_dispatcher(self, gates_dispatch: Array, topk=None):
+  def _create_dispatcher(self, gates_dispatch: Array, topk=None, _metrics=None):
     dispatcher_kwargs = dict(**(self.dispatcher or {}))
     use_bfloat16 = dispatcher_kwargs.pop("bfloat16", False)
     dispatcher = vmoe_amd.moe.get_top_experts_per_item_dispatcher(
         gates_dispatch, num_selected_experts=self.num_selected_experts, _topk=topk,
-        **dispatcher_kwargs)
+        _metrics=_metrics, **dispatcher_kwargs)
     if use_bfloat16:
       dispatcher = vmoe_amd.moe.Bfloat16Dispatcher(dispatcher)
     return dispatcher
