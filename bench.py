@@ -172,6 +172,32 @@ def soft_main(args):
                    "traffic": None, "launch_ms": mlp_ms / 2, "bytes_per_layer": bytes_mlp},
       "stage_ms": stage_ms, "cpu_baseline": None,
   }
+  if not args.no_cpu_baseline:
+    # The oracle's Soft MoE layer on the first groups of the same batch (the expert
+    # MLPs see `groups` rows each instead of G, all 128 experts' weights are read).
+    from oracle import moe_oracle as O
+    groups = 32
+    f = lambda t: t.detach().float().cpu().numpy()
+    x_np, mu_np, w0_np, w1_np = f(xs[0][:groups]), f(mu), f(w0), f(w1)
+    b0_np, b1_np = np.zeros((n, M), np.float32), np.zeros((n, D), np.float32)
+
+    def run():
+      odisp, _ = O.soft_router(x_np, mu_np, 1.0, O.BF16, compute_similarity_metrics=False)
+      return O.sparse_moe(odisp, lambda b: O.mlp_block(b, w0_np, b0_np, w1_np, b1_np, O.BF16), x_np)
+    run()
+    times = []
+    for _ in range(3):
+      t0 = time.perf_counter()
+      run()
+      times.append(time.perf_counter() - t0)
+    t = float(np.median(times))
+    result["cpu_baseline"] = {
+        "value": groups * m / t, "unit": "tokens/s", "cores": int(torch.get_num_threads()),
+        "kind": "port",
+        "sample": (f"oracle/moe_oracle.py soft_router + sparse_moe(mlp_block) on {groups} of {G} "
+                   f"groups ({groups * m} tokens, all {n} experts), median of 3 runs of {t:.2f} s; "
+                   "NumPy BLAS + torch CPU threads"),
+        "host_cpus": os.cpu_count()}
   print(json.dumps(result))
 
 
