@@ -177,7 +177,19 @@ __device__ __forceinline__ void store_tile(floatx16 (&acc)[TM / 32][TN / 32], un
     const int row = wrow0 + rl;
     const int col = wcol0 + oc;
     uint4 v = *reinterpret_cast<const uint4*>(so + rl * OLD + oc);
-    if (row < live && col + 8 <= N) *reinterpret_cast<uint4*>(Cb + (size_t)row * N + col) = v;
+    if (row < live && col + 8 <= N) {
+      // The activated hidden layer (hundreds of MB, read back once by the second product)
+      // is larger than any cache: it leaves with streaming stores so that it does not
+      // evict the operands.  The second product's output is read next by combine and
+      // stays cacheable.
+      if constexpr (EPI != kEpiBias) {
+        typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+        __builtin_nontemporal_store(__builtin_bit_cast(u32x4_t, v),
+                                    reinterpret_cast<u32x4_t*>(Cb + (size_t)row * N + col));
+      } else {
+        *reinterpret_cast<uint4*>(Cb + (size_t)row * N + col) = v;
+      }
+    }
   }
 }
 
