@@ -17,13 +17,30 @@ template <> struct Vec4<float> {
   __device__ static __forceinline__ float4 load(const float* p) {
     return *reinterpret_cast<const float4*>(p);
   }
+  __device__ static __forceinline__ float4 load_stream(const float* p) {
+    typedef float f32x4_t __attribute__((ext_vector_type(4)));
+    const f32x4_t t = __builtin_nontemporal_load(reinterpret_cast<const f32x4_t*>(p));
+    return make_float4(t.x, t.y, t.z, t.w);
+  }
   __device__ static __forceinline__ void store(float* p, float4 v) {
     *reinterpret_cast<float4*>(p) = v;
+  }
+  // For data that is not read again soon (the residual stream between two blocks'
+  // norms: another few hundred MB pass through the caches first).
+  __device__ static __forceinline__ void store_stream(float* p, float4 v) {
+    typedef float f32x4_t __attribute__((ext_vector_type(4)));
+    f32x4_t t = {v.x, v.y, v.z, v.w};
+    __builtin_nontemporal_store(t, reinterpret_cast<f32x4_t*>(p));
   }
 };
 template <> struct Vec4<bf16_t> {
   __device__ static __forceinline__ float4 load(const bf16_t* p) {
     const uint2 u = *reinterpret_cast<const uint2*>(p);
+    return make_float4(bf_lo(u.x), bf_hi(u.x), bf_lo(u.y), bf_hi(u.y));
+  }
+  __device__ static __forceinline__ float4 load_stream(const bf16_t* p) {
+    typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
+    const u32x2_t u = __builtin_nontemporal_load(reinterpret_cast<const u32x2_t*>(p));
     return make_float4(bf_lo(u.x), bf_hi(u.x), bf_lo(u.y), bf_hi(u.y));
   }
   __device__ static __forceinline__ void store(bf16_t* p, float4 v) {
@@ -74,12 +91,12 @@ __global__ __launch_bounds__(kLnThreads) void add_layer_norm_kernel(
       const int c = lane + 64 * i;
       v[i] = make_float4(0.f, 0.f, 0.f, 0.f);
       if (c < chunks) {
-        v[i] = Vec4<float>::load(residual + base + 4 * c);
+        v[i] = Vec4<float>::load_stream(residual + base + 4 * c);
         if (branch != nullptr) {
-          const float4 b = Vec4<TB>::load(branch + base + 4 * c);
+          const float4 b = Vec4<TB>::load_stream(branch + base + 4 * c);
           v[i].x += b.x; v[i].y += b.y; v[i].z += b.z; v[i].w += b.w;
         }
-        if (residual_out != nullptr) Vec4<float>::store(residual_out + base + 4 * c, v[i]);
+        if (residual_out != nullptr) Vec4<float>::store_stream(residual_out + base + 4 * c, v[i]);
       }
       s += (v[i].x + v[i].y) + (v[i].z + v[i].w);
       s2 += (v[i].x * v[i].x + v[i].y * v[i].y) + (v[i].z * v[i].z + v[i].w * v[i].w);
