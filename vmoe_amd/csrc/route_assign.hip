@@ -31,17 +31,25 @@ __host__ __device__ inline int pow2ceil(int v) {
 }
 
 // One side of a compare-exchange: the smaller (take_min) or larger of two keys.
-__device__ __forceinline__ uint64_t pick(uint64_t mine, uint64_t other, bool take_min) {
+template <typename KeyT>
+__device__ __forceinline__ KeyT pick(KeyT mine, KeyT other, bool take_min) {
   return ((other < mine) == take_min) ? other : mine;
 }
 
-template <int R, int ST>
-__device__ __forceinline__ void bitonic_in_thread(uint64_t (&key)[R], int size, int tid) {
+__device__ __forceinline__ uint64_t lane_exchange(uint64_t v, int lane_xor) {
+  return __shfl_xor((unsigned long long)v, lane_xor, kWave);
+}
+__device__ __forceinline__ uint32_t lane_exchange(uint32_t v, int lane_xor) {
+  return __shfl_xor(v, lane_xor, kWave);
+}
+
+template <int R, int ST, typename KeyT>
+__device__ __forceinline__ void bitonic_in_thread(KeyT (&key)[R], int size, int tid) {
 #pragma unroll
   for (int r = 0; r < R; ++r) {
     if ((r & ST) == 0 && r + ST < R) {
       const bool up = (((tid * R + r) & size) == 0);
-      const uint64_t a = key[r], b = key[r + ST];
+      const KeyT a = key[r], b = key[r + ST];
       const bool swap = (b < a) == up;
       key[r] = swap ? b : a;
       key[r + ST] = swap ? a : b;
@@ -49,43 +57,52 @@ __device__ __forceinline__ void bitonic_in_thread(uint64_t (&key)[R], int size, 
   }
 }
 
-// Ascending bitonic sort of the first SP (a power of two) of 1024*R keys, element
-// tid*R + r in key[r] of thread tid.  Every thread of the workgroup calls it; `xch`
-// holds 1024*R keys.
-template <int R>
-__device__ __forceinline__ void bitonic_sort_regs(uint64_t (&key)[R], uint64_t* xch, int SP,
-                                                  int tid) {
+// Ascending bitonic sort of SP (a power of two) keys, element tid*R + r in key[r] of
+// thread tid < nact = SP / R.  Every thread of the workgroup calls it (the LDS stages
+// have barriers); `xch` holds SP keys.
+template <int R, typename KeyT>
+__device__ __forceinline__ void bitonic_sort_regs(KeyT (&key)[R], KeyT* xch, int SP, int tid,
+                                                  int nact) {
+  const bool act = tid < nact;
   for (int size = 2; size <= SP; size <<= 1) {
     for (int stride = size >> 1; stride > 0; stride >>= 1) {
       if (stride >= 64 * R) {
+        if (act) {
 #pragma unroll
-        for (int r = 0; r < R; ++r) xch[tid * R + r] = key[r];
-        __syncthreads();
-#pragma unroll
-        for (int r = 0; r < R; ++r) {
-          const int i = tid * R + r;
-          key[r] = pick(key[r], xch[i ^ stride], ((i & stride) == 0) == ((i & size) == 0));
+          for (int r = 0; r < R; ++r) xch[tid * R + r] = key[r];
         }
         __syncthreads();
+        if (act) {
+#pragma unroll
+          for (int r = 0; r < R; ++r) {
+            const int i = tid * R + r;
+            key[r] = pick<KeyT>(key[r], xch[i ^ stride], ((i & stride) == 0) == ((i & size) == 0));
+          }
+        }
+        __syncthreads();
+      } else if (!act) {
+        continue;
       } else if (stride >= R) {
         const int lane_xor = stride / R;
 #pragma unroll
         for (int r = 0; r < R; ++r) {
           const int i = tid * R + r;
-          const uint64_t other = __shfl_xor((unsigned long long)key[r], lane_xor, kWave);
+          const KeyT other = lane_exchange(key[r], lane_xor);
           key[r] = pick(key[r], other, ((i & stride) == 0) == ((i & size) == 0));
         }
       } else {
-        if constexpr (R > 4) { if (stride == 4) bitonic_in_thread<R, 4>(key, size, tid); }
-        if constexpr (R > 2) { if (stride == 2) bitonic_in_thread<R, 2>(key, size, tid); }
-        if constexpr (R > 1) { if (stride == 1) bitonic_in_thread<R, 1>(key, size, tid); }
+        if constexpr (R > 4) { if (stride == 4) bitonic_in_thread<R, 4, KeyT>(key, size, tid); }
+        if constexpr (R > 2) { if (stride == 2) bitonic_in_thread<R, 2, KeyT>(key, size, tid); }
+        if constexpr (R > 1) { if (stride == 1) bitonic_in_thread<R, 1, KeyT>(key, size, tid); }
       }
     }
   }
 }
 
-// Keys per thread for a sort of SP keys by 1024 threads; 0 = the keys do not fit in
-// registers and are sorted in LDS.
+// Keys per thread for a sort of SP keys: as many threads as the workgroup has take part
+// (a stage costs a wave its shuffles and selects per key, so more waves with fewer keys
+// are faster: eight keys on an eighth of the threads took 35 us where two keys on all
+// take 25); 0 = the keys do not fit in the registers and are sorted in LDS.
 inline int keys_per_thread(int SP) {
   const int r = SP <= kRouteThreads ? 1 : SP / kRouteThreads;
   return r <= 8 ? r : 0;
@@ -135,16 +152,43 @@ __device__ __forceinline__ void route_assign_group(
       bitonic_sort_lds(keys, SP, tid);
       for (int r = tid; r < S; r += kRouteThreads) rank[(uint32_t)keys[r]] = r;
     } else {
-      uint64_t key[R];
+      // Gates that came out of a bfloat16 router are non-negative floats whose low 16
+      // bits are zero: gate and item index then fit one 32-bit key (S <= 65536), and the
+      // sort's compare-exchanges, which are what bounds this kernel, cost half as much.
+      const int nact = SP / R;
+      uint32_t bits[R];
+      bool narrow_ok = S <= 65536;
 #pragma unroll
       for (int r = 0; r < R; ++r) {
         const int s = tid * R + r;
-        key[r] = s < S ? ((uint64_t)(~orderable(val[(size_t)s * K])) << 32) | (uint32_t)s : ~0ull;
+        bits[r] = (tid < nact && s < S) ? __builtin_bit_cast(uint32_t, val[(size_t)s * K]) : 0u;
+        narrow_ok = narrow_ok && (bits[r] & 0x8000ffffu) == 0u;
       }
-      bitonic_sort_regs<R>(key, keys, SP, tid);
+      if (__syncthreads_and(narrow_ok)) {
+        uint32_t key[R];
 #pragma unroll
-      for (int r = 0; r < R; ++r)
-        if (tid * R + r < S) rank[(uint32_t)key[r]] = tid * R + r;
+        for (int r = 0; r < R; ++r) {
+          const int s = tid * R + r;
+          key[r] = s < S ? ((~orderable(__builtin_bit_cast(float, bits[r]))) & 0xffff0000u) | (uint32_t)s
+                         : ~0u;
+        }
+        bitonic_sort_regs<R, uint32_t>(key, reinterpret_cast<uint32_t*>(keys), SP, tid, nact);
+#pragma unroll
+        for (int r = 0; r < R; ++r)
+          if (tid < nact && tid * R + r < S) rank[key[r] & 0xffffu] = tid * R + r;
+      } else {
+        uint64_t key[R];
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+          const int s = tid * R + r;
+          key[r] = s < S ? ((uint64_t)(~orderable(__builtin_bit_cast(float, bits[r]))) << 32) | (uint32_t)s
+                         : ~0ull;
+        }
+        bitonic_sort_regs<R, uint64_t>(key, keys, SP, tid, nact);
+#pragma unroll
+        for (int r = 0; r < R; ++r)
+          if (tid < nact && tid * R + r < S) rank[(uint32_t)key[r]] = tid * R + r;
+      }
     }
   } else {
     for (int s = tid; s < S; s += kRouteThreads) rank[s] = s;
@@ -290,17 +334,19 @@ __global__ __launch_bounds__(kRouteThreads) void top_items_kernel(
     bitonic_sort_lds(keys, SP, tid);
     for (int r = tid; r < S; r += kRouteThreads) emit(r, (int)(uint32_t)keys[r]);
   } else {
+    const int nact = SP / R;
     uint64_t key[R];
 #pragma unroll
     for (int r = 0; r < R; ++r) {
       const int s = tid * R + r;
-      key[r] = s < S ? ((uint64_t)(~orderable(Elt<T>::load(col + (size_t)s * E))) << 32) | (uint32_t)s
-                     : ~0ull;
+      key[r] = (tid < nact && s < S)
+                   ? ((uint64_t)(~orderable(Elt<T>::load(col + (size_t)s * E))) << 32) | (uint32_t)s
+                   : ~0ull;
     }
-    bitonic_sort_regs<R>(key, keys, SP, tid);
+    bitonic_sort_regs<R, uint64_t>(key, keys, SP, tid, nact);
 #pragma unroll
     for (int r = 0; r < R; ++r)
-      if (tid * R + r < S) emit(tid * R + r, (int)(uint32_t)key[r]);
+      if (tid < nact && tid * R + r < S) emit(tid * R + r, (int)(uint32_t)key[r]);
   }
   for (int c = S + tid; c < C; c += kRouteThreads) slot_token[slot_row(e, g, c, G, E, C)] = -1;
 }
@@ -477,7 +523,7 @@ static int launch_route_assign(const VmoeRouteAssignParams* p, const VmoeRouterM
   const int SP = pow2ceil(p->S);
   const int W = (p->S * p->K + 31) / 32;
   const int R = keys_per_thread(SP);
-  const int NK = R == 0 ? SP : kRouteThreads * R;
+  const int NK = SP;
   size_t lds = (p->batch_priority ? (size_t)NK * 8 : 0) + (size_t)p->E * W * 8 +
                (size_t)p->S * 4 + (size_t)p->E * 4;
   RouterMetricsArgs ma{};
@@ -583,7 +629,7 @@ extern "C" int vmoe_top_items_per_expert(const VmoeTopItemsParams* p, vmoe_strea
     return VMOE_E_OVERFLOW;
   const int SP = pow2ceil(p->S < 2 ? 2 : p->S);
   const int R = keys_per_thread(SP);
-  const size_t lds = (size_t)(R == 0 ? SP : kRouteThreads * R) * 8;
+  const size_t lds = (size_t)SP * 8;
   if (lds > 160 * 1024) return VMOE_E_UNSUPPORTED;
   dim3 grid(p->E, p->G);
   auto launch = [&](auto kern, auto* gates) -> int {
