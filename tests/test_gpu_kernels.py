@@ -176,6 +176,43 @@ def test_route_assign_with_metrics_equals_separate_calls(K, G, S, E, k, C, dtype
     assert torch.equal(a, b)
 
 
+def test_route_assign_random_shapes(K):
+  """Seeded sweep over group sizes around the sort's switch points (keys per thread,
+  partial waves), expert counts, gate flavours (float32, bfloat16-valued -> 32-bit sort
+  keys, coarse values with many ties, negative and zero gates) against the sequential
+  C statement of the assignment."""
+  rng = np.random.default_rng(2024)
+  sizes = [1, 2, 3, 31, 32, 33, 63, 64, 65, 127, 128, 129, 255, 256, 257, 511, 512, 513, 1000,
+           1023, 1024, 1025, 1500, 2047, 2048, 2049, 3000, 4095, 4096, 4097]
+  for case, S in enumerate(sizes * 2):
+    E = int(rng.integers(1, 41))
+    k = int(rng.integers(1, min(E, 4) + 1))
+    G = int(rng.integers(1, 4))
+    C = int(rng.integers(1, max(2, (S * k) // E + 3)))
+    flavour = case % 4
+    pow2 = 1 << max(0, (S - 1).bit_length())
+    lds = 8 * max(1024, pow2) + 8 * E * ((S * k + 31) // 32) + 4 * S + 4 * E
+    if lds > 160 * 1024:      # the entry point's documented limit: such shapes are refused
+      E = max(k, (160 * 1024 - 8 * max(1024, pow2) - 4 * S) // (8 * ((S * k + 31) // 32) + 4) - 1)
+    logits = rng.standard_normal((G, S, E)).astype(np.float32) * 2
+    if flavour == 0:
+      gates = O.softmax(logits)
+    elif flavour == 1:
+      gates = O.bf16_round(O.softmax(logits))
+    elif flavour == 2:
+      gates = O.bf16_round(O.softmax(np.round(logits)))      # many equal gates
+    else:
+      gates = np.round(logits * 2).astype(np.float32) / 4       # negative, zero and tied "gates"
+    val, idx = K.topk(to_dev(gates), k)
+    got, _, _, fill = K.route_assign(val, idx, E, C, True)
+    want, want_w = route_c.route_batch(gates, k, True)
+    np.testing.assert_array_equal(to_np(got), want, err_msg=f"S={S} E={E} k={k} G={G} C={C} flavour={flavour}")
+    np.testing.assert_array_equal(to_np(val), want_w)
+    e = want[..., 0]
+    demand = np.stack([np.bincount(e[g].ravel(), minlength=E) for g in range(G)])
+    np.testing.assert_array_equal(to_np(fill), np.minimum(demand, C))
+
+
 def test_route_assign_golden(K, goldens):
   g = goldens["top_experts_per_item"]
   gates = np.asarray(g["gates"], np.float32)[None]
