@@ -49,6 +49,14 @@ GATE_CASES = [
     (2, 64, 264, 40, 4, O.BF16),
     (2, 37, 128, 100, 2, O.F32),
     (1, 1568, 768, 32, 2, O.BF16),
+    (1, 33000, 1024, 32, 2, O.BF16),   # eight-wave workgroups (one staged router kernel per CU)
+    (2, 77, 2048, 32, 2, O.BF16),      # router kernel staged in two chunks along D
+    (2, 45, 768, 16, 2, O.BF16),       # experts padded to the 32-wide tile
+    (2, 45, 320, 12, 3, O.BF16),       # expert count not a multiple of 8: element-wise staging
+    (3, 31, 72, 8, 1, O.BF16),         # D not a multiple of 64
+    (2, 50, 256, 64, 2, O.BF16),       # two expert tiles
+    (1, 70, 192, 128, 4, O.BF16),      # four expert tiles
+    (1, 70, 96, 128, 4, O.F32),
 ]
 
 
