@@ -497,7 +497,7 @@ def test_compact_rows(K, G, S, E, Kk, C, bpr):
 
 
 @pytest.mark.parametrize("dtype", [O.F32, O.BF16])
-@pytest.mark.parametrize("E", [5, 20])      # planned launch (few experts per die) / static order
+@pytest.mark.parametrize("E", [5, 20])      # fewer / more experts than dies in the launch plan
 def test_expert_mlp_rows_per_expert(K, dtype, E):
   """Leading rows equal the full computation bit for bit; the other rows are not written."""
   rng = np.random.default_rng(3)
@@ -517,6 +517,32 @@ def test_expert_mlp_rows_per_expert(K, dtype, E):
   for e, n in enumerate(rows):
     np.testing.assert_array_equal(to_np(out[e, :n]), to_np(full[e, :n]))
     assert (to_np(out[e, n:]) == 7.0).all()
+
+
+def test_expert_mlp_planned_launch_random_fill(K):
+  """bf16 expert products over packed rows with a die-balanced launch plan: random row
+  counts (empty, one row, tile boundaries, full), expert counts below and above the
+  number of dies, row capacities below and above a tile."""
+  rng = np.random.default_rng(11)
+  dtype = O.BF16
+  for E, R, D, M in [(1, 700, 64, 96), (3, 130, 96, 64), (8, 520, 64, 128), (9, 257, 128, 64),
+                     (17, 300, 64, 64), (40, 100, 64, 96), (64, 33, 96, 64)]:
+    x = to_dev(O.cast(rng.standard_normal((E, R, D)).astype(np.float32), dtype), dtype)
+    w0 = to_dev(O.cast(rng.standard_normal((E, D, M)).astype(np.float32) / 8, dtype), dtype)
+    w1 = to_dev(O.cast(rng.standard_normal((E, M, D)).astype(np.float32) / 11, dtype), dtype)
+    b0 = to_dev(O.cast(rng.standard_normal((E, M)).astype(np.float32) * 0.1, dtype), dtype)
+    b1 = to_dev(O.cast(rng.standard_normal((E, D)).astype(np.float32) * 0.1, dtype), dtype)
+    full = K.expert_mlp(x, w0, b0, w1, b1)
+    for trial in range(3):
+      special = np.asarray([0, 1, 127, 128, 129, 255, 256, 257, R], np.int64)
+      rows = np.where(rng.random(E) < 0.5, rng.integers(0, R + 1, E), rng.choice(special, E))
+      rows = np.minimum(rows, R).astype(np.int32)
+      out = torch.full_like(full, 7.0)
+      K.expert_mlp(x, w0, b0, w1, b1, out=out, rows_per_expert=to_dev(rows))
+      for e, n in enumerate(rows):
+        np.testing.assert_array_equal(to_np(out[e, :n]), to_np(full[e, :n]),
+                                      err_msg=f"E={E} R={R} rows={rows.tolist()} expert {e}")
+        assert (to_np(out[e, n:]) == 7.0).all(), f"E={E} R={R} rows={rows.tolist()} expert {e}"
 
 
 @pytest.mark.parametrize("G,S,N,dtype", [(3, 50, 16, O.F32), (4, 196, 128, O.BF16), (2, 7, 300, O.BF16), (3, 196, 128, O.F32),
