@@ -70,12 +70,26 @@ def test_indices(moe, goldens, case):
   _run_dispatcher_test(goldens, d, case)
 
 
-def test_indices_duplicate_slots_raise(moe):
-  idx = to_dev(np.asarray([[[[0, 0]], [[0, 0]]]], np.int32))
-  cw = torch.ones((1, 2, 1), device=dev())
-  d = moe.ExpertIndicesDispatcher(indices=idx, combine_weights=cw, num_experts=2, capacity=2)
-  with pytest.raises(ValueError, match="same"):
-    d.dispatch(torch.ones((1, 2, 4), device=dev()))
+@pytest.mark.parametrize("dtype", [O.F32, O.BF16])
+def test_indices_shared_slots_accumulate(moe, dtype):
+  """Hand-made indices that send several items to one slot: dispatch adds them up, as the
+  reference's scatter-add does (vmoe/moe.py:190-197, :522-544); combine gathers as usual."""
+  rng = np.random.default_rng(8)
+  G, S, Kk, E, C, D = 3, 40, 2, 4, 5, 24
+  idx = np.stack([rng.integers(0, E + 1, (G, S, Kk)), rng.integers(0, C + 2, (G, S, Kk))], -1).astype(np.int32)
+  idx[0, :4, 0] = (1, 2)                       # four items in one slot
+  cw = rng.random((G, S, Kk)).astype(np.float32)
+  x = O.cast(rng.standard_normal((G, S, D)), dtype)
+  d = moe.ExpertIndicesDispatcher(indices=to_dev(idx), combine_weights=to_dev(cw), num_experts=E, capacity=C)
+  od = O.ExpertIndicesDispatcher(idx, cw, E, C)
+  buf = d.dispatch(to_dev(x, dtype))
+  want = od.dispatch(x.astype(np.float32))
+  assert_close(to_np(buf), O.cast(want, dtype), 1e-6 if dtype == O.F32 else 1e-2, "accumulated dispatch")
+  y = O.cast(rng.standard_normal((E, G * C, D)), dtype)
+  np.testing.assert_allclose(to_np(d.combine(to_dev(y, dtype))), O.cast(od.combine(y.astype(np.float32)), dtype),
+                             rtol=1e-5 if dtype == O.F32 else 2e-2, atol=1e-5 if dtype == O.F32 else 2e-2)
+  # a second call reuses the per-occurrence maps
+  assert torch.equal(d.dispatch(to_dev(x, dtype)), buf)
 
 
 # ------------------------------------------------------------------ GetTopExpertsPerItemDispatcherTest

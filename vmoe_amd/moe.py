@@ -106,8 +106,10 @@ class ExpertIndicesDispatcher(BaseDispatcher):
     combine_weights: (G, S, K).
     num_experts, capacity: static sizes of the expert buffer.
 
-  Unlike the reference's scatter-add, two items may not share a slot (routers
-  never produce that); such hand-made indices raise ValueError.
+  Routers give every slot at most one item.  Hand-made indices that send several items
+  to one slot are accumulated as the reference's scatter-add does (vmoe/moe.py:190-197,
+  :522-544): dispatch then runs once per "occurrence" (the r-th item of every slot) and
+  the passes are added in float32, in item order.
   """
 
   def __init__(self, indices: Array, combine_weights: Array, num_experts: int, capacity: int,
@@ -122,6 +124,7 @@ class ExpertIndicesDispatcher(BaseDispatcher):
     self._weights_f32 = None                      # float32 copy of combine_weights, if on hand
     self.fill = None                              # (G, E) kept items per (group, expert), if known
     self._packed_maps = None                      # (token_row (G,S,K), rows_per_expert (E,))
+    self._rounds = None                           # per-occurrence slot maps when slots are shared
 
   @property
   def combine_weights(self) -> Array:
@@ -144,16 +147,47 @@ class ExpertIndicesDispatcher(BaseDispatcher):
       if invalid:
         raise ValueError("ExpertIndicesDispatcher: negative indices are not supported.")
       if dups:
-        raise ValueError("ExpertIndicesDispatcher: several items target the same "
-                         "(expert, position) slot; accumulating dispatch is not supported.")
+        self._rounds = self._occurrence_rounds(token_slot, slot_token.numel())
       self._slots = (token_slot, slot_token)
     return self._slots
+
+  @staticmethod
+  def _occurrence_rounds(token_slot: Array, num_slots: int):
+    """Splits the assignments so that no slot appears twice in a part: part r holds, for
+    every slot, its r-th assignment in item order.  Returns [(token_slot_r, slot_token_r)]."""
+    flat = token_slot.reshape(-1).to(torch.int64)
+    K_ = token_slot.shape[-1]
+    order = torch.argsort(flat, stable=True)
+    sorted_slots = flat[order]
+    first = torch.ones_like(sorted_slots, dtype=torch.bool)
+    first[1:] = sorted_slots[1:] != sorted_slots[:-1]
+    pos = torch.arange(flat.numel(), device=flat.device)
+    start = torch.where(first, pos, torch.zeros_like(pos)).cummax(0).values
+    occurrence = torch.empty_like(flat)
+    occurrence[order] = pos - start
+    occurrence[flat < 0] = -1
+    rounds = []
+    for r in range(int(occurrence.max().item()) + 1):
+      mine = occurrence == r
+      ts_r = torch.where(mine, flat, torch.full_like(flat, -1)).to(torch.int32)
+      st_r = torch.full((num_slots,), -1, dtype=torch.int32, device=flat.device)
+      st_r[flat[mine]] = (pos[mine] // K_).to(torch.int32)
+      rounds.append((ts_r.view(-1, K_).contiguous(), st_r))
+    return rounds
 
   def dispatch(self, data: Array) -> Array:
     G, S, Kk, _ = self.indices.shape
     token_slot, slot_token = self._maps()
     rows, item_shape, width = _as_rows(data, 2)
-    if _wants_grad(rows):
+    if self._rounds is not None:
+      if _wants_grad(rows):
+        raise NotImplementedError("gradients through a dispatch with shared slots")
+      acc = None
+      for ts_r, st_r in self._rounds:
+        part = K.dispatch(rows, ts_r, st_r).to(torch.float32)
+        acc = part if acc is None else acc + part
+      out = acc.to(rows.dtype)
+    elif _wants_grad(rows):
       out = _DispatchFn.apply(rows, token_slot.view(G * S, Kk), slot_token, slot_token.numel())
     else:
       out = K.dispatch(rows, token_slot.view(G * S, Kk), slot_token)
