@@ -6,7 +6,10 @@
 // Work split: a wave owns a tile of 32 items.  The router kernel W (D x E) is
 // staged once per workgroup in LDS (bf16: transposed to [expert][k] so that a
 // lane's MFMA B fragment is one 16-byte read; f32: kept [k][expert]).  Item rows
-// stream from HBM with 16-byte loads, 64 contiguous bytes per lane per step.
+// stream from HBM with 16-byte loads, 64 contiguous bytes per lane per step; in
+// bf16 they pass through two register buffers that are refilled as soon as their
+// MFMAs are issued, and the first loads go out before the router kernel is staged,
+// so that every workgroup of the launch is resident and loading from the start.
 // After the K loop the logits tile passes through a wave-private LDS tile, so
 // that each lane holds half of one item's row: softmax and top-K are serial per
 // lane, with one xor-32 shuffle per reduction to join the two halves.
