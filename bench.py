@@ -88,6 +88,14 @@ def cpu_baseline(cfg, x_np, params_np, bias_np, groups):
     times.append(time.perf_counter() - t0)
   t = float(np.median(times))
   import torch
+  # The same layer in the formulation the reference's released configs use (the einsum
+  # dispatcher with its dense (G, S, E, C) weights, vmoe/moe.py:127-161), on two groups.
+  eg = min(2, groups)
+  xe = x_np[:eg * cfg.group_images]
+  t0 = time.perf_counter()
+  O.mlp_moe_block(xe, params_np, group_size=S, num_selected_experts=cfg.num_selected_experts,
+                  dispatcher_kwargs=cfg.dispatcher_kwargs("einsum"), dtype=dtype, logit_bias=bias_np)
+  te = time.perf_counter() - t0
   return {
       "value": groups * S / t, "unit": "tokens/s", "cores": int(torch.get_num_threads()),
       "kind": "port",
@@ -95,6 +103,9 @@ def cpu_baseline(cfg, x_np, params_np, bias_np, groups):
                  f"{cfg.num_groups} groups ({groups * S} tokens, all {cfg.num_experts} experts), "
                  f"median of 3 runs of {t:.2f} s; NumPy BLAS + torch CPU threads"),
       "host_cpus": os.cpu_count(),
+      "einsum_dispatcher_formulation": {
+          "value": eg * S / te, "unit": "tokens/s",
+          "sample": f"same oracle with the einsum dispatcher on {eg} groups ({eg * S} tokens), one run of {te:.2f} s"},
   }
 
 
