@@ -344,6 +344,9 @@ typedef struct {
   size_t workspace_bytes;
   int32_t G, S, D, N;
   int32_t dtype;
+  int32_t workspace_prepared; /* 1: `workspace` still holds what an earlier call with the same mu,
+                                 scale, dtype and (G, S, D, N) left there; the slot parameters are
+                                 not normalised again (they are constants at inference) */
 } VmoeSoftRouteParams;
 size_t vmoe_soft_route_workspace_bytes(const VmoeSoftRouteParams* p);
 int vmoe_soft_route(const VmoeSoftRouteParams* p, vmoe_stream_t stream);

@@ -795,3 +795,38 @@ def test_layer_replays_from_hip_graph(dtype, dkw):
       for key in metrics:
         assert torch.equal(metrics[key], eager[i][1][key]), (rep, i, key)
       layer.apply(variables, xs[(i + 1) % 3])   # eager work between replays
+
+
+def test_soft_router_reuses_prepared_slot_parameters():
+  """The normalised slot parameters are kept between calls; a changed mu or scale
+  (new tensor or in-place update) must not be served from the kept copy."""
+  from vmoe_amd.projects.soft_moe import router
+  rng = np.random.default_rng(12)
+  G, m, D, n = 3, 40, 64, 8
+  x = to_dev(O.cast(rng.standard_normal((G, m, D)), O.BF16), O.BF16)
+  mu = to_dev((rng.standard_normal((D, n, 1)) / np.sqrt(D)).astype(np.float32))
+  scale = torch.tensor(1.5, device=dev())
+  layer = router.SoftRouter(num_experts=n, num_slots=1, compute_similarity_metrics=False)
+
+  def weights(r, mu_, scale_):
+    d, _ = r.apply({"params": {"mu": mu_, "scale": scale_}}, x)
+    return d.dispatcher.combine_weights.clone(), d.dispatcher.dispatch_weights.clone()
+
+  def fresh(mu_, scale_):
+    return weights(router.SoftRouter(num_experts=n, num_slots=1, compute_similarity_metrics=False),
+                   mu_, scale_)
+
+  first = weights(layer, mu, scale)
+  again = weights(layer, mu, scale)
+  for a, b in zip(first, again):
+    assert torch.equal(a, b)
+  mu.mul_(-1.0)                                  # in-place parameter update
+  for a, b in zip(weights(layer, mu, scale), fresh(mu, scale)):
+    assert torch.equal(a, b)
+  assert not torch.equal(weights(layer, mu, scale)[0], first[0])
+  scale.fill_(0.5)
+  for a, b in zip(weights(layer, mu, scale), fresh(mu, scale)):
+    assert torch.equal(a, b)
+  mu2 = mu.clone() * 2.0 + 0.1                   # another tensor
+  for a, b in zip(weights(layer, mu2, scale), fresh(mu2, scale)):
+    assert torch.equal(a, b)

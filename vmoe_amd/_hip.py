@@ -170,7 +170,7 @@ class SoftRouteParams(ctypes.Structure):
   _fields_ = [("x", c_void_p), ("mu", c_void_p), ("scale", c_float), ("dispatch_w", c_void_p),
               ("combine_w", c_void_p), ("logits", c_void_p), ("workspace", c_void_p),
               ("workspace_bytes", c_size_t), ("G", c_int32), ("S", c_int32), ("D", c_int32),
-              ("N", c_int32), ("dtype", c_int32)]
+              ("N", c_int32), ("dtype", c_int32), ("workspace_prepared", c_int32)]
 
 
 class EinsumParams(ctypes.Structure):

@@ -758,8 +758,9 @@ extern "C" int vmoe_soft_route(const VmoeSoftRouteParams* p, vmoe_stream_t strea
   const SoftLds L = soft_lds_layout(p->D, SP, NP);
   if (p->dtype == VMOE_BF16 && p->N <= 128 && p->N % 8 == 0 && soft_fast_width(p->D) && L.total <= 160 * 1024 && aligned16(p->dispatch_w) && aligned16(p->combine_w) &&
       (p->logits == nullptr || aligned16(p->logits))) {
-    hipLaunchKernelGGL(soft_prep_mu_kernel<bf16_t>, dim3(p->N), dim3(256), 0, stream,
-                       (const bf16_t*)p->mu, (bf16_t*)p->workspace, p->scale, !scale_x, p->D, p->N);
+    if (!p->workspace_prepared)
+      hipLaunchKernelGGL(soft_prep_mu_kernel<bf16_t>, dim3(p->N), dim3(256), 0, stream,
+                         (const bf16_t*)p->mu, (bf16_t*)p->workspace, p->scale, !scale_x, p->D, p->N);
     auto kern = p->D == 1024 ? soft_route_bf16_kernel<32>
                 : p->D == 768 ? soft_route_bf16_kernel<24>
                 : p->D == 512 ? soft_route_bf16_kernel<16>
@@ -774,8 +775,9 @@ extern "C" int vmoe_soft_route(const VmoeSoftRouteParams* p, vmoe_stream_t strea
   } else if (lds > 160 * 1024) {
     return VMOE_E_UNSUPPORTED;
   } else if (p->dtype == VMOE_BF16) {
-    hipLaunchKernelGGL(soft_prep_mu_kernel<bf16_t>, dim3(p->N), dim3(256), 0, stream,
-                       (const bf16_t*)p->mu, (bf16_t*)p->workspace, p->scale, !scale_x, p->D, p->N);
+    if (!p->workspace_prepared)
+      hipLaunchKernelGGL(soft_prep_mu_kernel<bf16_t>, dim3(p->N), dim3(256), 0, stream,
+                         (const bf16_t*)p->mu, (bf16_t*)p->workspace, p->scale, !scale_x, p->D, p->N);
     auto kern = soft_route_kernel<bf16_t>;
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
@@ -784,8 +786,9 @@ extern "C" int vmoe_soft_route(const VmoeSoftRouteParams* p, vmoe_stream_t strea
                        (const bf16_t*)p->workspace, (bf16_t*)p->dispatch_w, (bf16_t*)p->combine_w,
                        (bf16_t*)p->logits, p->scale, scale_x, p->S, p->D, p->N, SP, NP);
   } else {
-    hipLaunchKernelGGL(soft_prep_mu_kernel<float>, dim3(p->N), dim3(256), 0, stream,
-                       (const float*)p->mu, (float*)p->workspace, p->scale, !scale_x, p->D, p->N);
+    if (!p->workspace_prepared)
+      hipLaunchKernelGGL(soft_prep_mu_kernel<float>, dim3(p->N), dim3(256), 0, stream,
+                         (const float*)p->mu, (float*)p->workspace, p->scale, !scale_x, p->D, p->N);
     auto kern = soft_route_kernel<float>;
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);

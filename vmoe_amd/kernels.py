@@ -302,8 +302,13 @@ def expert_mlp_workspace_bytes(E, R, D, M, dtype, prepacked: bool) -> int:
   return int(H.lib().vmoe_expert_mlp_workspace_bytes(H.ctypes.byref(p)))
 
 
-def soft_route(x: torch.Tensor, mu: torch.Tensor, scale: float, return_logits: bool = False):
-  """x (G,S,D), mu (D,N) -> dispatch_w (G,S,N), combine_w (G,S,N) [, logits]."""
+def soft_route(x: torch.Tensor, mu: torch.Tensor, scale: float, return_logits: bool = False,
+               prepared: Optional[dict] = None):
+  """x (G,S,D), mu (D,N) -> dispatch_w (G,S,N), combine_w (G,S,N) [, logits].
+
+  ``prepared``: a dict the caller keeps for as long as mu, scale, dtype and the shapes stay
+  the same; the unit-norm, scaled slot parameters are computed on the first call, kept in
+  it, and reused by the later ones."""
   G, S, D = x.shape
   N = mu.shape[1]
   x = x.contiguous()
@@ -312,9 +317,17 @@ def soft_route(x: torch.Tensor, mu: torch.Tensor, scale: float, return_logits: b
   cw = torch.empty_like(dw)
   logits = torch.empty_like(dw) if return_logits else None
   p = H.SoftRouteParams(H.ptr(x), H.ptr(mu), float(scale), H.ptr(dw), H.ptr(cw), H.ptr(logits),
-                        None, 0, G, S, D, N, H.dtype_code(x.dtype))
-  need = H.lib().vmoe_soft_route_workspace_bytes(H.ctypes.byref(p))
-  ws = torch.empty(max(need, 16), dtype=torch.uint8, device=x.device)
+                        None, 0, G, S, D, N, H.dtype_code(x.dtype), 0)
+  key = (G, S, D, N, x.dtype, float(scale), str(x.device))
+  ws = prepared.get(key) if prepared is not None else None
+  if ws is None:
+    need = H.lib().vmoe_soft_route_workspace_bytes(H.ctypes.byref(p))
+    ws = torch.empty(max(need, 16), dtype=torch.uint8, device=x.device)
+    if prepared is not None:
+      prepared.clear()
+      prepared[key] = ws
+  else:
+    p.workspace_prepared = 1
   p.workspace = H.ptr(ws)
   p.workspace_bytes = ws.numel()
   H.call("vmoe_soft_route", p)

@@ -62,7 +62,8 @@ class SoftRouter(module.Module):
       raise ValueError(f"mu has shape {tuple(mu.shape)}, expected {(dim, self.num_experts, num_slots)}")
     n, s = self.num_experts, num_slots
     mu_c = self._cast_mu(mu, dtype)
-    dw, cw = K.soft_route(x, mu_c.reshape(dim, n * s), self._scale_value(p["scale"]))
+    dw, cw = K.soft_route(x, mu_c.reshape(dim, n * s), self._scale_value(p["scale"]),
+                          prepared=self._prepared_mu(mu_c, p["scale"]))
     dispatch_weights = dw.view(G, m, n, s)
     combine_weights = cw.view(G, m, n, s)
     dispatcher = EinsumDispatcher(combine_weights, dispatch_weights,
@@ -78,6 +79,13 @@ class SoftRouter(module.Module):
       return mu
     cache = self.__dict__.setdefault("_mu_cache", module.ParamCache())
     return cache.get((mu,), dtype, lambda: K.cast(mu, dtype))
+
+  def _prepared_mu(self, mu_c: Array, scale) -> dict:
+    """Holder of the normalised, scaled slot parameters of this (mu, scale) pair: they are
+    computed by the first call and reused until either tensor changes."""
+    cache = self.__dict__.setdefault("_prepared_cache", module.ParamCache())
+    tensors = (mu_c, scale) if isinstance(scale, torch.Tensor) else (mu_c,)
+    return cache.get(tensors, "prepared", dict)
 
   def _scale_value(self, scale) -> float:
     """The scalar parameter as a host float.  Reading a device scalar waits for the
