@@ -67,6 +67,18 @@ def device_weights(cfg, torch, dev, seed):
   return w0, w1, torch.zeros((E, M), dtype=tdt, device=dev), torch.zeros((E, D), dtype=tdt, device=dev)
 
 
+def host_cpu_model():
+  """Model name of the host CPU the baseline ran on (first entry of /proc/cpuinfo)."""
+  try:
+    with open("/proc/cpuinfo") as f:
+      for line in f:
+        if line.lower().startswith("model name"):
+          return line.split(":", 1)[1].strip()
+  except OSError:
+    pass
+  return "unknown"
+
+
 def cpu_baseline(cfg, x_np, params_np, bias_np, groups):
   """Times the CPU oracle (NumPy/torch-CPU restatement of the reference path) on
   the first `groups` groups of the same workload."""
@@ -102,7 +114,7 @@ def cpu_baseline(cfg, x_np, params_np, bias_np, groups):
       "sample": (f"oracle/moe_oracle.py mlp_moe_block (indices dispatcher) on {groups} of "
                  f"{cfg.num_groups} groups ({groups * S} tokens, all {cfg.num_experts} experts), "
                  f"median of 3 runs of {t:.2f} s; NumPy BLAS + torch CPU threads"),
-      "host_cpus": os.cpu_count(),
+      "host_cpus": os.cpu_count(), "cpu_model": host_cpu_model(),
       "einsum_dispatcher_formulation": {
           "value": eg * S / te, "unit": "tokens/s",
           "sample": f"same oracle with the einsum dispatcher on {eg} groups ({eg * S} tokens), one run of {te:.2f} s"},
@@ -208,7 +220,7 @@ def soft_main(args):
         "sample": (f"oracle/moe_oracle.py soft_router + sparse_moe(mlp_block) on {groups} of {G} "
                    f"groups ({groups * m} tokens, all {n} experts), median of 3 runs of {t:.2f} s; "
                    "NumPy BLAS + torch CPU threads"),
-        "host_cpus": os.cpu_count()}
+        "host_cpus": os.cpu_count(), "cpu_model": host_cpu_model()}
   print(json.dumps(result))
 
 
@@ -362,7 +374,7 @@ def vit_main(args):
         "sample": (f"oracle/vit_oracle.py vision_transformer_moe (bfloat16 rounding modelled) on "
                    f"{n_img} of {B} images (one routing group), one run of {t:.2f} s; NumPy BLAS + "
                    "torch CPU threads"),
-        "host_cpus": os.cpu_count()}
+        "host_cpus": os.cpu_count(), "cpu_model": host_cpu_model()}
   else:
     result["cpu_baseline"] = None
   print(json.dumps(result))
