@@ -127,6 +127,9 @@ int transpose(const void* in, void* out, int batch, int rows, int cols, int dtyp
 // one 256x256 workgroup per CU for the highest arithmetic intensity.
 using CfgUp = GemmCfg<128, 256, 2, 2, 32, 3, 2>;
 using CfgDown = GemmCfg<256, 256, 2, 2, 32, 4, 1>;
+// The persistent form of the second product keeps 35 KB of LDS for staging its output
+// and so has three stages; tile shape and launch plan are CfgDown's.
+using CfgDownPersistent = GemmCfg<256, 256, 2, 2, 32, 3, 1>;
 
 // Register-resident MFMA loop: the arithmetic ceiling that the expert GEMMs are
 // compared with.  Every wave keeps a 128 x 128 accumulator tile (16 MFMA tiles,
@@ -317,6 +320,10 @@ extern "C" int vmoe_expert_mlp(const VmoeExpertMlpParams* p, vmoe_stream_t strea
       return launch_gemm_bf16<CfgUp, kEpiBias>((const bf16_t*)hidden, (const bf16_t*)w1t,
                                               (const bf16_t*)p->b1, (bf16_t*)p->out, p->E, p->R,
                                               p->D, p->M, stream, nullptr, nullptr);
+    if (persistent_gemm_ok<CfgDownPersistent>(p->E, p->R, p->D, p->M, p->rows_per_expert, plan_down))
+      return launch_gemm_bf16_persistent<CfgDownPersistent, kEpiBias>(
+          (const bf16_t*)hidden, (const bf16_t*)w1t, (const bf16_t*)p->b1, (bf16_t*)p->out, p->E,
+          p->R, p->D, p->M, stream, plan_down);
     return launch_gemm_bf16<CfgDown, kEpiBias>((const bf16_t*)hidden, (const bf16_t*)w1t,
                                               (const bf16_t*)p->b1, (bf16_t*)p->out, p->E, p->R,
                                               p->D, p->M, stream, p->rows_per_expert, plan_down);

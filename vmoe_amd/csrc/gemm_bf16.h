@@ -549,6 +549,254 @@ __global__ __launch_bounds__(Cfg::kThreads, Cfg::kBlocksPerCu) void gemm_bf16_ke
 
 // Generic path (any Kd % 8 == 0): 128x128 tile, operands staged through
 // registers into padded LDS rows, out-of-range k chunks zero-filled.
+// Persistent variant for long k (the second product of an MLP): one workgroup per CU
+// walks its die's tiles.  The operand ring is never drained between tiles (the last
+// NSTAGE iterations of a tile request the first k tiles of the next one, so a tile's
+// first loads and the store traffic of the one before are off the critical path), and
+// the output leaves through a staging region of its own, 32 rows per wave at a time.
+// Operand offsets are relative to the whole arrays (the next tile may belong to another
+// batch): batch * R * Kd * 2 and batch * N * Kd * 2 must fit 32 bits.
+constexpr int kCusPerXcd = 32;
+
+template <typename Cfg>
+struct PersistentLds {
+  static constexpr int kOutLd = Cfg::TN + 8;
+  static constexpr size_t kRing = (size_t)Cfg::NSTAGE * Cfg::kStageBytes;
+  static constexpr size_t kStaging = (size_t)Cfg::kWaves * 32 * kOutLd * sizeof(bf16_t);
+  static constexpr size_t kBytes = kRing + kStaging;
+  static_assert(kBytes <= 160 * 1024, "LDS budget");
+};
+
+// HAS_BIAS is a template parameter: a run-time choice between two epilogues keeps the
+// accumulators alive across a branch and costs 556 bytes of scratch per lane.
+template <typename Cfg, int EPI, bool HAS_BIAS>
+__global__ __launch_bounds__(Cfg::kThreads, 1) void gemm_bf16_persistent_kernel(
+    const bf16_t* __restrict__ A, const bf16_t* __restrict__ Bt, const bf16_t* __restrict__ bias,
+    bf16_t* __restrict__ C, int R, int N, int Kd, int tiles_m, int tiles_n, int num_tiles,
+    int tiles_per_xcd, int panel_rows, const int4* __restrict__ plan, int plan_blocks) {
+#if defined(__HIP_DEVICE_COMPILE__)   // buffer-resource builtins exist in the device pass only
+  extern __shared__ __align__(1024) unsigned char smem[];
+  constexpr int BM = Cfg::BM, BN = Cfg::BN, BK = Cfg::BK;
+  constexpr int FM = Cfg::FM, FN = Cfg::FN;
+  constexpr int RB = Cfg::kRowBytes;
+  constexpr int NS = Cfg::NSTAGE, PD = NS - 1, L = Cfg::kLoads;
+  static_assert(BK == 32, "two k slices per tile");
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave / Cfg::WN, wn = wave % Cfg::WN;
+  const int m = lane & 31, h = lane >> 5;
+  const int xcd = blockIdx.x % kNumXcd, slot = blockIdx.x / kNumXcd;
+  constexpr int CPR = Cfg::kChunksPerRow;
+  constexpr int RPL = Cfg::kRowsPerLoad;
+  const int lrow = lane / CPR;
+  const int chunk = (lane % CPR) ^ (((wave * RPL + lrow) >> Cfg::kSwzShift) & (CPR - 1));
+
+  // Tile i of this workgroup: every kCusPerXcd-th entry of its die's run (the plan of a
+  // ragged launch, else the static order of map_tile), so that the tiles in flight on a
+  // die at any time are neighbours in that order.
+  struct TileCtx {
+    int b, row0, col0, live;
+    uint32_t a[Cfg::kAIssues], bo[Cfg::kBIssues];
+  };
+  auto setup_tile = [&](int i, TileCtx& t) -> bool {
+    const int s_ = slot + i * kCusPerXcd;
+    int tile_m, tile_n;
+    if (plan != nullptr) {
+      const int vblock = s_ * kNumXcd + xcd;
+      if (vblock >= plan_blocks) return false;
+      const int4 mine = plan[vblock];
+      if (mine.x < 0) return false;      // a die's run is dense from slot 0: nothing follows
+      t.b = mine.x;
+      tile_m = mine.y;
+      tile_n = mine.z;
+      t.live = mine.w;
+    } else {
+      const int logical = xcd * tiles_per_xcd + s_;
+      if (s_ >= tiles_per_xcd || logical >= num_tiles) return false;
+      const int per_batch = tiles_m * tiles_n;
+      t.b = logical / per_batch;
+      const int rem = logical - t.b * per_batch;
+      const int panel = rem / (panel_rows * tiles_n);
+      const int in_panel = rem - panel * panel_rows * tiles_n;
+      const int rows_here = min(panel_rows, tiles_m - panel * panel_rows);
+      tile_n = in_panel / rows_here;
+      tile_m = panel * panel_rows + in_panel - tile_n * rows_here;
+      t.live = R;
+    }
+    t.row0 = tile_m * BM;
+    t.col0 = tile_n * BN;
+#pragma unroll
+    for (int u = 0; u < Cfg::kAIssues; ++u) {
+      const int r = (u * Cfg::kWaves + wave) * RPL + lrow;
+      t.a[u] = (uint32_t)(t.b * R + min(t.row0 + r, R - 1)) * (uint32_t)Kd * 2u + chunk * 16;
+    }
+#pragma unroll
+    for (int u = 0; u < Cfg::kBIssues; ++u) {
+      const int r = (u * Cfg::kWaves + wave) * RPL + lrow;
+      t.bo[u] = (uint32_t)(t.b * N + min(t.col0 + r, N - 1)) * (uint32_t)Kd * 2u + chunk * 16;
+    }
+    return true;
+  };
+  const __amdgpu_buffer_rsrc_t a_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<bf16_t*>(A), 0, -1, 0x00020000);
+  const __amdgpu_buffer_rsrc_t b_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<bf16_t*>(Bt), 0, -1, 0x00020000);
+  auto load_ktile = [&](const TileCtx& t, int stage, int k0) {
+    unsigned char* s = smem + stage * Cfg::kStageBytes;
+#pragma unroll
+    for (int u = 0; u < Cfg::kAIssues; ++u)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(a_rsrc, (lds_ptr_t)(s + (u * Cfg::kWaves + wave) * RPL * RB),
+                                               16, t.a[u], k0 * 2, 0, 0);
+#pragma unroll
+    for (int u = 0; u < Cfg::kBIssues; ++u)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(
+          b_rsrc, (lds_ptr_t)(s + BM * RB + (u * Cfg::kWaves + wave) * RPL * RB), 16, t.bo[u], k0 * 2,
+          0, 0);
+  };
+
+  floatx16 acc[FM][FN];
+#pragma unroll
+  for (int i = 0; i < FM; ++i)
+#pragma unroll
+    for (int j = 0; j < FN; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+  bf16x8 fa[2][FM], fb[2][FN];
+  const int a_row_off = (wm * Cfg::TM + m) * RB;
+  const int b_row_off = BM * RB + (wn * Cfg::TN + m) * RB;
+  const int swz = (m >> Cfg::kSwzShift) & (CPR - 1);
+  auto load_frags = [&](int buf, int stage, int ks) {
+    const unsigned char* s = smem + stage * Cfg::kStageBytes + (((2 * ks + h) ^ swz) * 16);
+#pragma unroll
+    for (int i = 0; i < FM; ++i)
+      fa[buf][i] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(s + a_row_off + i * 32 * RB));
+#pragma unroll
+    for (int j = 0; j < FN; ++j)
+      fb[buf][j] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(s + b_row_off + j * 32 * RB));
+  };
+  auto mfma_slice = [&](int buf) {
+#pragma unroll
+    for (int i = 0; i < FM; ++i)
+#pragma unroll
+      for (int j = 0; j < FN; ++j)
+        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[buf][j], fa[buf][i], acc[i][j], 0, 0, 0);
+  };
+  // Same issue order inside a k slice as gemm_bf16_kernel: fragment reads behind the first
+  // MFMAs, the DMA loads (second slice only) spread over the rest.
+  constexpr int kReads = FM + FN, kMfmas = FM * FN;
+  auto slice_schedule = [&](auto vmem_c) {
+    constexpr int vmem = decltype(vmem_c)::value;
+    constexpr int kLead = kReads < kMfmas ? kReads : kMfmas;
+    constexpr int kReadsPer = (kReads + kLead - 1) / kLead;
+    constexpr int kRest = kMfmas - kLead;
+#pragma unroll
+    for (int g = 0; g < kLead; ++g) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, kReadsPer, 0);
+    }
+    if constexpr (vmem > 0 && kRest > 0) {
+#pragma unroll
+      for (int g = 0; g < kRest; ++g) {
+        if (g * vmem / kRest != (g + 1) * vmem / kRest)
+          __builtin_amdgcn_sched_group_barrier(0x020, (vmem + kRest - 1) / kRest, 0);
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  // One k tile.  WAITED = the k tile needed next is known to be complete (every wave
+  // drained its loads before the last output was staged, or in the prologue).  A macro:
+  // as a lambda taking the tile by reference the offsets end up in scratch memory.
+#define VMOE_PERSISTENT_K_ITERATION(SRC, K0, WAITED) do { \
+    const int next_stage = stage + 1 == NS ? 0 : stage + 1; \
+    load_frags(1, stage, 1); \
+    mfma_slice(0); \
+    slice_schedule(std::integral_constant<int, 0>{}); \
+    if constexpr (!(WAITED)) wait_vmcnt<(PD - 1) * L>(); \
+    wait_lgkmcnt0(); \
+    raw_barrier(); \
+    load_frags(0, next_stage, 0); \
+    load_ktile(SRC, stage, (K0)); \
+    mfma_slice(1); \
+    slice_schedule(std::integral_constant<int, L>{}); \
+    stage = next_stage; \
+  } while (0)
+
+  const int nk = Kd / BK;      // at least 2 * NS
+  TileCtx cur, nxt;
+  if (!setup_tile(0, cur)) return;
+#pragma unroll
+  for (int t = 0; t < NS; ++t) load_ktile(cur, t, t * BK);
+  wait_vmcnt<0>();
+  raw_barrier();
+  load_frags(0, 0, 0);
+  int stage = 0;
+  constexpr int OLD = PersistentLds<Cfg>::kOutLd;
+  bf16_t* so = reinterpret_cast<bf16_t*>(smem + PersistentLds<Cfg>::kRing) + (size_t)wave * 32 * OLD;
+  for (int ti = 0;; ++ti) {
+    const bool has_next = setup_tile(ti + 1, nxt);
+    if (!has_next) nxt = cur;   // the last tile requests its own first k tiles again: in bounds, never read
+    uint2 bias_pk[Cfg::TN / 8];
+    load_bias<Cfg::TN>(bias_pk, bias, cur.b, N, cur.col0 + wn * Cfg::TN, lane);
+#pragma unroll
+    for (int kt = 0; kt < NS - 1; ++kt) VMOE_PERSISTENT_K_ITERATION(cur, (kt + NS) * BK, true);
+    for (int kt = NS - 1; kt < nk - NS; ++kt) VMOE_PERSISTENT_K_ITERATION(cur, (kt + NS) * BK, false);
+    for (int kt = nk - NS; kt < nk; ++kt) VMOE_PERSISTENT_K_ITERATION(nxt, (kt + NS - nk) * BK, false);
+    // The first NS k tiles of the next tile are complete before the staging region is
+    // touched (no load that writes LDS is pending while the output is staged), and the
+    // first NS - 1 iterations of the next tile need no wait of their own.
+    wait_vmcnt<0>();
+    mfma_result_fence();
+    bf16_t* Cb = C + (size_t)cur.b * R * N;
+    const int wrow0 = cur.row0 + wm * Cfg::TM, wcol0 = cur.col0 + wn * Cfg::TN;
+    constexpr int kChunksOut = Cfg::TN / 8;
+    constexpr int kRowsPerPass = 64 / kChunksOut;
+    static_assert(64 % kChunksOut == 0 && 32 % kRowsPerPass == 0, "wave tile width must divide a wave");
+    const int oc = (lane % kChunksOut) * 8;
+    const int orow = lane / kChunksOut;
+#pragma unroll
+    for (int i = 0; i < FM; ++i) {
+#pragma unroll
+      for (int j = 0; j < FN; ++j) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const int cl = j * 32 + q * 8 + h * 4;
+          const uint2 bp = bias_pk[j * 4 + q];
+          const float bv[4] = {bf_lo(bp.x), bf_hi(bp.x), bf_lo(bp.y), bf_hi(bp.y)};
+          const uint32_t p0 = epilogue_pair<EPI, HAS_BIAS>(acc[i][j][q * 4], acc[i][j][q * 4 + 1], bv[0], bv[1]);
+          const uint32_t p1 = epilogue_pair<EPI, HAS_BIAS>(acc[i][j][q * 4 + 2], acc[i][j][q * 4 + 3], bv[2], bv[3]);
+          *reinterpret_cast<uint2*>(so + m * OLD + cl) = make_uint2(p0, p1);
+#pragma unroll
+          for (int v = 0; v < 4; ++v) acc[i][j][q * 4 + v] = 0.f;
+        }
+      }
+      // A wave reads back only what it wrote (its LDS operations complete in order).
+#pragma unroll
+      for (int r0 = 0; r0 < 32; r0 += kRowsPerPass) {
+        const int rl = r0 + orow;
+        const int row = wrow0 + i * 32 + rl;
+        const int col = wcol0 + oc;
+        const uint4 v = *reinterpret_cast<const uint4*>(so + rl * OLD + oc);
+        if (row < cur.live && col + 8 <= N) {
+          if constexpr (EPI != kEpiBias) {   // hidden layer: streaming store, as in store_tile
+            typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+            __builtin_nontemporal_store(__builtin_bit_cast(u32x4_t, v),
+                                        reinterpret_cast<u32x4_t*>(Cb + (size_t)row * N + col));
+          } else {
+            *reinterpret_cast<uint4*>(Cb + (size_t)row * N + col) = v;
+          }
+        }
+      }
+    }
+    if (!has_next) break;
+    cur = nxt;
+  }
+  wait_vmcnt<0>();
+#undef VMOE_PERSISTENT_K_ITERATION
+#endif
+}
+
 template <int EPI>
 __global__ __launch_bounds__(256) void gemm_bf16_generic_kernel(
     const bf16_t* __restrict__ A, const bf16_t* __restrict__ Bt, const bf16_t* __restrict__ bias,
@@ -694,6 +942,39 @@ int launch_gemm_bf16(const bf16_t* A, const bf16_t* Bt, const bf16_t* bias, bf16
   hipLaunchKernelGGL(kern, dim3(blocks), dim3(Cfg::kThreads), Cfg::kLdsBytes, stream, A, Bt, bias,
                      C, R, N, Kd, g.tiles_m, g.tiles_n, (int)g.tiles, g.tiles_per_xcd, g.panel_rows,
                      rows, plan, a_rows);
+  return launch_status();
+}
+
+// Whether gemm_bf16_persistent_kernel covers the product: fast geometry, at least
+// 2 * NSTAGE k tiles, operands addressable with 32-bit byte offsets from their start,
+// and a ragged launch only with its plan.
+template <typename Cfg>
+bool persistent_gemm_ok(int batch, int R, int N, int Kd, const int32_t* rows, const int4* plan) {
+  const GemmGeom g = gemm_geometry<Cfg>(batch, R, N, Kd);
+  const uint64_t lim = 1ull << 32;
+  return g.fast && Kd / Cfg::BK >= 2 * Cfg::NSTAGE && (N & 7) == 0 &&
+         (uint64_t)batch * R * Kd * 2 < lim && (uint64_t)batch * N * Kd * 2 < lim &&
+         g.tiles <= 0x7ffffff0LL && (rows == nullptr || plan != nullptr);
+}
+
+// Launches the persistent kernel; the caller checked persistent_gemm_ok.  `plan`, if
+// given, was filled by plan_ragged_tiles_kernel for gemm_geometry<Cfg> (BM, BN and
+// workgroups per CU decide it, not the number of stages).
+template <typename Cfg, int EPI>
+int launch_gemm_bf16_persistent(const bf16_t* A, const bf16_t* Bt, const bf16_t* bias, bf16_t* C,
+                                int batch, int R, int N, int Kd, hipStream_t stream,
+                                const int4* plan = nullptr) {
+  const GemmGeom g = gemm_geometry<Cfg>(batch, R, N, Kd);
+  auto kern = bias != nullptr ? gemm_bf16_persistent_kernel<Cfg, EPI, true>
+                              : gemm_bf16_persistent_kernel<Cfg, EPI, false>;
+  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                     hipFuncAttributeMaxDynamicSharedMemorySize,
+                                     (int)PersistentLds<Cfg>::kBytes);
+  if (e != hipSuccess) return (int)e;
+  const int plan_blocks = plan != nullptr ? (int)(g.ragged_slots * kNumXcd) : 0;
+  hipLaunchKernelGGL(kern, dim3(kCusPerXcd * kNumXcd), dim3(Cfg::kThreads),
+                     PersistentLds<Cfg>::kBytes, stream, A, Bt, bias, C, R, N, Kd, g.tiles_m,
+                     g.tiles_n, (int)g.tiles, g.tiles_per_xcd, g.panel_rows, plan, plan_blocks);
   return launch_status();
 }
 
