@@ -190,7 +190,7 @@ def soft_main(args):
       "vs_baseline": None, "dtype": "bf16", "data": "synthetic (seeded N(0,1) tokens and parameters)",
       "config": {"workload": cfg.name, "tokens": T, "d_model": D, "mlp_dim": M, "experts": n,
                  "slots_per_expert": p, "groups": G, "group_size": m},
-      "roofline": {"bound": "hbm", "kernel": "gemm_bf16_kernel", "achieved": achieved,
+      "roofline": {"bound": "hbm", "kernel": "gemm_bf16_kernel (first product) / gemm_bf16_persistent_kernel (second product)", "achieved": achieved,
                    "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": achieved / PEAK_HBM_GBS,
                    "traffic": None, "launch_ms": mlp_ms / 2, "bytes_per_layer": bytes_mlp},
       "stage_ms": stage_ms, "cpu_baseline": None,
@@ -345,7 +345,7 @@ def vit_main(args):
                  "tokens": T, "blocks": enc["num_layers"], "moe_blocks": list(moe_cfg["layers"]),
                  "experts": moe_cfg["num_experts"], "selected": 2, "group_size": moe_cfg["group_size"],
                  "capacity_factor": 1.05},
-      "roofline": {"bound": "mfma", "kernel": "gemm_bf16_kernel", "achieved": achieved,
+      "roofline": {"bound": "mfma", "kernel": "gemm_bf16_kernel (first product) / gemm_bf16_persistent_kernel (second product)", "achieved": achieved,
                    "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": achieved / PEAK_BF16_TFLOPS,
                    "traffic": None, "launch_ms": mlp_ms / (2 * enc["num_layers"]),
                    "flops_all_mlps": flops_mlp, "kept_rows_per_moe_block": kept_per_block,
@@ -480,7 +480,8 @@ def main():
   flops_per_launch = 2.0 * kept * D * M
   achieved_tflops = flops_per_launch / (gemm_ms * 1e-3) / 1e12
   peak = PEAK_BF16_TFLOPS if tdt == torch.bfloat16 else PEAK_FP32_MATRIX_TFLOPS
-  roofline = {"bound": "mfma", "kernel": "gemm_bf16_kernel" if b == 2 else "gemm_f32_kernel",
+  roofline = {"bound": "mfma",
+              "kernel": "gemm_bf16_kernel (first product) / gemm_bf16_persistent_kernel (second product)" if b == 2 else "gemm_f32_kernel",
               "achieved": achieved_tflops, "peak": peak, "unit": "TFLOP/s",
               "frac": achieved_tflops / peak, "traffic": MEASURED_TRAFFIC_BYTES.get(cfg.name),
               "launch_ms": gemm_ms, "flops_per_launch": flops_per_launch, "kept_rows": kept,
