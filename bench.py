@@ -35,9 +35,9 @@ PEAK_HBM_GBS = 8000.0
 # HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc runs
 # (FETCH_SIZE + WRITE_SIZE, scaled by a copy kernel of known size); None until measured.
 MEASURED_TRAFFIC_BYTES = {
-    # mean of the two GEMM launches of a layer: (639 + 565 + 1103 + 169) / 2 MiB;
+    # mean of the two GEMM launches of a layer: (638 + 565 + 1098 + 141) / 2 MiB;
     # FETCH_SIZE x 2.0, WRITE_SIZE x 1.0 (copy-kernel calibration).
-    "vmoe_b16_layer_E32_k2_bpr": 1.298e9,
+    "vmoe_b16_layer_E32_k2_bpr": 1.280e9,
 }
 
 
