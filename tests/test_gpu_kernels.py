@@ -545,6 +545,41 @@ def test_expert_mlp_planned_launch_random_fill(K):
         assert (to_np(out[e, n:]) == 7.0).all(), f"E={E} R={R} rows={rows.tolist()} expert {e}"
 
 
+@pytest.mark.parametrize("with_bias", [True, False])
+def test_expert_mlp_second_product_walks_several_tiles(K, with_bias):
+  """The second product's workgroups walk a list of tiles and fetch a tile's first
+  operands while they finish the tile before: enough tiles (480 of 256 x 256, 60 per die)
+  that most workgroups compute two, dense and over packed rows with a launch plan, the
+  last column tile 8 wide.  Checked against a float32 restatement with the bfloat16
+  rounding points of flax's Dense (accumulator, + bias) on the device, tolerance one
+  bfloat16 step; packed rows against the dense result bit for bit."""
+  rng = np.random.default_rng(23)
+  E, R, D, M = 16, 2321, 520, 256
+  bf = torch.bfloat16
+  x = to_dev(O.cast(rng.standard_normal((E, R, D)).astype(np.float32), O.BF16), O.BF16)
+  w0 = to_dev(O.cast(rng.standard_normal((E, D, M)).astype(np.float32) / np.sqrt(D), O.BF16), O.BF16)
+  w1 = to_dev(O.cast(rng.standard_normal((E, M, D)).astype(np.float32) / np.sqrt(M), O.BF16), O.BF16)
+  b0 = to_dev(O.cast(rng.standard_normal((E, M)).astype(np.float32) * 0.1, O.BF16), O.BF16) if with_bias else None
+  b1 = to_dev(O.cast(rng.standard_normal((E, D)).astype(np.float32) * 0.1, O.BF16), O.BF16) if with_bias else None
+  full = K.expert_mlp(x, w0, b0, w1, b1)
+  for e in range(E):                       # one expert at a time: plain 2-D products
+    h = (x[e].float() @ w0[e].float()).to(bf)
+    if with_bias:
+      h = (h.float() + b0[e].float()).to(bf)
+    h = torch.nn.functional.gelu(h.float(), approximate="tanh").to(bf)
+    y = (h.float() @ w1[e].float()).to(bf)
+    if with_bias:
+      y = (y.float() + b1[e].float()).to(bf)
+    np.testing.assert_allclose(to_np(full[e]), to_np(y), rtol=2e-2, atol=2e-2, err_msg=f"expert {e}")
+  rows = rng.integers(0, R + 1, E).astype(np.int32)
+  rows[:4] = [R, 0, 257, 1]
+  out = torch.full_like(full, 7.0)
+  K.expert_mlp(x, w0, b0, w1, b1, out=out, rows_per_expert=to_dev(rows))
+  for e, n in enumerate(rows):
+    np.testing.assert_array_equal(to_np(out[e, :n]), to_np(full[e, :n]), err_msg=f"expert {e}")
+    assert (to_np(out[e, n:]) == 7.0).all(), f"expert {e}"
+
+
 @pytest.mark.parametrize("G,S,N,dtype", [(3, 50, 16, O.F32), (4, 196, 128, O.BF16), (2, 7, 300, O.BF16), (3, 196, 128, O.F32),
                           (2, 9, 96, O.BF16), (5, 33, 8, O.BF16), (2, 300, 512, O.BF16)])
 def test_soft_router_stats(K, G, S, N, dtype):
