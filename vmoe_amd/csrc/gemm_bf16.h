@@ -30,6 +30,10 @@
 // logical tile (w % 8) * ceil(tiles/8) + w / 8, so that an XCD walks a contiguous
 // run of tiles (whole experts), and within an expert tiles are ordered in panels
 // of 8 row tiles so that the tiles in flight on an XCD share A and B panels.
+//
+// Two kernels share this scheme: gemm_bf16_kernel computes one tile per workgroup;
+// gemm_bf16_persistent_kernel (long k, one workgroup per CU) walks a list of tiles
+// and keeps the operand ring full across tile boundaries.
 #ifndef VMOE_GEMM_BF16_H_
 #define VMOE_GEMM_BF16_H_
 
