@@ -545,6 +545,34 @@ def test_expert_mlp_planned_launch_random_fill(K):
         assert (to_np(out[e, n:]) == 7.0).all(), f"E={E} R={R} rows={rows.tolist()} expert {e}"
 
 
+def test_expert_mlp_hidden_layer_beyond_4_gib(K):
+  """A hidden layer of 4.3 GiB: the second product cannot address it with 32-bit byte
+  offsets from its start, which the tile-walking kernel needs, so the one-tile-per-
+  workgroup kernel (offsets per expert) must take over.  Sampled rows of every expert
+  against a float32 restatement on the device."""
+  rng = np.random.default_rng(31)
+  E, R, D, M = 8, 70000, 64, 4096
+  assert E * R * M * 2 >= 1 << 32
+  bf = torch.bfloat16
+  gen = torch.Generator(device=dev())
+  gen.manual_seed(5)
+  x = torch.randn((E, R, D), generator=gen, device=dev()).to(bf)
+  w0 = (torch.randn((E, D, M), generator=gen, device=dev()) / D ** 0.5).to(bf)
+  w1 = (torch.randn((E, M, D), generator=gen, device=dev()) / M ** 0.5).to(bf)
+  b0 = (torch.randn((E, M), generator=gen, device=dev()) * 0.1).to(bf)
+  b1 = (torch.randn((E, D), generator=gen, device=dev()) * 0.1).to(bf)
+  out = K.expert_mlp(x, w0, b0, w1, b1)
+  pick = torch.from_numpy(np.unique(np.concatenate(
+      [[0, 1, 255, 256, R - 257, R - 2, R - 1], rng.integers(0, R, 50)]))).to(dev())
+  for e in range(E):
+    h = ((x[e, pick].float() @ w0[e].float()).to(bf).float() + b0[e].float()).to(bf)
+    h = torch.nn.functional.gelu(h.float(), approximate="tanh").to(bf)
+    y = ((h.float() @ w1[e].float()).to(bf).float() + b1[e].float()).to(bf)
+    np.testing.assert_allclose(to_np(out[e, pick]), to_np(y), rtol=2e-2, atol=2e-2, err_msg=f"expert {e}")
+  del out, x
+  torch.cuda.empty_cache()
+
+
 @pytest.mark.parametrize("with_bias", [True, False])
 def test_expert_mlp_second_product_walks_several_tiles(K, with_bias):
   """The second product's workgroups walk a list of tiles and fetch a tile's first
