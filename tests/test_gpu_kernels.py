@@ -318,6 +318,7 @@ MLP_CASES = [
     (8, 512, 512, 2048, O.F32),       # S/32-style layer, full size
     (3, 100, 72, 136, O.BF16),        # ragged everything
     (2, 300, 256, 512, O.BF16),
+    (3, 300, 64, 192, O.BF16),        # shortest second product the tile-walking kernel takes (6 k tiles)
     (4, 3200, 768, 3072, O.BF16),     # B/16 experts (4 of 32)
 ]
 
@@ -526,7 +527,8 @@ def test_expert_mlp_planned_launch_random_fill(K):
   rng = np.random.default_rng(11)
   dtype = O.BF16
   for E, R, D, M in [(1, 700, 64, 96), (3, 130, 96, 64), (8, 520, 64, 128), (9, 257, 128, 64),
-                     (17, 300, 64, 64), (40, 100, 64, 96), (64, 33, 96, 64)]:
+                     (17, 300, 64, 64), (40, 100, 64, 96), (64, 33, 96, 64),
+                     (5, 520, 64, 224), (12, 700, 520, 192)]:   # tile-walking second product
     x = to_dev(O.cast(rng.standard_normal((E, R, D)).astype(np.float32), dtype), dtype)
     w0 = to_dev(O.cast(rng.standard_normal((E, D, M)).astype(np.float32) / 8, dtype), dtype)
     w1 = to_dev(O.cast(rng.standard_normal((E, M, D)).astype(np.float32) / 11, dtype), dtype)
