@@ -570,7 +570,26 @@ def main():
       torch.cuda.synchronize()
       lib[name] = 2.0 * kept * D * M * 10 / (e0.elapsed_time(e1) * 1e-3) / 1e12
     roofline["library_gemm_same_shapes_TFLOPs"] = lib
-    del a_up, a_dn, w_up, w_dn
+    # What bounds a GEMM of this tiling on this part: the rate at which the second
+    # product's operand tiles (256 x 256 x 32, 128 flop per operand byte) can be moved
+    # from global memory into LDS at all, measured by a kernel that issues exactly those
+    # loads and nothing else, on operands of the layer's shape (E experts with their own
+    # weights, the kept rows spread evenly over them).
+    a_e = a_dn[: E * (kept // E)].view(E, kept // E, M)
+    w_e = (torch.randn((E, D, M), device=dev) * M ** -0.5).to(tdt)
+    for _ in range(3):
+      kernels.operand_delivery_probe(a_e, w_e)
+    e0.record()
+    for _ in range(10):
+      moved = kernels.operand_delivery_probe(a_e, w_e)
+    e1.record()
+    torch.cuda.synchronize()
+    tbps = moved * 10 / (e0.elapsed_time(e1) * 1e-3) / 1e12
+    roofline["operand_delivery"] = {
+        "TBps": tbps, "flop_per_byte": 128.0, "ceiling_TFLOPs": tbps * 128.0,
+        "frac_of_ceiling": achieved_tflops / (tbps * 128.0),
+        "note": "load-only kernel, second product's tiles; the first product's 128 x 256 tiles have 85 flop per byte"}
+    del a_up, a_dn, w_up, w_dn, a_e, w_e
   # The same K steps replayed from HIP graphs (one per rotating input buffer), as a
   # serving loop would run the layer; reported beside the eager figure, never as `value`.
   graph_ms = None

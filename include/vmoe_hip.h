@@ -453,6 +453,15 @@ int vmoe_copy_bytes(const void* in, void* out, size_t n, vmoe_stream_t stream);
 int vmoe_mfma_probe(const void* seed, size_t seed_bytes, void* sink, int32_t blocks,
                     int32_t iters, double* flops, vmoe_stream_t stream);
 
+/* Load-only counterpart of the 256 x 256 expert product (no counterpart in the
+ * reference; measurement aid like vmoe_mfma_probe): issues exactly the operand-tile
+ * loads of C[b] = A[b] (rows x kd) . Bt[b] (n x kd)^T, bfloat16, global memory -> LDS, in
+ * the product's tile order and does nothing with them.  *bytes is set to the operand
+ * bytes moved (tiles x 512 rows x kd x 2); bytes / time is the rate that bounds any
+ * kernel of this tiling, and x 128 flop/byte its ceiling in FLOP/s.  kd % 32 == 0. */
+int vmoe_operand_delivery_probe(const void* a, const void* bt, int32_t batch, int32_t rows,
+                                int32_t n, int32_t kd, double* bytes, vmoe_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

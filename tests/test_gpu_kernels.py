@@ -547,6 +547,22 @@ def test_expert_mlp_planned_launch_random_fill(K):
         assert (to_np(out[e, n:]) == 7.0).all(), f"E={E} R={R} rows={rows.tolist()} expert {e}"
 
 
+def test_operand_delivery_probe(K):
+  """The load-only measurement kernel reports the operand bytes of the 256 x 256 tiling
+  and refuses what the tiling refuses."""
+  from vmoe_amd import _hip as H
+  a = torch.randn((3, 700, 256), device=dev()).to(torch.bfloat16)
+  bt = torch.randn((3, 520, 256), device=dev()).to(torch.bfloat16)
+  moved = K.operand_delivery_probe(a, bt)
+  torch.cuda.synchronize()
+  assert moved == 3 * 3 * 3 * 512 * 256 * 2          # 3 batches x (3 x 3) tiles x 512 rows x K x 2 bytes
+  assert K.operand_delivery_probe(a[0], bt[0]) == 3 * 3 * 512 * 256 * 2
+  with pytest.raises(H.VmoeError):                     # K not a multiple of 32
+    K.operand_delivery_probe(a[:, :, :40].contiguous(), bt[:, :, :40].contiguous())
+  with pytest.raises(ValueError):
+    K.operand_delivery_probe(a.float(), bt.float())
+
+
 def test_expert_mlp_hidden_layer_beyond_4_gib(K):
   """A hidden layer of 4.3 GiB: the second product cannot address it with 32-bit byte
   offsets from its start, which the tile-walking kernel needs, so the one-tile-per-

@@ -176,6 +176,53 @@ __global__ __launch_bounds__(256) void mfma_probe_kernel(const uint4* __restrict
   sink[(size_t)blockIdx.x * 256 + threadIdx.x] = t;
 }
 
+// Load-only counterpart of the 256x256 product: every workgroup issues the LDS-DMA
+// loads of its tile's k tiles (same addresses, request shapes, tile order and ring of
+// four stages as gemm_bf16_kernel with CfgDown) and nothing else, two k tiles in flight.
+// The rate at which it moves operand tiles is the ceiling of any kernel of this tiling.
+__global__ __launch_bounds__(256, 1) void operand_delivery_probe_kernel(
+    const bf16_t* __restrict__ A, const bf16_t* __restrict__ Bt, int R, int N, int Kd,
+    int tiles_m, int tiles_n, int num_tiles, int tiles_per_xcd, int panel_rows) {
+#if defined(__HIP_DEVICE_COMPILE__)   // buffer-resource builtins exist in the device pass only
+  extern __shared__ __align__(1024) unsigned char smem[];
+  using Cfg = CfgDown;
+  int b, tile_m, tile_n;
+  if (!map_tile(tiles_m, tiles_n, num_tiles, tiles_per_xcd, panel_rows, b, tile_m, tile_n)) return;
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  constexpr int CPR = Cfg::kChunksPerRow, RPL = Cfg::kRowsPerLoad, RB = Cfg::kRowBytes;
+  const int lrow = lane / CPR, chunk = lane % CPR;
+  uint32_t a_off[Cfg::kAIssues], b_off[Cfg::kBIssues];
+#pragma unroll
+  for (int i = 0; i < Cfg::kAIssues; ++i)
+    a_off[i] = (uint32_t)min(tile_m * Cfg::BM + (i * Cfg::kWaves + wave) * RPL + lrow, R - 1) *
+                   (uint32_t)Kd * 2u + chunk * 16;
+#pragma unroll
+  for (int i = 0; i < Cfg::kBIssues; ++i)
+    b_off[i] = (uint32_t)min(tile_n * Cfg::BN + (i * Cfg::kWaves + wave) * RPL + lrow, N - 1) *
+                   (uint32_t)Kd * 2u + chunk * 16;
+  const __amdgpu_buffer_rsrc_t a_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<bf16_t*>(A + (size_t)b * R * Kd), 0, -1, 0x00020000);
+  const __amdgpu_buffer_rsrc_t b_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<bf16_t*>(Bt + (size_t)b * N * Kd), 0, -1, 0x00020000);
+  const int nk = Kd / Cfg::BK;
+  for (int kt = 0; kt < nk; ++kt) {
+    unsigned char* s = smem + (kt % Cfg::NSTAGE) * Cfg::kStageBytes;
+#pragma unroll
+    for (int i = 0; i < Cfg::kAIssues; ++i)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(a_rsrc, (lds_ptr_t)(s + (i * Cfg::kWaves + wave) * RPL * RB),
+                                               16, a_off[i], kt * Cfg::BK * 2, 0, 0);
+#pragma unroll
+    for (int i = 0; i < Cfg::kBIssues; ++i)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(
+          b_rsrc, (lds_ptr_t)(s + Cfg::BM * RB + (i * Cfg::kWaves + wave) * RPL * RB), 16, b_off[i],
+          kt * Cfg::BK * 2, 0, 0);
+    wait_vmcnt<2 * Cfg::kLoads>();   // a stage is written again four k tiles later
+  }
+  wait_vmcnt<0>();
+#endif
+}
+
 size_t align256(size_t v) { return (v + 255) / 256 * 256; }
 
 // The second product's 256x256 tiles run one per CU, in whole rounds of kNumCu tiles:
@@ -340,6 +387,27 @@ extern "C" int vmoe_expert_mlp(const VmoeExpertMlpParams* p, vmoe_stream_t strea
   return launch_gemm_f32<kEpiBias>((const float*)hidden, (const float*)p->w1, (const float*)p->b1,
                                    (float*)p->out, p->E, p->R, p->D, p->M, stream,
                                    p->rows_per_expert);
+}
+
+extern "C" int vmoe_operand_delivery_probe(const void* a, const void* bt, int32_t batch, int32_t rows,
+                                           int32_t n, int32_t kd, double* bytes,
+                                           vmoe_stream_t stream) {
+  if (a == nullptr || bt == nullptr || bytes == nullptr) return VMOE_E_NULL;
+  if (batch < 1 || rows < 1 || n < 1 || kd < 1) return VMOE_E_SHAPE;
+  if (!aligned16(a) || !aligned16(bt)) return VMOE_E_ALIGN;
+  const GemmGeom g = gemm_geometry<CfgDown>(batch, rows, n, kd);
+  if (!g.fast) return VMOE_E_UNSUPPORTED;    // kd % 32 != 0 or an operand beyond 32-bit offsets
+  if (g.tiles > 0x7ffffff0LL) return VMOE_E_OVERFLOW;
+  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(operand_delivery_probe_kernel),
+                                     hipFuncAttributeMaxDynamicSharedMemorySize,
+                                     (int)CfgDown::kLdsBytes);
+  if (e != hipSuccess) return (int)e;
+  hipLaunchKernelGGL(operand_delivery_probe_kernel, dim3((unsigned)g.tiles_per_xcd * kNumXcd),
+                     dim3(CfgDown::kThreads), CfgDown::kLdsBytes, as_stream(stream),
+                     (const bf16_t*)a, (const bf16_t*)bt, rows, n, kd, g.tiles_m, g.tiles_n,
+                     (int)g.tiles, g.tiles_per_xcd, g.panel_rows);
+  *bytes = (double)g.tiles * (CfgDown::BM + CfgDown::BN) * (double)kd * 2.0;
+  return launch_status();
 }
 
 extern "C" int vmoe_pack_expert_weights(const VmoeTransposeParams* p, vmoe_stream_t stream) {

@@ -469,6 +469,22 @@ def copy_bytes(src: torch.Tensor, dst: torch.Tensor) -> None:
           "vmoe_copy_bytes")
 
 
+def operand_delivery_probe(a: torch.Tensor, bt: torch.Tensor) -> float:
+  """Launches the load-only counterpart of the 256 x 256 product a (B, R, K) . bt (B, N, K)^T
+  (bfloat16, contiguous); returns the operand bytes it moves (time it with events)."""
+  if a.dim() == 2:
+    a, bt = a[None], bt[None]
+  if a.dtype != torch.bfloat16 or bt.dtype != torch.bfloat16 or not (a.is_contiguous() and bt.is_contiguous()):
+    raise ValueError("operand_delivery_probe: contiguous bfloat16 operands")
+  if a.shape[0] != bt.shape[0] or a.shape[2] != bt.shape[2]:
+    raise ValueError("operand_delivery_probe: a (B, R, K) and bt (B, N, K)")
+  moved = H.ctypes.c_double(0.0)
+  H.check(H.lib().vmoe_operand_delivery_probe(H.ptr(a), H.ptr(bt), a.shape[0], a.shape[1], bt.shape[1],
+                                              a.shape[2], H.ctypes.byref(moved), H.stream()),
+          "vmoe_operand_delivery_probe")
+  return float(moved.value)
+
+
 def mfma_probe(seed: torch.Tensor, blocks: int = 256, iters: int = 2000) -> float:
   """Launches the register-resident MFMA loop on operands read from `seed`;
   returns the floating-point operations it issues (time it with events)."""
