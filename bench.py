@@ -79,9 +79,12 @@ def host_cpu_model():
   return "unknown"
 
 
-def cpu_baseline(cfg, x_np, params_np, bias_np, groups):
+def cpu_baseline(cfg, x_np, params_np, bias_np, groups, gpu_out=None):
   """Times the CPU oracle (NumPy/torch-CPU restatement of the reference path) on
-  the first `groups` groups of the same workload."""
+  the first `groups` groups of the same workload.  With gpu_out (the layer's output
+  for the same items, float32 NumPy) the oracle's output is also compared with it:
+  an item is bad if any element differs by more than 2e-2 * (rms + |want|)
+  (bfloat16; 2e-5 in float32)."""
   from oracle import moe_oracle as O
   S = cfg.group_size
   imgs = groups * cfg.group_images
@@ -92,7 +95,7 @@ def cpu_baseline(cfg, x_np, params_np, bias_np, groups):
                            num_selected_experts=cfg.num_selected_experts,
                            dispatcher_kwargs=cfg.dispatcher_kwargs("indices"), dtype=dtype,
                            logit_bias=bias_np)
-  run()
+  want, _ = run()
   times = []
   for _ in range(3):
     t0 = time.perf_counter()
@@ -100,6 +103,17 @@ def cpu_baseline(cfg, x_np, params_np, bias_np, groups):
     times.append(time.perf_counter() - t0)
   t = float(np.median(times))
   import torch
+  parity = None
+  if gpu_out is not None:
+    D = want.shape[-1]
+    want = np.asarray(want, np.float32).reshape(-1, D)
+    got = np.asarray(gpu_out, np.float32).reshape(-1, D)[: want.shape[0]]
+    tol = 2e-2 if dtype == O.BF16 else 2e-5
+    rms = float(np.sqrt((want.astype(np.float64) ** 2).mean()))
+    bad = (np.abs(got - want) > tol * (rms + np.abs(want))).any(-1)
+    parity = {"items": int(bad.size), "bad": int(bad.sum()), "rtol": tol,
+              "allowed_bad_fraction": 0.01 if dtype == O.BF16 else 0.0,
+              "note": "timed path's output for input buffer 0 vs oracle/moe_oracle.py mlp_moe_block"}
   # The same layer in the formulation the reference's released configs use (the einsum
   # dispatcher with its dense (G, S, E, C) weights, vmoe/moe.py:127-161), on two groups.
   eg = min(2, groups)
@@ -108,7 +122,7 @@ def cpu_baseline(cfg, x_np, params_np, bias_np, groups):
   O.mlp_moe_block(xe, params_np, group_size=S, num_selected_experts=cfg.num_selected_experts,
                   dispatcher_kwargs=cfg.dispatcher_kwargs("einsum"), dtype=dtype, logit_bias=bias_np)
   te = time.perf_counter() - t0
-  return {
+  return parity, {
       "value": groups * S / t, "unit": "tokens/s", "cores": int(torch.get_num_threads()),
       "kind": "port",
       "sample": (f"oracle/moe_oracle.py mlp_moe_block (indices dispatcher) on {groups} of "
@@ -446,17 +460,26 @@ def main():
   # fully instrumented pass of the same K steps right after.
   sink = _hip.TimingSink(pairs=args.steps * 2, only=("vmoe_expert_mlp",))
   _hip.set_timing_sink(sink)
+  # One event per step boundary: the per-step times whose median is reported.
+  marks = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps + 1)]
+  for ev in marks:
+    ev.record()
   torch.cuda.synchronize()
   t0 = time.perf_counter()
+  marks[0].record()
   for i in range(args.steps):
     out, metrics = step(i)
+    marks[i + 1].record()
   t_enqueued = time.perf_counter()      # the host has issued everything; the GPU is still running
   torch.cuda.synchronize()
   t1 = time.perf_counter()
   _hip.set_timing_sink(None)
-  ms_per_step = (t1 - t0) * 1e3 / args.steps
+  wall_ms_per_step = (t1 - t0) * 1e3 / args.steps
+  step_ms = [marks[i].elapsed_time(marks[i + 1]) for i in range(args.steps)]
+  ms_per_step = float(np.median(step_ms))
   host_ms_per_step = (t_enqueued - t0) * 1e3 / args.steps
   tokens_per_s = T / (ms_per_step * 1e-3)
+  out0 = step(0)[0].float().cpu().numpy() if not args.no_cpu_baseline else None
 
   def per_step(pairs_by_name):
     return {name: float(np.mean([a.elapsed_time(b) for a, b in pairs])) * (len(pairs) / args.steps)
@@ -646,16 +669,29 @@ def main():
       "hbm": hbm,
       "hip_graph_ms_per_step": graph_ms,
       "host_enqueue_ms_per_step": host_ms_per_step,
+      "wall_ms_per_step": wall_ms_per_step,
+      "ms_per_step_note": ("ms_per_step and value: median of the K per-step times between events "
+                           "recorded at the step boundaries; wall_ms_per_step: host clock around "
+                           "the same K steps, synchronised on both sides, divided by K"),
+      "step_ms_min_max": [float(min(step_ms)), float(max(step_ms))],
   }
   if not args.no_cpu_baseline:
     params_np = {
         "Router": {"dense": {"kernel": router_np}},
         "Mlp": {"Dense_0": {"kernel": w0.float().cpu().numpy(), "bias": b0.float().cpu().numpy()},
                 "Dense_1": {"kernel": w1.float().cpu().numpy(), "bias": b1.float().cpu().numpy()}}}
-    result["cpu_baseline"] = cpu_baseline(cfg, xs_np[0], params_np, bias_np, min(args.cpu_groups, G))
+    parity, result["cpu_baseline"] = cpu_baseline(cfg, xs_np[0], params_np, bias_np,
+                                                  min(args.cpu_groups, G), gpu_out=out0)
+    result["parity_checked"] = parity
   else:
     result["cpu_baseline"] = None
+    result["parity_checked"] = None
   print(json.dumps(result))
+  parity = result["parity_checked"]
+  if parity and parity["bad"] > parity["allowed_bad_fraction"] * parity["items"]:
+    print(f"bench.py: the timed path's output differs from the oracle on {parity['bad']} of "
+          f"{parity['items']} items", file=sys.stderr)
+    sys.exit(1)
 
 
 def cfg_capacity(cfg):

@@ -234,7 +234,9 @@ def test_dense_einsum_dispatcher(moe, dtype):
   G, S, E, D = 2, 20, 4, 32
   cw = O.cast(O.softmax(rng.standard_normal((G, S, E)).astype(np.float32)), dtype)
   data = O.cast(rng.standard_normal((G, S, D)).astype(np.float32), dtype)
-  d = moe.DenseEinsumDispatcher(combine_weights=to_dev(cw, dtype))
+  # through the public factory (vmoe/moe.py:260-264), which passes its keyword arguments on
+  d = moe.get_dense_einsum_dispatcher(to_dev(cw, dtype), partition_spec=None)
+  assert isinstance(d, moe.DenseEinsumDispatcher)
   ref = O.DenseEinsumDispatcher(cw)
   out = d.dispatch(to_dev(data, dtype))
   want = ref.dispatch(data)
@@ -631,14 +633,29 @@ def test_soft_moe_b16_shape_vs_oracle(moe):
   assert_close(to_np(out), want, 3e-2, "soft moe b16 shape")
 
 
-@pytest.mark.parametrize("name", ["vmoe_s32_layer", "vmoe_l16_384_layer_cf0.5"])
+# groups of each benchmark configuration that the layer test runs (None = all of them)
+LAYER_CONFIG_GROUPS = {
+    "vmoe_s32_layer": None,                 # fp32, full size
+    "vmoe_b16_layer_E32_k2_bpr": None,      # the headline layer at full size: 32 groups, E = 32,
+                                            # C = 100: gathered first product, planned ragged
+                                            # launches, persistent second product
+    "vmoe_l16_384_layer_cf0.5": 2,          # 2 of 16 groups, all 32 experts
+    "vmoe_b16_model_layer_E8": 8,           # the full model's MoE layer: E = 8, C = 412, 8 of 64 groups
+}
+
+
+@pytest.mark.parametrize("name", sorted(LAYER_CONFIG_GROUPS))
 def test_layer_configs_vs_oracle(name):
-  """The fp32 S/32-style layer at full size, and the L/16@384 layer (capacity
-  factor 0.5, skewed logits) on 2 of its 16 groups with all 32 experts."""
+  """The benchmark configurations' layers through MlpMoeBlock.apply against the oracle:
+  the fp32 S/32-style layer and the headline B/16 layer (E = 32, top-2 with batch
+  priority routing, D/M = 768/3072) at full size, the L/16@384 layer (capacity factor
+  0.5, skewed logits) and the full B/16 model's layer (E = 8, C = 412) on some of
+  their groups."""
   from vmoe_amd import configs
   from vmoe_amd.nn import vit_moe
   cfg = configs.CONFIGS[name]
-  imgs = cfg.num_images if name == "vmoe_s32_layer" else 2 * cfg.group_images
+  groups = LAYER_CONFIG_GROUPS[name]
+  imgs = cfg.num_images if groups is None else groups * cfg.group_images
   x, params, bias = configs.make_layer_inputs(cfg, seed=5, num_images=imgs)
   dtype = O.BF16 if cfg.dtype == "bfloat16" else O.F32
   x = O.cast(x, dtype)
@@ -664,6 +681,85 @@ def test_layer_configs_vs_oracle(name):
   if name.startswith("vmoe_l16"):
     # capacity factor 0.5: at least half of the assignments are dropped -> many all-zero rows
     assert (np.abs(got).max(-1) == 0).mean() > 0.1
+  for key in ("auxiliary_loss", "gshard_loss", "importance_loss"):
+    np.testing.assert_allclose(to_np(metrics[key]), wmetrics[key], rtol=2e-2 if dtype == O.BF16 else 1e-4)
+
+
+# ------------------------------------------------------------------ routers chosen by name
+ROUTERS_BY_NAME = {
+    "default": {},
+    "bare_top_experts": {"name": "NoisyTopExpertsPerItemRouter"},
+    "bare_top_items": {"name": "NoisyTopItemsPerExpertRouter"},
+    "dotted_soft": {"name": "vmoe_amd.projects.soft_moe.router.SoftRouter"},
+    "call_syntax": {"name": "NoisyTopExpertsPerItemRouter(num_selected_experts=2)"},
+}
+
+
+@pytest.mark.parametrize("dtype", [O.F32, O.BF16])
+@pytest.mark.parametrize("which", sorted(ROUTERS_BY_NAME))
+def test_mlp_moe_block_router_by_name(which, dtype):
+  """MlpMoeBlock.create_router resolves `router={'name': ...}` with utils.parse_call
+  (vmoe/nn/vit_moe.py:76-88, vmoe/utils.py:59-109): no name (the default router), bare
+  names looked up in nn.routing, a dotted path (the Soft MoE router lives outside
+  nn.routing), and the call syntax.  Each block is run and compared with the oracle."""
+  from vmoe_amd.nn import routing, vit_moe
+  from vmoe_amd.projects.soft_moe import router as soft_router
+  rng = np.random.default_rng(23)
+  N, L, D, M, E, gs = 4, 48, 64, 128, 8, 96
+  tol = 2e-5 if dtype == O.F32 else 3e-2
+  x = O.cast(rng.standard_normal((N, L, D)), dtype)
+  mlp_np = _layer_params(rng, D, M, E, dtype, bias_scale=0.1)["Mlp"]
+  mlp_dev = {k: {kk: to_dev(vv, dtype) for kk, vv in v.items()} for k, v in mlp_np.items()}
+  fn = lambda b: O.mlp_block(b, mlp_np["Dense_0"]["kernel"], mlp_np["Dense_0"]["bias"],
+                             mlp_np["Dense_1"]["kernel"], mlp_np["Dense_1"]["bias"], dtype)
+  xg = x.reshape(-1, gs, D)
+  spec = dict(ROUTERS_BY_NAME[which])
+  if which == "dotted_soft":
+    spec.update(num_slots=2, compute_similarity_metrics=False)
+    mu = (rng.standard_normal((D, E, 2)) / np.sqrt(D)).astype(np.float32)
+    router_params = {"mu": to_dev(mu), "scale": torch.tensor(1.25, device=dev())}
+    odisp, _ = O.soft_router(xg, mu, 1.25, dtype, compute_similarity_metrics=False)
+    want_cls = soft_router.SoftRouter
+    tol = max(tol, 1e-4)      # data passes through bfloat16 in both einsums
+  else:
+    kernel = (rng.standard_normal((D, E)) / np.sqrt(D)).astype(np.float32)
+    router_params = {"dense": {"kernel": to_dev(kernel)}}
+    if which == "bare_top_items":
+      C = 16
+      spec.update(dispatcher=dict(name="einsum", capacity=C))
+      gates = O.router_gates(xg, kernel, dtype)
+      cws = [O.top_items_per_expert_einsum(gates[g], C) for g in range(gates.shape[0])]
+      odisp = O.EinsumDispatcher(np.stack([c[0] for c in cws]), np.stack([c[1] for c in cws]))
+      want_cls = routing.NoisyTopItemsPerExpertRouter
+    else:
+      dkw = dict(name="indices", batch_priority=True, capacity_factor=1.0)
+      spec.update(dispatcher=dkw)
+      if which != "call_syntax":
+        spec.update(num_selected_experts=2)
+      odisp, _, _ = O.noisy_top_experts_per_item_router(xg, kernel, 2, dkw, dtype)
+      want_cls = routing.NoisyTopExpertsPerItemRouter
+  layer = vit_moe.MlpMoeBlock(mlp_dim=M, num_experts=E, group_size=gs, deterministic=True,
+                              router=spec, dtype=tdtype(dtype))
+  router_module = layer.create_router()
+  assert type(router_module) is want_cls
+  assert router_module.deterministic is True and router_module.num_experts == E
+  assert router_module.dtype == tdtype(dtype)
+  out, metrics = layer.apply({"params": {"Router": router_params, "Mlp": mlp_dev}}, to_dev(x, dtype))
+  assert out.shape == (N, L, D) and out.dtype == tdtype(dtype) and "auxiliary_loss" in metrics
+  want = O.cast(O.sparse_moe(odisp, fn, xg), dtype).reshape(-1, D)
+  got = to_np(out).reshape(-1, D)
+  rms = np.sqrt((want ** 2).mean())
+  bad_items = (np.abs(got - want) > tol * (rms + np.abs(want))).any(-1)
+  # a gate that differs in its last place may change one routing decision
+  assert bad_items.mean() <= (0.0 if dtype == O.F32 or which == "dotted_soft" else 0.02), bad_items.sum()
+
+
+def test_mlp_moe_block_router_unknown_name():
+  from vmoe_amd.nn import vit_moe
+  layer = vit_moe.MlpMoeBlock(mlp_dim=8, num_experts=2, group_size=4, deterministic=True,
+                              router={"name": "NoSuchRouter"})
+  with pytest.raises(AttributeError):
+    layer.create_router()
 
 
 @pytest.mark.parametrize("dtype,bf16_dispatcher", [(O.F32, False), (O.BF16, False), (O.F32, True)])

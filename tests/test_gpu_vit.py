@@ -300,6 +300,33 @@ def test_model_bf16_vs_oracle(vit_moe):
   assert np.isfinite(to_np(metrics["auxiliary_loss"])).all()
 
 
+def test_model_b16_width_bf16_vs_oracle(vit_moe):
+  """The full model's real width (hidden 768, 12 heads of 64, mlp 3072, 224 px images in
+  16 x 16 patches, 1000 classes, global average pooling, bfloat16 encoder) on three
+  blocks, the middle one sparse as in the B/16 model (E = 8, top-2 with batch priority
+  routing, capacity factor 1.05, groups of 8 images): 16 images, two routing groups."""
+  from vmoe_amd import configs
+  cfg = configs.vit_b16_moe_model(dtype=None)
+  cfg["encoder"]["num_layers"] = 3
+  cfg["encoder"]["moe"]["layers"] = (1,)
+  cfg.pop("deterministic")
+  cfg.pop("head_kernel_zero_init")
+  rng = np.random.default_rng(21)
+  images = rng.uniform(-1, 1, (16, 224, 224, 3)).astype(np.float32)
+  params = V.init_params(rng, images.shape, **cfg)
+  want, want_metrics = V.vision_transformer_moe(images, params, **oracle_config(cfg, O.BF16))
+  model = vit_moe.VisionTransformerMoe(**product_config(cfg, O.BF16))
+  got, metrics = model.apply({"params": tree_to_dev(params)}, tree_to_dev(images))
+  assert got.dtype == torch.float32 and tuple(got.shape) == want.shape == (16, 1000)
+  err = np.abs(to_np(got) - want)
+  scale = float(np.sqrt(np.mean(want ** 2)))
+  bad_images = (err.max(axis=1) > 2e-2 * (scale + np.abs(want).max(axis=1))).sum()
+  print(f"b16 width: images outside 2e-2: {bad_images} / {len(want)}; max err {err.max():.3e}, scale {scale:.3f}")
+  assert bad_images <= 1, f"{bad_images} of {len(want)} images outside 2e-2 (scale {scale:.3f})"
+  np.testing.assert_allclose(to_np(metrics["auxiliary_loss"]),
+                             np.asarray(want_metrics["auxiliary_loss"]), rtol=2e-2, atol=1e-4)
+
+
 def test_model_from_checkpoint_files(vit_moe, tmp_path):
   """A dense model's parameters written in the reference's sharded checkpoint format,
   read back, upcycled (every expert a copy of the dense MLP) and run on the GPU."""

@@ -34,6 +34,12 @@ __device__ __forceinline__ void store_stream(uint4* p, const uint4& v) {
   __builtin_nontemporal_store(__builtin_bit_cast(u32x4, v), reinterpret_cast<u32x4*>(p));
 }
 
+// A slot row outside [0, num_slots) counts as a dropped assignment (-1): maps that do not
+// come from the slot-assignment kernels cannot make a row mover leave the buffer.
+__device__ __forceinline__ int checked_slot(int slot, int num_slots) {
+  return (unsigned)slot < (unsigned)num_slots ? slot : -1;
+}
+
 // idx / cpr for idx < 2^16 with magic = ceil(2^32 / cpr); magic == 0 encodes cpr == 1.
 __device__ __forceinline__ int div_chunks(int idx, uint32_t magic) {
   return magic == 0 ? idx : (int)__umulhi((uint32_t)idx, magic);
@@ -53,7 +59,7 @@ __global__ __launch_bounds__(kMoveThreads) void dispatch_kernel(
     const int t0 = blockIdx.x * kRowsPerBlock;
     if (tid < kRowsPerBlock * K) {
       const int r = tid / K;
-      slots[tid] = t0 + r < num_items ? token_slot[(size_t)t0 * K + tid] : -1;
+      slots[tid] = t0 + r < num_items ? checked_slot(token_slot[(size_t)t0 * K + tid], num_slots) : -1;
     }
     __syncthreads();
     for (int idx = tid; idx < total; idx += kMoveThreads) {
@@ -92,7 +98,7 @@ __global__ __launch_bounds__(kMoveThreads) void dispatch_generic_kernel(
     for (int ch = lane; ch < cpr; ch += kWave) {
       const uint4 v = x[(size_t)wave * cpr + ch];
       for (int k = 0; k < K; ++k) {
-        int slot = token_slot[(size_t)wave * K + k];
+        const int slot = checked_slot(token_slot[(size_t)wave * K + k], num_slots);
         if (slot >= 0) out[(size_t)slot * cpr + ch] = v;
       }
     }
@@ -136,8 +142,8 @@ template <> struct Chunk<bf16_t> {
 template <typename T>
 __global__ __launch_bounds__(kMoveThreads) void combine_kernel(
     const uint4* __restrict__ y, const int32_t* __restrict__ token_slot,
-    const float* __restrict__ weights, uint4* __restrict__ out, int num_items, int K, int cpr,
-    uint32_t magic) {
+    const float* __restrict__ weights, uint4* __restrict__ out, int num_items, int num_slots,
+    int K, int cpr, uint32_t magic) {
   constexpr int N = Chunk<T>::n;
   __shared__ int32_t slots[kRowsPerBlock * kMaxK];
   __shared__ float wts[kRowsPerBlock * kMaxK];
@@ -146,7 +152,7 @@ __global__ __launch_bounds__(kMoveThreads) void combine_kernel(
   if (tid < kRowsPerBlock * K) {
     const int r = tid / K;
     const bool ok = t0 + r < num_items;
-    slots[tid] = ok ? token_slot[(size_t)t0 * K + tid] : -1;
+    slots[tid] = ok ? checked_slot(token_slot[(size_t)t0 * K + tid], num_slots) : -1;
     wts[tid] = ok ? weights[(size_t)t0 * K + tid] : 0.f;
   }
   __syncthreads();
@@ -193,7 +199,8 @@ __global__ __launch_bounds__(kMoveThreads) void combine_kernel(
 template <typename T>
 __global__ __launch_bounds__(kMoveThreads) void combine_generic_kernel(
     const uint4* __restrict__ y, const int32_t* __restrict__ token_slot,
-    const float* __restrict__ weights, uint4* __restrict__ out, int num_items, int K, int cpr) {
+    const float* __restrict__ weights, uint4* __restrict__ out, int num_items, int num_slots,
+    int K, int cpr) {
   constexpr int N = Chunk<T>::n;
   const int lane = threadIdx.x & 63;
   const int t = __builtin_amdgcn_readfirstlane(
@@ -204,7 +211,7 @@ __global__ __launch_bounds__(kMoveThreads) void combine_generic_kernel(
 #pragma unroll
     for (int j = 0; j < N; ++j) acc[j] = 0.f;
     for (int k = 0; k < K; ++k) {
-      int slot = token_slot[(size_t)t * K + k];
+      const int slot = checked_slot(token_slot[(size_t)t * K + k], num_slots);
       if (slot < 0) continue;
       float w = weights[(size_t)t * K + k];
       float a[N];
@@ -278,7 +285,7 @@ __global__ __launch_bounds__(kMoveThreads) void scatter_scaled_kernel(
       float a[N];
       Chunk<T>::unpack(g[(size_t)wave * cpr + ch], a);
       for (int k = 0; k < K; ++k) {
-        const int slot = token_slot[(size_t)wave * K + k];
+        const int slot = checked_slot(token_slot[(size_t)wave * K + k], num_slots);
         if (slot < 0) continue;
         const float w = weights[(size_t)wave * K + k];
         float b[N];
@@ -297,15 +304,15 @@ __global__ __launch_bounds__(kMoveThreads) void scatter_scaled_kernel(
 template <typename T>
 __global__ __launch_bounds__(kMoveThreads) void row_dots_kernel(
     const uint4* __restrict__ g, const uint4* __restrict__ y,
-    const int32_t* __restrict__ token_slot, float* __restrict__ dw, int num_items, int K,
-    int cpr) {
+    const int32_t* __restrict__ token_slot, float* __restrict__ dw, int num_items, int num_slots,
+    int K, int cpr) {
   constexpr int N = Chunk<T>::n;
   const int lane = threadIdx.x & 63;
   const int t = __builtin_amdgcn_readfirstlane(
       (int)((blockIdx.x * (unsigned)kMoveThreads + threadIdx.x) >> 6));
   if (t >= num_items) return;
   for (int k = 0; k < K; ++k) {
-    const int slot = token_slot[(size_t)t * K + k];
+    const int slot = checked_slot(token_slot[(size_t)t * K + k], num_slots);
     float acc = 0.f;
     if (slot >= 0) {
       for (int ch = lane; ch < cpr; ch += kWave) {
@@ -377,21 +384,21 @@ extern "C" int vmoe_combine(const VmoeCombineParams* p, vmoe_stream_t stream) {
     if (bf16)
       hipLaunchKernelGGL(combine_kernel<bf16_t>, dim3(blocks), dim3(kMoveThreads), 0,
                          as_stream(stream), (const uint4*)p->y, p->token_slot, p->weights,
-                         (uint4*)p->out, p->num_items, p->K, cpr, chunk_magic(cpr));
+                         (uint4*)p->out, p->num_items, p->num_slots, p->K, cpr, chunk_magic(cpr));
     else
       hipLaunchKernelGGL(combine_kernel<float>, dim3(blocks), dim3(kMoveThreads), 0,
                          as_stream(stream), (const uint4*)p->y, p->token_slot, p->weights,
-                         (uint4*)p->out, p->num_items, p->K, cpr, chunk_magic(cpr));
+                         (uint4*)p->out, p->num_items, p->num_slots, p->K, cpr, chunk_magic(cpr));
   } else {
     const int blocks = (p->num_items + 3) / 4;
     if (bf16)
       hipLaunchKernelGGL(combine_generic_kernel<bf16_t>, dim3(blocks), dim3(kMoveThreads), 0,
                          as_stream(stream), (const uint4*)p->y, p->token_slot, p->weights,
-                         (uint4*)p->out, p->num_items, p->K, cpr);
+                         (uint4*)p->out, p->num_items, p->num_slots, p->K, cpr);
     else
       hipLaunchKernelGGL(combine_generic_kernel<float>, dim3(blocks), dim3(kMoveThreads), 0,
                          as_stream(stream), (const uint4*)p->y, p->token_slot, p->weights,
-                         (uint4*)p->out, p->num_items, p->K, cpr);
+                         (uint4*)p->out, p->num_items, p->num_slots, p->K, cpr);
   }
   return launch_status();
 }
@@ -455,10 +462,10 @@ extern "C" int vmoe_combine_backward_weights(const VmoeCombineBackwardParams* p,
   if (p->dtype == VMOE_BF16)
     hipLaunchKernelGGL(row_dots_kernel<bf16_t>, dim3(blocks), dim3(kMoveThreads), 0,
                        as_stream(stream), (const uint4*)p->dout, (const uint4*)p->y, p->token_slot,
-                       p->dweights, p->num_items, p->K, cpr);
+                       p->dweights, p->num_items, p->num_slots, p->K, cpr);
   else
     hipLaunchKernelGGL(row_dots_kernel<float>, dim3(blocks), dim3(kMoveThreads), 0,
                        as_stream(stream), (const uint4*)p->dout, (const uint4*)p->y, p->token_slot,
-                       p->dweights, p->num_items, p->K, cpr);
+                       p->dweights, p->num_items, p->num_slots, p->K, cpr);
   return launch_status();
 }

@@ -290,6 +290,9 @@ static int check_mlp(const VmoeExpertMlpParams* p) {
   }
   if (!aligned16(p->x) || !aligned16(p->out)) return VMOE_E_ALIGN;
   if ((int64_t)p->E * p->R >= INT32_MAX) return VMOE_E_OVERFLOW;
+  // Unpacked weights are transposed with the expert as the grid's z dimension.
+  if (p->dtype == VMOE_BF16 && (p->w0t == nullptr || p->w1t == nullptr) && p->E > 65535)
+    return VMOE_E_UNSUPPORTED;
   return VMOE_OK;
 }
 

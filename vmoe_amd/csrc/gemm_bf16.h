@@ -322,7 +322,7 @@ __global__ __launch_bounds__(Cfg::kThreads, Cfg::kBlocksPerCu) void gemm_bf16_ke
     const bf16_t* __restrict__ A, const bf16_t* __restrict__ Bt, const bf16_t* __restrict__ bias,
     bf16_t* __restrict__ C, int R, int N, int Kd, int tiles_m, int tiles_n, int num_tiles,
     int tiles_per_xcd, int panel_rows, const int32_t* __restrict__ rows,
-    const int4* __restrict__ plan, const int32_t* __restrict__ a_rows) {
+    const int4* __restrict__ plan, const int32_t* __restrict__ a_rows, int a_items) {
 #if defined(__HIP_DEVICE_COMPILE__)   // buffer-resource builtins exist in the device pass only
   extern __shared__ __align__(1024) unsigned char smem[];
   constexpr int BM = Cfg::BM, BN = Cfg::BN, BK = Cfg::BK;
@@ -374,7 +374,11 @@ __global__ __launch_bounds__(Cfg::kThreads, Cfg::kBlocksPerCu) void gemm_bf16_ke
   for (int i = 0; i < Cfg::kAIssues; ++i) {
     int r = (i * Cfg::kWaves + wave) * RPL + lrow;
     int arow = min(row0 + r, (a_rows != nullptr ? live : R) - 1);
-    if (a_rows != nullptr) arow = a_rows[(size_t)b * R + arow];
+    // an entry outside the item matrix reads item 0 instead of leaving the buffer
+    if (a_rows != nullptr) {
+      arow = a_rows[(size_t)b * R + arow];
+      arow = (unsigned)arow < (unsigned)a_items ? arow : 0;
+    }
     a_goff[i] = (uint32_t)arow * (uint32_t)Kd * 2u + chunk * 16;
   }
 #pragma unroll
@@ -945,7 +949,7 @@ int launch_gemm_bf16(const bf16_t* A, const bf16_t* Bt, const bf16_t* bias, bf16
   if (e != hipSuccess) return (int)e;
   hipLaunchKernelGGL(kern, dim3(blocks), dim3(Cfg::kThreads), Cfg::kLdsBytes, stream, A, Bt, bias,
                      C, R, N, Kd, g.tiles_m, g.tiles_n, (int)g.tiles, g.tiles_per_xcd, g.panel_rows,
-                     rows, plan, a_rows);
+                     rows, plan, a_rows, (int)a_items);
   return launch_status();
 }
 

@@ -428,6 +428,12 @@ def compute_capacity(num_tokens: int, num_experts: int, capacity_factor: float,
   return capacity
 
 
+def get_dense_einsum_dispatcher(gates: Array, **dispatcher_kwargs) -> DenseEinsumDispatcher:
+  """Every item goes to every expert: nothing to route, the gates (G, S, E) are the
+  combine weights; vmoe/moe.py:260-264."""
+  return DenseEinsumDispatcher(combine_weights=gates, **dispatcher_kwargs)
+
+
 def get_top_experts_per_item_dispatcher(
     gates: Array, name: str, num_selected_experts: int, batch_priority: bool,
     capacity: Optional[int] = None, capacity_factor: Optional[float] = None,

@@ -62,6 +62,17 @@ def lecun_normal(gen: torch.Generator, shape, fan_in: int, dtype=torch.float32, 
   return t.to(dtype).to(device) if device is not None else t.to(dtype)
 
 
+def require_no_grad(what: str, *tensors) -> None:
+  """The gating, routing and expert kernels are forward-only (inference).  Called with
+  the parameters and inputs of such a module: raises instead of silently cutting the
+  graph when autograd is recording and one of them requires a gradient."""
+  if torch.is_grad_enabled() and any(
+      isinstance(t, torch.Tensor) and t.requires_grad for t in tensors):
+    raise NotImplementedError(
+        f"{what} has no backward pass (inference path): call it under torch.no_grad() or "
+        "detach its parameters and inputs.")
+
+
 def make_rngs(rngs, device):
   """``rngs={'gating': seed or torch.Generator}`` (flax's ``rngs=`` argument of apply)
   with every seed turned into a generator on ``device``, so that modules that draw

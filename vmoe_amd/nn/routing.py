@@ -71,6 +71,7 @@ class NoisyTopExpertsPerItemRouter(module.Module):
     if kernel.shape != (inputs.shape[-1], num_experts):
       raise ValueError(f"Router kernel has shape {tuple(kernel.shape)}, expected "
                        f"{(inputs.shape[-1], num_experts)}")
+    module.require_no_grad(type(self).__name__, inputs, kernel)
     dtype = self.dtype or inputs.dtype
     x = K.cast(inputs, dtype)
     w = self._cast_kernel(kernel, dtype)
@@ -152,6 +153,7 @@ class NoisyTopItemsPerExpertRouter(module.Module):
     if kernel.shape != (inputs.shape[-1], self.num_experts):
       raise ValueError(f"Router kernel has shape {tuple(kernel.shape)}, expected "
                        f"{(inputs.shape[-1], self.num_experts)}")
+    module.require_no_grad(type(self).__name__, inputs, kernel)
     dtype = self.dtype or inputs.dtype
     if self.deterministic or self.noise_std == 0.0:
       gates, _, _ = K.gate_topk(K.cast(inputs, dtype), K.cast(kernel, dtype), 1)

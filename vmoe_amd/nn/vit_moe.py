@@ -60,9 +60,10 @@ class MlpBlock(module.Module):
     computed; the other rows of the result are not written."""
     p = variables["params"]
     dtype = self.dtype or inputs.dtype
-    x = K.cast(inputs, dtype)
     w0, b0 = p["Dense_0"]["kernel"], p["Dense_0"].get("bias")
     w1, b1 = p["Dense_1"]["kernel"], p["Dense_1"].get("bias")
+    module.require_no_grad("MlpBlock", inputs, w0, b0, w1, b1)
+    x = K.cast(inputs, dtype)
     cast = lambda t: None if t is None else K.cast(t, dtype)
     if dtype == torch.bfloat16:
       return K.expert_mlp(x, None, cast(b0), None, cast(b1), w0t=self._pack(w0, dtype),
@@ -86,6 +87,7 @@ class MlpBlock(module.Module):
     dtype = self.dtype or items.dtype
     w0, b0 = p["Dense_0"]["kernel"], p["Dense_0"].get("bias")
     w1, b1 = p["Dense_1"]["kernel"], p["Dense_1"].get("bias")
+    module.require_no_grad("MlpBlock", items, w0, b0, w1, b1)
     cast = lambda t: None if t is None else K.cast(t, dtype)
     return K.expert_mlp(K.cast(items, dtype), None, cast(b0), None, cast(b1),
                         w0t=self._pack(w0, dtype), w1t=self._pack(w1, dtype),

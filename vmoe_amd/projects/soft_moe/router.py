@@ -53,6 +53,7 @@ class SoftRouter(module.Module):
     if not self.deterministic and self.noise_std > 0:
       raise NotImplementedError("Router noise is a training-time feature and is not implemented.")
     p = variables["params"]
+    module.require_no_grad("SoftRouter", inputs, p["mu"], p["scale"])
     dtype = self.dtype or inputs.dtype
     x = K.cast(inputs, dtype)
     G, m, dim = x.shape
