@@ -212,6 +212,17 @@ typedef struct {
 } VmoeCompactRowsParams;
 int vmoe_compact_rows(const VmoeCompactRowsParams* p, vmoe_stream_t stream);
 
+/* vmoe_compact_rows without a scratch argument (no counterpart in the reference).  For
+ * callers that cannot allocate device memory: code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc.  `prefix` is ignored; the (G, E) scratch is a
+ * static device array inside the library, VMOE_COMPACT_ROWS_STATIC_MAX_GE int32 per
+ * device (256 KiB, held until the process ends).  G * E beyond that returns
+ * VMOE_E_WORKSPACE.  The call allocates and frees nothing.  All calls on one device share
+ * the array: calls that overlap on one device (two streams, two host threads) race; calls
+ * on one stream, or otherwise ordered, do not.  Results equal vmoe_compact_rows'. */
+#define VMOE_COMPACT_ROWS_STATIC_MAX_GE 65536
+int vmoe_compact_rows_static(const VmoeCompactRowsParams* p, vmoe_stream_t stream);
+
 /* ------------------------------------------------------------------ dispatch / combine
  * dispatch replaces ExpertIndicesDispatcher.dispatch (vmoe/moe.py:190-197:
  * repeat + scatter_nd into zeros + _dispatch layout): out[slot] = x[item] for

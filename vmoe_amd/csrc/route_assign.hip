@@ -16,6 +16,7 @@
 //      lookup plus one masked popcount.
 // The kernel also emits the two maps the data-movement kernels use: item ->
 // slot row (-1 when over capacity) and slot row -> item (-1 when empty).
+#include <mutex>
 #include "vmoe_common.h"
 #include "router_metrics.h"
 
@@ -661,12 +662,9 @@ extern "C" int vmoe_top_items_per_expert(const VmoeTopItemsParams* p, vmoe_strea
   }
 }
 
-extern "C" int vmoe_compact_rows(const VmoeCompactRowsParams* p, vmoe_stream_t stream) {
-  if (p == nullptr || p->fill == nullptr || p->token_slot == nullptr || p->token_row == nullptr ||
-      p->rows_per_expert == nullptr || p->prefix == nullptr)
-    return VMOE_E_NULL;
-  int rc = check_route_shapes(p->G, p->S, p->E, p->K, p->C);
-  if (rc != VMOE_OK) return rc;
+// Launches the row compaction with `prefix` as the (G, E) scratch of its two-launch form.
+static int launch_compact_rows(const VmoeCompactRowsParams* p, int32_t* prefix,
+                               vmoe_stream_t stream) {
   const size_t n = (size_t)p->G * p->S * p->K;
   const int parts = p->E <= 256 ? 256 / p->E : 1;
   if (p->E <= 256 && (int64_t)p->S * p->K >= 256 && (p->G + parts - 1) / parts <= 16) {
@@ -676,9 +674,66 @@ extern "C" int vmoe_compact_rows(const VmoeCompactRowsParams* p, vmoe_stream_t s
     return launch_status();
   }
   hipLaunchKernelGGL(fill_prefix_kernel, dim3(p->E), dim3(256), 0, as_stream(stream), p->fill,
-                     p->prefix, p->rows_per_expert, p->G, p->E);
+                     prefix, p->rows_per_expert, p->G, p->E);
   hipLaunchKernelGGL(compact_rows_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0,
-                     as_stream(stream), p->prefix, p->token_slot, p->token_row, p->row_token, p->G,
+                     as_stream(stream), prefix, p->token_slot, p->token_row, p->row_token, p->G,
                      p->E, p->C, p->S * p->K, p->K, n);
   return launch_status();
+}
+
+static int check_compact_rows(const VmoeCompactRowsParams* p) {
+  if (p == nullptr || p->fill == nullptr || p->token_slot == nullptr || p->token_row == nullptr ||
+      p->rows_per_expert == nullptr)
+    return VMOE_E_NULL;
+  return check_route_shapes(p->G, p->S, p->E, p->K, p->C);
+}
+
+extern "C" int vmoe_compact_rows(const VmoeCompactRowsParams* p, vmoe_stream_t stream) {
+  int rc = check_compact_rows(p);
+  if (rc != VMOE_OK) return rc;
+  if (p->prefix == nullptr) return VMOE_E_NULL;
+  return launch_compact_rows(p, p->prefix, stream);
+}
+
+// ---------------------------------------------------------------- no allocation
+// vmoe_compact_rows for callers that cannot allocate: the (G, E) scratch is a file-scope
+// device array.  Its name is only a host-side handle; the device address is asked for once
+// per device (each device holds its own copy) and only that address is given to kernels.
+static __device__ __align__(256) int32_t scratch[VMOE_COMPACT_ROWS_STATIC_MAX_GE];
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::mutex scratch_mutex;
+int32_t* scratch_ptr[kMaxDevices];   // device address of `scratch` on each device, null until asked
+}  // namespace
+
+// Device address of this device's copy of `scratch` (the current device), or null with *err set.
+static int32_t* scratch_address(int* err) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) { *err = (int)e; return nullptr; }
+  if (dev < 0 || dev >= kMaxDevices) { *err = VMOE_E_UNSUPPORTED; return nullptr; }
+  std::lock_guard<std::mutex> lock(scratch_mutex);
+  if (scratch_ptr[dev] == nullptr) {
+    void* ptr = nullptr;
+    e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || ptr == nullptr) {
+      *err = e != hipSuccess ? (int)e : (int)hipErrorInvalidSymbol;
+      return nullptr;
+    }
+    scratch_ptr[dev] = static_cast<int32_t*>(ptr);
+  }
+  return scratch_ptr[dev];
+}
+
+extern "C" int vmoe_compact_rows_static(const VmoeCompactRowsParams* p, vmoe_stream_t stream) {
+  int rc = check_compact_rows(p);
+  if (rc != VMOE_OK) return rc;
+  if ((int64_t)p->G * p->E > VMOE_COMPACT_ROWS_STATIC_MAX_GE) return VMOE_E_WORKSPACE;
+  int err = VMOE_OK;
+  int32_t* prefix = scratch_address(&err);
+  if (prefix == nullptr) return err;
+  // Every entry of the scratch that the second launch reads (g < G, e < E) is written by the
+  // first one: nothing has to start at zero, whatever an earlier call left behind.
+  return launch_compact_rows(p, prefix, stream);
 }
