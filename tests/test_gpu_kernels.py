@@ -547,6 +547,39 @@ def test_expert_mlp_planned_launch_random_fill(K):
         assert (to_np(out[e, n:]) == 7.0).all(), f"E={E} R={R} rows={rows.tolist()} expert {e}"
 
 
+@pytest.mark.parametrize("E,R,D,M", [(64, 384, 1024, 128), (32, 1152, 1024, 256), (90, 384, 520, 160)])
+def test_expert_mlp_wide_second_product(K, E, R, D, M):
+  """Shapes whose second product takes the wide kernel (384 x 256 tiles, eight waves: chosen
+  where the 256 x 256 tiles would need at least 1.38 times as many rounds of one tile per
+  compute unit): all rows against the oracle, then packed rows with a launch plan
+  (row counts around the tile height, empty experts) bit for bit against the dense launch."""
+  rng = np.random.default_rng(E + R)
+  dtype = O.BF16
+  x = O.cast(rng.standard_normal((E, R, D)).astype(np.float32), dtype)
+  w0 = O.cast(rng.standard_normal((E, D, M)).astype(np.float32) / np.sqrt(D), dtype)
+  w1 = O.cast(rng.standard_normal((E, M, D)).astype(np.float32) / np.sqrt(M), dtype)
+  b0 = O.cast(rng.standard_normal((E, M)).astype(np.float32) * 0.1, dtype)
+  b1 = O.cast(rng.standard_normal((E, D)).astype(np.float32) * 0.1, dtype)
+  dx, dw0, db0, dw1, db1 = (to_dev(a, dtype) for a in (x, w0, b0, w1, b1))
+  full = K.expert_mlp(dx, dw0, db0, dw1, db1)
+  pick = np.unique(np.concatenate([[0, E - 1], rng.integers(0, E, 4)]))
+  want = O.mlp_block(x[pick], w0[pick], b0[pick], w1[pick], b1[pick], dtype)
+  assert_close(to_np(full)[pick], want, 2e-2, "wide second product")
+  nobias = K.expert_mlp(dx, dw0, db0, dw1, None)
+  want = O.mlp_block(x[pick[:2]], w0[pick[:2]], b0[pick[:2]], w1[pick[:2]], None, dtype)
+  assert_close(to_np(nobias)[pick[:2]], want, 2e-2, "wide second product, no bias")
+  special = np.asarray([0, 1, 95, 96, 97, 383, 384, 385, R - 1, R], np.int64)
+  for trial in range(3):
+    rows = np.where(rng.random(E) < 0.5, rng.integers(0, R + 1, E), rng.choice(special, E))
+    rows = np.minimum(rows, R).astype(np.int32)
+    out = torch.full_like(full, 7.0)
+    K.expert_mlp(dx, dw0, db0, dw1, db1, out=out, rows_per_expert=to_dev(rows))
+    got, ref = to_np(out), to_np(full)
+    for e, n in enumerate(rows):
+      np.testing.assert_array_equal(got[e, :n], ref[e, :n], err_msg=f"rows={rows.tolist()} expert {e}")
+      assert (got[e, n:] == 7.0).all(), f"rows={rows.tolist()} expert {e}"
+
+
 def test_operand_delivery_probe(K):
   """The load-only measurement kernel reports the operand bytes of the 256 x 256 tiling
   and refuses what the tiling refuses."""

@@ -4,7 +4,7 @@
 // vit_jax.models_vit.MlpBlock (vmoe/nn/vit_moe.py:38-45): a GEMM batched over
 // the expert axis with the bias add and the GELU fused into the epilogue of the
 // first product and the bias add into the second.
-#include "gemm_bf16.h"
+#include "gemm_bf16_wide.h"
 
 namespace vmoe {
 namespace {
@@ -127,9 +127,11 @@ int transpose(const void* in, void* out, int batch, int rows, int cols, int dtyp
 // one 256x256 workgroup per CU for the highest arithmetic intensity.
 using CfgUp = GemmCfg<128, 256, 2, 2, 32, 3, 2>;
 using CfgDown = GemmCfg<256, 256, 2, 2, 32, 4, 1>;
-// The persistent form of the second product keeps 35 KB of LDS for staging its output
-// and so has three stages; tile shape and launch plan are CfgDown's.
-using CfgDownPersistent = GemmCfg<256, 256, 2, 2, 32, 3, 1>;
+// The persistent form of the second product takes k in 64-wide tiles, two stages: a DMA
+// load then requests whole 128-byte lines of an operand row (64-byte halves of a line,
+// requested a k tile apart, move at two thirds of the rate when the line comes from
+// beyond L2).  18 KB of LDS stage its output; tile shape and launch plan are CfgDown's.
+using CfgDownPersistent = GemmCfg<256, 256, 2, 2, 64, 2, 1>;
 
 // Register-resident MFMA loop: the arithmetic ceiling that the expert GEMMs are
 // compared with.  Every wave keeps a 128 x 128 accumulator tile (16 MFMA tiles,
@@ -239,16 +241,35 @@ bool down_prefers_half_tiles(int E, int R, int N) {
   return t_half < 0.9 * t_full;
 }
 
+// The second product takes the wide kernel (384 x 256 tiles, eight waves: about a tenth
+// faster per flop than the 256 x 256 persistent kernel) where its coarser tiles do not cost
+// more in idle compute units than that buys: both kernels run their tiles in rounds of one
+// per compute unit, and a last round that is nearly empty costs a whole tile's time.
+bool down_prefers_wide_tiles(int E, int R, int N, int Kd) {
+  if (!wide_gemm_ok(E, R, N, Kd, nullptr, nullptr, nullptr, 0)) return false;
+  constexpr int64_t kNumCu = kCusPerXcd * kNumXcd;
+  const int64_t tn = (N + 255) / 256;
+  const int64_t wide = (int64_t)E * ((R + WideCfg::BM - 1) / WideCfg::BM) * tn;
+  const int64_t square = (int64_t)E * ((R + 255) / 256) * tn;
+  const double t_wide = 1.5 * 0.92 * (double)((wide + kNumCu - 1) / kNumCu);
+  const double t_square = (double)((square + kNumCu - 1) / kNumCu);
+  return t_wide < t_square;
+}
+
 // Launch plans of the two ragged products of an MLP: geometry, bytes, one planning launch.
 struct MlpPlans {
   GemmGeom up, down;
+  bool down_wide = false;
+  int down_bm = CfgDown::BM;
   size_t up_bytes = 0, down_bytes = 0;   // 0: that product keeps the static tile order
 };
 
 MlpPlans mlp_plans(int E, int R, int D, int M) {
   MlpPlans m;
   m.up = gemm_geometry<CfgUp>(E, R, M, D);
-  m.down = gemm_geometry<CfgDown>(E, R, D, M);
+  m.down_wide = down_prefers_wide_tiles(E, R, D, M);
+  m.down = m.down_wide ? gemm_geometry<WideCfg>(E, R, D, M) : gemm_geometry<CfgDown>(E, R, D, M);
+  m.down_bm = m.down_wide ? WideCfg::BM : CfgDown::BM;
   // Ragged launches are planned whenever the geometry allows: with whole experts per
   // die in a static order the die that drew the fullest experts sets the time (a layer
   // with capacity factor 0.5 and a skewed router: 399 -> 267 us for the two products,
@@ -333,7 +354,7 @@ extern "C" int vmoe_expert_mlp(const VmoeExpertMlpParams* p, vmoe_stream_t strea
     if (plan_up != nullptr || plan_down != nullptr) {
       const RaggedGeom ga{CfgUp::BM, m.up.tiles_n, m.up.panel_rows,
                           plan_up ? (int)(m.up.ragged_slots * kNumXcd) : 0, plan_up};
-      const RaggedGeom gb{CfgDown::BM, m.down.tiles_n, m.down.panel_rows,
+      const RaggedGeom gb{m.down_bm, m.down.tiles_n, m.down.panel_rows,
                           plan_down ? (int)(m.down.ragged_slots * kNumXcd) : 0, plan_down};
       const int n = ga.num_blocks > gb.num_blocks ? ga.num_blocks : gb.num_blocks;
       hipLaunchKernelGGL(plan_ragged_tiles_kernel, dim3((n + 255) / 256), dim3(256),
@@ -370,6 +391,11 @@ extern "C" int vmoe_expert_mlp(const VmoeExpertMlpParams* p, vmoe_stream_t strea
       return launch_gemm_bf16<CfgUp, kEpiBias>((const bf16_t*)hidden, (const bf16_t*)w1t,
                                               (const bf16_t*)p->b1, (bf16_t*)p->out, p->E, p->R,
                                               p->D, p->M, stream, nullptr, nullptr);
+    if (down_prefers_wide_tiles(p->E, p->R, p->D, p->M) &&
+        (p->rows_per_expert == nullptr || plan_down != nullptr))
+      return launch_gemm_bf16_wide<kEpiBias>((const bf16_t*)hidden, (const bf16_t*)w1t,
+                                             (const bf16_t*)p->b1, (bf16_t*)p->out, p->E, p->R,
+                                             p->D, p->M, stream, plan_down);
     if (persistent_gemm_ok<CfgDownPersistent>(p->E, p->R, p->D, p->M, p->rows_per_expert, plan_down))
       return launch_gemm_bf16_persistent<CfgDownPersistent, kEpiBias>(
           (const bf16_t*)hidden, (const bf16_t*)w1t, (const bf16_t*)p->b1, (bf16_t*)p->out, p->E,

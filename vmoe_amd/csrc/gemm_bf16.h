@@ -568,10 +568,15 @@ constexpr int kCusPerXcd = 32;
 
 template <typename Cfg>
 struct PersistentLds {
-  static constexpr int kOutLd = Cfg::TN + 8;
   static constexpr size_t kRing = (size_t)Cfg::NSTAGE * Cfg::kStageBytes;
+  // The output is staged 32 rows per wave at a time, over the whole width of the wave tile
+  // where the ring leaves room for that, else in two halves.
+  static constexpr size_t kFullStaging = (size_t)Cfg::kWaves * 32 * (Cfg::TN + 8) * sizeof(bf16_t);
+  static constexpr int kStageCols = kRing + kFullStaging <= 160 * 1024 ? Cfg::TN : Cfg::TN / 2;
+  static constexpr int kOutLd = kStageCols + 8;
   static constexpr size_t kStaging = (size_t)Cfg::kWaves * 32 * kOutLd * sizeof(bf16_t);
   static constexpr size_t kBytes = kRing + kStaging;
+  static_assert(kStageCols % 32 == 0, "staging covers whole MFMA tiles");
   static_assert(kBytes <= 160 * 1024, "LDS budget");
 };
 
@@ -588,7 +593,7 @@ __global__ __launch_bounds__(Cfg::kThreads, 1) void gemm_bf16_persistent_kernel(
   constexpr int FM = Cfg::FM, FN = Cfg::FN;
   constexpr int RB = Cfg::kRowBytes;
   constexpr int NS = Cfg::NSTAGE, PD = NS - 1, L = Cfg::kLoads;
-  static_assert(BK == 32, "two k slices per tile");
+  constexpr int KS = BK / 16;    // k slices (one MFMA deep) per k tile: 2 or 4
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -718,15 +723,18 @@ __global__ __launch_bounds__(Cfg::kThreads, 1) void gemm_bf16_persistent_kernel(
   // as a lambda taking the tile by reference the offsets end up in scratch memory.
 #define VMOE_PERSISTENT_K_ITERATION(SRC, K0, WAITED) do { \
     const int next_stage = stage + 1 == NS ? 0 : stage + 1; \
-    load_frags(1, stage, 1); \
-    mfma_slice(0); \
-    slice_schedule(std::integral_constant<int, 0>{}); \
+    _Pragma("unroll") \
+    for (int ks = 0; ks + 1 < KS; ++ks) { \
+      load_frags((ks + 1) & 1, stage, ks + 1); \
+      mfma_slice(ks & 1); \
+      slice_schedule(std::integral_constant<int, 0>{}); \
+    } \
     if constexpr (!(WAITED)) wait_vmcnt<(PD - 1) * L>(); \
     wait_lgkmcnt0(); \
     raw_barrier(); \
     load_frags(0, next_stage, 0); \
     load_ktile(SRC, stage, (K0)); \
-    mfma_slice(1); \
+    mfma_slice((KS - 1) & 1); \
     slice_schedule(std::integral_constant<int, L>{}); \
     stage = next_stage; \
   } while (0)
@@ -758,41 +766,45 @@ __global__ __launch_bounds__(Cfg::kThreads, 1) void gemm_bf16_persistent_kernel(
     mfma_result_fence();
     bf16_t* Cb = C + (size_t)cur.b * R * N;
     const int wrow0 = cur.row0 + wm * Cfg::TM, wcol0 = cur.col0 + wn * Cfg::TN;
-    constexpr int kChunksOut = Cfg::TN / 8;
+    constexpr int SC = PersistentLds<Cfg>::kStageCols;   // columns staged at a time
+    constexpr int kChunksOut = SC / 8;
     constexpr int kRowsPerPass = 64 / kChunksOut;
-    static_assert(64 % kChunksOut == 0 && 32 % kRowsPerPass == 0, "wave tile width must divide a wave");
+    static_assert(64 % kChunksOut == 0 && 32 % kRowsPerPass == 0, "staged width must divide a wave");
     const int oc = (lane % kChunksOut) * 8;
     const int orow = lane / kChunksOut;
 #pragma unroll
     for (int i = 0; i < FM; ++i) {
 #pragma unroll
-      for (int j = 0; j < FN; ++j) {
+      for (int c0 = 0; c0 < Cfg::TN; c0 += SC) {
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          const int cl = j * 32 + q * 8 + h * 4;
-          const uint2 bp = bias_pk[j * 4 + q];
-          const float bv[4] = {bf_lo(bp.x), bf_hi(bp.x), bf_lo(bp.y), bf_hi(bp.y)};
-          const uint32_t p0 = epilogue_pair<EPI, HAS_BIAS>(acc[i][j][q * 4], acc[i][j][q * 4 + 1], bv[0], bv[1]);
-          const uint32_t p1 = epilogue_pair<EPI, HAS_BIAS>(acc[i][j][q * 4 + 2], acc[i][j][q * 4 + 3], bv[2], bv[3]);
-          *reinterpret_cast<uint2*>(so + m * OLD + cl) = make_uint2(p0, p1);
+        for (int j = c0 / 32; j < (c0 + SC) / 32; ++j) {
 #pragma unroll
-          for (int v = 0; v < 4; ++v) acc[i][j][q * 4 + v] = 0.f;
+          for (int q = 0; q < 4; ++q) {
+            const int cl = j * 32 - c0 + q * 8 + h * 4;
+            const uint2 bp = bias_pk[j * 4 + q];
+            const float bv[4] = {bf_lo(bp.x), bf_hi(bp.x), bf_lo(bp.y), bf_hi(bp.y)};
+            const uint32_t p0 = epilogue_pair<EPI, HAS_BIAS>(acc[i][j][q * 4], acc[i][j][q * 4 + 1], bv[0], bv[1]);
+            const uint32_t p1 = epilogue_pair<EPI, HAS_BIAS>(acc[i][j][q * 4 + 2], acc[i][j][q * 4 + 3], bv[2], bv[3]);
+            *reinterpret_cast<uint2*>(so + m * OLD + cl) = make_uint2(p0, p1);
+#pragma unroll
+            for (int v = 0; v < 4; ++v) acc[i][j][q * 4 + v] = 0.f;
+          }
         }
-      }
-      // A wave reads back only what it wrote (its LDS operations complete in order).
+        // A wave reads back only what it wrote (its LDS operations complete in order).
 #pragma unroll
-      for (int r0 = 0; r0 < 32; r0 += kRowsPerPass) {
-        const int rl = r0 + orow;
-        const int row = wrow0 + i * 32 + rl;
-        const int col = wcol0 + oc;
-        const uint4 v = *reinterpret_cast<const uint4*>(so + rl * OLD + oc);
-        if (row < cur.live && col + 8 <= N) {
-          if constexpr (EPI != kEpiBias) {   // hidden layer: streaming store, as in store_tile
-            typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
-            __builtin_nontemporal_store(__builtin_bit_cast(u32x4_t, v),
-                                        reinterpret_cast<u32x4_t*>(Cb + (size_t)row * N + col));
-          } else {
-            *reinterpret_cast<uint4*>(Cb + (size_t)row * N + col) = v;
+        for (int r0 = 0; r0 < 32; r0 += kRowsPerPass) {
+          const int rl = r0 + orow;
+          const int row = wrow0 + i * 32 + rl;
+          const int col = wcol0 + c0 + oc;
+          const uint4 v = *reinterpret_cast<const uint4*>(so + rl * OLD + oc);
+          if (row < cur.live && col + 8 <= N) {
+            if constexpr (EPI != kEpiBias) {   // hidden layer: streaming store, as in store_tile
+              typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+              __builtin_nontemporal_store(__builtin_bit_cast(u32x4_t, v),
+                                          reinterpret_cast<u32x4_t*>(Cb + (size_t)row * N + col));
+            } else {
+              *reinterpret_cast<uint4*>(Cb + (size_t)row * N + col) = v;
+            }
           }
         }
       }
