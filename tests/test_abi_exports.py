@@ -132,3 +132,38 @@ def test_two_block_entry_point_rejects_null():
   fn.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p]
   assert fn(None, None, None) < 0
   assert fn(ctypes.byref(_hip.RouteAssignParams()), ctypes.byref(_hip.RouterMetricsParams()), None) < 0
+
+
+# ------------------------------------------------------------------ the jax.ffi shim (source only)
+FFI_SOURCE = os.path.join(ROOT, "vmoe_amd", "csrc", "ffi", "vmoe_xla_ffi.cc")
+
+
+def _camel(name: str) -> str:
+  return "".join(part.capitalize() for part in name.split("_"))
+
+
+def test_xla_ffi_shim_covers_every_entry_point():
+  """The XLA FFI shim cannot be compiled here (no jaxlib headers), so its coverage is
+  checked on the text: every entry point of the header that takes a parameter block has
+  a handler symbol (the entry point's name in CamelCase) whose implementation calls it,
+  and every field of every parameter block is assigned somewhere in the shim."""
+  header = re.sub(r"/\*.*?\*/", "", open(HEADER).read(), flags=re.S)
+  shim = open(FFI_SOURCE).read()
+  code = re.sub(r"//[^\n]*", "", shim)
+  entry_points = re.findall(r"\bint\s+(vmoe_[a-z0-9_]+)\s*\(\s*const\s+(Vmoe\w+Params)\s*\*", header)
+  assert len(entry_points) >= 24
+  handlers = set(re.findall(r"XLA_FFI_DEFINE_HANDLER_SYMBOL\(\s*(\w+)\s*,", code))
+  for fn, _ in entry_points:
+    assert _camel(fn) in handlers, f"no XLA FFI handler symbol {_camel(fn)} for {fn}"
+    assert re.search(rf"\b{fn}\s*\(\s*&", code), f"the shim never calls {fn}"
+  assert len(handlers) == len(entry_points), sorted(handlers - {_camel(f) for f, _ in entry_points})
+  structs = {n: b for b, n in re.findall(r"typedef struct \{(.*?)\}\s*(\w+);", header, flags=re.S)}
+  for _, struct in set(entry_points):
+    for field in re.findall(r"(\w+)\s*(?:,|;)", re.sub(r"\[[^\]]*\]", "", structs[struct])):
+      if field in ("int32_t", "float", "size_t", "int64_t"):
+        continue
+      assert re.search(rf"(?:\.|->){field}\s*=", code), f"{struct}.{field} is never set in the shim"
+  # the registration loop of INTEGRATION.md names the same handlers
+  doc = open(os.path.join(ROOT, "INTEGRATION.md")).read()
+  for fn, _ in entry_points:
+    assert fn in doc, f"{fn} is not mentioned in INTEGRATION.md"

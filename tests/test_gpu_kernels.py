@@ -580,6 +580,67 @@ def test_expert_mlp_wide_second_product(K, E, R, D, M):
       assert (got[e, n:] == 7.0).all(), f"rows={rows.tolist()} expert {e}"
 
 
+def _sparse_signs(rng, shape, nonzeros, axis):
+  """Entries in {-1, 0, 1} with exactly `nonzeros` non-zero entries along `axis`."""
+  shape = list(shape)
+  n = shape.pop(axis)
+  flat = np.zeros((int(np.prod(shape)), n), np.float32)
+  for row in flat:
+    pos = rng.choice(n, size=min(nonzeros, n), replace=False)
+    row[pos] = rng.choice(np.asarray([-1.0, 1.0], np.float32), size=pos.size)
+  return np.ascontiguousarray(np.moveaxis(flat.reshape(*shape, n), -1, axis))
+
+
+@pytest.mark.parametrize("E,R,D,M", [
+    (2, 96, 64, 256),         # one-tile-per-workgroup first product (2 k tiles), tile-walking second product
+    (3, 200, 72, 136),        # widths outside the fast path: register-staged kernel, k edge
+    (64, 384, 1024, 128),     # wide second product
+    (2, 300, 256, 2048),      # long k loops on both kernels' steady state
+])
+def test_matrix_core_results_are_read_whole(K, E, R, D, M):
+  """Every accumulator register of the matrix-core loops must be complete when the
+  epilogue reads it: a v_mfma_f32_32x32x16_bf16 result read too early comes back with
+  its last register stale, which showed as wrong rows 27 and 31 of every 32-row tile (the
+  kernels put a fixed gap of wait states between the loop and the first read).  Operands
+  are small integers chosen so that every product, sum and rounding step of the MLP is
+  exact in bfloat16 and the GELU is the identity (pre-activations of 8 and more): the
+  result must equal the float64 answer bit for bit, in particular rows 27 and 31."""
+  rng = np.random.default_rng(D + M)
+  x = rng.integers(-1, 2, (E, R, D)).astype(np.float32)
+  w0 = _sparse_signs(rng, (E, D, M), 8, axis=1)             # |x @ w0| <= 8
+  b0 = np.full((E, M), 16.0, np.float32)                    # hidden = 16 + (x @ w0) in [8, 24]
+  w1 = _sparse_signs(rng, (E, M, D), 4, axis=1)             # |hidden @ w1| <= 96
+  b1 = rng.integers(-3, 4, (E, D)).astype(np.float32)
+  hidden = np.einsum("erd,edm->erm", x.astype(np.float64), w0.astype(np.float64)) + 16.0
+  assert hidden.min() >= 8 and hidden.max() <= 24
+  want = np.einsum("erm,emd->erd", hidden, w1.astype(np.float64)) + b1[:, None, :]
+  assert np.abs(want).max() <= 128
+  dtype = O.BF16
+  got = to_np(K.expert_mlp(*(to_dev(a, dtype) for a in (x, w0, b0, w1, b1)))).astype(np.float64)
+  rows = np.arange(R)
+  late = (rows % 32 == 27) | (rows % 32 == 31)
+  np.testing.assert_array_equal(got[:, late], want[:, late], err_msg="rows 27 / 31 of a 32-row tile")
+  np.testing.assert_array_equal(got, want)
+
+
+def test_gating_logits_are_read_whole(K):
+  """The gating kernel's matrix-core loop under the same check: integer operands, exact
+  float32 logits, all rows (27 and 31 of each 32-item tile first)."""
+  rng = np.random.default_rng(3)
+  G, S, D, E = 3, 100, 256, 32
+  x = rng.integers(-2, 3, (G, S, D)).astype(np.float32)
+  w = rng.integers(-1, 2, (D, E)).astype(np.float32)
+  want = (x.astype(np.float64) @ w.astype(np.float64))          # |sum| <= 512: exact in float32
+  want_bf = np.asarray(O.cast(want.astype(np.float32), O.BF16), np.float64)   # the logits are rounded to the dtype
+  for dtype, ref in ((O.F32, want), (O.BF16, want_bf)):
+    _, _, _, logits = K.gate_topk(to_dev(x, dtype), to_dev(w, dtype), 2, return_logits=True)
+    got = to_np(logits).astype(np.float64).reshape(G * S, E)
+    rows = np.arange(G * S)
+    late = (rows % 32 == 27) | (rows % 32 == 31)
+    np.testing.assert_array_equal(got[late], ref.reshape(G * S, E)[late], err_msg=f"{dtype}: rows 27 / 31")
+    np.testing.assert_array_equal(got, ref.reshape(G * S, E), err_msg=dtype)
+
+
 def test_operand_delivery_probe(K):
   """The load-only measurement kernel reports the operand bytes of the 256 x 256 tiling
   and refuses what the tiling refuses."""

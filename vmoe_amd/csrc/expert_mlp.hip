@@ -353,9 +353,9 @@ extern "C" int vmoe_expert_mlp(const VmoeExpertMlpParams* p, vmoe_stream_t strea
     ws += m.down_bytes;
     if (plan_up != nullptr || plan_down != nullptr) {
       const RaggedGeom ga{CfgUp::BM, m.up.tiles_n, m.up.panel_rows,
-                          plan_up ? (int)(m.up.ragged_slots * kNumXcd) : 0, plan_up};
+                          plan_up ? (int)(m.up.ragged_slots * kNumXcd) : 0, reinterpret_cast<PlanEntry*>(plan_up)};
       const RaggedGeom gb{m.down_bm, m.down.tiles_n, m.down.panel_rows,
-                          plan_down ? (int)(m.down.ragged_slots * kNumXcd) : 0, plan_down};
+                          plan_down ? (int)(m.down.ragged_slots * kNumXcd) : 0, reinterpret_cast<PlanEntry*>(plan_down)};
       const int n = ga.num_blocks > gb.num_blocks ? ga.num_blocks : gb.num_blocks;
       hipLaunchKernelGGL(plan_ragged_tiles_kernel, dim3((n + 255) / 256), dim3(256),
                          (size_t)(p->E + 1) * 8, stream, p->rows_per_expert, p->E, p->R, ga, gb);

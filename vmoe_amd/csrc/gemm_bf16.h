@@ -221,54 +221,15 @@ __device__ __forceinline__ bool map_tile(int tiles_m, int tiles_n, int num_tiles
 // panels as in map_tile.  plan[blockIdx] = (batch, tile_m, tile_n, live rows of the
 // batch), batch -1 for a workgroup without work.  One launch plans up to two products
 // (the two of an MLP differ in tile height and width).
-struct RaggedGeom {
-  int bm, tiles_n, panel_rows, num_blocks;
-  int4* plan;
-};
+// (RaggedGeom, PlanEntry and plan_entry, the scalar arithmetic of one plan entry, live in
+// route_index.h; the kernels read an entry as one int4.)
+static_assert(sizeof(PlanEntry) == sizeof(int4), "a plan entry is read as one int4");
 
 __device__ __forceinline__ void plan_one(const RaggedGeom& g, const int32_t* tile_prefix,
                                          const int32_t* __restrict__ rows, int batch, int R,
                                          int i) {
   if (g.plan == nullptr || i >= g.num_blocks) return;
-  const int total = tile_prefix[batch];
-  const int share = (total + kNumXcd - 1) / kNumXcd;
-  const int xcd = i % kNumXcd;
-  int slot = i / kNumXcd;
-  const int first = xcd * share;
-  const int last = min(first + share, total);      // this die's run of the tile list
-  int4 out = make_int4(-1, 0, 0, 0);
-  if (first < last && slot < (last - first) * g.tiles_n) {
-    int lo = 0, hi = batch;                        // tile_prefix[lo] <= first < tile_prefix[hi]
-    while (hi - lo > 1) {
-      const int mid = (lo + hi) >> 1;
-      if (tile_prefix[mid] <= first) lo = mid;
-      else hi = mid;
-    }
-    // Walk the run batch by batch; the tiles of one batch are cut into panels of about
-    // panel_rows row tiles (never across batches: a panel shares one batch's B operand),
-    // each swept column tile by column tile.
-    int pos = first;
-    for (int b = lo; b < batch && pos < last; ++b) {
-      const int seg_end = min(tile_prefix[b + 1], last);
-      const int seg = seg_end - pos;
-      if (seg <= 0) continue;
-      const int panels = max(1, (seg + g.panel_rows / 2) / g.panel_rows);
-      const int per_panel = (seg + panels - 1) / panels;
-      if (slot < seg * g.tiles_n) {
-        int q = slot / (per_panel * g.tiles_n);      // panels before the last are full
-        if (q > panels - 1) q = panels - 1;
-        const int rows_here = min(per_panel, seg - q * per_panel);
-        const int in_panel = slot - q * per_panel * g.tiles_n;
-        const int tile_n = in_panel / rows_here;
-        const int entry = pos + q * per_panel + (in_panel - tile_n * rows_here);
-        out = make_int4(b, entry - tile_prefix[b], tile_n, min(max(rows[b], 0), R));
-        break;
-      }
-      slot -= seg * g.tiles_n;
-      pos = seg_end;
-    }
-  }
-  g.plan[i] = out;
+  g.plan[i] = plan_entry(g, tile_prefix, rows, batch, R, i);
 }
 
 __global__ __launch_bounds__(256) void plan_ragged_tiles_kernel(

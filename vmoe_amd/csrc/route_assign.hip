@@ -146,7 +146,7 @@ __device__ __forceinline__ void route_assign_group(
     if constexpr (R == 0) {
       for (int s = tid; s < SP; s += kRouteThreads) {
         uint64_t key = ~0ull;
-        if (s < S) key = ((uint64_t)(~orderable(val[(size_t)s * K])) << 32) | (uint32_t)s;
+        if (s < S) key = bpr_key64(__builtin_bit_cast(uint32_t, val[(size_t)s * K]), s);
         keys[s] = key;
       }
       __syncthreads();
@@ -163,15 +163,14 @@ __device__ __forceinline__ void route_assign_group(
       for (int r = 0; r < R; ++r) {
         const int s = tid * R + r;
         bits[r] = (tid < nact && s < S) ? __builtin_bit_cast(uint32_t, val[(size_t)s * K]) : 0u;
-        narrow_ok = narrow_ok && (bits[r] & 0x8000ffffu) == 0u;
+        narrow_ok = narrow_ok && bpr_gate_is_narrow(bits[r]);
       }
       if (__syncthreads_and(narrow_ok)) {
         uint32_t key[R];
 #pragma unroll
         for (int r = 0; r < R; ++r) {
           const int s = tid * R + r;
-          key[r] = s < S ? ((~orderable(__builtin_bit_cast(float, bits[r]))) & 0xffff0000u) | (uint32_t)s
-                         : ~0u;
+          key[r] = s < S ? bpr_key32(bits[r], s) : ~0u;
         }
         bitonic_sort_regs<R, uint32_t>(key, reinterpret_cast<uint32_t*>(keys), SP, tid, nact);
 #pragma unroll
@@ -182,8 +181,7 @@ __device__ __forceinline__ void route_assign_group(
 #pragma unroll
         for (int r = 0; r < R; ++r) {
           const int s = tid * R + r;
-          key[r] = s < S ? ((uint64_t)(~orderable(__builtin_bit_cast(float, bits[r]))) << 32) | (uint32_t)s
-                         : ~0ull;
+          key[r] = s < S ? bpr_key64(bits[r], s) : ~0ull;
         }
         bitonic_sort_regs<R, uint64_t>(key, keys, SP, tid, nact);
 #pragma unroll
@@ -201,7 +199,7 @@ __device__ __forceinline__ void route_assign_group(
     int s = i / K, k = i - s * K;
     int e = idx[i];
     if (e >= 0 && e < E) {
-      int bit = k * S + rank[s];
+      const int bit = choice_bit(k, S, rank[s]);
       atomicOr(&bitmap[(size_t)e * W + (bit >> 5)], 1u << (bit & 31));
     }
   }
@@ -233,10 +231,9 @@ __device__ __forceinline__ void route_assign_group(
     int e = idx[i];
     int pos = -1, slot = -1;
     if (e >= 0 && e < E) {
-      int bit = k * S + rank[s];
-      int w = bit >> 5;
-      pos = (int)prefix[(size_t)e * W + w] +
-            __popc(bitmap[(size_t)e * W + w] & ((1u << (bit & 31)) - 1u));
+      const int bit = choice_bit(k, S, rank[s]);
+      const int w = bit >> 5;
+      pos = position_from_bitmap(prefix[(size_t)e * W + w], bitmap[(size_t)e * W + w], bit);
       if (pos < C) {
         slot = slot_row(e, g, pos, G, E, C);
         slot_token[slot] = g * S + s;
@@ -328,7 +325,7 @@ __global__ __launch_bounds__(kRouteThreads) void top_items_kernel(
   if constexpr (R == 0) {
     for (int s = tid; s < SP; s += kRouteThreads) {
       uint64_t key = ~0ull;
-      if (s < S) key = ((uint64_t)(~orderable(Elt<T>::load(col + (size_t)s * E))) << 32) | (uint32_t)s;
+      if (s < S) key = bpr_key64(__builtin_bit_cast(uint32_t, Elt<T>::load(col + (size_t)s * E)), s);
       keys[s] = key;
     }
     __syncthreads();
@@ -341,7 +338,7 @@ __global__ __launch_bounds__(kRouteThreads) void top_items_kernel(
     for (int r = 0; r < R; ++r) {
       const int s = tid * R + r;
       key[r] = (tid < nact && s < S)
-                   ? ((uint64_t)(~orderable(Elt<T>::load(col + (size_t)s * E))) << 32) | (uint32_t)s
+                   ? bpr_key64(__builtin_bit_cast(uint32_t, Elt<T>::load(col + (size_t)s * E)), s)
                    : ~0ull;
     }
     bitonic_sort_regs<R, uint64_t>(key, keys, SP, tid, nact);
@@ -364,15 +361,13 @@ __global__ __launch_bounds__(256) void indices_to_slots_kernel(
   size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
   size_t n = (size_t)G * S * K;
   if (i >= n) return;
-  int e = indices[2 * i], c = indices[2 * i + 1];
-  int slot = -1;
-  if (e < 0 || c < 0) {
-    atomicAdd(num_inv, 1);
-  } else if (e < E && c < C) {
-    size_t item = i / K;
-    int g = (int)(item / S);
-    slot = slot_row(e, g, c, G, E, C);
-    int prev = atomicExch(&slot_token[slot], (int)item);
+  const size_t item = i / K;
+  bool invalid;
+  const int slot = slot_of_index_pair(indices[2 * i], indices[2 * i + 1], (int)(item / S), G, E, C,
+                                      &invalid);
+  if (invalid) atomicAdd(num_inv, 1);
+  if (slot >= 0) {
+    const int prev = atomicExch(&slot_token[slot], (int)item);
     if (prev >= 0) atomicAdd(num_dup, 1);
   }
   token_slot[i] = slot;
@@ -436,11 +431,8 @@ __global__ __launch_bounds__(256) void compact_rows_kernel(
   const int slot = token_slot[i];
   int row = -1;
   if (slot >= 0) {
-    const int per_expert = G * C;
     const int g = (int)(i / per_group);
-    const int e = slot / per_expert;
-    const int c = (slot - e * per_expert) % C;
-    row = e * per_expert + prefix[(size_t)g * E + e] + c;
+    row = packed_row(slot, prefix[(size_t)g * E + slot_expert(slot, G, C)], G, C);
     if (row_token != nullptr) row_token[row] = (int)(i / K);
   }
   token_row[i] = row;
@@ -489,11 +481,8 @@ __global__ __launch_bounds__(256) void compact_rows_fused_kernel(
   const int slot = token_slot[i];
   int row = -1;
   if (slot >= 0) {
-    const int per_expert = G * C;
     const int g = (int)(i / per_group);
-    const int e = slot / per_expert;
-    const int c = (slot - e * per_expert) % C;
-    row = e * per_expert + before[g - g_lo][e] + c;
+    row = packed_row(slot, before[g - g_lo][slot_expert(slot, G, C)], G, C);
     if (row_token != nullptr) row_token[row] = (int)(i / K);
   }
   token_row[i] = row;

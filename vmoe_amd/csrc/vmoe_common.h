@@ -6,6 +6,7 @@
 #include <stdint.h>
 
 #include "vmoe_hip.h"
+#include "route_index.h"
 
 namespace vmoe {
 
@@ -61,26 +62,8 @@ __device__ __forceinline__ float gelu_erf(float x) {
 
 // Monotone map float32 -> uint32 (larger float -> larger uint); -0.0 == +0.0.
 __device__ __forceinline__ uint32_t orderable(float f) {
-  uint32_t u = __builtin_bit_cast(uint32_t, f);
-  if (u == 0x80000000u) u = 0u;
-  return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+  return orderable_bits(__builtin_bit_cast(uint32_t, f));
 }
-
-// Slot row of (expert e, group g, position c) in the (E, G*C) expert buffer.
-__device__ __forceinline__ int slot_row(int e, int g, int c, int G, int E, int C) {
-  int r;
-  if (G % E == 0) {
-    int q = G / E;
-    r = ((g % q) * E + g / q) * C + c;
-  } else {
-    r = g * C + c;
-  }
-  return e * (G * C) + r;
-}
-
-// Accelerator complex dies of the device; workgroup i is placed on die i % kNumXcd,
-// and each die has its own L2.
-constexpr int kNumXcd = 8;
 
 // s_waitcnt vmcnt(N) with lgkmcnt/expcnt left at their maxima.
 template <int N>
