@@ -234,6 +234,60 @@ static void check_index_pairs(std::mt19937& rng, int G, int S, int E, int K, int
   (void)dup;
 }
 
+
+// Stream-K share of a die's partial round (streamk_share): over die runs of 0 .. 200 tiles
+// and several k lengths, every k tile of every tile is computed exactly once by pieces of
+// at least three k tiles; the pieces of a tile wait for 0, 1, 2, ... deposits, in ascending
+// slot order, and exactly the one that waits for all the others runs the epilogue; shared,
+// the partial round costs a workgroup at most 0.85 of a tile's k tiles (plus rounding).
+static int check_streamk() {
+  int cases = 0;
+  const int slots = 32;
+  for (int sharing = 0; sharing < 2; ++sharing)
+    for (int nk : {4, 8, 12, 16, 48, 64, 80, 50})
+      for (int n = 0; n <= 200; ++n) {
+        ++cases;
+        struct Pc { int slot, kbeg, kcnt, last, waits; };
+        std::vector<std::vector<Pc>> tiles(n);
+        int maxpiece = 0;
+        for (int j = 0; j < slots; ++j) {
+          const StreamKShare s = streamk_share(n, slots, j, nk, sharing != 0);
+          CHECK(s.rounds == n / slots && s.pieces >= 0 && s.pieces <= 3, "share n=%d j=%d", n, j);
+          for (int i = 0; i < s.rounds; ++i) tiles[j + i * slots].push_back({j, 0, nk, 1, 0});
+          int work = 0;
+          for (int i = 0; i < s.pieces; ++i) {
+            const int tile = s.tile + i;
+            CHECK(tile >= s.rounds * slots && tile < n && tile - s.rounds * slots < slots && s.kbeg >= 0 &&
+                  s.kcnt >= 3 && s.kbeg + s.kcnt <= nk, "piece n=%d nk=%d j=%d", n, nk, j);
+            if (tile < 0 || tile >= n) continue;
+            tiles[tile].push_back({j, s.kbeg, s.kcnt, s.last, s.waits});
+            work += s.kcnt;
+          }
+          maxpiece = std::max(maxpiece, work);
+        }
+        for (int t = 0; t < n; ++t) {
+          auto& v = tiles[t];
+          std::sort(v.begin(), v.end(), [](const Pc& a, const Pc& b) { return a.kbeg < b.kbeg; });
+          int k = 0;
+          for (size_t a = 0; a < v.size(); ++a) {
+            CHECK(v[a].kbeg == k, "pieces consecutive n=%d nk=%d t=%d", n, nk, t);
+            k += v[a].kcnt;
+          }
+          CHECK(k == nk, "tile covered n=%d nk=%d t=%d", n, nk, t);
+          std::sort(v.begin(), v.end(), [](const Pc& a, const Pc& b) { return a.waits < b.waits; });
+          for (size_t a = 0; a < v.size(); ++a) {
+            CHECK(v[a].waits == (int)a, "deposit order n=%d nk=%d t=%d", n, nk, t);
+            if (a > 0) CHECK(v[a].slot > v[a - 1].slot, "a piece waits for lower slots only n=%d nk=%d t=%d", n, nk, t);
+            CHECK((v[a].last != 0) == (a + 1 == v.size()), "last piece n=%d nk=%d t=%d", n, nk, t);
+          }
+        }
+        const int r = n % slots;
+        if (sharing && nk % kStreamKGranule == 0 && nk >= 4 * kStreamKGranule && r > 0 && 4 * r <= 3 * slots)
+          CHECK(100 * maxpiece <= 85 * nk + 100 * kStreamKGranule, "partial round n=%d nk=%d: %d k tiles", n, nk, maxpiece);
+      }
+  return cases;
+}
+
 int main(int argc, char** argv) {
   std::mt19937 rng(argc > 1 ? (unsigned)atoi(argv[1]) : 2024u);
   const int sizes[] = {1, 2, 3, 31, 32, 33, 63, 64, 65, 127, 128, 129, 255, 256, 257, 511, 512, 513, 1000,
@@ -255,6 +309,7 @@ int main(int argc, char** argv) {
   check_routing(rng, 16, 300, 32, 2, 10, 0);
   check_routing(rng, 6, 50, 3, 1, 100, 3);
   cases += 4;
+  cases += check_streamk();
   printf("%d cases, %d failures\n", cases, failures);
   return failures == 0 ? 0 : 1;
 }

@@ -720,6 +720,92 @@ def test_expert_mlp_second_product_walks_several_tiles(K, with_bias):
     assert (to_np(out[e, n:]) == 7.0).all(), f"expert {e}"
 
 
+SHARED_ROUND_CASES = [
+    (16, 2321, 520, 1024),    # 60 tiles per die: one round, then 28 tiles shared by 32 workgroups (pieces of 12-16 k tiles)
+    (32, 768, 768, 768),      # 36 per die: 4 tiles in pieces of 4 k tiles, chains of three
+    (12, 2048, 1024, 512),    # 48 per die: 16 tiles, each halved
+    (40, 1300, 768, 1280),    # 90 per die: two rounds, then 26 tiles
+    (3, 500, 768, 1024),      # 2-3 tiles per die: no whole round, every tile in many pieces
+]
+
+
+@pytest.mark.parametrize("E,R,D,M", SHARED_ROUND_CASES)
+def test_expert_mlp_second_product_shares_partial_round(K, E, R, D, M):
+  """The tile-walking second product cuts the tiles of a die's last, partial round along k
+  among the die's workgroups; the float32 sums travel from piece to piece through memory.
+  Against the same experts computed one at a time and against a float32 restatement: a cut
+  changes the order of one float32 addition per output, so an output may differ from the
+  uncut computation by one bfloat16 step (few do); dense and over packed rows with a launch
+  plan (random row counts move the cuts); rows past a count are not written."""
+  rng = np.random.default_rng(E * 1000 + R)
+  bf = torch.bfloat16
+  x = to_dev(O.cast(rng.standard_normal((E, R, D)).astype(np.float32), O.BF16), O.BF16)
+  w0 = to_dev(O.cast(rng.standard_normal((E, D, M)).astype(np.float32) / np.sqrt(D), O.BF16), O.BF16)
+  w1 = to_dev(O.cast(rng.standard_normal((E, M, D)).astype(np.float32) / np.sqrt(M), O.BF16), O.BF16)
+  b0 = to_dev(O.cast(rng.standard_normal((E, M)).astype(np.float32) * 0.1, O.BF16), O.BF16)
+  b1 = to_dev(O.cast(rng.standard_normal((E, D)).astype(np.float32) * 0.1, O.BF16), O.BF16)
+  full = K.expert_mlp(x, w0, b0, w1, b1)
+  again = K.expert_mlp(x, w0, b0, w1, b1)
+  assert torch.equal(full, again), "two runs of the same launch differ"
+  ref = []
+  for e in range(E):                       # one expert at a time: plain 2-D products
+    h = ((x[e].float() @ w0[e].float()).to(bf).float() + b0[e].float()).to(bf)
+    h = torch.nn.functional.gelu(h.float(), approximate="tanh").to(bf)
+    ref.append(((h.float() @ w1[e].float()).to(bf).float() + b1[e].float()).to(bf))
+  ref = to_np(torch.stack(ref)).astype(np.float64)
+
+  def check(got, n_rows, what):
+    for e, n in enumerate(n_rows):
+      np.testing.assert_allclose(got[e, :n], ref[e, :n], rtol=2e-2, atol=2e-2, err_msg=f"{what} expert {e}")
+
+  got_full = to_np(full).astype(np.float64)
+  bias1 = to_np(b1).astype(np.float64)
+  check(got_full, [R] * E, "dense")
+  for trial in range(4):
+    rows = rng.integers(0, R + 1, E).astype(np.int32)
+    rows[:3] = [R, 0, 257]
+    out = torch.full_like(full, 7.0)
+    K.expert_mlp(x, w0, b0, w1, b1, out=out, rows_per_expert=to_dev(rows))
+    got = to_np(out).astype(np.float64)
+    check(got, rows, f"rows={rows.tolist()}")
+    differ = 0
+    for e, n in enumerate(rows):
+      assert (got[e, n:] == 7.0).all(), f"rows={rows.tolist()} expert {e}"
+      d = np.abs(got[e, :n] - got_full[e, :n])
+      # one step of the rounded accumulator (output minus bias), carried through the rounded sum with the bias
+      step = 2.0 ** -6 * (np.abs(got_full[e, :n]) + np.abs(bias1[e])[None, :])
+      assert (d <= step + 1e-30).all(), "more than one bfloat16 step from the dense launch"
+      differ += int((d > 0).sum())
+    assert differ <= 0.02 * max(1, int(rows.sum())) * D, f"{differ} outputs differ from the dense launch"
+
+
+@pytest.mark.parametrize("E,R,D,M", [(12, 2048, 1024, 512), (3, 500, 768, 1024)])
+def test_shared_partial_round_is_exact_on_exact_operands(K, E, R, D, M):
+  """The same cuts on operands whose every product, sum and rounding step is exact (small
+  integers, GELU the identity): whatever the order of the additions, the result must
+  equal the float64 answer bit for bit, dense and over packed rows."""
+  rng = np.random.default_rng(D + M)
+  x = rng.integers(-1, 2, (E, R, D)).astype(np.float32)
+  w0 = _sparse_signs(rng, (E, D, M), 8, axis=1)
+  b0 = np.full((E, M), 16.0, np.float32)
+  w1 = _sparse_signs(rng, (E, M, D), 4, axis=1)
+  b1 = rng.integers(-3, 4, (E, D)).astype(np.float32)
+  hidden = np.einsum("erd,edm->erm", x.astype(np.float64), w0.astype(np.float64)) + 16.0
+  want = np.einsum("erm,emd->erd", hidden, w1.astype(np.float64)) + b1[:, None, :]
+  assert hidden.min() >= 8 and hidden.max() <= 24 and np.abs(want).max() <= 128
+  dev_args = [to_dev(a, O.BF16) for a in (x, w0, b0, w1, b1)]
+  got = to_np(K.expert_mlp(*dev_args)).astype(np.float64)
+  np.testing.assert_array_equal(got, want)
+  rows = rng.integers(0, R + 1, E).astype(np.int32)
+  rows[0] = R
+  out = torch.full((E, R, D), 7.0, dtype=torch.bfloat16, device=dev())
+  K.expert_mlp(*dev_args, out=out, rows_per_expert=to_dev(rows))
+  got = to_np(out).astype(np.float64)
+  for e, n in enumerate(rows):
+    np.testing.assert_array_equal(got[e, :n], want[e, :n], err_msg=f"expert {e}")
+    assert (got[e, n:] == 7.0).all()
+
+
 @pytest.mark.parametrize("G,S,N,dtype", [(3, 50, 16, O.F32), (4, 196, 128, O.BF16), (2, 7, 300, O.BF16), (3, 196, 128, O.F32),
                           (2, 9, 96, O.BF16), (5, 33, 8, O.BF16), (2, 300, 512, O.BF16)])
 def test_soft_router_stats(K, G, S, N, dtype):

@@ -227,10 +227,15 @@ __global__ __launch_bounds__(256, 1) void operand_delivery_probe_kernel(
 
 size_t align256(size_t v) { return (v + 255) / 256 * 256; }
 
-// The second product's 256x256 tiles run one per CU, in whole rounds of kNumCu tiles:
-// 384 tiles (128 experts x 256 rows x 768 columns) take two rounds for 1.5 rounds of
-// work.  Tiles of 128x256, two per CU, waste less then; they are a few percent slower
-// per flop, so they are taken only where the rounds say 10 % or more.
+// Which kernel runs the second product (bfloat16).
+//  kDownShared: 256 x 256 tiles walked by one workgroup per CU, the last, partial round of a
+//    die shared along k (stream-K): its time follows the number of tiles, not of rounds.
+//  kDownWide: 384 x 256 tiles, eight waves; whole rounds of one tile per CU.
+//  kDownHalf: 128 x 256 tiles, two per CU (static launches the tile-walking kernels do not
+//    cover, where whole rounds of 256 x 256 tiles would waste a tenth or more).
+//  kDownPlain: 256 x 256 tiles, one workgroup per tile.
+enum DownKernel { kDownShared, kDownWide, kDownHalf, kDownPlain };
+
 bool down_prefers_half_tiles(int E, int R, int N) {
   constexpr int64_t kNumCu = 256;
   const int64_t tn = (N + 255) / 256;
@@ -241,48 +246,52 @@ bool down_prefers_half_tiles(int E, int R, int N) {
   return t_half < 0.9 * t_full;
 }
 
-// The second product takes the wide kernel (384 x 256 tiles, eight waves: about a tenth
-// faster per flop than the 256 x 256 persistent kernel) where its coarser tiles do not cost
-// more in idle compute units than that buys: both kernels run their tiles in rounds of one
-// per compute unit, and a last round that is nearly empty costs a whole tile's time.
-bool down_prefers_wide_tiles(int E, int R, int N, int Kd) {
-  if (!wide_gemm_ok(E, R, N, Kd, nullptr, nullptr, nullptr, 0)) return false;
-  constexpr int64_t kNumCu = kCusPerXcd * kNumXcd;
-  const int64_t tn = (N + 255) / 256;
-  const int64_t wide = (int64_t)E * ((R + WideCfg::BM - 1) / WideCfg::BM) * tn;
-  const int64_t square = (int64_t)E * ((R + 255) / 256) * tn;
-  const double t_wide = 1.5 * 0.92 * (double)((wide + kNumCu - 1) / kNumCu);
-  const double t_square = (double)((square + kNumCu - 1) / kNumCu);
-  return t_wide < t_square;
-}
-
 // Launch plans of the two ragged products of an MLP: geometry, bytes, one planning launch.
 struct MlpPlans {
   GemmGeom up, down;
-  bool down_wide = false;
+  DownKernel down_kernel = kDownPlain;
   int down_bm = CfgDown::BM;
   size_t up_bytes = 0, down_bytes = 0;   // 0: that product keeps the static tile order
+  size_t streamk_bytes = 0;              // exchange memory of kDownShared
 };
 
-MlpPlans mlp_plans(int E, int R, int D, int M) {
+MlpPlans mlp_plans(int E, int R, int D, int M, bool ragged) {
   MlpPlans m;
   m.up = gemm_geometry<CfgUp>(E, R, M, D);
-  m.down_wide = down_prefers_wide_tiles(E, R, D, M);
-  m.down = m.down_wide ? gemm_geometry<WideCfg>(E, R, D, M) : gemm_geometry<CfgDown>(E, R, D, M);
-  m.down_bm = m.down_wide ? WideCfg::BM : CfgDown::BM;
   // Ragged launches are planned whenever the geometry allows: with whole experts per
   // die in a static order the die that drew the fullest experts sets the time (a layer
   // with capacity factor 0.5 and a skewed router: 399 -> 267 us for the two products,
   // a third off the MoE blocks of the B/16 model with 8 experts), and on a balanced
   // layer the planned launch costs 0.3 %.
   auto bytes = [&](const GemmGeom& g) -> size_t {
-    if (!g.fast || g.ragged_slots * kNumXcd > 0x7ffffff0LL ||
+    if (!ragged || !g.fast || g.ragged_slots * kNumXcd > 0x7ffffff0LL ||
         (size_t)(E + 1) * 8 > 60000)
       return 0;
-    return align256((size_t)g.ragged_slots * kNumXcd * sizeof(int4));
+    return align256(((size_t)g.ragged_slots * kNumXcd + 1) * sizeof(int4));   // + the header entry
   };
   m.up_bytes = bytes(m.up);
+  const GemmGeom square = gemm_geometry<CfgDown>(E, R, D, M);
+  const GemmGeom wide = gemm_geometry<WideCfg>(E, R, D, M);
+  const int4* const planned = reinterpret_cast<const int4*>(&m);   // stands for "a plan exists"
+  const int32_t* const rows = ragged ? reinterpret_cast<const int32_t*>(&m) : nullptr;
+  const bool shared_ok = persistent_gemm_ok<CfgDownPersistent>(
+      E, R, D, M, rows, bytes(square) ? planned : nullptr) && M / CfgDownPersistent::BK % kStreamKGranule == 0;
+  const bool wide_ok = wide_gemm_ok(E, R, D, M, nullptr, nullptr, nullptr, 0) && (!ragged || bytes(wide));
+  constexpr double kNumCu = kCusPerXcd * kNumXcd;
+  // Time in units of one 256 x 256 tile on one CU.  The wide kernel's tile is 1.5 of them
+  // at about 0.92 of the time per flop, in whole rounds; the shared kernel pays for its
+  // tiles (the padding of the last row tile of a batch included) plus the exchange.
+  const double t_wide = 1.5 * 0.92 * std::ceil((double)wide.tiles / kNumCu);
+  const double t_shared = (double)square.tiles / kNumCu + 0.05;
+  if (shared_ok && (!wide_ok || t_shared <= t_wide)) m.down_kernel = kDownShared;
+  else if (wide_ok) m.down_kernel = kDownWide;
+  else if (!ragged && down_prefers_half_tiles(E, R, D)) m.down_kernel = kDownHalf;
+  else m.down_kernel = kDownPlain;
+  m.down = m.down_kernel == kDownWide ? wide : square;
+  m.down_bm = m.down_kernel == kDownWide ? WideCfg::BM : CfgDown::BM;
   m.down_bytes = bytes(m.down);
+  if (m.down_kernel == kDownShared)
+    m.streamk_bytes = align256(StreamKWorkspace<CfgDownPersistent>::kBytes);
   return m;
 }
 
@@ -321,9 +330,9 @@ extern "C" size_t vmoe_expert_mlp_workspace_bytes(const VmoeExpertMlpParams* p) 
   if (p == nullptr || p->E < 1 || p->R < 1 || p->D < 1 || p->M < 1) return 0;
   const size_t b = p->dtype == VMOE_BF16 ? 2 : 4;
   size_t bytes = align256((size_t)p->E * p->R * p->M * b);  // hidden activations
-  if (p->dtype == VMOE_BF16 && p->rows_per_expert != nullptr) {   // launch plans of the ragged products
-    const MlpPlans m = mlp_plans(p->E, p->R, p->D, p->M);
-    bytes += m.up_bytes + m.down_bytes;
+  if (p->dtype == VMOE_BF16) {   // launch plans of the ragged products, stream-K exchange
+    const MlpPlans m = mlp_plans(p->E, p->R, p->D, p->M, p->rows_per_expert != nullptr);
+    bytes += m.up_bytes + m.down_bytes + m.streamk_bytes;
   }
   if (p->dtype == VMOE_BF16) {
     if (p->w0t == nullptr) bytes += align256((size_t)p->E * p->D * p->M * b);
@@ -345,20 +354,27 @@ extern "C" int vmoe_expert_mlp(const VmoeExpertMlpParams* p, vmoe_stream_t strea
   ws += align256((size_t)p->E * p->R * p->M * b);
   int4* plan_up = nullptr;
   int4* plan_down = nullptr;
-  if (p->dtype == VMOE_BF16 && p->rows_per_expert != nullptr) {
-    const MlpPlans m = mlp_plans(p->E, p->R, p->D, p->M);
+  void* streamk = nullptr;
+  MlpPlans m;
+  if (p->dtype == VMOE_BF16) {
+    m = mlp_plans(p->E, p->R, p->D, p->M, p->rows_per_expert != nullptr);
     if (m.up_bytes) plan_up = reinterpret_cast<int4*>(ws);
     ws += m.up_bytes;
     if (m.down_bytes) plan_down = reinterpret_cast<int4*>(ws);
     ws += m.down_bytes;
+    if (m.streamk_bytes) streamk = ws;
+    ws += m.streamk_bytes;
     if (plan_up != nullptr || plan_down != nullptr) {
       const RaggedGeom ga{CfgUp::BM, m.up.tiles_n, m.up.panel_rows,
                           plan_up ? (int)(m.up.ragged_slots * kNumXcd) : 0, reinterpret_cast<PlanEntry*>(plan_up)};
       const RaggedGeom gb{m.down_bm, m.down.tiles_n, m.down.panel_rows,
                           plan_down ? (int)(m.down.ragged_slots * kNumXcd) : 0, reinterpret_cast<PlanEntry*>(plan_down)};
       const int n = ga.num_blocks > gb.num_blocks ? ga.num_blocks : gb.num_blocks;
+      using SK = StreamKWorkspace<CfgDownPersistent>;
       hipLaunchKernelGGL(plan_ragged_tiles_kernel, dim3((n + 255) / 256), dim3(256),
-                         (size_t)(p->E + 1) * 8, stream, p->rows_per_expert, p->E, p->R, ga, gb);
+                         (size_t)(p->E + 1) * 8, stream, p->rows_per_expert, p->E, p->R, ga, gb,
+                         streamk != nullptr ? SK::flags(streamk) : nullptr,
+                         streamk != nullptr ? SK::kFlags : 0);
     }
   }
   const bool tanh_gelu = p->gelu == VMOE_GELU_TANH;
@@ -387,22 +403,24 @@ extern "C" int vmoe_expert_mlp(const VmoeExpertMlpParams* p, vmoe_stream_t strea
                                                      p->R, p->M, p->D, stream, p->rows_per_expert,
                                                      plan_up, p->x_rows, p->num_items);
     if (rc != VMOE_OK) return rc;
-    if (p->rows_per_expert == nullptr && down_prefers_half_tiles(p->E, p->R, p->D))
-      return launch_gemm_bf16<CfgUp, kEpiBias>((const bf16_t*)hidden, (const bf16_t*)w1t,
-                                              (const bf16_t*)p->b1, (bf16_t*)p->out, p->E, p->R,
-                                              p->D, p->M, stream, nullptr, nullptr);
-    if (down_prefers_wide_tiles(p->E, p->R, p->D, p->M) &&
-        (p->rows_per_expert == nullptr || plan_down != nullptr))
-      return launch_gemm_bf16_wide<kEpiBias>((const bf16_t*)hidden, (const bf16_t*)w1t,
-                                             (const bf16_t*)p->b1, (bf16_t*)p->out, p->E, p->R,
-                                             p->D, p->M, stream, plan_down);
-    if (persistent_gemm_ok<CfgDownPersistent>(p->E, p->R, p->D, p->M, p->rows_per_expert, plan_down))
-      return launch_gemm_bf16_persistent<CfgDownPersistent, kEpiBias>(
-          (const bf16_t*)hidden, (const bf16_t*)w1t, (const bf16_t*)p->b1, (bf16_t*)p->out, p->E,
-          p->R, p->D, p->M, stream, plan_down);
-    return launch_gemm_bf16<CfgDown, kEpiBias>((const bf16_t*)hidden, (const bf16_t*)w1t,
-                                              (const bf16_t*)p->b1, (bf16_t*)p->out, p->E, p->R,
-                                              p->D, p->M, stream, p->rows_per_expert, plan_down);
+    switch (m.down_kernel) {
+      case kDownShared:
+        return launch_gemm_bf16_persistent<CfgDownPersistent, kEpiBias>(
+            (const bf16_t*)hidden, (const bf16_t*)w1t, (const bf16_t*)p->b1, (bf16_t*)p->out, p->E,
+            p->R, p->D, p->M, stream, plan_down, streamk, /*flags_clear=*/plan_down != nullptr);
+      case kDownWide:
+        return launch_gemm_bf16_wide<kEpiBias>((const bf16_t*)hidden, (const bf16_t*)w1t,
+                                               (const bf16_t*)p->b1, (bf16_t*)p->out, p->E, p->R,
+                                               p->D, p->M, stream, plan_down);
+      case kDownHalf:
+        return launch_gemm_bf16<CfgUp, kEpiBias>((const bf16_t*)hidden, (const bf16_t*)w1t,
+                                                (const bf16_t*)p->b1, (bf16_t*)p->out, p->E, p->R,
+                                                p->D, p->M, stream, nullptr, nullptr);
+      default:
+        return launch_gemm_bf16<CfgDown, kEpiBias>((const bf16_t*)hidden, (const bf16_t*)w1t,
+                                                  (const bf16_t*)p->b1, (bf16_t*)p->out, p->E, p->R,
+                                                  p->D, p->M, stream, p->rows_per_expert, plan_down);
+    }
   }
   if (tanh_gelu)
     rc = launch_gemm_f32<kEpiBiasGeluTanh>((const float*)p->x, (const float*)p->w0,
@@ -427,9 +445,7 @@ extern "C" int vmoe_operand_delivery_probe(const void* a, const void* bt, int32_
   const GemmGeom g = gemm_geometry<CfgDown>(batch, rows, n, kd);
   if (!g.fast) return VMOE_E_UNSUPPORTED;    // kd % 32 != 0 or an operand beyond 32-bit offsets
   if (g.tiles > 0x7ffffff0LL) return VMOE_E_OVERFLOW;
-  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(operand_delivery_probe_kernel),
-                                     hipFuncAttributeMaxDynamicSharedMemorySize,
-                                     (int)CfgDown::kLdsBytes);
+  hipError_t e = allow_dynamic_lds(reinterpret_cast<const void*>(operand_delivery_probe_kernel), CfgDown::kLdsBytes);
   if (e != hipSuccess) return (int)e;
   hipLaunchKernelGGL(operand_delivery_probe_kernel, dim3((unsigned)g.tiles_per_xcd * kNumXcd),
                      dim3(CfgDown::kThreads), CfgDown::kLdsBytes, as_stream(stream),

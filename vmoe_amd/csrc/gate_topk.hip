@@ -441,8 +441,7 @@ int launch_gate(const VmoeGateTopkParams* p, hipStream_t stream) {
   int blocks = (num_tiles + waves - 1) / waves;
   if (blocks > 1024) blocks = 1024;
   auto run = [&](auto kern) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    hipError_t e = allow_dynamic_lds(reinterpret_cast<const void*>(kern), lds);
     if (e != hipSuccess) return (int)e;
     hipLaunchKernelGGL(kern, dim3(blocks), dim3(waves * kWave), lds, stream,
                        (const T*)p->x, (const T*)p->w, p->logit_bias, (T*)p->gates, p->logits,

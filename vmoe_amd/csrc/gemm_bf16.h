@@ -38,6 +38,7 @@
 #define VMOE_GEMM_BF16_H_
 
 #include <cmath>
+#include <cstdlib>
 #include <type_traits>
 #include "vmoe_common.h"
 
@@ -232,8 +233,12 @@ __device__ __forceinline__ void plan_one(const RaggedGeom& g, const int32_t* til
   g.plan[i] = plan_entry(g, tile_prefix, rows, batch, R, i);
 }
 
+// Entry num_blocks of a plan (one past its last workgroup) holds the number of live row
+// tiles, from which a tile-walking kernel derives the length of its die's run; the
+// planning launch also clears the `clear_count` flags of the stream-K exchange.
 __global__ __launch_bounds__(256) void plan_ragged_tiles_kernel(
-    const int32_t* __restrict__ rows, int batch, int R, RaggedGeom ga, RaggedGeom gb) {
+    const int32_t* __restrict__ rows, int batch, int R, RaggedGeom ga, RaggedGeom gb,
+    int32_t* __restrict__ clear, int clear_count) {
   extern __shared__ int32_t tile_prefix[];      // 2 x (batch + 1): live row tiles before batch b
   __shared__ int32_t wsum[2][4];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -272,6 +277,16 @@ __global__ __launch_bounds__(256) void plan_ragged_tiles_kernel(
   const int i = blockIdx.x * 256 + tid;
   plan_one(ga, pa, rows, batch, R, i);
   plan_one(gb, pb, rows, batch, R, i);
+  if (blockIdx.x == 0) {
+    if (tid == 0 && ga.plan != nullptr) ga.plan[ga.num_blocks] = PlanEntry{pa[batch], 0, 0, 0};
+    if (tid == 0 && gb.plan != nullptr) gb.plan[gb.num_blocks] = PlanEntry{pb[batch], 0, 0, 0};
+    for (int c = tid; c < clear_count; c += 256) clear[c] = 0;
+  }
+}
+
+__global__ __launch_bounds__(256) void clear_i32_kernel(int32_t* __restrict__ p, int n) {
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  if (i < n) p[i] = 0;
 }
 
 // Fast path: Kd % BK == 0.  Global tiles go straight into LDS
@@ -547,7 +562,8 @@ template <typename Cfg, int EPI, bool HAS_BIAS>
 __global__ __launch_bounds__(Cfg::kThreads, 1) void gemm_bf16_persistent_kernel(
     const bf16_t* __restrict__ A, const bf16_t* __restrict__ Bt, const bf16_t* __restrict__ bias,
     bf16_t* __restrict__ C, int R, int N, int Kd, int tiles_m, int tiles_n, int num_tiles,
-    int tiles_per_xcd, int panel_rows, const int4* __restrict__ plan, int plan_blocks) {
+    int tiles_per_xcd, int panel_rows, const int4* __restrict__ plan, int plan_blocks,
+    float* __restrict__ sk_partials, int32_t* __restrict__ sk_flags) {
 #if defined(__HIP_DEVICE_COMPILE__)   // buffer-resource builtins exist in the device pass only
   extern __shared__ __align__(1024) unsigned char smem[];
   constexpr int BM = Cfg::BM, BN = Cfg::BN, BK = Cfg::BK;
@@ -566,21 +582,54 @@ __global__ __launch_bounds__(Cfg::kThreads, 1) void gemm_bf16_persistent_kernel(
   const int lrow = lane / CPR;
   const int chunk = (lane % CPR) ^ (((wave * RPL + lrow) >> Cfg::kSwzShift) & (CPR - 1));
 
-  // Tile i of this workgroup: every kCusPerXcd-th entry of its die's run (the plan of a
-  // ragged launch, else the static order of map_tile), so that the tiles in flight on a
-  // die at any time are neighbours in that order.
+  // Work of this workgroup: every kCusPerXcd-th entry of its die's run (the plan of a ragged
+  // launch, else the static order of map_tile), so that the tiles in flight on a die at
+  // any time are neighbours in that order, plus its share of the die's last, partial
+  // round (stream-K pieces, see streamk_share).
+  const int nk = Kd / BK;      // at least 2 * NS
+  int die_tiles;
+  if (plan != nullptr) {
+    const int total = plan[plan_blocks].x;               // live row tiles of all batches
+    const int share = (total + kNumXcd - 1) / kNumXcd;
+    die_tiles = max(0, min(xcd * share + share, total) - xcd * share) * tiles_n;
+  } else {
+    die_tiles = max(0, min(tiles_per_xcd, num_tiles - xcd * tiles_per_xcd));
+  }
+  die_tiles = __builtin_amdgcn_readfirstlane(die_tiles);
+  constexpr bool kCanShare = kStreamKGranule >= 2 * NS - 1;   // a piece covers the ring's fill and drain
+  const StreamKShare share_ =
+      streamk_share(die_tiles, kCusPerXcd, slot, nk, kCanShare && sk_partials != nullptr);
+  const int num_items = share_.rounds + share_.pieces;
   struct TileCtx {
     int b, row0, col0, live;
+    int kbeg, kcnt;       // k tiles of this item
+    int shared;           // index of the tile among the die's shared ones (its sums and counter)
+    int waits;            // deposits of the tile's other pieces that this item waits for and adds
+    int leaves_sums;      // 1: the item deposits its sums; 0: it runs the epilogue
     uint32_t a[Cfg::kAIssues], bo[Cfg::kBIssues];
   };
   auto setup_tile = [&](int i, TileCtx& t) -> bool {
-    const int s_ = slot + i * kCusPerXcd;
+    if (i >= num_items) return false;
+    int s_ = slot + i * kCusPerXcd;
+    t.kbeg = 0;
+    t.kcnt = nk;
+    t.shared = 0;
+    t.waits = 0;
+    t.leaves_sums = 0;
+    if (i >= share_.rounds) {
+      s_ = share_.tile + (i - share_.rounds);
+      t.kbeg = share_.kbeg;
+      t.kcnt = share_.kcnt;
+      t.shared = s_ - share_.rounds * kCusPerXcd;
+      t.waits = share_.waits;
+      t.leaves_sums = share_.last ? 0 : 1;
+    }
     int tile_m, tile_n;
     if (plan != nullptr) {
       const int vblock = s_ * kNumXcd + xcd;
       if (vblock >= plan_blocks) return false;
       const int4 mine = plan[vblock];
-      if (mine.x < 0) return false;      // a die's run is dense from slot 0: nothing follows
+      if (mine.x < 0) return false;
       t.b = mine.x;
       tile_m = mine.y;
       tile_n = mine.z;
@@ -598,8 +647,16 @@ __global__ __launch_bounds__(Cfg::kThreads, 1) void gemm_bf16_persistent_kernel(
       tile_m = panel * panel_rows + in_panel - tile_n * rows_here;
       t.live = R;
     }
-    t.row0 = tile_m * BM;
-    t.col0 = tile_n * BN;
+    // (wave-uniform values, kept in scalar registers)
+    t.b = __builtin_amdgcn_readfirstlane(t.b);
+    t.live = __builtin_amdgcn_readfirstlane(t.live);
+    t.row0 = __builtin_amdgcn_readfirstlane(tile_m * BM);
+    t.col0 = __builtin_amdgcn_readfirstlane(tile_n * BN);
+    t.kbeg = __builtin_amdgcn_readfirstlane(t.kbeg);
+    t.kcnt = __builtin_amdgcn_readfirstlane(t.kcnt);
+    t.shared = __builtin_amdgcn_readfirstlane(t.shared);
+    t.waits = __builtin_amdgcn_readfirstlane(t.waits);
+    t.leaves_sums = __builtin_amdgcn_readfirstlane(t.leaves_sums);
 #pragma unroll
     for (int u = 0; u < Cfg::kAIssues; ++u) {
       const int r = (u * Cfg::kWaves + wave) * RPL + lrow;
@@ -700,31 +757,78 @@ __global__ __launch_bounds__(Cfg::kThreads, 1) void gemm_bf16_persistent_kernel(
     stage = next_stage; \
   } while (0)
 
-  const int nk = Kd / BK;      // at least 2 * NS
   TileCtx cur, nxt;
   if (!setup_tile(0, cur)) return;
 #pragma unroll
-  for (int t = 0; t < NS; ++t) load_ktile(cur, t, t * BK);
+  for (int t = 0; t < NS; ++t) load_ktile(cur, t, (cur.kbeg + t) * BK);
   wait_vmcnt<0>();
   raw_barrier();
   load_frags(0, 0, 0);
   int stage = 0;
   constexpr int OLD = PersistentLds<Cfg>::kOutLd;
   bf16_t* so = reinterpret_cast<bf16_t*>(smem + PersistentLds<Cfg>::kRing) + (size_t)wave * 32 * OLD;
+  // Sums in memory: one tile per workgroup, in the order of the accumulator registers (a
+  // wave's store or load covers 1 KB of consecutive memory).
+  constexpr size_t kTileVecs = (size_t)BM * BN / 4;
+  const __amdgpu_buffer_rsrc_t sums_rsrc = __builtin_amdgcn_make_buffer_rsrc(sk_partials, 0, -1, 0x00020000);
+  const int vec0 = wave * FM * FN * 4 * 64 + lane;
   for (int ti = 0;; ++ti) {
     const bool has_next = setup_tile(ti + 1, nxt);
     if (!has_next) nxt = cur;   // the last tile requests its own first k tiles again: in bounds, never read
     uint2 bias_pk[Cfg::TN / 8];
     load_bias<Cfg::TN>(bias_pk, bias, cur.b, N, cur.col0 + wn * Cfg::TN, lane);
+    const int kc = __builtin_amdgcn_readfirstlane(cur.kcnt);
+    // (without the bounds the compiler plans for trip counts that cannot occur and spills)
+    __builtin_assume(kc >= 2 * NS && kc <= nk);
+    const int kb = __builtin_amdgcn_readfirstlane(cur.kbeg), nkb = __builtin_amdgcn_readfirstlane(nxt.kbeg);
 #pragma unroll
-    for (int kt = 0; kt < NS - 1; ++kt) VMOE_PERSISTENT_K_ITERATION(cur, (kt + NS) * BK, true);
-    for (int kt = NS - 1; kt < nk - NS; ++kt) VMOE_PERSISTENT_K_ITERATION(cur, (kt + NS) * BK, false);
-    for (int kt = nk - NS; kt < nk; ++kt) VMOE_PERSISTENT_K_ITERATION(nxt, (kt + NS - nk) * BK, false);
+    for (int kt = 0; kt < NS - 1; ++kt) VMOE_PERSISTENT_K_ITERATION(cur, (kb + kt + NS) * BK, true);
+    for (int kt = NS - 1; kt < kc - NS; ++kt) VMOE_PERSISTENT_K_ITERATION(cur, (kb + kt + NS) * BK, false);
+    for (int kt = kc - NS; kt < kc; ++kt) VMOE_PERSISTENT_K_ITERATION(nxt, (nkb + kt + NS - kc) * BK, false);
     // The first NS k tiles of the next tile are complete before the staging region is
     // touched (no load that writes LDS is pending while the output is staged), and the
     // first NS - 1 iterations of the next tile need no wait of their own.
     wait_vmcnt<0>();
     mfma_result_fence();
+    // A piece of a shared tile that is not the first to finish adds the sums deposited so
+    // far, chunk by chunk in the epilogue below, the loads kAhead chunks ahead of their
+    // use.  The other pieces were computed at the same time as this one, in workgroups
+    // with lower indices (placed before this one), so the wait is short; it is bounded
+    // all the same (sk_flags[kCusPerXcd * kNumXcd] counts the waits that gave up).
+    const int waits = __builtin_amdgcn_readfirstlane(cur.waits);
+    const bool adds_sums = waits > 0;
+    typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+    constexpr int kAhead = 8, kChunks = FM * FN * 4;
+    // The sums are written through to memory and read past the caches (sc0 sc1 on both
+    // sides): producer and consumer need no cache-wide write-back or invalidate (a
+    // device-scope fence here writes back the whole L2, once per wave), and the exchange
+    // does not depend on both workgroups sharing a die's L2.
+    constexpr int kSumsAux = 1 | 16;
+    const int shared_index = xcd * kCusPerXcd + __builtin_amdgcn_readfirstlane(cur.shared);
+    const int sums_base = shared_index * (int)(kTileVecs * 16);
+    u32x4_t ahead[kAhead];
+    if (adds_sums) {
+      if (tid == 0) {
+        const int32_t* f = sk_flags + shared_index;
+        int spins = 0;
+        while (__hip_atomic_load(f, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < waits) {
+          __builtin_amdgcn_s_sleep(16);
+          if (++spins > (1 << 22)) {
+            atomicAdd(sk_flags + kCusPerXcd * kNumXcd, 1);
+            break;
+          }
+        }
+      }
+      __syncthreads();
+#pragma unroll
+      for (int c = 0; c < kAhead; ++c)
+        ahead[c] = __builtin_amdgcn_raw_buffer_load_b128(sums_rsrc, vec0 * 16, sums_base + c * 1024, kSumsAux);
+    }
+    const bool leaves_sums = __builtin_amdgcn_readfirstlane(cur.leaves_sums) != 0;
+    // An item that ends inside its tile leaves its sums for the piece that continues it: the
+    // epilogue below stores each group of four as float32 on its way (one code path for the
+    // accumulators) and no row of the output.
+    const int live_rows = leaves_sums ? 0 : cur.live;
     bf16_t* Cb = C + (size_t)cur.b * R * N;
     const int wrow0 = cur.row0 + wm * Cfg::TM, wcol0 = cur.col0 + wn * Cfg::TN;
     constexpr int SC = PersistentLds<Cfg>::kStageCols;   // columns staged at a time
@@ -744,13 +848,35 @@ __global__ __launch_bounds__(Cfg::kThreads, 1) void gemm_bf16_persistent_kernel(
             const int cl = j * 32 - c0 + q * 8 + h * 4;
             const uint2 bp = bias_pk[j * 4 + q];
             const float bv[4] = {bf_lo(bp.x), bf_hi(bp.x), bf_lo(bp.y), bf_hi(bp.y)};
-            const uint32_t p0 = epilogue_pair<EPI, HAS_BIAS>(acc[i][j][q * 4], acc[i][j][q * 4 + 1], bv[0], bv[1]);
-            const uint32_t p1 = epilogue_pair<EPI, HAS_BIAS>(acc[i][j][q * 4 + 2], acc[i][j][q * 4 + 3], bv[2], bv[3]);
-            *reinterpret_cast<uint2*>(so + m * OLD + cl) = make_uint2(p0, p1);
+            // (read here and nowhere earlier: hoisted above the branches below, the reads
+            // of all 64 groups would need 256 registers at once)
+            floatx4 v;
 #pragma unroll
-            for (int v = 0; v < 4; ++v) acc[i][j][q * 4 + v] = 0.f;
+            for (int e = 0; e < 4; ++e) {
+              float x;
+              asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(x) : "a"(acc[i][j][q * 4 + e]));
+              v[e] = x;
+            }
+            const int cidx = (i * FN + j) * 4 + q;
+            if (adds_sums) {      // uniform over the workgroup
+              v += __builtin_bit_cast(floatx4, ahead[cidx % kAhead]);
+              if (cidx + kAhead < kChunks)
+                ahead[cidx % kAhead] = __builtin_amdgcn_raw_buffer_load_b128(
+                    sums_rsrc, vec0 * 16, sums_base + (cidx + kAhead) * 1024, kSumsAux);
+            }
+            if (leaves_sums) {    // uniform over the workgroup
+              __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4_t, v), sums_rsrc,
+                                                     vec0 * 16, sums_base + cidx * 1024, kSumsAux);
+            } else {
+              const uint32_t p0 = epilogue_pair<EPI, HAS_BIAS>(v[0], v[1], bv[0], bv[1]);
+              const uint32_t p1 = epilogue_pair<EPI, HAS_BIAS>(v[2], v[3], bv[2], bv[3]);
+              *reinterpret_cast<uint2*>(so + m * OLD + cl) = make_uint2(p0, p1);
+            }
+#pragma unroll
+            for (int e = 0; e < 4; ++e) acc[i][j][q * 4 + e] = 0.f;
           }
         }
+        if (leaves_sums) continue;
         // A wave reads back only what it wrote (its LDS operations complete in order).
 #pragma unroll
         for (int r0 = 0; r0 < 32; r0 += kRowsPerPass) {
@@ -758,7 +884,7 @@ __global__ __launch_bounds__(Cfg::kThreads, 1) void gemm_bf16_persistent_kernel(
           const int row = wrow0 + i * 32 + rl;
           const int col = wcol0 + c0 + oc;
           const uint4 v = *reinterpret_cast<const uint4*>(so + rl * OLD + oc);
-          if (row < cur.live && col + 8 <= N) {
+          if (row < live_rows && col + 8 <= N) {
             if constexpr (EPI != kEpiBias) {   // hidden layer: streaming store, as in store_tile
               typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
               __builtin_nontemporal_store(__builtin_bit_cast(u32x4_t, v),
@@ -769,6 +895,12 @@ __global__ __launch_bounds__(Cfg::kThreads, 1) void gemm_bf16_persistent_kernel(
           }
         }
       }
+    }
+    if (leaves_sums) {
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");    // every wave's sums have been written through
+      __syncthreads();
+      if (tid == 0)
+        __hip_atomic_store(sk_flags + shared_index, waits + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
     if (!has_next) break;
     cur = nxt;
@@ -916,9 +1048,7 @@ int launch_gemm_bf16(const bf16_t* A, const bf16_t* Bt, const bf16_t* bias, bf16
   if (g.tiles > 0x7ffffff0LL) return VMOE_E_OVERFLOW;
   const unsigned blocks = (unsigned)(plan != nullptr ? g.ragged_slots : g.tiles_per_xcd) * kNumXcd;
   auto kern = gemm_bf16_kernel<Cfg, EPI>;
-  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                     hipFuncAttributeMaxDynamicSharedMemorySize,
-                                     (int)Cfg::kLdsBytes);
+  hipError_t e = allow_dynamic_lds(reinterpret_cast<const void*>(kern), Cfg::kLdsBytes);
   if (e != hipSuccess) return (int)e;
   hipLaunchKernelGGL(kern, dim3(blocks), dim3(Cfg::kThreads), Cfg::kLdsBytes, stream, A, Bt, bias,
                      C, R, N, Kd, g.tiles_m, g.tiles_n, (int)g.tiles, g.tiles_per_xcd, g.panel_rows,
@@ -938,24 +1068,52 @@ bool persistent_gemm_ok(int batch, int R, int N, int Kd, const int32_t* rows, co
          g.tiles <= 0x7ffffff0LL && (rows == nullptr || plan != nullptr);
 }
 
+// Memory of the stream-K exchange of a tile-walking launch: one tile of float32 partial
+// sums per workgroup, then one flag per workgroup and the counter of abandoned waits.
+template <typename Cfg>
+struct StreamKWorkspace {
+  static constexpr int kBlocks = kCusPerXcd * kNumXcd;
+  static constexpr size_t kPartialBytes = (size_t)kBlocks * Cfg::BM * Cfg::BN * sizeof(float);
+  static constexpr int kFlags = kBlocks + 1;
+  static constexpr size_t kBytes = kPartialBytes + (size_t)(kFlags + 63) / 64 * 256;
+  static float* partials(void* ws) { return static_cast<float*>(ws); }
+  static int32_t* flags(void* ws) {
+    return reinterpret_cast<int32_t*>(static_cast<unsigned char*>(ws) + kPartialBytes);
+  }
+};
+
 // Launches the persistent kernel; the caller checked persistent_gemm_ok.  `plan`, if
 // given, was filled by plan_ragged_tiles_kernel for gemm_geometry<Cfg> (BM, BN and
-// workgroups per CU decide it, not the number of stages).
+// workgroups per CU decide it, not the number of stages).  `streamk`, if given, is
+// StreamKWorkspace<Cfg>::kBytes of memory: the die's last, partial round is then shared
+// along k.  `flags_clear`: the planning launch has already cleared its flags.
 template <typename Cfg, int EPI>
 int launch_gemm_bf16_persistent(const bf16_t* A, const bf16_t* Bt, const bf16_t* bias, bf16_t* C,
                                 int batch, int R, int N, int Kd, hipStream_t stream,
-                                const int4* plan = nullptr) {
+                                const int4* plan = nullptr, void* streamk = nullptr,
+                                bool flags_clear = false) {
   const GemmGeom g = gemm_geometry<Cfg>(batch, R, N, Kd);
   auto kern = bias != nullptr ? gemm_bf16_persistent_kernel<Cfg, EPI, true>
                               : gemm_bf16_persistent_kernel<Cfg, EPI, false>;
-  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                     hipFuncAttributeMaxDynamicSharedMemorySize,
-                                     (int)PersistentLds<Cfg>::kBytes);
+  hipError_t e = allow_dynamic_lds(reinterpret_cast<const void*>(kern), PersistentLds<Cfg>::kBytes);
   if (e != hipSuccess) return (int)e;
+  using SK = StreamKWorkspace<Cfg>;
+  float* partials = nullptr;
+  int32_t* flags = nullptr;
+  // (VMOE_WHOLE_TILES=1 in the environment keeps every tile whole: the switch behind the
+  // before / after figures of the shared round)
+  if (streamk != nullptr && getenv("VMOE_WHOLE_TILES") == nullptr) {
+    partials = SK::partials(streamk);
+    flags = SK::flags(streamk);
+    if (!flags_clear)
+      hipLaunchKernelGGL(clear_i32_kernel, dim3((SK::kFlags + 255) / 256), dim3(256), 0, stream,
+                         flags, SK::kFlags);
+  }
   const int plan_blocks = plan != nullptr ? (int)(g.ragged_slots * kNumXcd) : 0;
   hipLaunchKernelGGL(kern, dim3(kCusPerXcd * kNumXcd), dim3(Cfg::kThreads),
                      PersistentLds<Cfg>::kBytes, stream, A, Bt, bias, C, R, N, Kd, g.tiles_m,
-                     g.tiles_n, (int)g.tiles, g.tiles_per_xcd, g.panel_rows, plan, plan_blocks);
+                     g.tiles_n, (int)g.tiles, g.tiles_per_xcd, g.panel_rows, plan, plan_blocks,
+                     partials, flags);
   return launch_status();
 }
 

@@ -305,8 +305,7 @@ int launch_gemm_bf16_wide(const bf16_t* A, const bf16_t* Bt, const bf16_t* bias,
     kern = bias != nullptr ? gemm_bf16_wide_kernel<Cfg, EPI, true, true> : gemm_bf16_wide_kernel<Cfg, EPI, false, true>;
   else
     kern = bias != nullptr ? gemm_bf16_wide_kernel<Cfg, EPI, true, false> : gemm_bf16_wide_kernel<Cfg, EPI, false, false>;
-  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)Cfg::kLdsBytes);
+  hipError_t e = allow_dynamic_lds(reinterpret_cast<const void*>(kern), Cfg::kLdsBytes);
   if (e != hipSuccess) return (int)e;
   const int plan_blocks = plan != nullptr ? (int)(g.ragged_slots * kNumXcd) : 0;
   hipLaunchKernelGGL(kern, dim3(kCusPerXcd * kNumXcd), dim3(Cfg::kThreads), Cfg::kLdsBytes,

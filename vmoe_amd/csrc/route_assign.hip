@@ -528,8 +528,7 @@ static int launch_route_assign(const VmoeRouteAssignParams* p, const VmoeRouterM
   }
   if (lds > 160 * 1024) return VMOE_E_UNSUPPORTED;
   auto launch = [&](auto kern, auto... extra) -> int {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    hipError_t e = allow_dynamic_lds(reinterpret_cast<const void*>(kern), lds);
     if (e != hipSuccess) return (int)e;
     hipLaunchKernelGGL(kern, dim3(m != nullptr ? 2 * p->G : p->G), dim3(kRouteThreads), lds,
                        as_stream(stream), p->topk_val, p->topk_idx, p->indices, p->token_slot,
@@ -623,8 +622,7 @@ extern "C" int vmoe_top_items_per_expert(const VmoeTopItemsParams* p, vmoe_strea
   if (lds > 160 * 1024) return VMOE_E_UNSUPPORTED;
   dim3 grid(p->E, p->G);
   auto launch = [&](auto kern, auto* gates) -> int {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    hipError_t e = allow_dynamic_lds(reinterpret_cast<const void*>(kern), lds);
     if (e != hipSuccess) return (int)e;
     hipLaunchKernelGGL(kern, grid, dim3(kRouteThreads), lds, as_stream(stream), gates, p->indices,
                        p->token_slot, p->slot_token, p->weights, p->sel_minmax, p->G, p->S, p->E,

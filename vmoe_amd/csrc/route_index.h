@@ -139,5 +139,101 @@ VMOE_HD PlanEntry plan_entry(const RaggedGeom& g, const int32_t* tile_prefix, co
   return out;
 }
 
+// ---- stream-K share of a die's last, partial round (see gemm_bf16_persistent_kernel) ----
+// A die's run of n tiles is walked by `slots` workgroups, one tile per workgroup and round:
+// q = n / slots whole rounds, and r = n % slots tiles that would leave slots - r workgroups
+// idle for a whole tile's time.  Those r tiles are cut along k instead (at multiples of
+// kStreamKGranule k tiles), after the whole rounds, and always so that the workgroups
+// that run side by side compute the same k range of neighbouring tiles: the operands of
+// neighbours then meet in the die's L2, as they do in a whole round (pieces at staggered
+// k positions run at the rate of memory, which costs more than the idle workgroups did).
+//  * r <= slots / 2: every tile in p = min(slots / r, 4) equal pieces; piece c of tile t
+//    goes to slot c * r + t, so slots c * r .. c * r + r - 1 form a group in step.
+//  * r <= 3/4 slots: each of the first slots - r workgroups computes the tails of
+//    g = ceil(r / (slots - r)) <= 3 consecutive tiles, one after the other, and slot
+//    slots - r + t the head of tile t; the cut is placed so that both kinds finish
+//    together (a tail costs its k tiles and the store of its sums, a head its k tiles
+//    and an epilogue: about 0.04 and 0.1 of a tile).
+//  * more: the tiles run whole (a cut would save less than it costs).
+// The pieces of a tile exchange float32 sums through one tile of memory and a counter per
+// shared tile: a piece waits until the counter says that `waits` pieces have deposited,
+// adds the sums found there to its own, and either deposits the result (counter + 1) or,
+// as the tile's last piece, turns it into the output.  A piece only ever waits for
+// workgroups with lower indices (placed before its own), and those never wait for it.
+constexpr int kStreamKGranule = 4;
+struct StreamKShare {
+  int rounds;       // whole rounds: tiles slot + i * slots of the die's run, i < rounds
+  // After the rounds: `pieces` pieces of consecutive run entries tile, tile + 1, ..., all
+  // over k tiles kbeg .. kbeg + kcnt - 1, computed one after the other.
+  int pieces;
+  int tile, kbeg, kcnt;
+  int waits;        // deposits a piece waits for and adds (0: none)
+  int last;         // 1: the pieces run the epilogue; 0: they deposit their sums
+};
+VMOE_HD int streamk_cut(int U, int c, int parts) {     // k tile where part c of `parts` begins
+  return (int)(((long long)U * c + parts / 2) / parts) * kStreamKGranule;
+}
+VMOE_HD StreamKShare streamk_share(int n, int slots, int j, int nk, bool sharing) {
+  StreamKShare s{};
+  s.rounds = n / slots;
+  const int r = n - s.rounds * slots;
+  const int U = nk / kStreamKGranule;
+  const int base = s.rounds * slots;
+  if (r == 0) return s;
+  const bool cut = sharing && nk % kStreamKGranule == 0;
+  if (cut && 2 * r <= slots) {
+    int parts = slots / r;
+    if (parts > 4) parts = 4;
+    if (parts > U) parts = U;
+    if (parts >= 2) {
+      const int c = j / r, t = j - c * r;
+      if (c < parts) {
+        const int k0 = streamk_cut(U, c, parts), k1 = streamk_cut(U, c + 1, parts);
+        s.pieces = 1;
+        s.tile = base + t;
+        s.kbeg = k0;
+        s.kcnt = k1 - k0;
+        s.waits = c;
+        s.last = c + 1 == parts ? 1 : 0;
+      }
+      return s;
+    }
+  } else if (cut && 4 * r <= 3 * slots && U >= 4) {
+    const int others = slots - r;
+    const int g = (r + others - 1) / others;           // 2 or 3 tails per tail workgroup
+    // head + 0.1 = g * (tail + 0.04), head + tail = 1 (in tiles)
+    int head = (int)((U * (104LL * g - 10) + 50 * (g + 1)) / (100 * (g + 1)));
+    if (head > U - 1) head = U - 1;
+    if (head < 1) head = 1;
+    const int k1 = head * kStreamKGranule;
+    if (j >= others) {
+      s.pieces = 1;
+      s.tile = base + (j - others);
+      s.kbeg = 0;
+      s.kcnt = k1;
+      s.waits = 1;
+      s.last = 1;
+    } else {
+      const int t = g * j;
+      s.pieces = t < r ? plan_min(g, r - t) : 0;
+      s.tile = base + t;
+      s.kbeg = k1;
+      s.kcnt = nk - k1;
+      s.waits = 0;
+      s.last = 0;
+    }
+    return s;
+  }
+  if (j < r) {     // the tiles of the partial round run whole
+    s.pieces = 1;
+    s.tile = base + j;
+    s.kbeg = 0;
+    s.kcnt = nk;
+    s.waits = 0;
+    s.last = 1;
+  }
+  return s;
+}
+
 }  // namespace vmoe
 #endif  // VMOE_ROUTE_INDEX_H_

@@ -766,8 +766,7 @@ extern "C" int vmoe_soft_route(const VmoeSoftRouteParams* p, vmoe_stream_t strea
                 : p->D == 512 ? soft_route_bf16_kernel<16>
                 : p->D == 384 ? soft_route_bf16_kernel<12>
                               : soft_route_bf16_kernel<8>;
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)L.total);
+    hipError_t e = allow_dynamic_lds(reinterpret_cast<const void*>(kern), L.total);
     if (e != hipSuccess) return (int)e;
     hipLaunchKernelGGL(kern, dim3(p->G), dim3(kSrThreads), L.total, stream, (const bf16_t*)p->x,
                        (const bf16_t*)p->workspace, (bf16_t*)p->dispatch_w, (bf16_t*)p->combine_w,
@@ -779,8 +778,7 @@ extern "C" int vmoe_soft_route(const VmoeSoftRouteParams* p, vmoe_stream_t strea
       hipLaunchKernelGGL(soft_prep_mu_kernel<bf16_t>, dim3(p->N), dim3(256), 0, stream,
                          (const bf16_t*)p->mu, (bf16_t*)p->workspace, p->scale, !scale_x, p->D, p->N);
     auto kern = soft_route_kernel<bf16_t>;
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    hipError_t e = allow_dynamic_lds(reinterpret_cast<const void*>(kern), lds);
     if (e != hipSuccess) return (int)e;
     hipLaunchKernelGGL(kern, dim3(p->G), dim3(256), lds, stream, (const bf16_t*)p->x,
                        (const bf16_t*)p->workspace, (bf16_t*)p->dispatch_w, (bf16_t*)p->combine_w,
@@ -790,8 +788,7 @@ extern "C" int vmoe_soft_route(const VmoeSoftRouteParams* p, vmoe_stream_t strea
       hipLaunchKernelGGL(soft_prep_mu_kernel<float>, dim3(p->N), dim3(256), 0, stream,
                          (const float*)p->mu, (float*)p->workspace, p->scale, !scale_x, p->D, p->N);
     auto kern = soft_route_kernel<float>;
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    hipError_t e = allow_dynamic_lds(reinterpret_cast<const void*>(kern), lds);
     if (e != hipSuccess) return (int)e;
     hipLaunchKernelGGL(kern, dim3(p->G), dim3(256), lds, stream, (const float*)p->x,
                        (const float*)p->workspace, (float*)p->dispatch_w, (float*)p->combine_w,

@@ -440,8 +440,7 @@ extern "C" int vmoe_attention(const VmoeAttentionParams* p, vmoe_stream_t stream
   const size_t lds = (size_t)sk_pad * kKRow * 2 + (size_t)kHd * (sk_pad + 8) * 2 +
                      (size_t)waves * 32 * kStageRow * 2;
   if (lds > 160 * 1024) return VMOE_E_UNSUPPORTED;
-  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(attention_bf16_kernel),
-                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+  hipError_t e = allow_dynamic_lds(reinterpret_cast<const void*>(attention_bf16_kernel), lds);
   if (e != hipSuccess) return (int)e;
   const float scale_log2e = p->scale * 1.4426950408889634f;
   hipLaunchKernelGGL(attention_bf16_kernel, dim3((unsigned)(p->B * p->H)), dim3(waves * 64), lds,

@@ -5,6 +5,10 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <map>
+#include <mutex>
+#include <utility>
+
 #include "vmoe_hip.h"
 #include "route_index.h"
 
@@ -99,6 +103,23 @@ inline hipStream_t as_stream(vmoe_stream_t s) { return reinterpret_cast<hipStrea
 inline int launch_status() {
   hipError_t err = hipGetLastError();
   return err == hipSuccess ? VMOE_OK : (int)err;
+}
+
+// Raises a kernel's limit of dynamic LDS.  hipFuncSetAttribute takes a lock and walks the
+// runtime's tables on the host, so it is called once per (kernel, device) and limit: a
+// launch whose size the recorded limit already covers skips it.
+inline hipError_t allow_dynamic_lds(const void* kern, size_t bytes) {
+  static std::mutex mu;
+  static std::map<std::pair<const void*, int>, size_t> limit;
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return e;
+  std::lock_guard<std::mutex> lock(mu);
+  size_t& have = limit[std::make_pair(kern, dev)];
+  if (bytes <= have) return hipSuccess;
+  e = hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+  if (e == hipSuccess) have = bytes;
+  return e;
 }
 
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
