@@ -9,6 +9,7 @@ synthetic tokens already resident in HBM.  Prints ONE JSON line.
 from __future__ import annotations
 
 import argparse
+import gc
 import json
 import os
 import sys
@@ -174,13 +175,33 @@ def soft_main(args):
   # the other stages from a second, fully instrumented pass.
   sink = _hip.TimingSink(pairs=args.steps * 2, only=("vmoe_expert_mlp",))
   _hip.set_timing_sink(sink)
+  # One event per step boundary (the per-step times whose median is reported) and one
+  # host time stamp per step (which step, if any, kept the host waiting).
+  marks = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps + 1)]
+  for ev in marks:
+    ev.record()
+  torch.cuda.synchronize()
+  host_t = [0.0] * (args.steps + 1)
+  # A full collection of Python's cyclic garbage collector walks every object that torch and
+  # numpy have created (tens of milliseconds) and fires after a fixed number of allocations,
+  # i.e. at a fixed step: it runs now, and not inside the timed loop.
+  gc.collect()
+  gc.disable()
   t0 = time.perf_counter()
+  marks[0].record()
+  host_t[0] = t0
   for i in range(args.steps):
     step(i)
+    marks[i + 1].record()
+    host_t[i + 1] = time.perf_counter()
   t_enqueued = time.perf_counter()
   torch.cuda.synchronize()
   t1 = time.perf_counter()
-  ms = (t1 - t0) * 1e3 / args.steps
+  gc.enable()
+  step_ms = [marks[i].elapsed_time(marks[i + 1]) for i in range(args.steps)]
+  host_step_ms = [(host_t[i + 1] - host_t[i]) * 1e3 for i in range(args.steps)]
+  ms = float(np.median(step_ms))
+  wall_ms = (t1 - t0) * 1e3 / args.steps
   host_ms = (t_enqueued - t0) * 1e3 / args.steps
   full = _hip.TimingSink(pairs=args.steps * CALLS_PER_STEP)
   _hip.set_timing_sink(full)
@@ -209,7 +230,14 @@ def soft_main(args):
       "roofline": {"bound": "hbm", "kernel": "gemm_bf16_kernel", "achieved": achieved,
                    "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": achieved / PEAK_HBM_GBS,
                    "traffic": None, "launch_ms": mlp_ms / 2, "bytes_per_layer": bytes_mlp},
-      "stage_ms": stage_ms, "host_enqueue_ms_per_step": host_ms, "cpu_baseline": None,
+      "stage_ms": stage_ms, "host_enqueue_ms_per_step": host_ms, "wall_ms_per_step": wall_ms,
+      "ms_per_step_note": ("ms_per_step and value: median of the K per-step times between events "
+                           "recorded at the step boundaries; wall_ms_per_step: host clock around the "
+                           "same K steps, synchronised on both sides, divided by K"),
+      "step_ms_min_max": [float(min(step_ms)), float(max(step_ms))],
+      "slowest_step": {"gpu": int(np.argmax(step_ms)), "gpu_ms": float(max(step_ms)),
+                       "host": int(np.argmax(host_step_ms)), "host_ms": float(max(host_step_ms))},
+      "cpu_baseline": None,
   }
   if not args.no_cpu_baseline:
     # The oracle's Soft MoE layer on the first groups of the same batch (the expert
@@ -465,6 +493,8 @@ def main():
   for ev in marks:
     ev.record()
   torch.cuda.synchronize()
+  gc.collect()       # (a full collection fires after a fixed number of allocations and takes
+  gc.disable()       # tens of milliseconds: it runs here, not inside the timed loop)
   t0 = time.perf_counter()
   marks[0].record()
   for i in range(args.steps):
@@ -473,6 +503,7 @@ def main():
   t_enqueued = time.perf_counter()      # the host has issued everything; the GPU is still running
   torch.cuda.synchronize()
   t1 = time.perf_counter()
+  gc.enable()
   _hip.set_timing_sink(None)
   wall_ms_per_step = (t1 - t0) * 1e3 / args.steps
   step_ms = [marks[i].elapsed_time(marks[i + 1]) for i in range(args.steps)]

@@ -392,22 +392,27 @@ extern "C" int vmoe_expert_mlp(const VmoeExpertMlpParams* p, vmoe_stream_t strea
       if (rc != VMOE_OK) return rc;
       w1t = ws;
     }
+    // The counters of the second product's stream-K exchange are cleared by the planning
+    // launch, or else by the first product's.
+    using SK = StreamKWorkspace<CfgDownPersistent>;
+    const bool planned = plan_up != nullptr || plan_down != nullptr;
+    int32_t* clear = streamk != nullptr && !planned ? SK::flags(streamk) : nullptr;
     if (tanh_gelu)
       rc = launch_gemm_bf16<CfgUp, kEpiBiasGeluTanh>((const bf16_t*)p->x, (const bf16_t*)w0t,
                                                       (const bf16_t*)p->b0, (bf16_t*)hidden, p->E,
                                                       p->R, p->M, p->D, stream, p->rows_per_expert,
-                                                      plan_up, p->x_rows, p->num_items);
+                                                      plan_up, p->x_rows, p->num_items, clear, SK::kFlags);
     else
       rc = launch_gemm_bf16<CfgUp, kEpiBiasGeluErf>((const bf16_t*)p->x, (const bf16_t*)w0t,
                                                      (const bf16_t*)p->b0, (bf16_t*)hidden, p->E,
                                                      p->R, p->M, p->D, stream, p->rows_per_expert,
-                                                     plan_up, p->x_rows, p->num_items);
+                                                     plan_up, p->x_rows, p->num_items, clear, SK::kFlags);
     if (rc != VMOE_OK) return rc;
     switch (m.down_kernel) {
       case kDownShared:
         return launch_gemm_bf16_persistent<CfgDownPersistent, kEpiBias>(
             (const bf16_t*)hidden, (const bf16_t*)w1t, (const bf16_t*)p->b1, (bf16_t*)p->out, p->E,
-            p->R, p->D, p->M, stream, plan_down, streamk, /*flags_clear=*/plan_down != nullptr);
+            p->R, p->D, p->M, stream, plan_down, streamk, /*flags_clear=*/true);
       case kDownWide:
         return launch_gemm_bf16_wide<kEpiBias>((const bf16_t*)hidden, (const bf16_t*)w1t,
                                                (const bf16_t*)p->b1, (bf16_t*)p->out, p->E, p->R,

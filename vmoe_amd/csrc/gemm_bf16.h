@@ -298,13 +298,18 @@ __global__ __launch_bounds__(Cfg::kThreads, Cfg::kBlocksPerCu) void gemm_bf16_ke
     const bf16_t* __restrict__ A, const bf16_t* __restrict__ Bt, const bf16_t* __restrict__ bias,
     bf16_t* __restrict__ C, int R, int N, int Kd, int tiles_m, int tiles_n, int num_tiles,
     int tiles_per_xcd, int panel_rows, const int32_t* __restrict__ rows,
-    const int4* __restrict__ plan, const int32_t* __restrict__ a_rows, int a_items) {
+    const int4* __restrict__ plan, const int32_t* __restrict__ a_rows, int a_items,
+    int32_t* __restrict__ clear, int clear_count) {
 #if defined(__HIP_DEVICE_COMPILE__)   // buffer-resource builtins exist in the device pass only
   extern __shared__ __align__(1024) unsigned char smem[];
   constexpr int BM = Cfg::BM, BN = Cfg::BN, BK = Cfg::BK;
   constexpr int FM = Cfg::FM, FN = Cfg::FN;
   constexpr int RB = Cfg::kRowBytes;
   const int tid = threadIdx.x;
+  // (a few words that the next launch on the stream wants cleared: the counters of its
+  // stream-K exchange, which would otherwise cost a launch of their own)
+  if (clear != nullptr && blockIdx.x == 0)
+    for (int c = tid; c < clear_count; c += Cfg::kThreads) clear[c] = 0;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave / Cfg::WN, wn = wave % Cfg::WN;
@@ -1032,8 +1037,13 @@ template <typename Cfg, int EPI>
 int launch_gemm_bf16(const bf16_t* A, const bf16_t* Bt, const bf16_t* bias, bf16_t* C, int batch,
                      int R, int N, int Kd, hipStream_t stream, const int32_t* rows = nullptr,
                      const int4* plan = nullptr, const int32_t* a_rows = nullptr,
-                     long long a_items = 0) {
+                     long long a_items = 0, int32_t* clear = nullptr, int clear_count = 0) {
   const GemmGeom g = gemm_geometry<Cfg>(batch, R, N, Kd);
+  if (clear != nullptr && !g.fast) {
+    hipLaunchKernelGGL(clear_i32_kernel, dim3((clear_count + 255) / 256), dim3(256), 0, stream, clear,
+                       clear_count);
+    clear = nullptr;
+  }
   if (a_rows != nullptr && (!g.fast || rows == nullptr ||
                             (unsigned long long)a_items * Kd * 2 >= (1ull << 32)))
     return VMOE_E_UNSUPPORTED;     // the gathering load exists in the LDS-DMA kernel only
@@ -1052,7 +1062,7 @@ int launch_gemm_bf16(const bf16_t* A, const bf16_t* Bt, const bf16_t* bias, bf16
   if (e != hipSuccess) return (int)e;
   hipLaunchKernelGGL(kern, dim3(blocks), dim3(Cfg::kThreads), Cfg::kLdsBytes, stream, A, Bt, bias,
                      C, R, N, Kd, g.tiles_m, g.tiles_n, (int)g.tiles, g.tiles_per_xcd, g.panel_rows,
-                     rows, plan, a_rows, (int)a_items);
+                     rows, plan, a_rows, (int)a_items, clear, clear_count);
   return launch_status();
 }
 
