@@ -36,9 +36,19 @@ PEAK_HBM_GBS = 8000.0
 # HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc runs
 # (FETCH_SIZE + WRITE_SIZE, scaled by a copy kernel of known size); None until measured.
 MEASURED_TRAFFIC_BYTES = {
-    # mean of the two GEMM launches of a layer: (638 + 565 + 1098 + 141) / 2 MiB;
-    # FETCH_SIZE x 2.0, WRITE_SIZE x 1.0 (copy-kernel calibration).
-    "vmoe_b16_layer_E32_k2_bpr": 1.280e9,
+    # mean of the two GEMM launches of a layer: (634 + 565 + 1102 + 181) / 2 MiB;
+    # FETCH_SIZE x 2.0, WRITE_SIZE x 1.0 (copy-kernel calibration);
+    # profiles/hbm_traffic__vmoe_b16_layer.md.
+    "vmoe_b16_layer_E32_k2_bpr": 1.301e9,
+}
+# Share of the launch during which the matrix cores are busy (SQ_VALU_MFMA_BUSY_CYCLES over
+# GRBM_GUI_ACTIVE x 1 024 SIMDs), from the rocprofv3 --pmc runs of this command summarised in
+# profiles/mfma_util__vmoe_b16_layer.md: counters cannot be read from inside the run.
+MEASURED_MFMA_BUSY = {
+    "vmoe_b16_layer_E32_k2_bpr": {
+        "first_product": 0.418, "second_product": 0.443, "vendor_gemm_second_product_shape": 0.535,
+        "register_resident_mfma_loop": 0.904,
+        "source": "profiles/mfma_util__vmoe_b16_layer.md (rocprofv3 --pmc, same command, 5 steps)"},
 }
 
 
@@ -542,6 +552,7 @@ def main():
               "kernel": "gemm_bf16_kernel (first product) / gemm_bf16_persistent_kernel (second product)" if b == 2 else "gemm_f32_kernel",
               "achieved": achieved_tflops, "peak": peak, "unit": "TFLOP/s",
               "frac": achieved_tflops / peak, "traffic": MEASURED_TRAFFIC_BYTES.get(cfg.name),
+              "mfma_busy": MEASURED_MFMA_BUSY.get(cfg.name),
               "launch_ms": gemm_ms, "flops_per_launch": flops_per_launch, "kept_rows": kept,
               "buffer_rows": E * G * C}
 

@@ -299,6 +299,12 @@ int vmoe_densify(const VmoeDensifyParams* p, vmoe_stream_t stream);
  * bf16 needs the kernels in K-contiguous order: pass w0t (E,M,D) / w1t (E,D,M)
  * made once by vmoe_pack_expert_weights; if they are null the call packs
  * w0/w1 into `workspace` first (extra HBM pass).  D % 8 == 0 and M % 8 == 0.
+ * `workspace` holds the hidden activations (E, R, M), the launch plans of a call with
+ * rows_per_expert and, for bf16, 64 MB through which the second product's workgroups
+ * exchange float32 partial sums when the tiles of a last, partial round are cut along k
+ * (results are deterministic; such a cut reorders one float32 addition per output, so
+ * outputs of a call with rows_per_expert may differ from those of a call without by one
+ * bfloat16 rounding step).  Calls that share a workspace must not overlap.
  */
 typedef struct {
   const void* x;    /* (E, R, D) dtype */

@@ -69,15 +69,18 @@ def test_hand_assembled_files(tmp_path):
   arr = np.arange(12, dtype=np.float32).reshape(4, 3)
   info_a = pk((pk(((4, 3), "float32", False, {})), (snd((0, 2), (0, 3)), snd((2, 4), (0, 3))), (0, 1)))
   info_b = pk((pk(((2,), "bfloat16", False, {})), (snd((0, 2)),), (1,)))
+  info_s = pk((pk(((), "int32", False, {})), (snd(),), (0,)))          # a scalar leaf: no slices
   index = msgpack.packb({"shard_count": 2, "version": "20220622",
-                         "index": {"w": msgpack.ExtType(8, info_a), "b": msgpack.ExtType(8, info_b)}})
+                         "index": {"w": msgpack.ExtType(8, info_a), "b": msgpack.ExtType(8, info_b),
+                                   "step": msgpack.ExtType(8, info_s)}})
   nd = lambda a, name=None: msgpack.ExtType(1, pk((a.shape, name or a.dtype.name, a.tobytes())))
   magic = "__msgpack_array_chunk_a87ca2__"
   bf = np.asarray([0x3F80, 0xC000], np.uint16)          # 1.0, -2.0
-  # leaf ids follow sorted keys: b = 0, w = 1
-  shard0 = msgpack.packb({magic: True, "1": [[[nd(arr[:2].reshape(-1))], msgpack.ExtType(6, snd((0, 2), (0, 3)))]]})
+  # leaf ids follow sorted keys: b = 0, step = 1, w = 2
+  shard0 = msgpack.packb({magic: True, "2": [[[nd(arr[:2].reshape(-1))], msgpack.ExtType(6, snd((0, 2), (0, 3)))]],
+                          "1": [[[nd(np.asarray([7], np.int32))], msgpack.ExtType(6, snd())]]})
   shard1 = msgpack.packb({magic: True,
-                          "1": [[[nd(arr[2:].reshape(-1)[:4]), nd(arr[2:].reshape(-1)[4:])],
+                          "2": [[[nd(arr[2:].reshape(-1)[:4]), nd(arr[2:].reshape(-1)[4:])],
                                  msgpack.ExtType(6, snd((2, 4), (0, 3)))]],
                           "0": [[[nd(bf, "bfloat16")], msgpack.ExtType(6, snd((0, 2)))]]})
   prefix = str(tmp_path / "c")
@@ -87,6 +90,7 @@ def test_hand_assembled_files(tmp_path):
   out = C.restore_checkpoint(prefix)
   np.testing.assert_array_equal(out["w"], arr)
   np.testing.assert_array_equal(out["b"], np.asarray([1.0, -2.0], np.float32))
+  assert np.asarray(out["step"]).shape == () and int(out["step"]) == 7
 
 
 def test_errors(tmp_path):
