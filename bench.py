@@ -21,9 +21,13 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 if ROOT not in sys.path:
   sys.path.insert(0, ROOT)
 
-# Steps run before the warm-up so that no one-time initialisation (first launches,
-# memory pools, event objects) falls into the warm-up or the timed steps.
-INIT_STEPS = 10
+# Steps run first so that no one-time initialisation (first launches, memory pools) falls
+# into the warm-up or the timed steps; the timing events are created after them.
+COLD_STEPS = 3
+# Steps run right in front of the W warm-up steps, after everything that leaves the GPU idle
+# (creating events, a garbage collection): an idle GPU takes about 25 ms of work to get its
+# clocks back, more than a few warm-up steps of a millisecond each.
+INIT_STEPS = 30
 # Entry-point calls of one layer step, rounded up: their timing events are created
 # before the timed region, which then only records them.
 CALLS_PER_STEP = 12
@@ -178,13 +182,13 @@ def soft_main(args):
     return mlp.apply(mvars, dispatcher, xs[i % 4])
 
   _hip.set_timing_sink({})
-  for i in range(INIT_STEPS + args.warmup):
+  for i in range(COLD_STEPS):
     step(i)
   torch.cuda.synchronize()
   # As in main(): events only around the dominant entry point inside the timed region,
   # the other stages from a second, fully instrumented pass.
   sink = _hip.TimingSink(pairs=args.steps * 2, only=("vmoe_expert_mlp",))
-  _hip.set_timing_sink(sink)
+  warm_sink = _hip.TimingSink(pairs=(INIT_STEPS + args.warmup) * 2, only=("vmoe_expert_mlp",))
   # One event per step boundary (the per-step times whose median is reported) and one
   # host time stamp per step (which step, if any, kept the host waiting).
   marks = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps + 1)]
@@ -194,9 +198,15 @@ def soft_main(args):
   host_t = [0.0] * (args.steps + 1)
   # A full collection of Python's cyclic garbage collector walks every object that torch and
   # numpy have created (tens of milliseconds) and fires after a fixed number of allocations,
-  # i.e. at a fixed step: it runs now, and not inside the timed loop.
+  # i.e. at a fixed step: it runs now, before the warm-up (an idle GPU takes several steps
+  # to get its clocks back), and stays off until the timed loop is over.
   gc.collect()
   gc.disable()
+  _hip.set_timing_sink(warm_sink)
+  for i in range(INIT_STEPS + args.warmup):
+    step(i)
+  torch.cuda.synchronize()
+  _hip.set_timing_sink(sink)
   t0 = time.perf_counter()
   marks[0].record()
   host_t[0] = t0
@@ -245,6 +255,7 @@ def soft_main(args):
                            "recorded at the step boundaries; wall_ms_per_step: host clock around the "
                            "same K steps, synchronised on both sides, divided by K"),
       "step_ms_min_max": [float(min(step_ms)), float(max(step_ms))],
+      "step_ms_p10_p50_p90": [float(np.percentile(step_ms, q)) for q in (10, 50, 90)],
       "slowest_step": {"gpu": int(np.argmax(step_ms)), "gpu_ms": float(max(step_ms)),
                        "host": int(np.argmax(host_step_ms)), "host_ms": float(max(host_step_ms))},
       "cpu_baseline": None,
@@ -485,10 +496,7 @@ def main():
   # Untimed: one-time costs (code objects, allocator pools, timing events) and
   # then the W warm-up steps, run exactly as the timed steps are.
   _hip.set_timing_sink({})
-  for i in range(INIT_STEPS):
-    out, metrics = step(i)
-  torch.cuda.synchronize()
-  for i in range(args.warmup):
+  for i in range(COLD_STEPS):
     out, metrics = step(i)
   torch.cuda.synchronize()
 
@@ -497,14 +505,25 @@ def main():
   # cost the layer about 6 % of its throughput; the other stages are timed in a second,
   # fully instrumented pass of the same K steps right after.
   sink = _hip.TimingSink(pairs=args.steps * 2, only=("vmoe_expert_mlp",))
-  _hip.set_timing_sink(sink)
+  warm_sink = _hip.TimingSink(pairs=(INIT_STEPS + args.warmup) * 2, only=("vmoe_expert_mlp",))
   # One event per step boundary: the per-step times whose median is reported.
   marks = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps + 1)]
   for ev in marks:
     ev.record()
   torch.cuda.synchronize()
-  gc.collect()       # (a full collection fires after a fixed number of allocations and takes
-  gc.disable()       # tens of milliseconds: it runs here, not inside the timed loop)
+  # A full collection of Python's cyclic garbage collector fires after a fixed number of
+  # allocations and takes tens of milliseconds: it runs here and stays off until the timed
+  # loop is over.  Everything that leaves the GPU idle (creating events, this collection)
+  # comes before the initialisation and warm-up steps, never between them and the timed
+  # steps: after 40 ms of idling the clocks take some twenty steps (25 ms) to come back,
+  # which is what the INIT_STEPS in front of the W warm-up steps are for.
+  gc.collect()
+  gc.disable()
+  _hip.set_timing_sink(warm_sink)
+  for i in range(INIT_STEPS + args.warmup):
+    out, metrics = step(i)
+  torch.cuda.synchronize()
+  _hip.set_timing_sink(sink)
   t0 = time.perf_counter()
   marks[0].record()
   for i in range(args.steps):
@@ -716,6 +735,9 @@ def main():
                            "recorded at the step boundaries; wall_ms_per_step: host clock around "
                            "the same K steps, synchronised on both sides, divided by K"),
       "step_ms_min_max": [float(min(step_ms)), float(max(step_ms))],
+      "step_ms_p10_p50_p90": [float(np.percentile(step_ms, q)) for q in (10, 50, 90)],
+      "step_ms_first_five": [float(v) for v in step_ms[:5]],
+      "untimed_steps_before_warmup": COLD_STEPS + INIT_STEPS,
   }
   if not args.no_cpu_baseline:
     params_np = {
