@@ -50,7 +50,7 @@ MEASURED_TRAFFIC_BYTES = {
 # profiles/mfma_util__vmoe_b16_layer.md: counters cannot be read from inside the run.
 MEASURED_MFMA_BUSY = {
     "vmoe_b16_layer_E32_k2_bpr": {
-        "first_product": 0.418, "second_product": 0.443, "vendor_gemm_second_product_shape": 0.535,
+        "first_product": 0.415, "second_product": 0.434, "vendor_gemm_second_product_shape": 0.535,
         "register_resident_mfma_loop": 0.904,
         "source": "profiles/mfma_util__vmoe_b16_layer.md (rocprofv3 --pmc, same command, 5 steps)"},
 }
