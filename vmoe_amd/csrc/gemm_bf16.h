@@ -367,9 +367,9 @@ __global__ __launch_bounds__(Cfg::kThreads, Cfg::kBlocksPerCu) void gemm_bf16_ke
     int r = (i * Cfg::kWaves + wave) * RPL + lrow;
     b_goff[i] = (uint32_t)min(col0 + r, N - 1) * (uint32_t)Kd * 2u + chunk * 16;
   }
-  // The DMA loads of a k tile are issued in two halves (A rows, then B rows), one
-  // under the MFMAs of each k slice: a wave sustains about one 1 KB DMA load per
-  // 80 clocks, so they must be spread out or the wave stalls behind them.
+  // A wave sustains about one 1 KB DMA load per 80 clocks, and a load that cannot be issued
+  // (address FIFO full) holds up the MFMAs behind it: the loads of a k tile are spread out,
+  // A rows under the second slice of one iteration, B rows under the first slice of the next.
   // Buffer addressing: the descriptor carries the operand's base, the lane's byte
   // offset is loop-invariant and the advance along k is a scalar, so a DMA load
   // needs no per-iteration address arithmetic and moves one address dword per
@@ -480,16 +480,56 @@ __global__ __launch_bounds__(Cfg::kThreads, Cfg::kBlocksPerCu) void gemm_bf16_ke
   // kt + NS go out right behind it, under the MFMAs of the second k slice.
   const int nk = Kd / BK;
   const int pro = min(NS, nk);
+  // Long k (more k tiles than stages): the B loads of a k tile go out one slice after its
+  // A loads, under the first slice of the following iteration, so that a wave's DMA
+  // requests come in two short bursts per iteration instead of one long one.
+  const bool split = nk > NS;
 #pragma unroll
   for (int t = 0; t < NS; ++t)
     if (t < pro) {
       load_a(t, t * BK);
-      load_b(t, t * BK);
+      if (!split || t + 1 < NS) load_b(t, t * BK);
     }
   wait_tile(pro - 1);
   raw_barrier();
   load_frags(0, 0, 0);
   int stage = 0;
+  if (split) {
+    const int steady = nk - NS;
+    int prev_stage = NS - 1;
+    for (int kt = 0; kt < steady; ++kt) {
+      const int next_stage = stage + 1 == NS ? 0 : stage + 1;
+      load_frags(1, stage, 1);
+      load_b(prev_stage, (kt + NS - 1) * BK);
+      mfma_slice(0);
+      slice_schedule(std::integral_constant<int, Cfg::kBIssues>{});
+      wait_vmcnt<(PD - 1) * L>();
+      wait_lgkmcnt0();
+      raw_barrier();
+      load_frags(0, next_stage, 0);
+      load_a(stage, (kt + NS) * BK);
+      mfma_slice(1);
+      slice_schedule(std::integral_constant<int, Cfg::kAIssues>{});
+      prev_stage = stage;
+      stage = next_stage;
+    }
+    for (int kt = steady; kt < nk; ++kt) {
+      const int next_stage = stage + 1 == NS ? 0 : stage + 1;
+      load_frags(1, stage, 1);
+      if (kt == steady) load_b(prev_stage, (nk - 1) * BK);
+      mfma_slice(0);
+      slice_schedule(std::integral_constant<int, 0>{});
+      if (kt + 1 < nk) {
+        wait_tile(nk - 2 - kt);
+        wait_lgkmcnt0();
+        raw_barrier();
+        load_frags(0, next_stage, 0);
+      }
+      mfma_slice(1);
+      slice_schedule(std::integral_constant<int, 0>{});
+      stage = next_stage;
+    }
+  } else {
   // Steady state: the body is one basic block (no branches), so that the
   // scheduling hints hold and the fragment reads / DMA loads really are issued
   // under the MFMAs.  Tile kt + 1 has landed when only the PD - 1 tiles issued
@@ -526,6 +566,7 @@ __global__ __launch_bounds__(Cfg::kThreads, Cfg::kBlocksPerCu) void gemm_bf16_ke
     mfma_slice(1);
     slice_schedule(std::integral_constant<int, 0>{});
     stage = next_stage;
+  }
   }
   wait_lgkmcnt0();
   __syncthreads();   // all waves are done with the operand tiles: LDS is reused below
