@@ -785,6 +785,47 @@ __global__ __launch_bounds__(Cfg::kThreads, 1) void gemm_bf16_persistent_kernel(
   // One k tile.  WAITED = the k tile needed next is known to be complete (every wave
   // drained its loads before the last output was staged, or in the prologue).  A macro:
   // as a lambda taking the tile by reference the offsets end up in scratch memory.
+  auto load_ktile_a = [&](const TileCtx& t, int stage, int k0) {
+    unsigned char* s = smem + stage * Cfg::kStageBytes;
+#pragma unroll
+    for (int u = 0; u < Cfg::kAIssues; ++u)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(a_rsrc, (lds_ptr_t)(s + (u * Cfg::kWaves + wave) * RPL * RB),
+                                               16, t.a[u], k0 * 2, 0, 0);
+  };
+  auto load_ktile_b = [&](const TileCtx& t, int stage, int k0) {
+    unsigned char* s = smem + stage * Cfg::kStageBytes;
+#pragma unroll
+    for (int u = 0; u < Cfg::kBIssues; ++u)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(
+          b_rsrc, (lds_ptr_t)(s + BM * RB + (u * Cfg::kWaves + wave) * RPL * RB), 16, t.bo[u], k0 * 2,
+          0, 0);
+  };
+  // Two stages: the A rows of k tile kt + 2 go out under the last slice of iteration kt (the
+  // barrier in front of it frees their stage), its B rows under the first slice of
+  // iteration kt + 1, into the same stage: two short bursts of DMA requests instead of one
+  // long one (a request that cannot be issued holds up the MFMAs behind it; second product of the
+  // headline layer: -17 us in six alternating A/B pairs).
+#define VMOE_PERSISTENT_K_ITERATION_SPLIT(SRC, K0, PSRC, PK0) do { \
+    const int next_stage = stage ^ 1; \
+    load_frags(1, stage, 1); \
+    load_ktile_b(PSRC, next_stage, (PK0)); \
+    mfma_slice(0); \
+    slice_schedule(std::integral_constant<int, Cfg::kBIssues>{}); \
+    _Pragma("unroll") \
+    for (int ks = 1; ks + 1 < KS; ++ks) { \
+      load_frags((ks + 1) & 1, stage, ks + 1); \
+      mfma_slice(ks & 1); \
+      slice_schedule(std::integral_constant<int, 0>{}); \
+    } \
+    wait_vmcnt<0>(); \
+    wait_lgkmcnt0(); \
+    raw_barrier(); \
+    load_frags(0, next_stage, 0); \
+    load_ktile_a(SRC, stage, (K0)); \
+    mfma_slice((KS - 1) & 1); \
+    slice_schedule(std::integral_constant<int, Cfg::kAIssues>{}); \
+    stage = next_stage; \
+  } while (0)
 #define VMOE_PERSISTENT_K_ITERATION(SRC, K0, WAITED) do { \
     const int next_stage = stage + 1 == NS ? 0 : stage + 1; \
     _Pragma("unroll") \
@@ -827,10 +868,17 @@ __global__ __launch_bounds__(Cfg::kThreads, 1) void gemm_bf16_persistent_kernel(
     // (without the bounds the compiler plans for trip counts that cannot occur and spills)
     __builtin_assume(kc >= 2 * NS && kc <= nk);
     const int kb = __builtin_amdgcn_readfirstlane(cur.kbeg), nkb = __builtin_amdgcn_readfirstlane(nxt.kbeg);
+    if constexpr (NS == 2 && KS >= 3) {
+      for (int kt = 0; kt < kc - NS; ++kt)
+        VMOE_PERSISTENT_K_ITERATION_SPLIT(cur, (kb + kt + NS) * BK, cur, (kb + kt + NS - 1) * BK);
+      VMOE_PERSISTENT_K_ITERATION_SPLIT(nxt, nkb * BK, cur, (kb + kc - 1) * BK);
+      VMOE_PERSISTENT_K_ITERATION_SPLIT(nxt, (nkb + 1) * BK, nxt, nkb * BK);
+    } else {
 #pragma unroll
-    for (int kt = 0; kt < NS - 1; ++kt) VMOE_PERSISTENT_K_ITERATION(cur, (kb + kt + NS) * BK, true);
-    for (int kt = NS - 1; kt < kc - NS; ++kt) VMOE_PERSISTENT_K_ITERATION(cur, (kb + kt + NS) * BK, false);
-    for (int kt = kc - NS; kt < kc; ++kt) VMOE_PERSISTENT_K_ITERATION(nxt, (nkb + kt + NS - kc) * BK, false);
+      for (int kt = 0; kt < NS - 1; ++kt) VMOE_PERSISTENT_K_ITERATION(cur, (kb + kt + NS) * BK, true);
+      for (int kt = NS - 1; kt < kc - NS; ++kt) VMOE_PERSISTENT_K_ITERATION(cur, (kb + kt + NS) * BK, false);
+      for (int kt = kc - NS; kt < kc; ++kt) VMOE_PERSISTENT_K_ITERATION(nxt, (nkb + kt + NS - kc) * BK, false);
+    }
     // The first NS k tiles of the next tile are complete before the staging region is
     // touched (no load that writes LDS is pending while the output is staged), and the
     // first NS - 1 iterations of the next tile need no wait of their own.
@@ -953,6 +1001,7 @@ __global__ __launch_bounds__(Cfg::kThreads, 1) void gemm_bf16_persistent_kernel(
   }
   wait_vmcnt<0>();
 #undef VMOE_PERSISTENT_K_ITERATION
+#undef VMOE_PERSISTENT_K_ITERATION_SPLIT
 #endif
 }
 
