@@ -590,15 +590,25 @@ constexpr int kCusPerXcd = 32;
 
 template <typename Cfg>
 struct PersistentLds {
-  static constexpr size_t kRing = (size_t)Cfg::NSTAGE * Cfg::kStageBytes;
+  // Two stages of 64-wide k tiles: the A rows get a ring of three slots and the B rows one
+  // of two (all of the 160 KB of LDS), so that a k tile's A rows can be requested two
+  // iterations ahead and stay in flight across the barrier of the iteration in between.
+  static constexpr bool kDeepA = Cfg::NSTAGE == 2 && Cfg::BK == 64 &&
+                                 (size_t)(3 * Cfg::BM + 2 * Cfg::BN) * Cfg::kRowBytes <= 160 * 1024;
+  static constexpr size_t kABytes = (size_t)Cfg::BM * Cfg::kRowBytes;
+  static constexpr size_t kBBytes = (size_t)Cfg::BN * Cfg::kRowBytes;
+  static constexpr size_t kRing = kDeepA ? 3 * kABytes + 2 * kBBytes : (size_t)Cfg::NSTAGE * Cfg::kStageBytes;
   // The output is staged 32 rows per wave at a time, over the whole width of the wave tile
-  // where the ring leaves room for that, else in two halves.
+  // where the ring leaves room for that, else in two halves.  With the deep A ring the
+  // staging region is the A slot that the finished tile's last k tile has just left.
   static constexpr size_t kFullStaging = (size_t)Cfg::kWaves * 32 * (Cfg::TN + 8) * sizeof(bf16_t);
-  static constexpr int kStageCols = kRing + kFullStaging <= 160 * 1024 ? Cfg::TN : Cfg::TN / 2;
+  static constexpr size_t kRoom = kDeepA ? kABytes : 160 * 1024 - kRing;
+  static constexpr int kStageCols = kFullStaging <= kRoom ? Cfg::TN : Cfg::TN / 2;
   static constexpr int kOutLd = kStageCols + 8;
   static constexpr size_t kStaging = (size_t)Cfg::kWaves * 32 * kOutLd * sizeof(bf16_t);
-  static constexpr size_t kBytes = kRing + kStaging;
+  static constexpr size_t kBytes = kDeepA ? kRing : kRing + kStaging;
   static_assert(kStageCols % 32 == 0, "staging covers whole MFMA tiles");
+  static_assert(kStaging <= kRoom, "staging region");
   static_assert(kBytes <= 160 * 1024, "LDS budget");
 };
 
@@ -782,50 +792,82 @@ __global__ __launch_bounds__(Cfg::kThreads, 1) void gemm_bf16_persistent_kernel(
     }
     __builtin_amdgcn_sched_barrier(0);
   };
-  // One k tile.  WAITED = the k tile needed next is known to be complete (every wave
-  // drained its loads before the last output was staged, or in the prologue).  A macro:
-  // as a lambda taking the tile by reference the offsets end up in scratch memory.
-  auto load_ktile_a = [&](const TileCtx& t, int stage, int k0) {
-    unsigned char* s = smem + stage * Cfg::kStageBytes;
+  // Deep A ring (PersistentLds::kDeepA).  Iteration j multiplies k tile j out of A slot
+  // j mod 3 and B slot j mod 2, four DMA requests per wave under each of its four slices:
+  //   slice 0   second half of the B rows of k tile j + 1 (into the other B slot)
+  //   slice 1   first half of the A rows of k tile j + 2 (into the A slot that k tile j - 1
+  //   slice 2   second half of them                       left at the last barrier)
+  //   wait until only those A requests are in flight; barrier (every wave has read the
+  //   last fragments of k tile j)
+  //   slice 3   first half of the B rows of k tile j + 2 (into k tile j's B slot)
+  // A k tile's A rows (the operand that comes from HBM) have about 1.5 iterations to
+  // arrive and stay in flight across a barrier, where two whole stages drained at every
+  // barrier allowed 1 and 0.6; and no slice carries more than four requests (a request
+  // that cannot be issued holds up the MFMAs behind it).  A model of the loop (these
+  // requests, the fragment reads and the MFMAs on the second product's shape) takes 386 us
+  // with two drained stages, 338 with the ring and two bursts of eight, 296 with this one.
+  constexpr bool kDeepA = PersistentLds<Cfg>::kDeepA;
+  constexpr int kABytes = (int)PersistentLds<Cfg>::kABytes, kBBytes = (int)PersistentLds<Cfg>::kBBytes;
+  constexpr int kHalfA = Cfg::kAIssues / 2, kHalfB = Cfg::kBIssues / 2;
+  auto ring_load_a = [&](const TileCtx& t, int slot_a, int k0, auto half) {
+    unsigned char* s = smem + slot_a * kABytes;
+    constexpr int u0 = decltype(half)::value * kHalfA;
 #pragma unroll
-    for (int u = 0; u < Cfg::kAIssues; ++u)
+    for (int u = u0; u < u0 + kHalfA; ++u)
       __builtin_amdgcn_raw_ptr_buffer_load_lds(a_rsrc, (lds_ptr_t)(s + (u * Cfg::kWaves + wave) * RPL * RB),
                                                16, t.a[u], k0 * 2, 0, 0);
   };
-  auto load_ktile_b = [&](const TileCtx& t, int stage, int k0) {
-    unsigned char* s = smem + stage * Cfg::kStageBytes;
+  auto ring_load_b = [&](const TileCtx& t, int slot_b, int k0, auto half) {
+    unsigned char* s = smem + 3 * kABytes + slot_b * kBBytes;
+    constexpr int u0 = decltype(half)::value * kHalfB;
 #pragma unroll
-    for (int u = 0; u < Cfg::kBIssues; ++u)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(
-          b_rsrc, (lds_ptr_t)(s + BM * RB + (u * Cfg::kWaves + wave) * RPL * RB), 16, t.bo[u], k0 * 2,
-          0, 0);
+    for (int u = u0; u < u0 + kHalfB; ++u)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(b_rsrc, (lds_ptr_t)(s + (u * Cfg::kWaves + wave) * RPL * RB),
+                                               16, t.bo[u], k0 * 2, 0, 0);
   };
-  // Two stages: the A rows of k tile kt + 2 go out under the last slice of iteration kt (the
-  // barrier in front of it frees their stage), its B rows under the first slice of
-  // iteration kt + 1, into the same stage: two short bursts of DMA requests instead of one
-  // long one (a request that cannot be issued holds up the MFMAs behind it; second product of the
-  // headline layer: -17 us in six alternating A/B pairs).
-#define VMOE_PERSISTENT_K_ITERATION_SPLIT(SRC, K0, PSRC, PK0) do { \
-    const int next_stage = stage ^ 1; \
-    load_frags(1, stage, 1); \
-    load_ktile_b(PSRC, next_stage, (PK0)); \
+  using Half0 = std::integral_constant<int, 0>;
+  using Half1 = std::integral_constant<int, 1>;
+  const int ring_b_row_off = 3 * kABytes + (wn * Cfg::TN + m) * RB;
+  auto ring_frags = [&](int buf, int slot_a, int slot_b, int ks) {
+    const int col = ((2 * ks + h) ^ swz) * 16;
+    const unsigned char* pa = smem + slot_a * kABytes + a_row_off + col;
+    const unsigned char* pb = smem + slot_b * kBBytes + ring_b_row_off + col;
+#pragma unroll
+    for (int i = 0; i < FM; ++i)
+      fa[buf][i] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(pa + i * 32 * RB));
+#pragma unroll
+    for (int j = 0; j < FN; ++j)
+      fb[buf][j] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(pb + j * 32 * RB));
+  };
+  // SRC, K0: k tile j + 2; PSRC, PK0: k tile j + 1.
+#define VMOE_PERSISTENT_K_ITERATION_RING(SRC, K0, PSRC, PK0) do { \
+    const int prev_a = sa == 0 ? 2 : sa - 1, next_a = sa == 2 ? 0 : sa + 1; \
+    ring_frags(1, sa, sb, 1); \
+    ring_load_b(PSRC, sb ^ 1, (PK0), Half1{}); \
     mfma_slice(0); \
-    slice_schedule(std::integral_constant<int, Cfg::kBIssues>{}); \
-    _Pragma("unroll") \
-    for (int ks = 1; ks + 1 < KS; ++ks) { \
-      load_frags((ks + 1) & 1, stage, ks + 1); \
-      mfma_slice(ks & 1); \
-      slice_schedule(std::integral_constant<int, 0>{}); \
-    } \
-    wait_vmcnt<0>(); \
+    slice_schedule(std::integral_constant<int, kHalfB>{}); \
+    ring_frags(0, sa, sb, 2); \
+    ring_load_a(SRC, prev_a, (K0), Half0{}); \
+    mfma_slice(1); \
+    slice_schedule(std::integral_constant<int, kHalfA>{}); \
+    ring_frags(1, sa, sb, 3); \
+    ring_load_a(SRC, prev_a, (K0), Half1{}); \
+    mfma_slice(0); \
+    slice_schedule(std::integral_constant<int, kHalfA>{}); \
+    wait_vmcnt<Cfg::kAIssues>(); \
     wait_lgkmcnt0(); \
     raw_barrier(); \
-    load_frags(0, next_stage, 0); \
-    load_ktile_a(SRC, stage, (K0)); \
-    mfma_slice((KS - 1) & 1); \
-    slice_schedule(std::integral_constant<int, Cfg::kAIssues>{}); \
-    stage = next_stage; \
+    ring_frags(0, next_a, sb ^ 1, 0); \
+    ring_load_b(SRC, sb, (K0), Half0{}); \
+    mfma_slice(1); \
+    slice_schedule(std::integral_constant<int, kHalfB>{}); \
+    sa = next_a; \
+    sb ^= 1; \
   } while (0)
+  // One k tile of the plain ring of NS stages.  WAITED = the k tile needed next is known to
+  // be complete (every wave drained its loads before the last output was staged, or in the
+  // prologue).  Macros: as lambdas taking the tile by reference the offsets end up in
+  // scratch memory.
 #define VMOE_PERSISTENT_K_ITERATION(SRC, K0, WAITED) do { \
     const int next_stage = stage + 1 == NS ? 0 : stage + 1; \
     _Pragma("unroll") \
@@ -846,14 +888,27 @@ __global__ __launch_bounds__(Cfg::kThreads, 1) void gemm_bf16_persistent_kernel(
 
   TileCtx cur, nxt;
   if (!setup_tile(0, cur)) return;
-#pragma unroll
-  for (int t = 0; t < NS; ++t) load_ktile(cur, t, (cur.kbeg + t) * BK);
-  wait_vmcnt<0>();
-  raw_barrier();
-  load_frags(0, 0, 0);
   int stage = 0;
+  int sa = 0, sb = 0;      // slots of the k tile that the next iteration multiplies (deep A ring)
+  if constexpr (kDeepA) {
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      ring_load_a(cur, t, (cur.kbeg + t) * BK, Half0{});
+      ring_load_a(cur, t, (cur.kbeg + t) * BK, Half1{});
+      ring_load_b(cur, t, (cur.kbeg + t) * BK, Half0{});
+      if (t == 0) ring_load_b(cur, t, (cur.kbeg + t) * BK, Half1{});   // (k tile 1's: first iteration)
+    }
+    wait_vmcnt<0>();
+    raw_barrier();
+    ring_frags(0, 0, 0, 0);
+  } else {
+#pragma unroll
+    for (int t = 0; t < NS; ++t) load_ktile(cur, t, (cur.kbeg + t) * BK);
+    wait_vmcnt<0>();
+    raw_barrier();
+    load_frags(0, 0, 0);
+  }
   constexpr int OLD = PersistentLds<Cfg>::kOutLd;
-  bf16_t* so = reinterpret_cast<bf16_t*>(smem + PersistentLds<Cfg>::kRing) + (size_t)wave * 32 * OLD;
   // Sums in memory: one tile per workgroup, in the order of the accumulator registers (a
   // wave's store or load covers 1 KB of consecutive memory).
   constexpr size_t kTileVecs = (size_t)BM * BN / 4;
@@ -868,11 +923,11 @@ __global__ __launch_bounds__(Cfg::kThreads, 1) void gemm_bf16_persistent_kernel(
     // (without the bounds the compiler plans for trip counts that cannot occur and spills)
     __builtin_assume(kc >= 2 * NS && kc <= nk);
     const int kb = __builtin_amdgcn_readfirstlane(cur.kbeg), nkb = __builtin_amdgcn_readfirstlane(nxt.kbeg);
-    if constexpr (NS == 2 && KS >= 3) {
-      for (int kt = 0; kt < kc - NS; ++kt)
-        VMOE_PERSISTENT_K_ITERATION_SPLIT(cur, (kb + kt + NS) * BK, cur, (kb + kt + NS - 1) * BK);
-      VMOE_PERSISTENT_K_ITERATION_SPLIT(nxt, nkb * BK, cur, (kb + kc - 1) * BK);
-      VMOE_PERSISTENT_K_ITERATION_SPLIT(nxt, (nkb + 1) * BK, nxt, nkb * BK);
+    if constexpr (kDeepA) {
+      for (int kt = 0; kt < kc - 2; ++kt)
+        VMOE_PERSISTENT_K_ITERATION_RING(cur, (kb + kt + 2) * BK, cur, (kb + kt + 1) * BK);
+      VMOE_PERSISTENT_K_ITERATION_RING(nxt, nkb * BK, cur, (kb + kc - 1) * BK);
+      VMOE_PERSISTENT_K_ITERATION_RING(nxt, (nkb + 1) * BK, nxt, nkb * BK);
     } else {
 #pragma unroll
       for (int kt = 0; kt < NS - 1; ++kt) VMOE_PERSISTENT_K_ITERATION(cur, (kb + kt + NS) * BK, true);
@@ -884,6 +939,12 @@ __global__ __launch_bounds__(Cfg::kThreads, 1) void gemm_bf16_persistent_kernel(
     // first NS - 1 iterations of the next tile need no wait of their own.
     wait_vmcnt<0>();
     mfma_result_fence();
+    // Staging region: behind the ring, or (deep A ring) the A slot of the k tile multiplied
+    // last, which no wave reads after that iteration's barrier and which the next request
+    // for A rows (first slice of the next tile's first iteration) will fill: the barrier
+    // at the end of the epilogue keeps that request behind every wave's staged rows.
+    bf16_t* so = reinterpret_cast<bf16_t*>(
+        smem + (kDeepA ? (size_t)(sa == 0 ? 2 : sa - 1) * kABytes : PersistentLds<Cfg>::kRing)) + (size_t)wave * 32 * OLD;
     // A piece of a shared tile that is not the first to finish adds the sums deposited so
     // far, chunk by chunk in the epilogue below, the loads kAhead chunks ahead of their
     // use.  The other pieces were computed at the same time as this one, in workgroups
@@ -997,11 +1058,12 @@ __global__ __launch_bounds__(Cfg::kThreads, 1) void gemm_bf16_persistent_kernel(
         __hip_atomic_store(sk_flags + shared_index, waits + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
     if (!has_next) break;
+    if constexpr (kDeepA) raw_barrier();
     cur = nxt;
   }
   wait_vmcnt<0>();
 #undef VMOE_PERSISTENT_K_ITERATION
-#undef VMOE_PERSISTENT_K_ITERATION_SPLIT
+#undef VMOE_PERSISTENT_K_ITERATION_RING
 #endif
 }
 
