@@ -769,6 +769,16 @@ __global__ __launch_bounds__(Cfg::kThreads, 1) void gemm_bf16_persistent_kernel(
       for (int j = 0; j < FN; ++j)
         acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[buf][j], fa[buf][i], acc[i][j], 0, 0, 0);
   };
+  // First slice of a tile: the sums start from zero in the MFMA itself, so the epilogue need
+  // not clear 256 accumulator registers.
+  auto mfma_slice_first = [&](int buf) {
+    const floatx16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int i = 0; i < FM; ++i)
+#pragma unroll
+      for (int j = 0; j < FN; ++j)
+        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[buf][j], fa[buf][i], zero, 0, 0, 0);
+  };
   // Same issue order inside a k slice as gemm_bf16_kernel: fragment reads behind the first
   // MFMAs, the DMA loads (second slice only) spread over the rest.
   constexpr int kReads = FM + FN, kMfmas = FM * FN;
@@ -840,11 +850,11 @@ __global__ __launch_bounds__(Cfg::kThreads, 1) void gemm_bf16_persistent_kernel(
       fb[buf][j] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(pb + j * 32 * RB));
   };
   // SRC, K0: k tile j + 2; PSRC, PK0: k tile j + 1.
-#define VMOE_PERSISTENT_K_ITERATION_RING(SRC, K0, PSRC, PK0) do { \
+#define VMOE_PERSISTENT_K_ITERATION_RING(SRC, K0, PSRC, PK0, FIRST) do { \
     const int prev_a = sa == 0 ? 2 : sa - 1, next_a = sa == 2 ? 0 : sa + 1; \
     ring_frags(1, sa, sb, 1); \
     ring_load_b(PSRC, sb ^ 1, (PK0), Half1{}); \
-    mfma_slice(0); \
+    if constexpr (FIRST) mfma_slice_first(0); else mfma_slice(0); \
     slice_schedule(std::integral_constant<int, kHalfB>{}); \
     ring_frags(0, sa, sb, 2); \
     ring_load_a(SRC, prev_a, (K0), Half0{}); \
@@ -924,10 +934,11 @@ __global__ __launch_bounds__(Cfg::kThreads, 1) void gemm_bf16_persistent_kernel(
     __builtin_assume(kc >= 2 * NS && kc <= nk);
     const int kb = __builtin_amdgcn_readfirstlane(cur.kbeg), nkb = __builtin_amdgcn_readfirstlane(nxt.kbeg);
     if constexpr (kDeepA) {
-      for (int kt = 0; kt < kc - 2; ++kt)
-        VMOE_PERSISTENT_K_ITERATION_RING(cur, (kb + kt + 2) * BK, cur, (kb + kt + 1) * BK);
-      VMOE_PERSISTENT_K_ITERATION_RING(nxt, nkb * BK, cur, (kb + kc - 1) * BK);
-      VMOE_PERSISTENT_K_ITERATION_RING(nxt, (nkb + 1) * BK, nxt, nkb * BK);
+      VMOE_PERSISTENT_K_ITERATION_RING(cur, (kb + 2) * BK, cur, (kb + 1) * BK, true);
+      for (int kt = 1; kt < kc - 2; ++kt)
+        VMOE_PERSISTENT_K_ITERATION_RING(cur, (kb + kt + 2) * BK, cur, (kb + kt + 1) * BK, false);
+      VMOE_PERSISTENT_K_ITERATION_RING(nxt, nkb * BK, cur, (kb + kc - 1) * BK, false);
+      VMOE_PERSISTENT_K_ITERATION_RING(nxt, (nkb + 1) * BK, nxt, nkb * BK, false);
     } else {
 #pragma unroll
       for (int kt = 0; kt < NS - 1; ++kt) VMOE_PERSISTENT_K_ITERATION(cur, (kb + kt + NS) * BK, true);
@@ -1025,8 +1036,6 @@ __global__ __launch_bounds__(Cfg::kThreads, 1) void gemm_bf16_persistent_kernel(
               const uint32_t p0 = epilogue_pair<EPI, HAS_BIAS>(v[0], v[1], bv[0], bv[1]);
               const uint32_t p1 = epilogue_pair<EPI, HAS_BIAS>(v[2], v[3], bv[2], bv[3]);
               *reinterpret_cast<uint2*>(so + m * OLD + cl) = make_uint2(p0, p1);
-#pragma unroll
-              for (int e = 0; e < 4; ++e) acc[i][j][q * 4 + e] = 0.f;
             }
           }
 #pragma unroll
@@ -1078,8 +1087,10 @@ __global__ __launch_bounds__(Cfg::kThreads, 1) void gemm_bf16_persistent_kernel(
               const uint32_t p1 = epilogue_pair<EPI, HAS_BIAS>(v[2], v[3], bv[2], bv[3]);
               *reinterpret_cast<uint2*>(so + m * OLD + cl) = make_uint2(p0, p1);
             }
+            if constexpr (!kDeepA) {
 #pragma unroll
-            for (int e = 0; e < 4; ++e) acc[i][j][q * 4 + e] = 0.f;
+              for (int e = 0; e < 4; ++e) acc[i][j][q * 4 + e] = 0.f;
+            }
           }
         }
         if (leaves_sums) continue;
