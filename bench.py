@@ -40,18 +40,18 @@ PEAK_HBM_GBS = 8000.0
 # HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc runs
 # (FETCH_SIZE + WRITE_SIZE, scaled by a copy kernel of known size); None until measured.
 MEASURED_TRAFFIC_BYTES = {
-    # mean of the two GEMM launches of a layer: (633 + 565 + 1124 + 181) / 2 MiB;
+    # mean of the two GEMM launches of a layer: (633 + 565 + 1099 + 182) / 2 MiB;
     # FETCH_SIZE x 2.0, WRITE_SIZE x 1.0 (copy-kernel calibration);
     # profiles/hbm_traffic__vmoe_b16_layer.md.
-    "vmoe_b16_layer_E32_k2_bpr": 1.312e9,
+    "vmoe_b16_layer_E32_k2_bpr": 1.300e9,
 }
 # Share of the launch during which the matrix cores are busy (SQ_VALU_MFMA_BUSY_CYCLES over
 # GRBM_GUI_ACTIVE x 1 024 SIMDs), from the rocprofv3 --pmc runs of this command summarised in
 # profiles/mfma_util__vmoe_b16_layer.md: counters cannot be read from inside the run.
 MEASURED_MFMA_BUSY = {
     "vmoe_b16_layer_E32_k2_bpr": {
-        "first_product": 0.427, "second_product": 0.458, "vendor_gemm_second_product_shape": 0.542,
-        "register_resident_mfma_loop": 0.900,
+        "first_product": 0.436, "second_product": 0.606, "vendor_gemm_second_product_shape": 0.545,
+        "register_resident_mfma_loop": 0.947,
         "source": "profiles/mfma_util__vmoe_b16_layer.md (rocprofv3 --pmc, same command, 5 steps)"},
 }
 
@@ -654,25 +654,32 @@ def main():
       torch.cuda.synchronize()
       lib[name] = 2.0 * kept * D * M * 10 / (e0.elapsed_time(e1) * 1e-3) / 1e12
     roofline["library_gemm_same_shapes_TFLOPs"] = lib
-    # What bounds a GEMM of this tiling on this part: the rate at which the second
-    # product's operand tiles (256 x 256 x 32, 128 flop per operand byte) can be moved
-    # from global memory into LDS at all, measured by a kernel that issues exactly those
-    # loads and nothing else, on operands of the layer's shape (E experts with their own
-    # weights, the kept rows spread evenly over them).
+    # The rate at which operand tiles can be moved from global memory into LDS at all,
+    # measured by a kernel that issues exactly the DMA requests of a 256 x 256 product and
+    # nothing else, on operands of the layer's shape (E experts with their own weights, the
+    # kept rows spread evenly over them): with 32-wide k tiles (64-byte row segments per
+    # request, as the first product issues them) and with 64-wide ones (128-byte segments,
+    # the second product's).  Times the flop per operand byte of a tiling it is the
+    # FLOP/s that no kernel of that tiling and request shape can exceed.
     a_e = a_dn[: E * (kept // E)].view(E, kept // E, M)
     w_e = (torch.randn((E, D, M), device=dev) * M ** -0.5).to(tdt)
-    for _ in range(3):
-      kernels.operand_delivery_probe(a_e, w_e)
-    e0.record()
-    for _ in range(10):
-      moved = kernels.operand_delivery_probe(a_e, w_e)
-    e1.record()
-    torch.cuda.synchronize()
-    tbps = moved * 10 / (e0.elapsed_time(e1) * 1e-3) / 1e12
-    roofline["operand_delivery"] = {
-        "TBps": tbps, "flop_per_byte": 128.0, "ceiling_TFLOPs": tbps * 128.0,
-        "frac_of_ceiling": achieved_tflops / (tbps * 128.0),
-        "note": "load-only kernel, second product's tiles; the first product's 128 x 256 tiles have 85 flop per byte"}
+    delivery = {}
+    for name, k_tile, seg, fpb, what in (
+        ("first_product", 32, 64, 2.0 * 128 * 256 / ((128 + 256) * 2), "128 x 256 tiles"),
+        ("second_product", 64, 128, 2.0 * 256 * 256 / ((256 + 256) * 2), "256 x 256 tiles")):
+      for _ in range(3):
+        kernels.operand_delivery_probe(a_e, w_e, k_tile=k_tile)
+      e0.record()
+      for _ in range(10):
+        moved = kernels.operand_delivery_probe(a_e, w_e, k_tile=k_tile)
+      e1.record()
+      torch.cuda.synchronize()
+      tbps = moved * 10 / (e0.elapsed_time(e1) * 1e-3) / 1e12
+      delivery[name] = {"row_segment_bytes": seg, "TBps": tbps, "tiling": what, "flop_per_byte": fpb,
+                        "ceiling_TFLOPs": tbps * fpb}
+    delivery["note"] = ("load-only kernel on 256 x 256 tiles of the second product's operands; the rate depends "
+                        "on the shape of the requests, the ceiling on the product's own flop per operand byte")
+    roofline["operand_delivery"] = delivery
     del a_up, a_dn, w_up, w_dn, a_e, w_e
   # The same K steps replayed from HIP graphs (one per rotating input buffer), as a
   # serving loop would run the layer; reported beside the eager figure, never as `value`.

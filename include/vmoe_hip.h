@@ -479,6 +479,12 @@ int vmoe_mfma_probe(const void* seed, size_t seed_bytes, void* sink, int32_t blo
 int vmoe_operand_delivery_probe(const void* a, const void* bt, int32_t batch, int32_t rows,
                                 int32_t n, int32_t kd, double* bytes, vmoe_stream_t stream);
 
+/* The same with 64-wide k tiles, as the tile-walking second product requests them: a row
+ * segment of a request is 128 bytes instead of 64 and one to two k tiles stay in flight
+ * (no counterpart in the reference; measurement aid).  kd % 64 == 0. */
+int vmoe_operand_delivery_probe_k64(const void* a, const void* bt, int32_t batch, int32_t rows,
+                                    int32_t n, int32_t kd, double* bytes, vmoe_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

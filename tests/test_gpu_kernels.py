@@ -651,6 +651,10 @@ def test_operand_delivery_probe(K):
   torch.cuda.synchronize()
   assert moved == 3 * 3 * 3 * 512 * 256 * 2          # 3 batches x (3 x 3) tiles x 512 rows x K x 2 bytes
   assert K.operand_delivery_probe(a[0], bt[0]) == 3 * 3 * 512 * 256 * 2
+  assert K.operand_delivery_probe(a, bt, k_tile=64) == moved     # same tiles, 128-byte row segments
+  torch.cuda.synchronize()
+  with pytest.raises(H.VmoeError):                     # K not a multiple of 64
+    K.operand_delivery_probe(a[:, :, :96].contiguous(), bt[:, :, :96].contiguous(), k_tile=64)
   with pytest.raises(H.VmoeError):                     # K not a multiple of 32
     K.operand_delivery_probe(a[:, :, :40].contiguous(), bt[:, :, :40].contiguous())
   with pytest.raises(ValueError):

@@ -130,7 +130,9 @@ using CfgDown = GemmCfg<256, 256, 2, 2, 32, 4, 1>;
 // The persistent form of the second product takes k in 64-wide tiles, two stages: a DMA
 // load then requests whole 128-byte lines of an operand row (64-byte halves of a line,
 // requested a k tile apart, move at two thirds of the rate when the line comes from
-// beyond L2).  18 KB of LDS stage its output; tile shape and launch plan are CfgDown's.
+// beyond L2).  Its A rows sit in a ring of three LDS slots, its B rows in one of two (all of
+// the 160 KB); the output is staged in the A slot that the tile's last k tile has left.
+// Tile shape and launch plan are CfgDown's.
 using CfgDownPersistent = GemmCfg<256, 256, 2, 2, 64, 2, 1>;
 
 // Register-resident MFMA loop: the arithmetic ceiling that the expert GEMMs are
@@ -179,15 +181,20 @@ __global__ __launch_bounds__(256) void mfma_probe_kernel(const uint4* __restrict
 }
 
 // Load-only counterpart of the 256x256 product: every workgroup issues the LDS-DMA
-// loads of its tile's k tiles (same addresses, request shapes, tile order and ring of
-// four stages as gemm_bf16_kernel with CfgDown) and nothing else, two k tiles in flight.
-// The rate at which it moves operand tiles is the ceiling of any kernel of this tiling.
+// loads of its tile's k tiles (same addresses, request shapes and tile order as the product
+// kernels) and nothing else; no barrier, no wait except the one that keeps a stage from
+// being requested again while a request for it is in flight.  PCfg = CfgDown: 32-wide k
+// tiles (64-byte row segments), a ring of four stages, two k tiles in flight;
+// PCfg = CfgDownPersistent: 64-wide k tiles (128-byte row segments), two stages, one to two
+// k tiles in flight.  The rate at which it moves operand tiles is the ceiling of any kernel
+// with requests of that shape.
+template <typename PCfg>
 __global__ __launch_bounds__(256, 1) void operand_delivery_probe_kernel(
     const bf16_t* __restrict__ A, const bf16_t* __restrict__ Bt, int R, int N, int Kd,
     int tiles_m, int tiles_n, int num_tiles, int tiles_per_xcd, int panel_rows) {
 #if defined(__HIP_DEVICE_COMPILE__)   // buffer-resource builtins exist in the device pass only
   extern __shared__ __align__(1024) unsigned char smem[];
-  using Cfg = CfgDown;
+  using Cfg = PCfg;
   int b, tile_m, tile_n;
   if (!map_tile(tiles_m, tiles_n, num_tiles, tiles_per_xcd, panel_rows, b, tile_m, tile_n)) return;
   const int lane = threadIdx.x & 63;
@@ -219,7 +226,7 @@ __global__ __launch_bounds__(256, 1) void operand_delivery_probe_kernel(
       __builtin_amdgcn_raw_ptr_buffer_load_lds(
           b_rsrc, (lds_ptr_t)(s + Cfg::BM * RB + (i * Cfg::kWaves + wave) * RPL * RB), 16, b_off[i],
           kt * Cfg::BK * 2, 0, 0);
-    wait_vmcnt<2 * Cfg::kLoads>();   // a stage is written again four k tiles later
+    wait_vmcnt<(Cfg::NSTAGE >= 4 ? 2 : 1) * Cfg::kLoads>();   // a stage is written again NSTAGE k tiles later
   }
   wait_vmcnt<0>();
 #endif
@@ -441,23 +448,35 @@ extern "C" int vmoe_expert_mlp(const VmoeExpertMlpParams* p, vmoe_stream_t strea
                                    p->rows_per_expert);
 }
 
-extern "C" int vmoe_operand_delivery_probe(const void* a, const void* bt, int32_t batch, int32_t rows,
-                                           int32_t n, int32_t kd, double* bytes,
-                                           vmoe_stream_t stream) {
+template <typename PCfg>
+static int launch_operand_delivery_probe(const void* a, const void* bt, int32_t batch, int32_t rows,
+                                         int32_t n, int32_t kd, double* bytes, vmoe_stream_t stream) {
   if (a == nullptr || bt == nullptr || bytes == nullptr) return VMOE_E_NULL;
   if (batch < 1 || rows < 1 || n < 1 || kd < 1) return VMOE_E_SHAPE;
   if (!aligned16(a) || !aligned16(bt)) return VMOE_E_ALIGN;
-  const GemmGeom g = gemm_geometry<CfgDown>(batch, rows, n, kd);
-  if (!g.fast) return VMOE_E_UNSUPPORTED;    // kd % 32 != 0 or an operand beyond 32-bit offsets
+  const GemmGeom g = gemm_geometry<PCfg>(batch, rows, n, kd);
+  if (!g.fast) return VMOE_E_UNSUPPORTED;    // kd not a multiple of the k tile, or an operand beyond 32-bit offsets
   if (g.tiles > 0x7ffffff0LL) return VMOE_E_OVERFLOW;
-  hipError_t e = allow_dynamic_lds(reinterpret_cast<const void*>(operand_delivery_probe_kernel), CfgDown::kLdsBytes);
+  hipError_t e = allow_dynamic_lds(reinterpret_cast<const void*>(operand_delivery_probe_kernel<PCfg>), PCfg::kLdsBytes);
   if (e != hipSuccess) return (int)e;
-  hipLaunchKernelGGL(operand_delivery_probe_kernel, dim3((unsigned)g.tiles_per_xcd * kNumXcd),
-                     dim3(CfgDown::kThreads), CfgDown::kLdsBytes, as_stream(stream),
+  hipLaunchKernelGGL(operand_delivery_probe_kernel<PCfg>, dim3((unsigned)g.tiles_per_xcd * kNumXcd),
+                     dim3(PCfg::kThreads), PCfg::kLdsBytes, as_stream(stream),
                      (const bf16_t*)a, (const bf16_t*)bt, rows, n, kd, g.tiles_m, g.tiles_n,
                      (int)g.tiles, g.tiles_per_xcd, g.panel_rows);
-  *bytes = (double)g.tiles * (CfgDown::BM + CfgDown::BN) * (double)kd * 2.0;
+  *bytes = (double)g.tiles * (PCfg::BM + PCfg::BN) * (double)kd * 2.0;
   return launch_status();
+}
+
+extern "C" int vmoe_operand_delivery_probe(const void* a, const void* bt, int32_t batch, int32_t rows,
+                                           int32_t n, int32_t kd, double* bytes,
+                                           vmoe_stream_t stream) {
+  return launch_operand_delivery_probe<CfgDown>(a, bt, batch, rows, n, kd, bytes, stream);
+}
+
+extern "C" int vmoe_operand_delivery_probe_k64(const void* a, const void* bt, int32_t batch,
+                                               int32_t rows, int32_t n, int32_t kd, double* bytes,
+                                               vmoe_stream_t stream) {
+  return launch_operand_delivery_probe<CfgDownPersistent>(a, bt, batch, rows, n, kd, bytes, stream);
 }
 
 extern "C" int vmoe_pack_expert_weights(const VmoeTransposeParams* p, vmoe_stream_t stream) {

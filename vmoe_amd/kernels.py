@@ -469,9 +469,13 @@ def copy_bytes(src: torch.Tensor, dst: torch.Tensor) -> None:
           "vmoe_copy_bytes")
 
 
-def operand_delivery_probe(a: torch.Tensor, bt: torch.Tensor) -> float:
+def operand_delivery_probe(a: torch.Tensor, bt: torch.Tensor, k_tile: int = 32) -> float:
   """Launches the load-only counterpart of the 256 x 256 product a (B, R, K) . bt (B, N, K)^T
-  (bfloat16, contiguous); returns the operand bytes it moves (time it with events)."""
+  (bfloat16, contiguous); returns the operand bytes it moves (time it with events).
+  k_tile = 32: 64-byte row segments per request (first product, plain second product);
+  k_tile = 64: 128-byte segments (tile-walking second product)."""
+  if k_tile not in (32, 64):
+    raise ValueError("operand_delivery_probe: k_tile is 32 or 64")
   if a.dim() == 2:
     a, bt = a[None], bt[None]
   if a.dtype != torch.bfloat16 or bt.dtype != torch.bfloat16 or not (a.is_contiguous() and bt.is_contiguous()):
@@ -479,9 +483,9 @@ def operand_delivery_probe(a: torch.Tensor, bt: torch.Tensor) -> float:
   if a.shape[0] != bt.shape[0] or a.shape[2] != bt.shape[2]:
     raise ValueError("operand_delivery_probe: a (B, R, K) and bt (B, N, K)")
   moved = H.ctypes.c_double(0.0)
-  H.check(H.lib().vmoe_operand_delivery_probe(H.ptr(a), H.ptr(bt), a.shape[0], a.shape[1], bt.shape[1],
-                                              a.shape[2], H.ctypes.byref(moved), H.stream()),
-          "vmoe_operand_delivery_probe")
+  fn = H.lib().vmoe_operand_delivery_probe if k_tile == 32 else H.lib().vmoe_operand_delivery_probe_k64
+  H.check(fn(H.ptr(a), H.ptr(bt), a.shape[0], a.shape[1], bt.shape[1], a.shape[2],
+             H.ctypes.byref(moved), H.stream()), "vmoe_operand_delivery_probe")
   return float(moved.value)
 
 
