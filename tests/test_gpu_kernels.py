@@ -49,7 +49,11 @@ GATE_CASES = [
     (2, 64, 264, 40, 4, O.BF16),
     (2, 37, 128, 100, 2, O.F32),
     (1, 1568, 768, 32, 2, O.BF16),
-    (1, 33000, 1024, 32, 2, O.BF16),   # eight-wave workgroups (one staged router kernel per CU)
+    (1, 33000, 1024, 32, 2, O.BF16),   # streaming kernel, rings of two slots (the router kernel takes 66 KB)
+    (1, 8200, 768, 32, 2, O.BF16),     # streaming kernel, rings of three slots, a last tile of 8 items
+    (3, 2741, 768, 8, 2, O.BF16),      # streaming kernel, experts padded to the 32-wide tile
+    (2, 4100, 256, 24, 3, O.BF16),     # streaming kernel, four chunks of k
+    (1, 8192, 64, 16, 1, O.BF16),      # streaming kernel, a single chunk of k
     (2, 77, 2048, 32, 2, O.BF16),      # router kernel staged in two chunks along D
     (2, 45, 768, 16, 2, O.BF16),       # experts padded to the 32-wide tile
     (2, 45, 320, 12, 3, O.BF16),       # expert count not a multiple of 8: element-wise staging
@@ -88,6 +92,41 @@ def test_gate_topk_logit_bias(K):
   b = (rng.standard_normal(E) * 2).astype(np.float32)
   gates, _, _ = K.gate_topk(to_dev(x, O.BF16), to_dev(w, O.BF16), 2, logit_bias=to_dev(b))
   assert_close(to_np(gates), O.router_gates(x, w, O.BF16, b), 2e-2, "gates with bias")
+
+
+def test_gate_topk_streaming_and_direct_loads_agree(K, monkeypatch):
+  """The two forms of the bfloat16 gating kernel (item rows through LDS by DMA, or by direct
+  loads: VMOE_GATE_DIRECT_LOADS=1) add the same products in a different order of k: equal
+  bit for bit where every partial sum is exact, within a few bfloat16 steps otherwise; the
+  logit bias and a call without the gates output take the streaming form too."""
+  rng = np.random.default_rng(11)
+  n, D, E = 8192 + 40, 768, 32
+  xi = rng.integers(-2, 3, (1, n, D)).astype(np.float32)          # exact in bfloat16, sums below 2^24
+  wi = rng.integers(-2, 3, (D, E)).astype(np.float32) / 64
+  b = (rng.integers(-8, 9, E) / 4).astype(np.float32)
+  xr = O.cast(rng.standard_normal((1, n, D)), O.BF16)
+  wr = O.cast(rng.standard_normal((D, E)) / np.sqrt(D), O.BF16)
+  for x, w, exact in ((xi, wi, True), (xr, wr, False)):
+    monkeypatch.delenv("VMOE_GATE_DIRECT_LOADS", raising=False)
+    g_s, v_s, i_s = K.gate_topk(to_dev(x, O.BF16), to_dev(w, O.BF16), 2, logit_bias=to_dev(b))
+    _, v_n, i_n = K.gate_topk(to_dev(x, O.BF16), to_dev(w, O.BF16), 2, logit_bias=to_dev(b), return_gates=False)
+    monkeypatch.setenv("VMOE_GATE_DIRECT_LOADS", "1")
+    g_d, v_d, i_d = K.gate_topk(to_dev(x, O.BF16), to_dev(w, O.BF16), 2, logit_bias=to_dev(b))
+    monkeypatch.delenv("VMOE_GATE_DIRECT_LOADS")
+    np.testing.assert_array_equal(to_np(i_s), to_np(i_n))
+    np.testing.assert_array_equal(to_np(v_s), to_np(v_n))
+    if exact:
+      np.testing.assert_array_equal(to_np(g_s), to_np(g_d))
+      np.testing.assert_array_equal(to_np(i_s), to_np(i_d))
+      np.testing.assert_array_equal(to_np(v_s), to_np(v_d))
+      assert_close(to_np(g_s), O.router_gates(x, w, O.BF16, b), 2e-2, "gates")
+    else:
+      gs, gd = to_np(g_s).astype(np.float64), to_np(g_d).astype(np.float64)
+      # (a logit of magnitude 2 .. 4 that rounds the other way moves by 2^-6, its gate by
+      # 1.6 %, and the other gates of the item through the sum)
+      assert np.all(np.abs(gs - gd) <= 2.0 ** -5 * np.maximum(np.abs(gs), np.abs(gd)) + 1e-30)
+      assert float((gs != gd).mean()) < 0.05
+      assert int((to_np(i_s) != to_np(i_d)).any(-1).sum()) <= n // 100
 
 
 def test_router_metrics(K, goldens):
