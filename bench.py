@@ -40,18 +40,18 @@ PEAK_HBM_GBS = 8000.0
 # HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc runs
 # (FETCH_SIZE + WRITE_SIZE, scaled by a copy kernel of known size); None until measured.
 MEASURED_TRAFFIC_BYTES = {
-    # mean of the two GEMM launches of a layer: (633 + 565 + 1099 + 182) / 2 MiB;
+    # mean of the two GEMM launches of a layer: (632 + 565 + 1099 + 182) / 2 MiB;
     # FETCH_SIZE x 2.0, WRITE_SIZE x 1.0 (copy-kernel calibration);
     # profiles/hbm_traffic__vmoe_b16_layer.md.
-    "vmoe_b16_layer_E32_k2_bpr": 1.300e9,
+    "vmoe_b16_layer_E32_k2_bpr": 1.299e9,
 }
 # Share of the launch during which the matrix cores are busy (SQ_VALU_MFMA_BUSY_CYCLES over
 # GRBM_GUI_ACTIVE x 1 024 SIMDs), from the rocprofv3 --pmc runs of this command summarised in
 # profiles/mfma_util__vmoe_b16_layer.md: counters cannot be read from inside the run.
 MEASURED_MFMA_BUSY = {
     "vmoe_b16_layer_E32_k2_bpr": {
-        "first_product": 0.436, "second_product": 0.606, "vendor_gemm_second_product_shape": 0.545,
-        "register_resident_mfma_loop": 0.947,
+        "first_product": 0.424, "second_product": 0.598, "vendor_gemm_second_product_shape": 0.539,
+        "register_resident_mfma_loop": 0.938,
         "source": "profiles/mfma_util__vmoe_b16_layer.md (rocprofv3 --pmc, same command, 5 steps)"},
 }
 
