@@ -404,16 +404,18 @@ extern "C" int vmoe_expert_mlp(const VmoeExpertMlpParams* p, vmoe_stream_t strea
     using SK = StreamKWorkspace<CfgDownPersistent>;
     const bool planned = plan_up != nullptr || plan_down != nullptr;
     int32_t* clear = streamk != nullptr && !planned ? SK::flags(streamk) : nullptr;
+    static_assert(std::is_same<CfgUp, GemmCfg<128, 256, 2, 2, 32, 3, 2>>::value,
+                  "launch_gemm_bf16_first runs CfgUp's geometry");
     if (tanh_gelu)
-      rc = launch_gemm_bf16<CfgUp, kEpiBiasGeluTanh>((const bf16_t*)p->x, (const bf16_t*)w0t,
-                                                      (const bf16_t*)p->b0, (bf16_t*)hidden, p->E,
-                                                      p->R, p->M, p->D, stream, p->rows_per_expert,
-                                                      plan_up, p->x_rows, p->num_items, clear, SK::kFlags);
+      rc = launch_gemm_bf16_first<kEpiBiasGeluTanh>((const bf16_t*)p->x, (const bf16_t*)w0t,
+                                                    (const bf16_t*)p->b0, (bf16_t*)hidden, p->E,
+                                                    p->R, p->M, p->D, stream, p->rows_per_expert,
+                                                    plan_up, p->x_rows, p->num_items, clear, SK::kFlags);
     else
-      rc = launch_gemm_bf16<CfgUp, kEpiBiasGeluErf>((const bf16_t*)p->x, (const bf16_t*)w0t,
-                                                     (const bf16_t*)p->b0, (bf16_t*)hidden, p->E,
-                                                     p->R, p->M, p->D, stream, p->rows_per_expert,
-                                                     plan_up, p->x_rows, p->num_items, clear, SK::kFlags);
+      rc = launch_gemm_bf16_first<kEpiBiasGeluErf>((const bf16_t*)p->x, (const bf16_t*)w0t,
+                                                   (const bf16_t*)p->b0, (bf16_t*)hidden, p->E,
+                                                   p->R, p->M, p->D, stream, p->rows_per_expert,
+                                                   plan_up, p->x_rows, p->num_items, clear, SK::kFlags);
     if (rc != VMOE_OK) return rc;
     switch (m.down_kernel) {
       case kDownShared:

@@ -577,6 +577,217 @@ __global__ __launch_bounds__(Cfg::kThreads, Cfg::kBlocksPerCu) void gemm_bf16_ke
 #endif
 }
 
+// First-product form of gemm_bf16_kernel for k a multiple of 64 (128 x 256 tile, four waves,
+// two workgroups per CU, same launch geometry and plan as GemmCfg<128, 256, 2, 2, 32, 3, 2>).
+// The launch is bound by the rate at which the load path takes its DMA requests, and that
+// rate depends on their shape: 64-byte row segments (32-wide k tiles) move at 9.5 TB/s,
+// 128-byte segments at 13 and more.  The LDS that two workgroups per CU leave (80 KB each)
+// does not hold two 64-wide stages of both operands, but it holds them for the B rows (the
+// weights: two thirds of the requests): B sits in two slots of 64-wide k tiles (128-byte
+// segments, 2 x 32 KB), A in two slots of 32-wide ones (64-byte segments, 2 x 8 KB).
+// Iterations are 32 wide; the pair 2 J, 2 J + 1 multiplies B slot J mod 2.
+//   iteration 2 J      slice 0: second half of the B rows of pair J + 1
+//                      wait (that half may stay in flight), barrier
+//                      slice 1: A rows of k tile 2 J + 2
+//   iteration 2 J + 1  slice 0: nothing
+//                      wait for everything, barrier (B slot J mod 2 is free from here on)
+//                      slice 1: A rows of k tile 2 J + 3, first half of the B rows of pair J + 2
+// A load-only model of the launch: 350 us with 64-byte segments for both operands, 271 - 287
+// with this mix.
+template <int EPI>
+__global__ __launch_bounds__(256, 2) void gemm_bf16_mixed_kernel(
+    const bf16_t* __restrict__ A, const bf16_t* __restrict__ Bt, const bf16_t* __restrict__ bias,
+    bf16_t* __restrict__ C, int R, int N, int Kd, int tiles_m, int tiles_n, int num_tiles,
+    int tiles_per_xcd, int panel_rows, const int32_t* __restrict__ rows,
+    const int4* __restrict__ plan, const int32_t* __restrict__ a_rows, int a_items,
+    int32_t* __restrict__ clear, int clear_count) {
+#if defined(__HIP_DEVICE_COMPILE__)   // buffer-resource builtins exist in the device pass only
+  extern __shared__ __align__(1024) unsigned char smem[];
+  constexpr int BM = 128, BN = 256, TM = 64, TN = 128, FM = 2, FN = 4, kWaves = 4;
+  constexpr int kASlot = BM * 64, kBSlot = BN * 128, kBBase = 2 * kASlot;
+  const int tid = threadIdx.x;
+  if (clear != nullptr && blockIdx.x == 0)
+    for (int c = tid; c < clear_count; c += 256) clear[c] = 0;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave >> 1, wn = wave & 1;
+  const int m = lane & 31, h = lane >> 5;
+
+  int b, tile_m, tile_n;
+  int live = R;
+  if (plan != nullptr) {
+    const int4 mine = plan[blockIdx.x];
+    if (mine.x < 0) return;
+    b = mine.x;
+    tile_m = mine.y;
+    tile_n = mine.z;
+    live = mine.w;
+  } else {
+    if (!map_tile(tiles_m, tiles_n, num_tiles, tiles_per_xcd, panel_rows, b, tile_m, tile_n)) return;
+    if (rows != nullptr) {
+      live = min(rows[b], R);
+      if (tile_m * BM >= live) return;
+    }
+  }
+  const int row0 = tile_m * BM, col0 = tile_n * BN;
+  const unsigned char* Ab = reinterpret_cast<const unsigned char*>(
+      a_rows != nullptr ? A : A + (size_t)b * R * Kd);
+  const unsigned char* Bb = reinterpret_cast<const unsigned char*>(Bt + (size_t)b * N * Kd);
+
+  // A request of A rows fills 16 rows x 64 bytes, one of B rows 8 rows x 128 bytes; lane L
+  // lands in LDS position L of the request and fetches the piece that the XOR swizzle of its
+  // row puts there (64-byte rows: four rows share a 256-byte bank line, 128-byte rows: two).
+  uint32_t a_goff[2], b_goff[8];
+  {
+    const int lrow = lane >> 2;
+    const int piece = (lane & 3) ^ (((wave * 16 + lrow) >> 2) & 3);
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int r = (i * kWaves + wave) * 16 + lrow;
+      int arow = min(row0 + r, (a_rows != nullptr ? live : R) - 1);
+      if (a_rows != nullptr) {
+        arow = a_rows[(size_t)b * R + arow];
+        arow = (unsigned)arow < (unsigned)a_items ? arow : 0;
+      }
+      a_goff[i] = (uint32_t)arow * (uint32_t)Kd * 2u + piece * 16;
+    }
+  }
+  {
+    const int lrow = lane >> 3;
+    const int piece = (lane & 7) ^ (((wave * 8 + lrow) >> 1) & 7);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int r = (i * kWaves + wave) * 8 + lrow;
+      b_goff[i] = (uint32_t)min(col0 + r, N - 1) * (uint32_t)Kd * 2u + piece * 16;
+    }
+  }
+  const __amdgpu_buffer_rsrc_t a_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<unsigned char*>(Ab), 0, -1, 0x00020000);
+  const __amdgpu_buffer_rsrc_t b_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<unsigned char*>(Bb), 0, -1, 0x00020000);
+  auto load_a = [&](int slot, int kt) {           // k tile kt (32 wide) -> A slot
+    unsigned char* s = smem + slot * kASlot;
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(a_rsrc, (lds_ptr_t)(s + (i * kWaves + wave) * 1024), 16,
+                                               a_goff[i], kt * 64, 0, 0);
+  };
+  auto load_b_half = [&](int slot, int pair, auto half) {   // pair of k tiles (64 wide) -> B slot
+    unsigned char* s = smem + kBBase + slot * kBSlot;
+    constexpr int i0 = decltype(half)::value * 4;
+#pragma unroll
+    for (int i = i0; i < i0 + 4; ++i)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(b_rsrc, (lds_ptr_t)(s + (i * kWaves + wave) * 1024), 16,
+                                               b_goff[i], pair * 128, 0, 0);
+  };
+  using Half0 = std::integral_constant<int, 0>;
+  using Half1 = std::integral_constant<int, 1>;
+
+  floatx16 acc[FM][FN];
+#pragma unroll
+  for (int i = 0; i < FM; ++i)
+#pragma unroll
+    for (int j = 0; j < FN; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+  bf16x8 fa[2][FM], fb[2][FN];
+  const int a_row_off = (wm * TM + m) * 64;
+  const int b_row_off = kBBase + (wn * TN + m) * 128;
+  const int swz_a = (m >> 2) & 3, swz_b = (m >> 1) & 7;
+  // Fragments of slice ks (0, 1) of k tile kt.
+  auto load_frags = [&](int buf, int kt, int ks) {
+    const unsigned char* pa = smem + (kt & 1) * kASlot + a_row_off + (((2 * ks + h) ^ swz_a) * 16);
+    const unsigned char* pb = smem + ((kt >> 1) & 1) * kBSlot + b_row_off +
+                              ((((kt & 1) * 4 + 2 * ks + h) ^ swz_b) * 16);
+#pragma unroll
+    for (int i = 0; i < FM; ++i)
+      fa[buf][i] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(pa + i * 32 * 64));
+#pragma unroll
+    for (int j = 0; j < FN; ++j)
+      fb[buf][j] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(pb + j * 32 * 128));
+  };
+  auto mfma_slice = [&](int buf) {
+#pragma unroll
+    for (int i = 0; i < FM; ++i)
+#pragma unroll
+      for (int j = 0; j < FN; ++j)
+        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[buf][j], fa[buf][i], acc[i][j], 0, 0, 0);
+  };
+  // Issue order inside a slice as in gemm_bf16_kernel: the fragment reads of the next slice
+  // behind the first MFMAs, the DMA requests spread over the rest.
+  constexpr int kReads = FM + FN, kMfmas = FM * FN;
+  auto slice_schedule = [&](auto vmem_c) {
+    constexpr int vmem = decltype(vmem_c)::value;
+    constexpr int kLead = kReads < kMfmas ? kReads : kMfmas;
+    constexpr int kRest = kMfmas - kLead;
+#pragma unroll
+    for (int g = 0; g < kLead; ++g) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+    }
+    if constexpr (vmem > 0) {
+#pragma unroll
+      for (int g = 0; g < kRest; ++g) {
+        if (g * vmem / kRest != (g + 1) * vmem / kRest)
+          __builtin_amdgcn_sched_group_barrier(0x020, (vmem + kRest - 1) / kRest, 0);
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  uint2 bias_pk[TN / 8];
+  load_bias<TN>(bias_pk, bias, b, N, col0 + wn * TN, lane);
+
+  const int nk = Kd / 32;          // even, at least 4: the launcher checks
+  load_a(0, 0);
+  load_b_half(0, 0, Half0{});
+  load_b_half(0, 0, Half1{});
+  load_a(1, 1);
+  load_b_half(1, 1, Half0{});
+  wait_vmcnt<6>();                 // k tile 0 has landed: A rows of k tile 1 and half a B slot may be in flight
+  raw_barrier();
+  load_frags(0, 0, 0);
+  // B1: pair J + 1 exists; A2 / A3: k tiles 2 J + 2 / 2 J + 3 exist; B2: pair J + 2 exists.
+#define VMOE_MIXED_PAIR(J, B1, A2, A3, B2) do { \
+    const int kt_ = 2 * (J); \
+    load_frags(1, kt_, 1); \
+    if constexpr (B1) load_b_half(((J) + 1) & 1, (J) + 1, Half1{}); \
+    mfma_slice(0); \
+    slice_schedule(std::integral_constant<int, (B1) ? 4 : 0>{}); \
+    wait_vmcnt<(B1) ? 4 : 0>(); \
+    wait_lgkmcnt0(); \
+    raw_barrier(); \
+    load_frags(0, kt_ + 1, 0); \
+    if constexpr (A2) load_a(0, kt_ + 2); \
+    mfma_slice(1); \
+    slice_schedule(std::integral_constant<int, (A2) ? 2 : 0>{}); \
+    load_frags(1, kt_ + 1, 1); \
+    mfma_slice(0); \
+    slice_schedule(std::integral_constant<int, 0>{}); \
+    if constexpr (A2) { \
+      wait_vmcnt<0>(); \
+      wait_lgkmcnt0(); \
+      raw_barrier(); \
+      load_frags(0, kt_ + 2, 0); \
+    } \
+    if constexpr (A3) load_a(1, kt_ + 3); \
+    if constexpr (B2) load_b_half((J) & 1, (J) + 2, Half0{}); \
+    mfma_slice(1); \
+    slice_schedule(std::integral_constant<int, ((A3) ? 2 : 0) + ((B2) ? 4 : 0)>{}); \
+  } while (0)
+  const int npairs = nk / 2;
+  for (int J = 0; J < npairs - 2; ++J) VMOE_MIXED_PAIR(J, true, true, true, true);
+  VMOE_MIXED_PAIR(npairs - 2, true, true, true, false);
+  VMOE_MIXED_PAIR(npairs - 1, false, false, false, false);
+#undef VMOE_MIXED_PAIR
+  wait_lgkmcnt0();
+  __syncthreads();   // all waves are done with the operand tiles: LDS is reused below
+  mfma_result_fence();
+  store_tile<EPI, TM, TN>(acc, smem, wave, lane, bias_pk, bias != nullptr, C, b, R, live, N,
+                          row0 + wm * TM, col0 + wn * TN);
+#endif
+}
+
 // Generic path (any Kd % 8 == 0): 128x128 tile, operands staged through
 // registers into padded LDS rows, out-of-range k chunks zero-filled.
 // Persistent variant for long k (the second product of an MLP): one workgroup per CU
@@ -1278,6 +1489,36 @@ int launch_gemm_bf16(const bf16_t* A, const bf16_t* Bt, const bf16_t* bias, bf16
   hipLaunchKernelGGL(kern, dim3(blocks), dim3(Cfg::kThreads), Cfg::kLdsBytes, stream, A, Bt, bias,
                      C, R, N, Kd, g.tiles_m, g.tiles_n, (int)g.tiles, g.tiles_per_xcd, g.panel_rows,
                      rows, plan, a_rows, (int)a_items, clear, clear_count);
+  return launch_status();
+}
+
+// The first product of an MLP: gemm_bf16_mixed_kernel where it applies (k a multiple of 64
+// and at least 128), else gemm_bf16_kernel with the same tiling; launch geometry and plan are
+// those of GemmCfg<128, 256, 2, 2, 32, 3, 2> either way.  VMOE_FIRST_PRODUCT_K32=1 in the
+// environment keeps the 32-wide k tiles for both operands (the switch behind the before /
+// after figures).
+template <int EPI>
+int launch_gemm_bf16_first(const bf16_t* A, const bf16_t* Bt, const bf16_t* bias, bf16_t* C,
+                           int batch, int R, int N, int Kd, hipStream_t stream,
+                           const int32_t* rows, const int4* plan, const int32_t* a_rows,
+                           long long a_items, int32_t* clear, int clear_count) {
+  using Cfg = GemmCfg<128, 256, 2, 2, 32, 3, 2>;
+  const GemmGeom g = gemm_geometry<Cfg>(batch, R, N, Kd);
+  const bool gather_ok = a_rows == nullptr ||
+                         (rows != nullptr && (unsigned long long)a_items * Kd * 2 < (1ull << 32));
+  if (!g.fast || Kd % 64 != 0 || Kd < 128 || !gather_ok || g.tiles > 0x7ffffff0LL ||
+      getenv("VMOE_FIRST_PRODUCT_K32") != nullptr)
+    return launch_gemm_bf16<Cfg, EPI>(A, Bt, bias, C, batch, R, N, Kd, stream, rows, plan, a_rows,
+                                      a_items, clear, clear_count);
+  constexpr size_t kLds = 2 * 128 * 64 + 2 * 256 * 128;
+  static_assert(kLds * 2 <= 160 * 1024, "two workgroups per CU");
+  const unsigned blocks = (unsigned)(plan != nullptr ? g.ragged_slots : g.tiles_per_xcd) * kNumXcd;
+  auto kern = gemm_bf16_mixed_kernel<EPI>;
+  hipError_t e = allow_dynamic_lds(reinterpret_cast<const void*>(kern), kLds);
+  if (e != hipSuccess) return (int)e;
+  hipLaunchKernelGGL(kern, dim3(blocks), dim3(256), kLds, stream, A, Bt, bias, C, R, N, Kd,
+                     g.tiles_m, g.tiles_n, (int)g.tiles, g.tiles_per_xcd, g.panel_rows, rows, plan,
+                     a_rows, (int)a_items, clear, clear_count);
   return launch_status();
 }
 
