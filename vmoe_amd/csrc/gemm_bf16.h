@@ -672,11 +672,15 @@ __global__ __launch_bounds__(256, 2) void gemm_bf16_mixed_kernel(
       __builtin_amdgcn_raw_ptr_buffer_load_lds(a_rsrc, (lds_ptr_t)(s + (i * kWaves + wave) * 1024), 16,
                                                a_goff[i], kt * 64, 0, 0);
   };
+  // B requests of a pair that go out with the first part (2, 3 and 4 measure the same, 5 and
+  // 6 cost 3 and 11 us)
+  constexpr int kBFirst = 4;
   auto load_b_half = [&](int slot, int pair, auto half) {   // pair of k tiles (64 wide) -> B slot
     unsigned char* s = smem + kBBase + slot * kBSlot;
-    constexpr int i0 = decltype(half)::value * 4;
+    constexpr int i0 = decltype(half)::value ? kBFirst : 0;
+    constexpr int i1 = decltype(half)::value ? 8 : kBFirst;
 #pragma unroll
-    for (int i = i0; i < i0 + 4; ++i)
+    for (int i = i0; i < i1; ++i)
       __builtin_amdgcn_raw_ptr_buffer_load_lds(b_rsrc, (lds_ptr_t)(s + (i * kWaves + wave) * 1024), 16,
                                                b_goff[i], pair * 128, 0, 0);
   };
@@ -744,7 +748,7 @@ __global__ __launch_bounds__(256, 2) void gemm_bf16_mixed_kernel(
   load_b_half(0, 0, Half1{});
   load_a(1, 1);
   load_b_half(1, 1, Half0{});
-  wait_vmcnt<6>();                 // k tile 0 has landed: A rows of k tile 1 and half a B slot may be in flight
+  wait_vmcnt<2 + kBFirst>();       // k tile 0 has landed: A rows of k tile 1 and the first part of a B slot may be in flight
   raw_barrier();
   load_frags(0, 0, 0);
   // B1: pair J + 1 exists; A2 / A3: k tiles 2 J + 2 / 2 J + 3 exist; B2: pair J + 2 exists.
@@ -753,8 +757,8 @@ __global__ __launch_bounds__(256, 2) void gemm_bf16_mixed_kernel(
     load_frags(1, kt_, 1); \
     if constexpr (B1) load_b_half(((J) + 1) & 1, (J) + 1, Half1{}); \
     mfma_slice(0); \
-    slice_schedule(std::integral_constant<int, (B1) ? 4 : 0>{}); \
-    wait_vmcnt<(B1) ? 4 : 0>(); \
+    slice_schedule(std::integral_constant<int, (B1) ? 8 - kBFirst : 0>{}); \
+    wait_vmcnt<(B1) ? 8 - kBFirst : 0>(); \
     wait_lgkmcnt0(); \
     raw_barrier(); \
     load_frags(0, kt_ + 1, 0); \
@@ -773,7 +777,7 @@ __global__ __launch_bounds__(256, 2) void gemm_bf16_mixed_kernel(
     if constexpr (A3) load_a(1, kt_ + 3); \
     if constexpr (B2) load_b_half((J) & 1, (J) + 2, Half0{}); \
     mfma_slice(1); \
-    slice_schedule(std::integral_constant<int, ((A3) ? 2 : 0) + ((B2) ? 4 : 0)>{}); \
+    slice_schedule(std::integral_constant<int, ((A3) ? 2 : 0) + ((B2) ? kBFirst : 0)>{}); \
   } while (0)
   const int npairs = nk / 2;
   for (int J = 0; J < npairs - 2; ++J) VMOE_MIXED_PAIR(J, true, true, true, true);
