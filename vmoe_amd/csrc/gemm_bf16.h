@@ -176,6 +176,31 @@ __device__ __forceinline__ void store_tile(floatx16 (&acc)[TM / 32][TN / 32], un
   static_assert(64 % kChunksOut == 0, "wave tile width must divide a wave");
   const int oc = (lane % kChunksOut) * 8;
   const int orow = lane / kChunksOut;
+#if defined(__HIP_DEVICE_COMPILE__)
+  // Rows and columns past the edge leave through the range check of a buffer store (the
+  // lane's part of the address in the vector offset, which the check sees, the pass's part in
+  // the scalar offset) instead of a branch around every store.
+  if ((uint64_t)R * N * 2 < (1ull << 31)) {
+    typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+    const uint64_t cb_bits = reinterpret_cast<uint64_t>(Cb);      // the same in every lane
+    bf16_t* cb_uniform = reinterpret_cast<bf16_t*>(
+        ((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(cb_bits >> 32)) << 32) |
+        (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)cb_bits));
+    const __amdgpu_buffer_rsrc_t c_rsrc = __builtin_amdgcn_make_buffer_rsrc(cb_uniform, 0, R * N * 2, 0x00020000);
+    const uint32_t lane_off = (uint32_t)(orow * N + oc) * 2u;
+    const int row_u = __builtin_amdgcn_readfirstlane(wrow0), col_u = __builtin_amdgcn_readfirstlane(wcol0);
+    const bool col_ok = oc + 8 <= N - col_u;
+#pragma unroll
+    for (int r0 = 0; r0 < TM; r0 += kRowsPerPass) {
+      const uint4 v = *reinterpret_cast<const uint4*>(so + (r0 + orow) * OLD + oc);
+      const bool ok = col_ok && orow < live - (row_u + r0);
+      __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4_t, v), c_rsrc,
+                                             ok ? lane_off : 0xfffffff0u,
+                                             ((row_u + r0) * N + col_u) * 2, EPI != kEpiBias ? 2 : 0);
+    }
+    return;
+  }
+#endif
 #pragma unroll
   for (int r0 = 0; r0 < TM; r0 += kRowsPerPass) {
     const int rl = r0 + orow;
