@@ -24,6 +24,16 @@ if ROOT not in sys.path:
 # Steps run first so that no one-time initialisation (first launches, memory pools) falls
 # into the warm-up or the timed steps; the timing events are created after them.
 COLD_STEPS = 3
+# The expert MLP's two products run under vmoe_expert_mlp or, when the packed rows were
+# computed in the launch that plans them (vmoe_compact_rows_planned), under
+# vmoe_expert_mlp_planned; the stage tables report the two as vmoe_expert_mlp.
+MLP_CALLS = ("vmoe_expert_mlp", "vmoe_expert_mlp_planned")
+
+
+def merge_mlp_calls(stage_ms):
+  if "vmoe_expert_mlp_planned" in stage_ms:
+    stage_ms["vmoe_expert_mlp"] = stage_ms.get("vmoe_expert_mlp", 0.0) + stage_ms.pop("vmoe_expert_mlp_planned")
+  return stage_ms
 # Steps run right in front of the W warm-up steps, after everything that leaves the GPU idle
 # (creating events, a garbage collection): an idle GPU takes about 25 ms of work to get its
 # clocks back, more than a few warm-up steps of a millisecond each.
@@ -187,8 +197,8 @@ def soft_main(args):
   torch.cuda.synchronize()
   # As in main(): events only around the dominant entry point inside the timed region,
   # the other stages from a second, fully instrumented pass.
-  sink = _hip.TimingSink(pairs=args.steps * 2, only=("vmoe_expert_mlp",))
-  warm_sink = _hip.TimingSink(pairs=(INIT_STEPS + args.warmup) * 2, only=("vmoe_expert_mlp",))
+  sink = _hip.TimingSink(pairs=args.steps * 2, only=MLP_CALLS)
+  warm_sink = _hip.TimingSink(pairs=(INIT_STEPS + args.warmup) * 2, only=MLP_CALLS)
   # One event per step boundary (the per-step times whose median is reported) and one
   # host time stamp per step (which step, if any, kept the host waiting).
   marks = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps + 1)]
@@ -231,8 +241,8 @@ def soft_main(args):
   _hip.set_timing_sink(None)
   per_step = lambda d: {name: float(np.mean([a.elapsed_time(b) for a, b in pairs])) *
                         (len(pairs) / args.steps) for name, pairs in d.items()}
-  stage_ms = per_step(full)
-  stage_ms.update(per_step(sink))
+  stage_ms = merge_mlp_calls(per_step(full))
+  stage_ms.update(merge_mlp_calls(per_step(sink)))
   T = G * m
   # Dominant kernel: the expert GEMM, weight-bandwidth bound here (1.2 GB of weights
   # for 309 GFLOP): algorithmic bytes = weights + slot activations in and out + hidden.
@@ -337,7 +347,7 @@ def vit_main(args):
   # Timed region: events only around the dominant entry point (the MLP GEMMs); module
   # spans and the other stages come from a second, fully instrumented pass of the same
   # steps (events between kernels serialise their hand-over and would slow the pass).
-  sink = _hip.TimingSink(pairs=args.steps * 14, only=("vmoe_expert_mlp",))
+  sink = _hip.TimingSink(pairs=args.steps * 14, only=MLP_CALLS)
   _hip.set_timing_sink(sink)
   t0 = time.perf_counter()
   for i in range(args.steps):
@@ -360,8 +370,8 @@ def vit_main(args):
   module_ms = {k: float(sum(a.elapsed_time(b) for a, b in v)) / args.steps for k, v in spans.items()}
   per_step = lambda d: {name: float(np.mean([a.elapsed_time(b) for a, b in pairs])) *
                         (len(pairs) / args.steps) for name, pairs in d.items()}
-  stage_ms = per_step(full)
-  stage_ms.update(per_step(sink))
+  stage_ms = merge_mlp_calls(per_step(full))
+  stage_ms.update(merge_mlp_calls(per_step(sink)))
   module_ms["other (patch embedding, layer norms, residuals, head)"] = ms_instrumented - sum(
       module_ms.values())
   module_ms["instrumented_pass_ms_per_step"] = ms_instrumented
@@ -386,10 +396,18 @@ def vit_main(args):
     recording.keep.append(self)            # keeps ids distinct until they are read
     return maps
   recording.keep = []
+  set_maps = moe_lib.ExpertIndicesDispatcher.set_packed_maps
+
+  def recording_set(self, maps):           # (packed rows computed by the expert's planning launch)
+    set_maps(self, maps)
+    live_rows[id(self)] = maps[1]
+    recording.keep.append(self)
   moe_lib.ExpertIndicesDispatcher._packed = recording
+  moe_lib.ExpertIndicesDispatcher.set_packed_maps = recording_set
   step(0)
   torch.cuda.synchronize()
   moe_lib.ExpertIndicesDispatcher._packed = packed
+  moe_lib.ExpertIndicesDispatcher.set_packed_maps = set_maps
   live_rows = list(live_rows.values())
   kept_per_block = [int(r.sum()) for r in live_rows]
   assert len(kept_per_block) == n_moe
@@ -504,8 +522,8 @@ def main():
   # An event between two kernels serialises their hand-over, and eight pairs per step
   # cost the layer about 6 % of its throughput; the other stages are timed in a second,
   # fully instrumented pass of the same K steps right after.
-  sink = _hip.TimingSink(pairs=args.steps * 2, only=("vmoe_expert_mlp",))
-  warm_sink = _hip.TimingSink(pairs=(INIT_STEPS + args.warmup) * 2, only=("vmoe_expert_mlp",))
+  sink = _hip.TimingSink(pairs=args.steps * 2, only=MLP_CALLS)
+  warm_sink = _hip.TimingSink(pairs=(INIT_STEPS + args.warmup) * 2, only=MLP_CALLS)
   # One event per step boundary: the per-step times whose median is reported.
   marks = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps + 1)]
   for ev in marks:
@@ -550,9 +568,9 @@ def main():
     step(i)
   torch.cuda.synchronize()
   _hip.set_timing_sink(None)
-  stage_ms = per_step(full)
+  stage_ms = merge_mlp_calls(per_step(full))
   stage_ms_instrumented_mlp = stage_ms["vmoe_expert_mlp"]
-  stage_ms.update(per_step(sink))          # the GEMMs' time is the one of the timed region
+  stage_ms.update(merge_mlp_calls(per_step(sink)))    # the GEMMs' time is the one of the timed region
 
   # Kept assignments (rows that carry an item) for the algorithmic flop count.
   gates, val, idx = kernels.gate_topk(xs[0].view(G, S, D), variables["params"]["Router"]["dense"]["kernel"].to(tdt), K,

@@ -334,6 +334,19 @@ typedef struct {
 size_t vmoe_expert_mlp_workspace_bytes(const VmoeExpertMlpParams* p);
 int vmoe_expert_mlp(const VmoeExpertMlpParams* p, vmoe_stream_t stream);
 
+/* vmoe_compact_rows and the planning launch of vmoe_expert_mlp in one launch (no counterpart
+ * in the reference: the packed rows have none).  `mlp` is the parameter block of the MLP call
+ * that follows, with its workspace and with rows_per_expert = c->rows_per_expert, x_rows =
+ * c->row_token where the first product gathers its rows (only E, R, D, M, dtype, the
+ * workspace and rows_per_expert are looked at here); that call is then made as
+ * vmoe_expert_mlp_planned, which takes the launch plans in the workspace as written.
+ * VMOE_E_UNSUPPORTED where the compaction needs its two-launch form (E > 256, fewer than 256
+ * assignments per group, many groups of few experts) or the MLP plans nothing (float32):
+ * make the separate calls.  Results equal those of the separate calls. */
+int vmoe_compact_rows_planned(const VmoeCompactRowsParams* c, const VmoeExpertMlpParams* mlp,
+                              vmoe_stream_t stream);
+int vmoe_expert_mlp_planned(const VmoeExpertMlpParams* p, vmoe_stream_t stream);
+
 /* (batch, rows, cols) -> (batch, cols, rows), 2- or 4-byte elements. */
 typedef struct {
   const void* in;

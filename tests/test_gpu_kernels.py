@@ -700,6 +700,46 @@ def test_operand_delivery_probe(K):
     K.operand_delivery_probe(a.float(), bt.float())
 
 
+@pytest.mark.parametrize("G,S,E,k,C,D,M", [
+    (4, 1568, 32, 2, 100, 256, 512),     # headline routing shapes, a narrow MLP
+    (2, 1568, 8, 2, 412, 128, 256),      # few experts, many rows each
+    (3, 300, 5, 3, 200, 128, 192),       # expert count that does not divide 256
+])
+def test_expert_mlp_with_compaction_in_the_planning_launch(K, monkeypatch, G, S, E, k, C, D, M):
+  """expert_mlp(compact=...) (vmoe_compact_rows_planned + vmoe_expert_mlp_planned) against
+  vmoe_compact_rows followed by vmoe_expert_mlp: the integer maps bit for bit, the output
+  rows of kept assignments bit for bit as well (the same kernels run on the same plan)."""
+  rng = np.random.default_rng(G * 100 + E)
+  gates = O.softmax(rng.standard_normal((G, S, E)).astype(np.float32) * 2)
+  val, idx = K.topk(to_dev(gates), k)
+  _, token_slot, _, fill = K.route_assign(val, idx, E, C, True)
+  items = to_dev(O.cast(rng.standard_normal((G * S, D)), O.BF16), O.BF16)
+  w0 = to_dev(O.cast(rng.standard_normal((E, D, M)) / np.sqrt(D), O.BF16), O.BF16)
+  w1 = to_dev(O.cast(rng.standard_normal((E, M, D)) / np.sqrt(M), O.BF16), O.BF16)
+  b0 = to_dev(O.cast(rng.standard_normal((E, M)) * 0.1, O.BF16), O.BF16)
+  b1 = to_dev(O.cast(rng.standard_normal((E, D)) * 0.1, O.BF16), O.BF16)
+  w0t, w1t = K.pack_expert_weights(w0), K.pack_expert_weights(w1)
+  token_row, rows, row_token = K.compact_rows(fill, token_slot, C)
+  want = K.expert_mlp(items, None, b0, None, b1, w0t=w0t, w1t=w1t, rows_per_expert=rows, x_rows=row_token)
+  for separate in (False, True):
+    if separate:
+      monkeypatch.setenv("VMOE_PLAN_SEPARATE_LAUNCH", "1")
+    else:
+      monkeypatch.delenv("VMOE_PLAN_SEPARATE_LAUNCH", raising=False)
+    for _ in range(2):
+      got, maps = K.expert_mlp(items, None, b0, None, b1, w0t=w0t, w1t=w1t,
+                               compact=(fill, token_slot, C))
+      np.testing.assert_array_equal(to_np(maps[0]), to_np(token_row))
+      np.testing.assert_array_equal(to_np(maps[1]), to_np(rows))
+      r = to_np(rows)
+      g_np, w_np = to_np(got), to_np(want)
+      rt_g, rt_w = to_np(maps[2]), to_np(row_token)
+      for e in range(E):
+        np.testing.assert_array_equal(rt_g[e, :r[e]], rt_w[e, :r[e]])
+        np.testing.assert_array_equal(g_np[e, :r[e]], w_np[e, :r[e]])
+  monkeypatch.delenv("VMOE_PLAN_SEPARATE_LAUNCH", raising=False)
+
+
 def test_expert_mlp_hidden_layer_beyond_4_gib(K):
   """A hidden layer of 4.3 GiB: the second product cannot address it with 32-bit byte
   offsets from its start, which the tile-walking kernel needs, so the one-tile-per-

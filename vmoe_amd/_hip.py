@@ -22,7 +22,7 @@ W_F32, W_BF16, W_BOOL = 0, 1, 2
 EXPORTS = [
     "vmoe_abi_version", "vmoe_error_string", "vmoe_gate_topk", "vmoe_topk", "vmoe_router_metrics",
     "vmoe_route_assign", "vmoe_route_assign_metrics", "vmoe_top_items_per_expert", "vmoe_indices_to_slots", "vmoe_dispatch", "vmoe_combine", "vmoe_densify",
-    "vmoe_expert_mlp_workspace_bytes", "vmoe_expert_mlp", "vmoe_pack_expert_weights",
+    "vmoe_expert_mlp_workspace_bytes", "vmoe_expert_mlp", "vmoe_expert_mlp_planned", "vmoe_compact_rows_planned", "vmoe_pack_expert_weights",
     "vmoe_soft_route_workspace_bytes", "vmoe_soft_route", "vmoe_einsum_dispatch",
     "vmoe_einsum_combine", "vmoe_cast", "vmoe_copy_bytes", "vmoe_mfma_probe", "vmoe_operand_delivery_probe", "vmoe_operand_delivery_probe_k64",
     "vmoe_add_layer_norm", "vmoe_attention", "vmoe_noisy_gates", "vmoe_compact_rows", "vmoe_compact_rows_static",
@@ -264,6 +264,28 @@ def call2(name: str, first: ctypes.Structure, second: ctypes.Structure) -> None:
   stop.record()
   sink.setdefault(name, []).append((start, stop))
   check(code, name)
+
+
+def call_blocks(name: str, *args, accept=()) -> int:
+  """An entry point that takes several parameter blocks before the stream (passed by
+  reference).  Timed like call().  Return codes listed in `accept` are returned, not raised."""
+  fn = getattr(lib(), name)
+  cargs = [ctypes.byref(a) if isinstance(a, ctypes.Structure) else a for a in args]
+  sink = _timing_sink
+  if sink is None or (getattr(sink, "only", None) is not None and name not in sink.only):
+    code = fn(*cargs, stream())
+  else:
+    take = getattr(sink, "take", None)
+    start, stop = take() if take is not None else (
+        torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
+    start.record()
+    code = fn(*cargs, stream())
+    stop.record()
+    sink.setdefault(name, []).append((start, stop))
+  if code in accept:
+    return code
+  check(code, name)
+  return code
 
 
 def call(name: str, params: ctypes.Structure) -> None:

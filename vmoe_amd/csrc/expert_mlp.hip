@@ -5,6 +5,7 @@
 // the expert axis with the bias add and the GELU fused into the epilogue of the
 // first product and the bias add into the second.
 #include "gemm_bf16_wide.h"
+#include "compact_rows.h"
 
 namespace vmoe {
 namespace {
@@ -232,6 +233,25 @@ __global__ __launch_bounds__(256, 1) void operand_delivery_probe_kernel(
 #endif
 }
 
+// Row compaction and the launch plans of the expert MLP's ragged products in one launch:
+// workgroups 0 .. compact_blocks - 1 renumber the assignments (compact_rows_fused_block),
+// the others plan (plan_ragged_tiles_block, row counts from the fill counts).  Neither part
+// reads what the other writes.
+__global__ __launch_bounds__(256) void compact_rows_planned_kernel(
+    const int32_t* __restrict__ fill, const int32_t* __restrict__ token_slot,
+    int32_t* __restrict__ token_row, int32_t* __restrict__ row_token,
+    int32_t* __restrict__ rows_per_expert, int G, int E, int C, int per_group, int K, size_t n,
+    unsigned compact_blocks, int R, RaggedGeom ga, RaggedGeom gb, int32_t* __restrict__ clear,
+    int clear_count) {
+  extern __shared__ int32_t tile_prefix[];
+  if (blockIdx.x < compact_blocks)
+    compact_rows_fused_block(fill, token_slot, token_row, row_token, rows_per_expert, G, E, C,
+                             per_group, K, n, blockIdx.x);
+  else
+    plan_ragged_tiles_block(nullptr, fill, G, E, R, ga, gb, clear, clear_count,
+                            blockIdx.x - compact_blocks, tile_prefix);
+}
+
 size_t align256(size_t v) { return (v + 255) / 256 * 256; }
 
 // Which kernel runs the second product (bfloat16).
@@ -272,7 +292,7 @@ MlpPlans mlp_plans(int E, int R, int D, int M, bool ragged) {
   // layer the planned launch costs 0.3 %.
   auto bytes = [&](const GemmGeom& g) -> size_t {
     if (!ragged || !g.fast || g.ragged_slots * kNumXcd > 0x7ffffff0LL ||
-        (size_t)(E + 1) * 8 > 60000)
+        plan_ragged_tiles_lds(E) > 60000)
       return 0;
     return align256(((size_t)g.ragged_slots * kNumXcd + 1) * sizeof(int4));   // + the header entry
   };
@@ -348,41 +368,70 @@ extern "C" size_t vmoe_expert_mlp_workspace_bytes(const VmoeExpertMlpParams* p) 
   return bytes;
 }
 
-extern "C" int vmoe_expert_mlp(const VmoeExpertMlpParams* p, vmoe_stream_t stream_) {
+// Where the pieces of a bfloat16 MLP's workspace lie, and what the planning launch is given.
+struct MlpWorkspace {
+  void* hidden = nullptr;
+  int4* plan_up = nullptr;
+  int4* plan_down = nullptr;
+  void* streamk = nullptr;
+  unsigned char* rest = nullptr;     // transposed weights, where the caller did not pack them
+  MlpPlans m;
+  RaggedGeom ga{}, gb{};
+  int plan_blocks = 0;               // workgroups of the planning launch (0: nothing to plan)
+};
+
+MlpWorkspace mlp_workspace(const VmoeExpertMlpParams* p) {
+  MlpWorkspace w;
+  unsigned char* ws = static_cast<unsigned char*>(p->workspace);
+  const size_t b = p->dtype == VMOE_BF16 ? 2 : 4;
+  w.hidden = ws;
+  ws += align256((size_t)p->E * p->R * p->M * b);
+  if (p->dtype == VMOE_BF16) {
+    w.m = mlp_plans(p->E, p->R, p->D, p->M, p->rows_per_expert != nullptr);
+    if (w.m.up_bytes) w.plan_up = reinterpret_cast<int4*>(ws);
+    ws += w.m.up_bytes;
+    if (w.m.down_bytes) w.plan_down = reinterpret_cast<int4*>(ws);
+    ws += w.m.down_bytes;
+    if (w.m.streamk_bytes) w.streamk = ws;
+    ws += w.m.streamk_bytes;
+    if (w.plan_up != nullptr || w.plan_down != nullptr) {
+      w.ga = RaggedGeom{CfgUp::BM, w.m.up.tiles_n, w.m.up.panel_rows,
+                        w.plan_up ? (int)(w.m.up.ragged_slots * kNumXcd) : 0,
+                        reinterpret_cast<PlanEntry*>(w.plan_up)};
+      w.gb = RaggedGeom{w.m.down_bm, w.m.down.tiles_n, w.m.down.panel_rows,
+                        w.plan_down ? (int)(w.m.down.ragged_slots * kNumXcd) : 0,
+                        reinterpret_cast<PlanEntry*>(w.plan_down)};
+      const int n = w.ga.num_blocks > w.gb.num_blocks ? w.ga.num_blocks : w.gb.num_blocks;
+      w.plan_blocks = (n + 255) / 256;
+    }
+  }
+  w.rest = ws;
+  return w;
+}
+
+// `planned`: the launch plans in the workspace have been written (vmoe_compact_rows_planned).
+static int run_expert_mlp(const VmoeExpertMlpParams* p, vmoe_stream_t stream_, bool planned_already) {
   int rc = check_mlp(p);
   if (rc != VMOE_OK) return rc;
   const size_t need = vmoe_expert_mlp_workspace_bytes(p);
   if (p->workspace == nullptr || p->workspace_bytes < need || !aligned16(p->workspace))
     return VMOE_E_WORKSPACE;
   hipStream_t stream = as_stream(stream_);
-  unsigned char* ws = static_cast<unsigned char*>(p->workspace);
   const size_t b = p->dtype == VMOE_BF16 ? 2 : 4;
-  void* hidden = ws;
-  ws += align256((size_t)p->E * p->R * p->M * b);
-  int4* plan_up = nullptr;
-  int4* plan_down = nullptr;
-  void* streamk = nullptr;
-  MlpPlans m;
-  if (p->dtype == VMOE_BF16) {
-    m = mlp_plans(p->E, p->R, p->D, p->M, p->rows_per_expert != nullptr);
-    if (m.up_bytes) plan_up = reinterpret_cast<int4*>(ws);
-    ws += m.up_bytes;
-    if (m.down_bytes) plan_down = reinterpret_cast<int4*>(ws);
-    ws += m.down_bytes;
-    if (m.streamk_bytes) streamk = ws;
-    ws += m.streamk_bytes;
-    if (plan_up != nullptr || plan_down != nullptr) {
-      const RaggedGeom ga{CfgUp::BM, m.up.tiles_n, m.up.panel_rows,
-                          plan_up ? (int)(m.up.ragged_slots * kNumXcd) : 0, reinterpret_cast<PlanEntry*>(plan_up)};
-      const RaggedGeom gb{m.down_bm, m.down.tiles_n, m.down.panel_rows,
-                          plan_down ? (int)(m.down.ragged_slots * kNumXcd) : 0, reinterpret_cast<PlanEntry*>(plan_down)};
-      const int n = ga.num_blocks > gb.num_blocks ? ga.num_blocks : gb.num_blocks;
-      using SK = StreamKWorkspace<CfgDownPersistent>;
-      hipLaunchKernelGGL(plan_ragged_tiles_kernel, dim3((n + 255) / 256), dim3(256),
-                         (size_t)(p->E + 1) * 8, stream, p->rows_per_expert, p->E, p->R, ga, gb,
-                         streamk != nullptr ? SK::flags(streamk) : nullptr,
-                         streamk != nullptr ? SK::kFlags : 0);
-    }
+  const MlpWorkspace w = mlp_workspace(p);
+  void* hidden = w.hidden;
+  int4* plan_up = w.plan_up;
+  int4* plan_down = w.plan_down;
+  void* streamk = w.streamk;
+  const MlpPlans& m = w.m;
+  unsigned char* ws = w.rest;
+  if (planned_already && w.plan_blocks == 0) return VMOE_E_UNSUPPORTED;
+  if (w.plan_blocks > 0 && !planned_already) {
+    using SK = StreamKWorkspace<CfgDownPersistent>;
+    hipLaunchKernelGGL(plan_ragged_tiles_kernel, dim3(w.plan_blocks), dim3(256),
+                       plan_ragged_tiles_lds(p->E), stream, p->rows_per_expert, p->E, p->R, w.ga, w.gb,
+                       streamk != nullptr ? SK::flags(streamk) : nullptr,
+                       streamk != nullptr ? SK::kFlags : 0);
   }
   const bool tanh_gelu = p->gelu == VMOE_GELU_TANH;
   if (p->dtype == VMOE_BF16) {
@@ -448,6 +497,47 @@ extern "C" int vmoe_expert_mlp(const VmoeExpertMlpParams* p, vmoe_stream_t strea
   return launch_gemm_f32<kEpiBias>((const float*)hidden, (const float*)p->w1, (const float*)p->b1,
                                    (float*)p->out, p->E, p->R, p->D, p->M, stream,
                                    p->rows_per_expert);
+}
+
+extern "C" int vmoe_expert_mlp(const VmoeExpertMlpParams* p, vmoe_stream_t stream) {
+  return run_expert_mlp(p, stream, false);
+}
+
+extern "C" int vmoe_expert_mlp_planned(const VmoeExpertMlpParams* p, vmoe_stream_t stream) {
+  return run_expert_mlp(p, stream, true);
+}
+
+extern "C" int vmoe_compact_rows_planned(const VmoeCompactRowsParams* c,
+                                         const VmoeExpertMlpParams* mlp, vmoe_stream_t stream) {
+  if (c == nullptr || mlp == nullptr || c->fill == nullptr || c->token_slot == nullptr ||
+      c->token_row == nullptr || c->rows_per_expert == nullptr)
+    return VMOE_E_NULL;
+  if (c->G < 1 || c->S < 1 || c->E < 1 || c->K < 1 || c->C < 1 || c->K > c->E) return VMOE_E_SHAPE;
+  if ((int64_t)c->G * c->S * c->K * 2 >= INT32_MAX || (int64_t)c->E * c->G * c->C >= INT32_MAX)
+    return VMOE_E_OVERFLOW;
+  int rc = check_mlp(mlp);
+  if (rc != VMOE_OK) return rc;
+  if (mlp->E != c->E || (int64_t)mlp->R != (int64_t)c->G * c->C ||
+      mlp->rows_per_expert != c->rows_per_expert)
+    return VMOE_E_SHAPE;
+  if (mlp->workspace == nullptr || mlp->workspace_bytes < vmoe_expert_mlp_workspace_bytes(mlp) ||
+      !aligned16(mlp->workspace))
+    return VMOE_E_WORKSPACE;
+  // One launch needs the one-launch form of the compaction and an MLP whose products are planned.
+  if (!compact_rows_fused_ok(c->G, c->S, c->E, c->K) || mlp->dtype != VMOE_BF16)
+    return VMOE_E_UNSUPPORTED;
+  const MlpWorkspace w = mlp_workspace(mlp);
+  if (w.plan_blocks == 0) return VMOE_E_UNSUPPORTED;
+  const size_t n = (size_t)c->G * c->S * c->K;
+  const unsigned compact_blocks = (unsigned)((n + 255) / 256);
+  using SK = StreamKWorkspace<CfgDownPersistent>;
+  hipLaunchKernelGGL(compact_rows_planned_kernel, dim3(compact_blocks + (unsigned)w.plan_blocks),
+                     dim3(256), plan_ragged_tiles_lds(c->E), as_stream(stream), c->fill,
+                     c->token_slot, c->token_row, c->row_token, c->rows_per_expert, c->G, c->E, c->C,
+                     c->S * c->K, c->K, n, compact_blocks, mlp->R, w.ga, w.gb,
+                     w.streamk != nullptr ? SK::flags(w.streamk) : nullptr,
+                     w.streamk != nullptr ? SK::kFlags : 0);
+  return launch_status();
 }
 
 template <typename PCfg>

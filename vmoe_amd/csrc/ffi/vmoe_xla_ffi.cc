@@ -405,6 +405,86 @@ XLA_FFI_DEFINE_HANDLER_SYMBOL(VmoeExpertMlp, ExpertMlpImpl,
                                   .Attr<bool>("packed").Attr<bool>("has_bias").Attr<bool>("ragged")
                                   .Attr<bool>("gather").Attr<int32_t>("gelu"));
 
+// The MLP with its launch plans already in `workspace` (written by vmoe_compact_rows_planned
+// for the same shapes): bind `workspace` as a result that aliases the operand holding them
+// (input_output_aliases).  Operands and attributes as VmoeExpertMlp with ragged = gather = true.
+static ffi::Error ExpertMlpPlannedImpl(hipStream_t stream, Any x, Any w0, Any b0, Any w1, Any b1,
+                                       S32 rows_per_expert, S32 x_rows, AnyOut out, AnyOut workspace,
+                                       bool packed, bool has_bias, int32_t gelu) {
+  VmoeExpertMlpParams p{};
+  p.x = x.untyped_data();
+  if (packed) {
+    p.w0t = w0.untyped_data();
+    p.w1t = w1.untyped_data();
+  } else {
+    p.w0 = w0.untyped_data();
+    p.w1 = w1.untyped_data();
+  }
+  p.b0 = has_bias ? b0.untyped_data() : nullptr;
+  p.b1 = has_bias ? b1.untyped_data() : nullptr;
+  p.out = out->untyped_data();
+  p.workspace = workspace->untyped_data();
+  p.workspace_bytes = workspace->size_bytes();
+  p.E = (int32_t)out->dimensions()[0];
+  p.R = (int32_t)out->dimensions()[1];
+  p.D = (int32_t)out->dimensions()[2];
+  p.M = packed ? Dim(w0, 1) : Dim(w0, 2);
+  p.dtype = DType(x.element_type());
+  p.gelu = gelu;
+  p.rows_per_expert = rows_per_expert.typed_data();
+  p.x_rows = x_rows.typed_data();
+  p.num_items = (int32_t)(x.element_count() / p.D);
+  return Status(vmoe_expert_mlp_planned(&p, stream), "vmoe_expert_mlp_planned");
+}
+XLA_FFI_DEFINE_HANDLER_SYMBOL(VmoeExpertMlpPlanned, ExpertMlpPlannedImpl,
+                              ffi::Ffi::Bind().Ctx<Stream>().Arg<Any>().Arg<Any>().Arg<Any>().Arg<Any>()
+                                  .Arg<Any>().Arg<S32>().Arg<S32>().Ret<Any>().Ret<Any>()
+                                  .Attr<bool>("packed").Attr<bool>("has_bias").Attr<int32_t>("gelu"));
+
+// Row compaction, launch plans and the MLP of the gathered rows as one custom call (the form
+// in which XLA would use the pair vmoe_compact_rows_planned / vmoe_expert_mlp_planned):
+// fill (G,E), token_slot (G,S,K), items (T,D), weights as VmoeExpertMlp -> token_row (G,S,K),
+// rows_per_expert (E,), row_token (E, G*C), out (E, G*C, D), workspace.
+static ffi::Error CompactRowsPlannedImpl(hipStream_t stream, S32 fill, S32 token_slot, Any x, Any w0,
+                                         Any b0, Any w1, Any b1, S32Out token_row,
+                                         S32Out rows_per_expert, S32Out row_token, AnyOut out,
+                                         AnyOut workspace, int32_t capacity, bool packed,
+                                         bool has_bias, int32_t gelu) {
+  VmoeCompactRowsParams c{};
+  FillCompact(&c, fill, token_slot, token_row, rows_per_expert, row_token, capacity);
+  VmoeExpertMlpParams p{};
+  p.x = x.untyped_data();
+  if (packed) {
+    p.w0t = w0.untyped_data();
+    p.w1t = w1.untyped_data();
+  } else {
+    p.w0 = w0.untyped_data();
+    p.w1 = w1.untyped_data();
+  }
+  p.b0 = has_bias ? b0.untyped_data() : nullptr;
+  p.b1 = has_bias ? b1.untyped_data() : nullptr;
+  p.out = out->untyped_data();
+  p.workspace = workspace->untyped_data();
+  p.workspace_bytes = workspace->size_bytes();
+  p.E = (int32_t)out->dimensions()[0];
+  p.R = (int32_t)out->dimensions()[1];
+  p.D = (int32_t)out->dimensions()[2];
+  p.M = packed ? Dim(w0, 1) : Dim(w0, 2);
+  p.dtype = DType(x.element_type());
+  p.gelu = gelu;
+  p.rows_per_expert = rows_per_expert->typed_data();
+  p.x_rows = row_token->typed_data();
+  p.num_items = (int32_t)(x.element_count() / p.D);
+  ffi::Error e = Status(vmoe_compact_rows_planned(&c, &p, stream), "vmoe_compact_rows_planned");
+  if (e.failure()) return e;
+  return Status(vmoe_expert_mlp_planned(&p, stream), "vmoe_expert_mlp_planned");
+}
+XLA_FFI_DEFINE_HANDLER_SYMBOL(VmoeCompactRowsPlanned, CompactRowsPlannedImpl,
+                              ffi::Ffi::Bind().Ctx<Stream>().Arg<S32>().Arg<S32>().Arg<Any>().Arg<Any>()
+                                  .Arg<Any>().Arg<Any>().Arg<Any>().Ret<S32>().Ret<S32>().Ret<S32>()
+                                  .Ret<Any>().Ret<Any>().Attr<int32_t>("capacity").Attr<bool>("packed")
+                                  .Attr<bool>("has_bias").Attr<int32_t>("gelu"));
+
 // in (batch, rows, cols) -> out (batch, cols, rows)
 static ffi::Error PackExpertWeightsImpl(hipStream_t stream, Any in, AnyOut out) {
   VmoeTransposeParams p{};

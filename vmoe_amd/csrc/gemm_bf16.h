@@ -261,18 +261,33 @@ __device__ __forceinline__ void plan_one(const RaggedGeom& g, const int32_t* til
 // Entry num_blocks of a plan (one past its last workgroup) holds the number of live row
 // tiles, from which a tile-walking kernel derives the length of its die's run; the
 // planning launch also clears the `clear_count` flags of the stream-K exchange.
-__global__ __launch_bounds__(256) void plan_ragged_tiles_kernel(
-    const int32_t* __restrict__ rows, int batch, int R, RaggedGeom ga, RaggedGeom gb,
-    int32_t* __restrict__ clear, int clear_count) {
-  extern __shared__ int32_t tile_prefix[];      // 2 x (batch + 1): live row tiles before batch b
+// One workgroup of the planning launch (block = its index among the planning workgroups).
+// With `fill` (G x batch fill counts of the slot assignment) the row counts are its column
+// sums, added up here, and `rows` is not read: the plan then does not wait for the launch
+// that writes the row counts and can share a launch with it.
+__device__ __forceinline__ void plan_ragged_tiles_block(
+    const int32_t* __restrict__ rows, const int32_t* __restrict__ fill, int G, int batch, int R,
+    const RaggedGeom& ga, const RaggedGeom& gb, int32_t* __restrict__ clear, int clear_count,
+    unsigned block, int32_t* tile_prefix) {
+  // tile_prefix: 2 x (batch + 1) live row tiles before batch b, then `batch` row counts
   __shared__ int32_t wsum[2][4];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   int32_t* pa = tile_prefix;
   int32_t* pb = tile_prefix + batch + 1;
+  int32_t* rows_here = tile_prefix + 2 * (batch + 1);
   int carry_a = 0, carry_b = 0;
   for (int b0 = 0; b0 < batch; b0 += 256) {     // every workgroup scans all batches (few)
     const int bb = b0 + tid;
-    const int n = bb < batch ? min(max(rows[bb], 0), R) : 0;
+    int n = 0;
+    if (bb < batch) {
+      if (fill != nullptr) {
+        for (int g = 0; g < G; ++g) n += fill[(size_t)g * batch + bb];
+      } else {
+        n = rows[bb];
+      }
+      n = min(max(n, 0), R);
+      rows_here[bb] = n;
+    }
     const int ta = (n + ga.bm - 1) / ga.bm, tb = (n + gb.bm - 1) / gb.bm;
     int xa = ta, xb = tb;
 #pragma unroll
@@ -299,14 +314,24 @@ __global__ __launch_bounds__(256) void plan_ragged_tiles_kernel(
   }
   if (tid == 0) { pa[batch] = carry_a; pb[batch] = carry_b; }
   __syncthreads();
-  const int i = blockIdx.x * 256 + tid;
-  plan_one(ga, pa, rows, batch, R, i);
-  plan_one(gb, pb, rows, batch, R, i);
-  if (blockIdx.x == 0) {
+  const int i = block * 256 + tid;
+  plan_one(ga, pa, rows_here, batch, R, i);
+  plan_one(gb, pb, rows_here, batch, R, i);
+  if (block == 0) {
     if (tid == 0 && ga.plan != nullptr) ga.plan[ga.num_blocks] = PlanEntry{pa[batch], 0, 0, 0};
     if (tid == 0 && gb.plan != nullptr) gb.plan[gb.num_blocks] = PlanEntry{pb[batch], 0, 0, 0};
     for (int c = tid; c < clear_count; c += 256) clear[c] = 0;
   }
+}
+
+// LDS of a planning workgroup.
+inline size_t plan_ragged_tiles_lds(int batch) { return ((size_t)2 * (batch + 1) + batch) * sizeof(int32_t); }
+
+__global__ __launch_bounds__(256) void plan_ragged_tiles_kernel(
+    const int32_t* __restrict__ rows, int batch, int R, RaggedGeom ga, RaggedGeom gb,
+    int32_t* __restrict__ clear, int clear_count) {
+  extern __shared__ int32_t tile_prefix[];
+  plan_ragged_tiles_block(rows, nullptr, 0, batch, R, ga, gb, clear, clear_count, blockIdx.x, tile_prefix);
 }
 
 __global__ __launch_bounds__(256) void clear_i32_kernel(int32_t* __restrict__ p, int n) {

@@ -19,6 +19,7 @@
 #include <mutex>
 #include "vmoe_common.h"
 #include "router_metrics.h"
+#include "compact_rows.h"
 
 namespace vmoe {
 namespace {
@@ -447,45 +448,8 @@ __global__ __launch_bounds__(256) void compact_rows_fused_kernel(
     const int32_t* __restrict__ fill, const int32_t* __restrict__ token_slot,
     int32_t* __restrict__ token_row, int32_t* __restrict__ row_token,
     int32_t* __restrict__ rows_per_expert, int G, int E, int C, int per_group, int K, size_t n) {
-  __shared__ int32_t part[256];
-  __shared__ int32_t before[2][256];
-  const int tid = threadIdx.x;
-  const size_t i0 = (size_t)blockIdx.x * 256;
-  const int g_lo = (int)(i0 / per_group);
-  const int parts = 256 / E;
-  const int e_t = tid % E, q = tid / E;
-  auto column_sum = [&](int g_end) {   // sum of fill[0 .. g_end) [e], valid in threads tid < E
-    int acc = 0;
-    if (q < parts)
-      for (int g = q; g < g_end; g += parts) acc += fill[(size_t)g * E + e_t];
-    part[tid] = acc;
-    __syncthreads();
-    int total = 0;
-    if (tid < E)
-      for (int j = 0; j < parts; ++j) total += part[j * E + tid];
-    __syncthreads();
-    return total;
-  };
-  const int lo = column_sum(g_lo);
-  if (tid < E) {
-    before[0][tid] = lo;
-    before[1][tid] = lo + (g_lo < G ? fill[(size_t)g_lo * E + tid] : 0);
-  }
-  if (blockIdx.x == 0) {
-    const int total = column_sum(G);
-    if (tid < E) rows_per_expert[tid] = total;
-  }
-  __syncthreads();
-  const size_t i = i0 + tid;
-  if (i >= n) return;
-  const int slot = token_slot[i];
-  int row = -1;
-  if (slot >= 0) {
-    const int g = (int)(i / per_group);
-    row = packed_row(slot, before[g - g_lo][slot_expert(slot, G, C)], G, C);
-    if (row_token != nullptr) row_token[row] = (int)(i / K);
-  }
-  token_row[i] = row;
+  compact_rows_fused_block(fill, token_slot, token_row, row_token, rows_per_expert, G, E, C,
+                           per_group, K, n, blockIdx.x);
 }
 
 }  // namespace
@@ -653,8 +617,7 @@ extern "C" int vmoe_top_items_per_expert(const VmoeTopItemsParams* p, vmoe_strea
 static int launch_compact_rows(const VmoeCompactRowsParams* p, int32_t* prefix,
                                vmoe_stream_t stream) {
   const size_t n = (size_t)p->G * p->S * p->K;
-  const int parts = p->E <= 256 ? 256 / p->E : 1;
-  if (p->E <= 256 && (int64_t)p->S * p->K >= 256 && (p->G + parts - 1) / parts <= 16) {
+  if (compact_rows_fused_ok(p->G, p->S, p->E, p->K)) {
     hipLaunchKernelGGL(compact_rows_fused_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0,
                        as_stream(stream), p->fill, p->token_slot, p->token_row, p->row_token,
                        p->rows_per_expert, p->G, p->E, p->C, p->S * p->K, p->K, n);

@@ -6,6 +6,7 @@ on a ROCm device and are used as raw device pointers on torch's current stream.
 from __future__ import annotations
 
 import ctypes
+import os
 from typing import Optional, Tuple
 
 import torch
@@ -91,6 +92,9 @@ def router_metrics(gates: torch.Tensor, topk_idx: torch.Tensor, gshard_loss_weig
                             topk_idx.shape[-1], H.dtype_code(gates.dtype))
   H.call("vmoe_router_metrics", p)
   return imp, gsh, aux
+
+
+_E_UNSUPPORTED = -6
 
 
 def route_assign(topk_val: Optional[torch.Tensor], topk_idx: torch.Tensor, num_experts: int,
@@ -261,11 +265,24 @@ def pack_expert_weights(w: torch.Tensor) -> torch.Tensor:
 def expert_mlp(x: torch.Tensor, w0, b0, w1, b1, w0t=None, w1t=None, approximate_gelu: bool = True,
                workspace: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None,
                rows_per_expert: Optional[torch.Tensor] = None,
-               x_rows: Optional[torch.Tensor] = None):
+               x_rows: Optional[torch.Tensor] = None, compact=None):
   """x (E,R,D) -> (E,R,D): gelu(x @ w0 + b0) @ w1 + b1 per expert; with rows_per_expert (E,)
   int32 only that many leading rows of every expert are computed.  With x_rows (E,R) int32,
   x is the (T,D) matrix of items and x_rows names the item of every row (gathered by the
-  first product; see expert_mlp_can_gather)."""
+  first product; see expert_mlp_can_gather).
+
+  With ``compact=(fill (G,E), token_slot (G,S,K), capacity)`` x is the (T,D) matrix of items
+  and the packed rows are computed here, in the launch that plans the products (what
+  compact_rows gives is returned as well): -> (out, (token_row, rows_per_expert, row_token))."""
+  maps = None
+  if compact is not None:
+    fill, token_slot, capacity = compact
+    G, E = fill.shape
+    _, S, K = token_slot.shape
+    token_row = _i32(G, S, K, device=fill.device)
+    rows_per_expert = _i32(E, device=fill.device)
+    x_rows = _i32(E, G * capacity, device=fill.device)
+    maps = (token_row, rows_per_expert, x_rows)
   num_items = 0
   if x_rows is not None:
     E, R = x_rows.shape
@@ -285,8 +302,23 @@ def expert_mlp(x: torch.Tensor, w0, b0, w1, b1, w0t=None, w1t=None, approximate_
     workspace = torch.empty(need, dtype=torch.uint8, device=x.device)
   p.workspace = H.ptr(workspace)
   p.workspace_bytes = workspace.numel() * workspace.element_size()
-  H.call("vmoe_expert_mlp", p)
-  return out
+  if compact is None:
+    H.call("vmoe_expert_mlp", p)
+    return out
+  c = H.CompactRowsParams(H.ptr(fill), H.ptr(token_slot), H.ptr(maps[0]), H.ptr(maps[1]),
+                          H.ptr(None), H.ptr(maps[2]), G, S, E, K, capacity)
+  # (VMOE_PLAN_SEPARATE_LAUNCH=1 in the environment keeps the planning launch apart: the
+  # switch behind the before / after figures)
+  rc = _E_UNSUPPORTED
+  if not os.environ.get("VMOE_PLAN_SEPARATE_LAUNCH"):
+    rc = H.call_blocks("vmoe_compact_rows_planned", c, p, accept=(_E_UNSUPPORTED,))
+  if rc == 0:
+    H.call("vmoe_expert_mlp_planned", p)
+  else:
+    c.prefix = H.ptr(_i32(G, E, device=fill.device))
+    H.call("vmoe_compact_rows", c)
+    H.call("vmoe_expert_mlp", p)
+  return out, maps
 
 
 def expert_mlp_can_gather(dtype: torch.dtype, D: int, num_items: int) -> bool:

@@ -223,6 +223,17 @@ class ExpertIndicesDispatcher(BaseDispatcher):
       self._packed_maps = K.compact_rows(self.fill, token_slot, self.capacity)
     return self._packed_maps
 
+  def pending_compaction(self):
+    """-> (fill, token_slot, capacity) while the packed rows have not been computed (an
+    expert that computes them itself hands them back with set_packed_maps), else None."""
+    if self._packed_maps is not None or self.fill is None:
+      return None
+    token_slot, _ = self._maps()
+    return self.fill, token_slot, self.capacity
+
+  def set_packed_maps(self, maps) -> None:
+    self._packed_maps = tuple(maps)
+
   def packed_rows(self):
     """-> (row_token (E, G * capacity) int32: the item (g * S + s) in every packed row,
     rows_per_expert (E,) int32): what an expert needs to gather its rows itself."""
@@ -359,6 +370,12 @@ class _SparseEinsumDispatcher(EinsumDispatcher):
 
   def packed_rows(self):
     return self._inner.packed_rows()
+
+  def pending_compaction(self):
+    return self._inner.pending_compaction()
+
+  def set_packed_maps(self, maps) -> None:
+    self._inner.set_packed_maps(maps)
 
   def combine_packed(self, data: Array) -> Array:
     return self._inner.combine_packed(data)
@@ -653,8 +670,15 @@ def sparse_moe_spmd(target, variable_axes: Optional[Mapping[str, Any]] = None,
         if (gather is not None and packed_rows is not None and x.ndim == 3
             and self.expert.can_gather(x)):
           # ... and fetches them from the items itself: no dispatched buffer at all.
-          row_token, rows_per_expert = packed_rows()
-          outputs = gather(variables, x.reshape(-1, x.shape[-1]), row_token, rows_per_expert)
+          routed = getattr(self.expert, "apply_experts_routed", None)
+          pending = getattr(dispatcher, "pending_compaction", None)
+          todo = pending() if (routed is not None and pending is not None) else None
+          if todo is not None:    # the packed rows come out of the expert's planning launch
+            outputs, maps = routed(variables, x.reshape(-1, x.shape[-1]), *todo)
+            dispatcher.set_packed_maps(maps)
+          else:
+            row_token, rows_per_expert = packed_rows()
+            outputs = gather(variables, x.reshape(-1, x.shape[-1]), row_token, rows_per_expert)
         else:
           dispatched, rows_per_expert = dispatcher.dispatch_packed(x)
           outputs = self.expert.apply_experts(variables, dispatched,

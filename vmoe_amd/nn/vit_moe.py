@@ -94,6 +94,23 @@ class MlpBlock(module.Module):
                         approximate_gelu=self.approximate_gelu, rows_per_expert=rows_per_expert,
                         x_rows=row_token)
 
+  def apply_experts_routed(self, variables, items: Array, fill: Array, token_slot: Array,
+                           capacity: int):
+    """apply_experts_gathered for a dispatcher whose packed rows are still to be computed:
+    items (T, D), fill (G, E) and token_slot (G, S, K) of the slot assignment -> (outputs
+    (E, G * capacity, D), (token_row, rows_per_expert, row_token)).  The renumbering of the
+    assignments shares a launch with the planning of the two products."""
+    p = variables["params"]
+    dtype = self.dtype or items.dtype
+    w0, b0 = p["Dense_0"]["kernel"], p["Dense_0"].get("bias")
+    w1, b1 = p["Dense_1"]["kernel"], p["Dense_1"].get("bias")
+    module.require_no_grad("MlpBlock", items, w0, b0, w1, b1)
+    cast = lambda t: None if t is None else K.cast(t, dtype)
+    return K.expert_mlp(K.cast(items, dtype), None, cast(b0), None, cast(b1),
+                        w0t=self._pack(w0, dtype), w1t=self._pack(w1, dtype),
+                        approximate_gelu=self.approximate_gelu,
+                        compact=(fill, token_slot, capacity))
+
   def apply(self, variables, inputs: Array) -> Array:
     """Single MLP: inputs (..., D)."""
     stacked = vmoe_amd.moe._tree_map(lambda t: t[None], variables)
