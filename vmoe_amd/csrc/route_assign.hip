@@ -126,6 +126,8 @@ __device__ __forceinline__ void bitonic_sort_lds(uint64_t* keys, int SP, int tid
   }
 }
 
+constexpr int kRankBins = 1024;    // bins of the counting rank: gates from 1 down to 2^-8
+
 template <int R>
 __device__ __forceinline__ void route_assign_group(
     const float* __restrict__ topk_val, const int32_t* __restrict__ topk_idx,
@@ -166,7 +168,70 @@ __device__ __forceinline__ void route_assign_group(
         bits[r] = (tid < nact && s < S) ? __builtin_bit_cast(uint32_t, val[(size_t)s * K]) : 0u;
         narrow_ok = narrow_ok && bpr_gate_is_narrow(bits[r]);
       }
-      if (__syncthreads_and(narrow_ok)) {
+      // Narrow gates within a factor 2^8 of 1 (the largest gate of a softmax over up to 128
+      // experts always is) take at most kRankBins distinct values, in descending order as
+      // the bin number 0x3F80 - (bits >> 16) ascends: the rank of an item is then the number
+      // of items in lower bins plus the number of items of its own bin with a lower index
+      // -- a histogram, a prefix sum, a scatter into the bins' segments and a count inside
+      // the item's own segment, four barriers in all, where the bitonic sort of 2 048 keys
+      // takes 66 compare-exchange steps (15 of the kernel's 22 us on the headline layer).
+      // Every step counts, none depends on the order in which the threads arrive, so the
+      // ranks are those of the sort.  A segment as long as the group (all gates equal) costs
+      // what the sort costs.
+      bool count_ok = narrow_ok;
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        const uint32_t hi = bits[r] >> 16;
+        if (tid < nact && tid * R + r < S) count_ok = count_ok && hi <= 0x3F80u && hi + kRankBins > 0x3F80u;
+      }
+      if (__syncthreads_and(count_ok)) {
+        uint32_t* hist = reinterpret_cast<uint32_t*>(keys);      // items per bin, then the bins' cursors
+        uint32_t* start = hist + kRankBins;                      // first rank of each bin
+        uint32_t* seg = start + kRankBins;                       // S items, bin by bin
+        for (int i = tid; i < kRankBins; i += kRouteThreads) hist[i] = 0u;
+        __syncthreads();
+        int bin[R];
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+          bin[r] = (int)(0x3F80u - (bits[r] >> 16));
+          if (tid < nact && tid * R + r < S) atomicAdd(&hist[bin[r]], 1u);
+        }
+        __syncthreads();
+        // Exclusive prefix over the bins: kRankBins == kRouteThreads, one bin per thread.
+        {
+          static_assert(kRankBins == kRouteThreads, "one bin per thread");
+          const int lane = tid & 63, wave = tid >> 6;
+          const uint32_t c = hist[tid];
+          uint32_t incl = c;
+#pragma unroll
+          for (int d = 1; d < 64; d <<= 1) {
+            const uint32_t o = __shfl_up(incl, d, kWave);
+            if (lane >= d) incl += o;
+          }
+          __shared__ uint32_t wave_total[kRouteThreads / 64];
+          if (lane == 63) wave_total[wave] = incl;
+          __syncthreads();
+          uint32_t before = 0;
+          for (int w = 0; w < wave; ++w) before += wave_total[w];
+          start[tid] = before + incl - c;
+          hist[tid] = before + incl - c;                       // cursor of the scatter
+        }
+        __syncthreads();
+#pragma unroll
+        for (int r = 0; r < R; ++r)
+          if (tid < nact && tid * R + r < S) seg[atomicAdd(&hist[bin[r]], 1u)] = (uint32_t)(tid * R + r);
+        __syncthreads();
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+          const int item = tid * R + r;
+          if (tid < nact && item < S) {
+            const uint32_t first = start[bin[r]], end = hist[bin[r]];
+            uint32_t lower = 0;
+            for (uint32_t q = first; q < end; ++q) lower += seg[q] < (uint32_t)item ? 1u : 0u;
+            rank[item] = (int)(first + lower);
+          }
+        }
+      } else if (__syncthreads_and(narrow_ok)) {
         uint32_t key[R];
 #pragma unroll
         for (int r = 0; r < R; ++r) {
@@ -477,7 +542,10 @@ static int launch_route_assign(const VmoeRouteAssignParams* p, const VmoeRouterM
   const int SP = pow2ceil(p->S);
   const int W = (p->S * p->K + 31) / 32;
   const int R = keys_per_thread(SP);
-  const int NK = SP;
+  // (the region of the sort keys also serves the counting rank: two arrays of kRankBins
+  // words and one of S)
+  const int rank_words = 2 * kRankBins + p->S;
+  const int NK = SP > (rank_words + 1) / 2 ? SP : (rank_words + 1) / 2;
   size_t lds = (p->batch_priority ? (size_t)NK * 8 : 0) + (size_t)p->E * W * 8 +
                (size_t)p->S * 4 + (size_t)p->E * 4;
   RouterMetricsArgs ma{};
