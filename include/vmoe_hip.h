@@ -131,8 +131,8 @@ int vmoe_router_metrics(const VmoeRouterMetricsParams* p, vmoe_stream_t stream);
  * the item index, or with batch_priority the stable descending order of
  * topk_val[:,0].  Positions are not clipped; an assignment is kept iff
  * position < C.  Experts outside [0,E) get position -1.
- * Limits: 8*max(1024, pow2ceil(S)) (with batch_priority) + 8*E*ceil(S*K/32) + 4*S + 4*E
- * bytes of LDS <= 160 KiB.
+ * Limits: 8*max(pow2ceil(S), 1024 + ceil(S/2)) (with batch_priority) + 8*E*ceil(S*K/32) +
+ * 4*S + 4*E bytes of LDS <= 160 KiB.
  */
 typedef struct {
   const float* topk_val;   /* (G, S, K); only [:, :, 0] is read, and only with batch_priority */
