@@ -50,18 +50,18 @@ PEAK_HBM_GBS = 8000.0
 # HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc runs
 # (FETCH_SIZE + WRITE_SIZE, scaled by a copy kernel of known size); None until measured.
 MEASURED_TRAFFIC_BYTES = {
-    # mean of the two GEMM launches of a layer: (632 + 565 + 1099 + 182) / 2 MiB;
+    # mean of the two GEMM launches of a layer: (630 + 565 + 1096 + 182) / 2 MiB;
     # FETCH_SIZE x 2.0, WRITE_SIZE x 1.0 (copy-kernel calibration);
     # profiles/hbm_traffic__vmoe_b16_layer.md.
-    "vmoe_b16_layer_E32_k2_bpr": 1.299e9,
+    "vmoe_b16_layer_E32_k2_bpr": 1.297e9,
 }
 # Share of the launch during which the matrix cores are busy (SQ_VALU_MFMA_BUSY_CYCLES over
 # GRBM_GUI_ACTIVE x 1 024 SIMDs), from the rocprofv3 --pmc runs of this command summarised in
 # profiles/mfma_util__vmoe_b16_layer.md: counters cannot be read from inside the run.
 MEASURED_MFMA_BUSY = {
     "vmoe_b16_layer_E32_k2_bpr": {
-        "first_product": 0.424, "second_product": 0.598, "vendor_gemm_second_product_shape": 0.539,
-        "register_resident_mfma_loop": 0.938,
+        "first_product": 0.451, "second_product": 0.599, "vendor_gemm_second_product_shape": 0.536,
+        "register_resident_mfma_loop": 0.937,
         "source": "profiles/mfma_util__vmoe_b16_layer.md (rocprofv3 --pmc, same command, 5 steps)"},
 }
 
@@ -428,7 +428,7 @@ def vit_main(args):
                  "tokens": T, "blocks": enc["num_layers"], "moe_blocks": list(moe_cfg["layers"]),
                  "experts": moe_cfg["num_experts"], "selected": 2, "group_size": moe_cfg["group_size"],
                  "capacity_factor": 1.05},
-      "roofline": {"bound": "mfma", "kernel": "gemm_bf16_kernel (first product) / gemm_bf16_persistent_kernel (second product)", "achieved": achieved,
+      "roofline": {"bound": "mfma", "kernel": "gemm_bf16_mixed_kernel (first product) / gemm_bf16_persistent_kernel (second product)", "achieved": achieved,
                    "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": achieved / PEAK_BF16_TFLOPS,
                    "traffic": None, "launch_ms": mlp_ms / (2 * enc["num_layers"]),
                    "flops_all_mlps": flops_mlp, "kept_rows_per_moe_block": kept_per_block,
@@ -586,7 +586,7 @@ def main():
   achieved_tflops = flops_per_launch / (gemm_ms * 1e-3) / 1e12
   peak = PEAK_BF16_TFLOPS if tdt == torch.bfloat16 else PEAK_FP32_MATRIX_TFLOPS
   roofline = {"bound": "mfma",
-              "kernel": "gemm_bf16_kernel (first product) / gemm_bf16_persistent_kernel (second product)" if b == 2 else "gemm_f32_kernel",
+              "kernel": "gemm_bf16_mixed_kernel (first product) / gemm_bf16_persistent_kernel (second product)" if b == 2 else "gemm_f32_kernel",
               "achieved": achieved_tflops, "peak": peak, "unit": "TFLOP/s",
               "frac": achieved_tflops / peak, "traffic": MEASURED_TRAFFIC_BYTES.get(cfg.name),
               "mfma_busy": MEASURED_MFMA_BUSY.get(cfg.name),
