@@ -370,7 +370,8 @@ typedef struct {
   void* dispatch_w;   /* out (G, S, N) dtype */
   void* combine_w;    /* out (G, S, N) dtype */
   void* logits;       /* optional out (G, S, N) dtype */
-  void* workspace;    /* D*N*sizeof(float) bytes for the unit-norm, scaled mu */
+  void* workspace;    /* vmoe_soft_route_workspace_bytes() bytes for the unit-norm, scaled mu (the
+                         order is the kernel's own: for bfloat16 the order of its MFMA fragments) */
   size_t workspace_bytes;
   int32_t G, S, D, N;
   int32_t dtype;

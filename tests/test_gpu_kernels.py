@@ -1,4 +1,5 @@
 """Parity of each HIP kernel (called through the C ABI) against the CPU oracle."""
+import os
 import numpy as np
 import pytest
 import torch
@@ -438,6 +439,10 @@ SOFT_CASES = [
     (1, 20, 768, 64, 2, O.BF16),      # inputs smaller than mu on the bf16 path
     (2, 64, 768, 20, 1, O.BF16),      # N % 8 != 0: generic path
     (2, 64, 320, 16, 1, O.BF16),      # width outside the fast path
+    # two-role kernel with 16-row item tiles (two 32-row tiles do not fit LDS beside the
+    # logits): dispatch softmax from registers (S <= 256) and in three passes
+    (1, 250, 768, 128, 1, O.BF16),
+    (2, 260, 768, 128, 1, O.BF16),
 ]
 
 
@@ -457,6 +462,29 @@ def test_soft_route(K, G, S, D, n, p, dtype):
   atol = 1e-4 if dtype == O.F32 else 3e-2
   np.testing.assert_allclose(to_np(dw).sum(1), 1.0, atol=atol)
   np.testing.assert_allclose(to_np(cw).sum(2), 1.0, atol=atol)
+
+
+@pytest.mark.parametrize("G,S,D,N", [(5, 196, 768, 128), (2, 250, 768, 128), (3, 100, 512, 64),
+                                     (2, 300, 256, 104), (2, 37, 384, 40)])
+def test_soft_route_two_roles_and_single_role_agree(K, G, S, D, N):
+  """The kernel whose waves split into producers and consumers against the single-role kernel
+  (VMOE_SOFT_ROUTE_SINGLE_ROLE=1): same arithmetic per element, different summation order in
+  the norms and softmax sums: a norm that rounds the other way moves a normalised item by one
+  bfloat16 step, a logit by about as much, and a weight by up to exp(step) - 1, in few places."""
+  rng = np.random.default_rng(G * S + N)
+  x = to_dev(O.cast(rng.standard_normal((G, S, D)), O.BF16), O.BF16)
+  mu = to_dev(O.cast(rng.standard_normal((D, N)) / np.sqrt(D), O.BF16), O.BF16)
+  got = [to_np(a) for a in K.soft_route(x, mu, 1.3, return_logits=True)]
+  os.environ["VMOE_SOFT_ROUTE_SINGLE_ROLE"] = "1"
+  try:
+    want = [to_np(a) for a in K.soft_route(x, mu, 1.3, return_logits=True)]
+  finally:
+    del os.environ["VMOE_SOFT_ROUTE_SINGLE_ROLE"]
+  for name, a, b in zip(("dispatch weights", "combine weights", "logits"), got, want):
+    diff = np.abs(a - b)
+    floor = 2.0 ** -7 * np.abs(b).max() if name == "logits" else 0.0
+    assert (diff <= 2.0 ** -5 * np.abs(b) + floor).all(), (name, float((diff / (np.abs(b) + 1e-30)).max()))
+    assert (diff > 0).mean() <= 1e-3, (name, float((diff > 0).mean()))
 
 
 EINSUM_CASES = [

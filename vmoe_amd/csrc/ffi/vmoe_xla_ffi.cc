@@ -498,7 +498,7 @@ XLA_FFI_DEFINE_HANDLER_SYMBOL(VmoePackExpertWeights, PackExpertWeightsImpl,
                               ffi::Ffi::Bind().Ctx<Stream>().Arg<Any>().Ret<Any>());
 
 // ---------------------------------------------------------------- Soft MoE
-// x (G,S,D), mu (D,N) -> dispatch_w, combine_w, logits (G,S,N), workspace (D*N f32)
+// x (G,S,D), mu (D,N) -> dispatch_w, combine_w, logits (G,S,N), workspace (vmoe_soft_route_workspace_bytes)
 static ffi::Error SoftRouteImpl(hipStream_t stream, Any x, Any mu, AnyOut dispatch_w, AnyOut combine_w,
                                 AnyOut logits, AnyOut workspace, float scale, bool want_logits) {
   VmoeSoftRouteParams p{};

@@ -4,7 +4,9 @@
 // group normalises the item rows, multiplies them with the unit-norm slot
 // parameters on the matrix cores, keeps the (S x N) logits of the group in LDS
 // and takes both softmaxes (over items for the dispatch weights, over slots for
-// the combine weights) from that one copy.
+// the combine weights) from that one copy.  The bfloat16 kernel for the model
+// widths up to 768 splits the waves of a workgroup into two roles
+// (soft_route_roles_kernel).
 //
 // einsum_dispatch / einsum_combine replace EinsumDispatcher.dispatch/.combine
 // (vmoe/moe.py:148-161) for dense weights, including the expert-buffer row
@@ -13,6 +15,8 @@
 // reference promotes bf16 data to the weights' dtype), and a lane's operands
 // are single scalars, so neither the (S, N) weights nor the (rows, D) data need
 // a transposed copy.
+#include <algorithm>
+
 #include "vmoe_common.h"
 #include "einsum_bf16.h"
 
@@ -38,12 +42,26 @@ __device__ __forceinline__ void store_any(void* p, size_t i, float v, int dtype)
 // Unit-normalise the columns of mu (D, N) and apply the scale when it belongs to
 // mu.  bf16: writes muT (N, D) so that a column's k run is contiguous;
 // f32: writes (D, N).
+// frag_ksw > 0 (bf16, D = 32 * frag_ksw): the order in which soft_route_roles_kernel's
+// consumer waves hold the parameters, [slot / 32][slot % 32 / 16][d / 32][lane][d % 8]
+// with lane = (d % 32 / 8) * 16 + slot % 16, so that every fragment load of a wave is
+// 1 KB of consecutive memory; the grid then covers the slots up to a multiple of 32 and
+// the ones past N are zeros.
 template <typename T>
 __global__ __launch_bounds__(256) void soft_prep_mu_kernel(const T* __restrict__ mu,
                                                            T* __restrict__ out, float scale,
-                                                           int scale_mu, int D, int N) {
+                                                           int scale_mu, int D, int N,
+                                                           int frag_ksw = 0) {
   __shared__ float red[256];
   const int n = blockIdx.x, tid = threadIdx.x;
+  auto frag_index = [&](int d) -> size_t {
+    const int lane = ((d & 31) >> 3) * 16 + (n & 15);
+    return ((((size_t)(n >> 5) * 2 + ((n & 31) >> 4)) * frag_ksw + (d >> 5)) * 64 + lane) * 8 + (d & 7);
+  };
+  if (n >= N) {     // padding slots of the fragment order
+    for (int d = tid; d < D; d += 256) Elt<T>::store(out + frag_index(d), 0.f);
+    return;
+  }
   float s = 0.f;
   for (int d = tid; d < D; d += 256) {
     float v = Elt<T>::load(mu + (size_t)d * N + n);
@@ -60,7 +78,8 @@ __global__ __launch_bounds__(256) void soft_prep_mu_kernel(const T* __restrict__
   for (int d = tid; d < D; d += 256) {
     float v = Elt<T>::round(Elt<T>::load(mu + (size_t)d * N + n) * inv);
     if (scale_mu) v = Elt<T>::round(v * sc);
-    if (sizeof(T) == 2) Elt<T>::store(out + (size_t)n * D + d, v);
+    if (frag_ksw > 0) Elt<T>::store(out + frag_index(d), v);
+    else if (sizeof(T) == 2) Elt<T>::store(out + (size_t)n * D + d, v);
     else Elt<T>::store(out + (size_t)d * N + n, v);
   }
 }
@@ -483,6 +502,423 @@ __global__ __launch_bounds__(kSrThreads) void soft_route_bf16_kernel(
   }
 }
 
+// Reductions over the 32 lanes of a half wave: four DPP steps inside a row of 16 lanes
+// (quad_perm [1,0,3,2], quad_perm [2,3,0,1], row_half_mirror, row_mirror), then one exchange
+// between the two rows.  Every lane ends with the result.
+template <int CTRL>
+__device__ __forceinline__ float dpp_lane(float v) {
+  return __builtin_bit_cast(
+      float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true));
+}
+__device__ __forceinline__ float half_wave_sum(float v) {
+  v += dpp_lane<0xB1>(v);
+  v += dpp_lane<0x4E>(v);
+  v += dpp_lane<0x141>(v);
+  v += dpp_lane<0x140>(v);
+  return v + __shfl_xor(v, 16, kWave);
+}
+__device__ __forceinline__ float half_wave_max(float v) {
+  v = fmaxf(v, dpp_lane<0xB1>(v));
+  v = fmaxf(v, dpp_lane<0x4E>(v));
+  v = fmaxf(v, dpp_lane<0x141>(v));
+  v = fmaxf(v, dpp_lane<0x140>(v));
+  return fmaxf(v, __shfl_xor(v, 16, kWave));
+}
+
+// soft_route_bf16_kernel with the waves of a workgroup in two roles (N <= 128 slots,
+// D = 32 * KSW <= 768).  In the single-role kernel every wave normalises rows (VALU), then
+// every wave multiplies (LDS reads and matrix cores), then every wave takes the row
+// softmax (VALU): the units take turns.  Here waves 0..3 only fetch and normalise item rows
+// (tile t + 1 into one of two LDS tiles) while waves 4..7, each with the unit-norm
+// parameters of 32 slots in registers, multiply tile t and take the combine weights of
+// tile t - 1; one barrier per tile hands the tiles over.  A consumer wave reads an item
+// tile once for 32 slots (the single-role kernel: once per 16), so the LDS reads halve as
+// well.  The arithmetic per element is that of soft_route_bf16_kernel.
+struct SoftPipeLds {
+  size_t xs, red, cmx, csum, lg, total;
+};
+inline SoftPipeLds soft_pipe_lds_layout(int D, int SP, int NP, int rows) {
+  SoftPipeLds l;
+  l.xs = 0;                                           // two tiles of `rows` normalised rows
+  l.red = 0;                                          // (the column reductions reuse them)
+  l.cmx = l.xs + (size_t)2 * rows * (D + 16) * 2;
+  l.csum = l.cmx + 128 * sizeof(float);
+  l.lg = l.csum + 128 * sizeof(float);
+  l.total = l.lg + (size_t)SP * (NP + 8) * 2;
+  return l;
+}
+
+constexpr int kTailRows = 8;   // rows per thread of the register-resident dispatch softmax
+template <int KSW, int ROWS, bool SCALE_X>
+__global__ __launch_bounds__(kSrThreads) void soft_route_roles_kernel(
+    const bf16_t* __restrict__ x, const bf16_t* __restrict__ muw, bf16_t* __restrict__ dispatch_w,
+    bf16_t* __restrict__ combine_w, bf16_t* __restrict__ logits_out, float scale, int S, int D,
+    int N, int SP, int NP, SoftPipeLds L) {
+  constexpr int CP = (KSW + 7) / 8;   // 16-byte pieces of an item row per lane of a half wave
+  constexpr int RPW = ROWS / 4;       // rows of a tile per producer wave
+  constexpr int PAIRS = RPW / 2;      // a half wave takes one row at a time
+  constexpr int RB = ROWS / 16;       // 16-row blocks of a tile
+  static_assert(ROWS == 16 || ROWS == 32, "tile height");
+  extern __shared__ __align__(16) unsigned char smem[];
+  bf16_t* xs = reinterpret_cast<bf16_t*>(smem + L.xs);
+  float* red = reinterpret_cast<float*>(smem + L.red);
+  float* cmx = reinterpret_cast<float*>(smem + L.cmx);
+  float* csum = reinterpret_cast<float*>(smem + L.csum);
+  bf16_t* lg = reinterpret_cast<bf16_t*>(smem + L.lg);
+  const int LDX = D + 16, LDW = NP + 8;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int m = lane & 31, h = lane >> 5;
+  const int g = blockIdx.x;
+  const bf16_t* xg = x + (size_t)g * S * D;
+  const float sc = bf16r(scale);
+  const int row_chunks = D / 8, row_tiles = SP / ROWS;
+  bf16_t* const xtile[2] = {xs, xs + (size_t)ROWS * LDX};
+
+  // Combine weights of the item rows [s_begin, s_end) of one tile: softmax over the N slots.
+  // The four waves of a role share the tile; half wave = one row, lane = four consecutive
+  // slots.  The producers take them (tile t - 1 while tile t is multiplied): the consumers'
+  // iteration is the longer one (its fragment reads keep the LDS busy).
+  constexpr int CR = ROWS / 8;    // rows of a tile per half wave: their chains overlap
+  auto combine_rows = [&](int s_begin, int s_end) {
+    {
+      const int s0 = s_begin + (wave & 3) * (ROWS / 4);
+      const int c = m * 4;
+      float l[CR][4], mx[CR];
+#pragma unroll
+      for (int r = 0; r < CR; ++r) {
+        const int s = s0 + 2 * r + h;
+#pragma unroll
+        for (int u = 0; u < 4; ++u) l[r][u] = -INFINITY;
+        if (s < s_end && c < N) {
+          const uint2 pr = *reinterpret_cast<const uint2*>(lg + (size_t)s * LDW + c);
+          l[r][0] = bf_lo(pr.x); l[r][1] = bf_hi(pr.x); l[r][2] = bf_lo(pr.y); l[r][3] = bf_hi(pr.y);
+        }
+        mx[r] = fmaxf(fmaxf(l[r][0], l[r][1]), fmaxf(l[r][2], l[r][3]));
+      }
+#pragma unroll
+      for (int r = 0; r < CR; ++r) mx[r] = half_wave_max(mx[r]);
+      float e[CR][4], sum[CR];
+#pragma unroll
+      for (int r = 0; r < CR; ++r) {
+        const float mb = mx[r] * kLog2e;
+        sum[r] = 0.f;
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          e[r][u] = __builtin_amdgcn_exp2f(fmaf(l[r][u], kLog2e, -mb));   // exp2(-inf) = 0 past N
+          sum[r] += e[r][u];
+        }
+      }
+#pragma unroll
+      for (int r = 0; r < CR; ++r) sum[r] = half_wave_sum(sum[r]);
+#pragma unroll
+      for (int r = 0; r < CR; ++r) {
+        const int s = s0 + 2 * r + h;
+        const float rs = __builtin_amdgcn_rcpf(sum[r]);
+        if (s < s_end && c < N)
+          *reinterpret_cast<uint2*>(combine_w + ((size_t)g * S + s) * N + c) = make_uint2(
+              pack_bf16x2(e[r][0] * rs, e[r][1] * rs), pack_bf16x2(e[r][2] * rs, e[r][3] * rs));
+      }
+    }
+  };
+  if (wave < 4) {
+    // ---- producers: item rows wave * RPW .. + RPW of every tile
+    auto load_rows = [&](uint4 (&raw)[PAIRS][CP], int t) {
+#pragma unroll
+      for (int i = 0; i < PAIRS; ++i) {
+        const int r = min(t * ROWS + wave * RPW + 2 * i + h, S - 1);   // rows past S: zeros below
+#pragma unroll
+        for (int ps = 0; ps < CP; ++ps) {
+          const int c = min(ps * 32 + m, row_chunks - 1);
+          raw[i][ps] = *reinterpret_cast<const uint4*>(xg + (size_t)r * D + c * 8);
+        }
+      }
+    };
+    auto norm_rows = [&](uint4 (&raw)[PAIRS][CP], int t, bf16_t* xt) {
+#pragma unroll
+      for (int i = 0; i < PAIRS; ++i) {
+        float sq = 0.f;
+#pragma unroll
+        for (int ps = 0; ps < CP; ++ps) {
+          const uint32_t w4[4] = {raw[i][ps].x, raw[i][ps].y, raw[i][ps].z, raw[i][ps].w};
+          float tsum = 0.f;
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            const float lo = bf_lo(w4[q]), hi = bf_hi(w4[q]);
+            tsum = fmaf(lo, lo, tsum);
+            tsum = fmaf(hi, hi, tsum);
+          }
+          if (KSW % 8 == 0 || ps * 32 + m < row_chunks) sq += tsum;
+        }
+        sq = half_wave_sum(sq);
+        const int lrow = wave * RPW + 2 * i + h;
+        const float inv = t * ROWS + lrow < S ? 1.0f / sqrtf(sq + kNormEps) : 0.f;
+#pragma unroll
+        for (int ps = 0; ps < CP; ++ps) {
+          const int c = ps * 32 + m;
+          const uint32_t w4[4] = {raw[i][ps].x, raw[i][ps].y, raw[i][ps].z, raw[i][ps].w};
+          uint32_t o4[4];
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            float lo = bf_lo(w4[q]) * inv, hi = bf_hi(w4[q]) * inv;
+            if (SCALE_X) { lo = bf16r(lo) * sc; hi = bf16r(hi) * sc; }
+            o4[q] = pack_bf16x2(lo, hi);
+          }
+          if (KSW % 8 == 0 || c < row_chunks)
+            *reinterpret_cast<uint4*>(xt + (size_t)lrow * LDX + c * 8) = make_uint4(o4[0], o4[1], o4[2], o4[3]);
+        }
+      }
+    };
+    // Tile t + 1 is normalised while tile t is multiplied; its registers then fetch tile
+    // t + 3, so the rows of two tiles are always on their way.
+    uint4 raw0[PAIRS][CP], raw1[PAIRS][CP];
+    load_rows(raw0, 0);
+    if (row_tiles > 1) load_rows(raw1, 1);
+    norm_rows(raw0, 0, xtile[0]);
+    if (row_tiles > 2) load_rows(raw0, 2);
+    wait_lgkmcnt0();
+    raw_barrier();
+    for (int t = 0; t < row_tiles; t += 2) {
+      if (t + 1 < row_tiles) {
+        norm_rows(raw1, t + 1, xtile[1]);
+        if (t + 3 < row_tiles) load_rows(raw1, t + 3);
+      }
+      // (the logits of tile t - 1 were complete at the last barrier)
+      if (t > 0) combine_rows((t - 1) * ROWS, min(t * ROWS, S));
+      wait_lgkmcnt0();
+      raw_barrier();
+      if (t + 1 < row_tiles) {
+        if (t + 2 < row_tiles) {
+          norm_rows(raw0, t + 2, xtile[0]);
+          if (t + 4 < row_tiles) load_rows(raw0, t + 4);
+        }
+        combine_rows(t * ROWS, min((t + 1) * ROWS, S));
+        wait_lgkmcnt0();
+        raw_barrier();
+      }
+    }
+    combine_rows((row_tiles - 1) * ROWS, S);
+  } else {
+    // ---- consumers: slots cw * 32 .. + 32 of every tile, and the combine weights
+    const int cw = wave - 4;
+    const int r16 = lane & 15, kq = lane >> 4;   // 16x16x32 fragment: row / column, k quarter
+    const bool mma_on = cw * 32 < NP;
+    bf16x8 bfr[2][KSW];   // (soft_prep_mu_kernel wrote them in this order: 1 KB per load)
+    if (mma_on) {
+#pragma unroll
+      for (int cb = 0; cb < 2; ++cb) {
+        const bf16_t* frag = muw + ((size_t)(cw * 2 + cb) * KSW * 64 + lane) * 8;
+#pragma unroll
+        for (int i = 0; i < KSW; ++i)
+          bfr[cb][i] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(frag + (size_t)i * 512));
+      }
+    }
+    auto multiply = [&](int t, const bf16_t* xt) {
+      if (!mma_on) return;
+      floatx4 acc[RB][2];
+#pragma unroll
+      for (int rh = 0; rh < RB; ++rh)
+#pragma unroll
+        for (int cb = 0; cb < 2; ++cb)
+#pragma unroll
+          for (int v = 0; v < 4; ++v) acc[rh][cb][v] = 0.f;
+      const bf16_t* arow = xt + (size_t)r16 * LDX + kq * 8;
+      // The item fragments of k step i + kAhead are requested before the MFMAs of step i
+      // (a ring of kAhead + 1 register sets; the scheduling barriers keep that order).
+      constexpr int kAhead = 2;
+      bf16x8 af[kAhead + 1][RB];
+      auto read_step = [&](int i, bf16x8 (&dst)[RB]) {
+#pragma unroll
+        for (int rh = 0; rh < RB; ++rh)
+          dst[rh] = __builtin_bit_cast(
+              bf16x8, *reinterpret_cast<const uint4*>(arow + (size_t)rh * 16 * LDX + i * 32));
+      };
+#pragma unroll
+      for (int i = 0; i < kAhead && i < KSW; ++i) read_step(i, af[i]);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int i = 0; i < KSW; ++i) {
+        if (i + kAhead < KSW) read_step(i + kAhead, af[(i + kAhead) % (kAhead + 1)]);
+#pragma unroll
+        for (int rh = 0; rh < RB; ++rh)
+#pragma unroll
+          for (int cb = 0; cb < 2; ++cb)
+            acc[rh][cb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af[i % (kAhead + 1)][rh], bfr[cb][i],
+                                                                 acc[rh][cb], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      mfma_result_fence();
+#pragma unroll
+      for (int rh = 0; rh < RB; ++rh)
+#pragma unroll
+        for (int cb = 0; cb < 2; ++cb)
+#pragma unroll
+          for (int v = 0; v < 4; ++v) {
+            const int row = t * ROWS + rh * 16 + kq * 4 + v;
+            lg[(size_t)row * LDW + cw * 32 + cb * 16 + r16] = f2bf(acc[rh][cb][v]);
+          }
+    };
+    raw_barrier();
+    for (int t = 0; t < row_tiles; ++t) {
+      multiply(t, xtile[t & 1]);
+      wait_lgkmcnt0();
+      raw_barrier();
+    }
+  }
+
+  // Thread -> (16-byte piece c of a weights row, rows s = sr, sr + rpp, ...).
+  const int lchunks = N / 8, rpp = kSrThreads / lchunks;
+  const int sr = tid / lchunks, pc = tid - sr * lchunks;
+  if (logits_out != nullptr && sr < rpp) {
+    for (int s = sr; s < S; s += rpp)
+      *reinterpret_cast<uint4*>(logits_out + ((size_t)g * S + s) * N + pc * 8) =
+          *reinterpret_cast<const uint4*>(lg + (size_t)s * LDW + pc * 8);
+  }
+
+  // Dispatch weights: softmax over the S items of each slot.
+  if (SP <= 32 * kTailRows) {
+    // Up to 256 items: a thread keeps one 16-byte piece (8 slots) of every 32nd row in
+    // registers, so the logits are read from LDS once and every exponential is taken once.
+    // Maxima and sums of a column meet across the lanes of a wave (rows 16 and 32 lanes
+    // apart), then across the waves in LDS (the item tiles, which nobody reads any more).
+    const int tc = tid & 15, tr = tid >> 4;
+    const bool col_on = tc * 8 < NP;
+    float* red_max = red;
+    float* red_sum = red + 8 * 128;
+    uint32_t lw[kTailRows][4];
+    float cm[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) cm[u] = -INFINITY;
+#pragma unroll
+    for (int j = 0; j < kTailRows; ++j) {
+      const int s_ = tr + 32 * j;
+      uint4 q = make_uint4(0xff80ff80u, 0xff80ff80u, 0xff80ff80u, 0xff80ff80u);   // -inf pairs
+      if (s_ < S && col_on) q = *reinterpret_cast<const uint4*>(lg + (size_t)s_ * LDW + tc * 8);
+      lw[j][0] = q.x; lw[j][1] = q.y; lw[j][2] = q.z; lw[j][3] = q.w;
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        cm[2 * u] = fmaxf(cm[2 * u], bf_lo(lw[j][u]));
+        cm[2 * u + 1] = fmaxf(cm[2 * u + 1], bf_hi(lw[j][u]));
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      cm[u] = fmaxf(cm[u], __shfl_xor(cm[u], 16, kWave));
+      cm[u] = fmaxf(cm[u], __shfl_xor(cm[u], 32, kWave));
+    }
+    if (lane < 16) {
+      *reinterpret_cast<float4*>(red_max + wave * 128 + tc * 8) = make_float4(cm[0], cm[1], cm[2], cm[3]);
+      *reinterpret_cast<float4*>(red_max + wave * 128 + tc * 8 + 4) = make_float4(cm[4], cm[5], cm[6], cm[7]);
+    }
+    __syncthreads();
+#pragma unroll
+    for (int w = 0; w < 8; ++w) {
+      const float4 a = *reinterpret_cast<const float4*>(red_max + w * 128 + tc * 8);
+      const float4 b = *reinterpret_cast<const float4*>(red_max + w * 128 + tc * 8 + 4);
+      const float v[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+#pragma unroll
+      for (int u = 0; u < 8; ++u) cm[u] = w == 0 ? v[u] : fmaxf(cm[u], v[u]);
+    }
+    float ev[kTailRows][8], cs[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      cm[u] *= kLog2e;
+      cs[u] = 0.f;
+    }
+#pragma unroll
+    for (int j = 0; j < kTailRows; ++j)
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        ev[j][2 * u] = __builtin_amdgcn_exp2f(fmaf(bf_lo(lw[j][u]), kLog2e, -cm[2 * u]));   // exp2(-inf) = 0
+        ev[j][2 * u + 1] = __builtin_amdgcn_exp2f(fmaf(bf_hi(lw[j][u]), kLog2e, -cm[2 * u + 1]));
+        cs[2 * u] += ev[j][2 * u];
+        cs[2 * u + 1] += ev[j][2 * u + 1];
+      }
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      cs[u] += __shfl_xor(cs[u], 16, kWave);
+      cs[u] += __shfl_xor(cs[u], 32, kWave);
+    }
+    if (lane < 16) {
+      *reinterpret_cast<float4*>(red_sum + wave * 128 + tc * 8) = make_float4(cs[0], cs[1], cs[2], cs[3]);
+      *reinterpret_cast<float4*>(red_sum + wave * 128 + tc * 8 + 4) = make_float4(cs[4], cs[5], cs[6], cs[7]);
+    }
+    __syncthreads();
+#pragma unroll
+    for (int w = 0; w < 8; ++w) {
+      const float4 a = *reinterpret_cast<const float4*>(red_sum + w * 128 + tc * 8);
+      const float4 b = *reinterpret_cast<const float4*>(red_sum + w * 128 + tc * 8 + 4);
+      const float v[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+#pragma unroll
+      for (int u = 0; u < 8; ++u) cs[u] = w == 0 ? v[u] : cs[u] + v[u];
+    }
+#pragma unroll
+    for (int u = 0; u < 8; ++u) cs[u] = __builtin_amdgcn_rcpf(cs[u]);
+#pragma unroll
+    for (int j = 0; j < kTailRows; ++j) {
+      const int s_ = tr + 32 * j;
+      if (s_ < S && tc * 8 < N)
+        *reinterpret_cast<uint4*>(dispatch_w + ((size_t)g * S + s_) * N + tc * 8) = make_uint4(
+            pack_bf16x2(ev[j][0] * cs[0], ev[j][1] * cs[1]), pack_bf16x2(ev[j][2] * cs[2], ev[j][3] * cs[3]),
+            pack_bf16x2(ev[j][4] * cs[4], ev[j][5] * cs[5]), pack_bf16x2(ev[j][6] * cs[6], ev[j][7] * cs[7]));
+    }
+  } else {
+    // More items: three passes over the logits in LDS.  For the maxima and sums a column
+    // is shared by RG threads that take every RG-th row and meet in LDS.
+    const int RG = kSrThreads / NP;
+    const int n = tid % NP, rg = tid / NP;
+    const bool act = rg < RG;
+    float mx = -INFINITY;
+    if (act)
+#pragma unroll 8
+      for (int s = rg; s < S; s += RG) mx = fmaxf(mx, bf2f(lg[(size_t)s * LDW + n]));
+    red[tid] = mx;
+    __syncthreads();
+    if (act) {
+      mx = -INFINITY;
+      for (int q = 0; q < RG; ++q) mx = fmaxf(mx, red[q * NP + n]);
+    }
+    __syncthreads();
+    const float mb = mx * kLog2e;
+    float sum = 0.f;
+    if (act)
+#pragma unroll 8
+      for (int s = rg; s < S; s += RG)
+        sum += __builtin_amdgcn_exp2f(fmaf(bf2f(lg[(size_t)s * LDW + n]), kLog2e, -mb));
+    red[tid] = sum;
+    __syncthreads();
+    if (act && rg == 0) {
+      sum = 0.f;
+      for (int q = 0; q < RG; ++q) sum += red[q * NP + n];
+      cmx[n] = mb;
+      csum[n] = __builtin_amdgcn_rcpf(sum);
+    }
+    __syncthreads();
+    if (sr < rpp) {
+      float cm[8], cr[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        cm[u] = cmx[pc * 8 + u];
+        cr[u] = csum[pc * 8 + u];
+      }
+#pragma unroll 4
+      for (int s = sr; s < S; s += rpp) {
+        const uint4 rawl = *reinterpret_cast<const uint4*>(lg + (size_t)s * LDW + pc * 8);
+        const uint32_t w4[4] = {rawl.x, rawl.y, rawl.z, rawl.w};
+        uint32_t o4[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          const float lo = __builtin_amdgcn_exp2f(fmaf(bf_lo(w4[u]), kLog2e, -cm[2 * u])) * cr[2 * u];
+          const float hi = __builtin_amdgcn_exp2f(fmaf(bf_hi(w4[u]), kLog2e, -cm[2 * u + 1])) * cr[2 * u + 1];
+          o4[u] = pack_bf16x2(lo, hi);
+        }
+        *reinterpret_cast<uint4*>(dispatch_w + ((size_t)g * S + s) * N + pc * 8) =
+            make_uint4(o4[0], o4[1], o4[2], o4[3]);
+      }
+    }
+  }
+}
+
 // Dense einsum between per-group weights and data on the float32 matrix cores.
 //   DISPATCH: out[slot(g,mm)] = sum_s w[g,s,mm] * data[g,s,:]      (M = E*C, Kd = S)
 //   COMBINE:  out[g,mm,:]     = sum_n w[g,mm,n] * data[slot(g,n)]  (M = S,   Kd = E*C)
@@ -734,7 +1170,9 @@ using namespace vmoe;
 
 extern "C" size_t vmoe_soft_route_workspace_bytes(const VmoeSoftRouteParams* p) {
   if (p == nullptr || p->D < 1 || p->N < 1) return 0;
-  return (size_t)p->D * p->N * sizeof(float);
+  // float32: (D, N) floats; bfloat16: the slots padded to a multiple of 32
+  const size_t padded = (size_t)p->D * ((p->N + 31) / 32 * 32) * 2;
+  return std::max((size_t)p->D * p->N * sizeof(float), padded);
 }
 
 extern "C" int vmoe_soft_route(const VmoeSoftRouteParams* p, vmoe_stream_t stream_) {
@@ -758,6 +1196,36 @@ extern "C" int vmoe_soft_route(const VmoeSoftRouteParams* p, vmoe_stream_t strea
   const SoftLds L = soft_lds_layout(p->D, SP, NP);
   if (p->dtype == VMOE_BF16 && p->N <= 128 && p->N % 8 == 0 && soft_fast_width(p->D) && L.total <= 160 * 1024 && aligned16(p->dispatch_w) && aligned16(p->combine_w) &&
       (p->logits == nullptr || aligned16(p->logits))) {
+    // Two roles per workgroup where the slot parameters of 32 slots fit a wave's registers
+    // (D <= 768) and two item tiles fit LDS beside the logits (tiles of 32 rows, else 16).
+    // (VMOE_SOFT_ROUTE_SINGLE_ROLE=1 in the environment keeps the single-role kernel: the
+    // switch behind the before / after figures)
+    const int tile_rows = soft_pipe_lds_layout(p->D, SP, NP, 32).total <= 160 * 1024 ? 32 : 16;
+    const SoftPipeLds PL = soft_pipe_lds_layout(p->D, SP, NP, tile_rows);
+    if (p->D <= 768 && PL.total <= 160 * 1024 && getenv("VMOE_SOFT_ROUTE_SINGLE_ROLE") == nullptr) {
+      using Kern = void (*)(const bf16_t*, const bf16_t*, bf16_t*, bf16_t*, bf16_t*, float, int, int,
+                            int, int, int, SoftPipeLds);
+      auto pick = [&](auto ksw) -> Kern {
+        constexpr int K = decltype(ksw)::value;
+        if (tile_rows == 32)
+          return scale_x ? soft_route_roles_kernel<K, 32, true> : soft_route_roles_kernel<K, 32, false>;
+        return scale_x ? soft_route_roles_kernel<K, 16, true> : soft_route_roles_kernel<K, 16, false>;
+      };
+      Kern kern = p->D == 768   ? pick(std::integral_constant<int, 24>{})
+                  : p->D == 512 ? pick(std::integral_constant<int, 16>{})
+                  : p->D == 384 ? pick(std::integral_constant<int, 12>{})
+                                : pick(std::integral_constant<int, 8>{});
+      hipError_t e = allow_dynamic_lds(reinterpret_cast<const void*>(kern), PL.total);
+      if (e != hipSuccess) return (int)e;
+      if (!p->workspace_prepared)
+        hipLaunchKernelGGL(soft_prep_mu_kernel<bf16_t>, dim3(NP), dim3(256), 0, stream,
+                           (const bf16_t*)p->mu, (bf16_t*)p->workspace, p->scale, !scale_x, p->D, p->N,
+                           p->D / 32);
+      hipLaunchKernelGGL(kern, dim3(p->G), dim3(kSrThreads), PL.total, stream, (const bf16_t*)p->x,
+                         (const bf16_t*)p->workspace, (bf16_t*)p->dispatch_w, (bf16_t*)p->combine_w,
+                         (bf16_t*)p->logits, p->scale, p->S, p->D, p->N, SP, NP, PL);
+      return launch_status();
+    }
     if (!p->workspace_prepared)
       hipLaunchKernelGGL(soft_prep_mu_kernel<bf16_t>, dim3(p->N), dim3(256), 0, stream,
                          (const bf16_t*)p->mu, (bf16_t*)p->workspace, p->scale, !scale_x, p->D, p->N);
