@@ -617,10 +617,19 @@ def test_expert_mlp_planned_launch_random_fill(K):
 
 @pytest.mark.parametrize("E,R,D,M", [(64, 384, 1024, 128), (32, 1152, 1024, 256), (90, 384, 520, 160)])
 def test_expert_mlp_wide_second_product(K, E, R, D, M):
-  """Shapes whose second product takes the wide kernel (384 x 256 tiles, eight waves: chosen
-  where the 256 x 256 tiles would need at least 1.38 times as many rounds of one tile per
-  compute unit): all rows against the oracle, then packed rows with a launch plan
-  (row counts around the tile height, empty experts) bit for bit against the dense launch."""
+  """Shapes whose second product takes the wide kernel (384 x 256 tiles, eight waves; it runs
+  where the tile-walking 256 x 256 kernel does not apply, and VMOE_SECOND_PRODUCT=wide asks
+  for it wherever it applies itself): all rows against the oracle, then packed rows with a
+  launch plan (row counts around the tile height, empty experts) bit for bit against the
+  dense launch."""
+  os.environ["VMOE_SECOND_PRODUCT"] = "wide"
+  try:
+    _wide_second_product(K, E, R, D, M)
+  finally:
+    del os.environ["VMOE_SECOND_PRODUCT"]
+
+
+def _wide_second_product(K, E, R, D, M):
   rng = np.random.default_rng(E + R)
   dtype = O.BF16
   x = O.cast(rng.standard_normal((E, R, D)).astype(np.float32), dtype)

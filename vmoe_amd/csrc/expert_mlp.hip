@@ -4,6 +4,8 @@
 // vit_jax.models_vit.MlpBlock (vmoe/nn/vit_moe.py:38-45): a GEMM batched over
 // the expert axis with the bias add and the GELU fused into the epilogue of the
 // first product and the bias add into the second.
+#include <cstring>
+
 #include "gemm_bf16_wide.h"
 #include "compact_rows.h"
 
@@ -306,14 +308,22 @@ MlpPlans mlp_plans(int E, int R, int D, int M, bool ragged) {
   const bool wide_ok = wide_gemm_ok(E, R, D, M, nullptr, nullptr, nullptr, 0) && (!ragged || bytes(wide));
   constexpr double kNumCu = kCusPerXcd * kNumXcd;
   // Time in units of one 256 x 256 tile on one CU.  The wide kernel's tile is 1.5 of them
-  // at about 0.92 of the time per flop, in whole rounds; the shared kernel pays for its
-  // tiles (the padding of the last row tile of a batch included) plus the exchange.
-  const double t_wide = 1.5 * 0.92 * std::ceil((double)wide.tiles / kNumCu);
+  // at about 1.04 of the time per flop (0.92 before the 256 x 256 kernel kept its A rows
+  // in a ring of three slots), in whole rounds; the shared kernel pays for its tiles (the
+  // padding of the last row tile of a batch included) plus the exchange.  With these
+  // figures the wide kernel only runs where the shared one does not apply.
+  const double t_wide = 1.5 * 1.04 * std::ceil((double)wide.tiles / kNumCu);
   const double t_shared = (double)square.tiles / kNumCu + 0.05;
   if (shared_ok && (!wide_ok || t_shared <= t_wide)) m.down_kernel = kDownShared;
   else if (wide_ok) m.down_kernel = kDownWide;
   else if (!ragged && down_prefers_half_tiles(E, R, D)) m.down_kernel = kDownHalf;
   else m.down_kernel = kDownPlain;
+  // (VMOE_SECOND_PRODUCT=shared|wide in the environment overrides the choice between those
+  // two where both apply: the switch behind the figures that the model above was fitted to)
+  if (const char* force = getenv("VMOE_SECOND_PRODUCT")) {
+    if (strcmp(force, "shared") == 0 && shared_ok) m.down_kernel = kDownShared;
+    if (strcmp(force, "wide") == 0 && wide_ok) m.down_kernel = kDownWide;
+  }
   m.down = m.down_kernel == kDownWide ? wide : square;
   m.down_bm = m.down_kernel == kDownWide ? WideCfg::BM : CfgDown::BM;
   m.down_bytes = bytes(m.down);
