@@ -464,6 +464,31 @@ def test_soft_route(K, G, S, D, n, p, dtype):
   np.testing.assert_allclose(to_np(cw).sum(2), 1.0, atol=atol)
 
 
+def test_soft_route_seeded_shapes(K):
+  """Seeded sweep over the shapes of the bfloat16 fast paths (model widths, N a multiple of 8 up
+  to 128, group sizes around the tile heights and around the 256 items that the
+  register-resident dispatch softmax holds) against the oracle."""
+  rng = np.random.default_rng(2024)
+  special_s = [1, 15, 16, 17, 31, 32, 33, 63, 64, 65, 223, 224, 225, 255, 256, 257, 300]
+  for trial in range(16):
+    D = int(rng.choice([256, 384, 512, 768, 1024]))
+    n = int(rng.integers(1, 17)) * 8
+    S = int(rng.choice(special_s)) if trial % 2 == 0 else int(rng.integers(1, 320))
+    G = int(rng.integers(1, 4))
+    x = O.cast(rng.standard_normal((G, S, D)), O.BF16)
+    mu = O.cast(rng.standard_normal((D, n, 1)) / np.sqrt(D), O.BF16)
+    scale = float(rng.uniform(0.5, 2.0))
+    dw, cw, lg = K.soft_route(to_dev(x, O.BF16), to_dev(mu.reshape(D, n), O.BF16), scale,
+                              return_logits=True)
+    wl, wd, wc, _ = O.soft_router_weights(x, mu, scale, O.BF16)
+    tag = f"G={G} S={S} D={D} N={n}"
+    assert_close(to_np(lg), wl.reshape(G, S, n), 2e-2, "logits " + tag)
+    assert_close(to_np(dw), wd.reshape(G, S, n), 8e-2, "dispatch weights " + tag)
+    assert_close(to_np(cw), wc.reshape(G, S, n), 8e-2, "combine weights " + tag)
+    np.testing.assert_allclose(to_np(dw).sum(1), 1.0, atol=3e-2, err_msg=tag)
+    np.testing.assert_allclose(to_np(cw).sum(2), 1.0, atol=3e-2, err_msg=tag)
+
+
 @pytest.mark.parametrize("G,S,D,N", [(5, 196, 768, 128), (2, 250, 768, 128), (3, 100, 512, 64),
                                      (2, 300, 256, 104), (2, 37, 384, 40)])
 def test_soft_route_two_roles_and_single_role_agree(K, G, S, D, N):
