@@ -163,7 +163,7 @@ def test_xla_ffi_shim_covers_every_entry_point():
       if field in ("int32_t", "float", "size_t", "int64_t"):
         continue
       assert re.search(rf"(?:\.|->){field}\s*=", code), f"{struct}.{field} is never set in the shim"
-  # the registration loop of INTEGRATION.md names the same handlers
+  # the registration loop of the integration guide names the same handlers
   doc = open(os.path.join(ROOT, "INTEGRATION.md")).read()
   for fn, _ in entry_points:
     assert fn in doc, f"{fn} is not mentioned in INTEGRATION.md"
