@@ -397,6 +397,15 @@ typedef struct {
   int32_t dtype;
 } VmoeSoftStatsParams;
 int vmoe_soft_router_stats(const VmoeSoftStatsParams* p, vmoe_stream_t stream);
+/* vmoe_soft_route and vmoe_soft_router_stats on its outputs in one call (SoftRouter.__call__
+ * with its get_metrics, vmoe/projects/soft_moe/router.py:57-125).  `stats` names the same
+ * combine_w / dispatch_w, G, S, N and dtype as `route`.  Where the routing kernel can, it
+ * leaves the (G, 4) partial sums itself (bfloat16, up to 256 items per group, the widths of
+ * its two-role kernel) and only the launch that adds them up follows; otherwise the two
+ * calls are made one after the other.  The scalars equal those of the separate calls up to
+ * the order in which float32 sums are taken. */
+int vmoe_soft_route_stats(const VmoeSoftRouteParams* route, const VmoeSoftStatsParams* stats,
+                          vmoe_stream_t stream);
 
 /* EinsumDispatcher.dispatch / .combine with dense weights
  * (vmoe/moe.py:148-161): per group,

@@ -952,6 +952,29 @@ def test_shared_partial_round_is_exact_on_exact_operands(K, E, R, D, M):
     assert (got[e, n:] == 7.0).all()
 
 
+@pytest.mark.parametrize("G,S,D,N", [(6, 196, 768, 128), (3, 250, 768, 128), (2, 37, 384, 40),
+                                     (4, 100, 512, 64), (2, 256, 256, 8), (1, 1, 768, 8),
+                                     (2, 300, 256, 104), (2, 33, 1024, 128), (2, 64, 768, 20)])
+def test_soft_route_with_stats(K, G, S, D, N):
+  """vmoe_soft_route_stats: the weights are those of vmoe_soft_route bit for bit, and the
+  scalars are the means of vmoe/projects/soft_moe/router.py:119-125 of exactly those stored
+  weights, whether the routing launch takes the partial sums itself (bfloat16, up to 256 items,
+  widths up to 768) or the separate launches run (the last three shapes)."""
+  rng = np.random.default_rng(G * S + N)
+  x = to_dev(O.cast(rng.standard_normal((G, S, D)), O.BF16), O.BF16)
+  mu = to_dev(O.cast(rng.standard_normal((D, N)) / np.sqrt(D), O.BF16), O.BF16)
+  dw0, cw0 = K.soft_route(x, mu, 1.2)
+  dw, cw, scalars = K.soft_route(x, mu, 1.2, with_stats=True)
+  np.testing.assert_array_equal(to_np(dw), to_np(dw0))
+  np.testing.assert_array_equal(to_np(cw), to_np(cw0))
+  d, c = to_np(dw).astype(np.float64), to_np(cw).astype(np.float64)
+  want = [c.min(axis=2).mean(), c.max(axis=2).mean(), d.min(axis=1).mean(), d.max(axis=1).mean()]
+  got = [float(v) for v in scalars]
+  np.testing.assert_allclose(got[:4], want, rtol=3e-6)
+  assert got[4] == 0.0
+  np.testing.assert_allclose(got[:4], [float(v) for v in K.soft_router_stats(cw, dw)][:4], rtol=3e-6)
+
+
 @pytest.mark.parametrize("G,S,N,dtype", [(3, 50, 16, O.F32), (4, 196, 128, O.BF16), (2, 7, 300, O.BF16), (3, 196, 128, O.F32),
                           (2, 9, 96, O.BF16), (5, 33, 8, O.BF16), (2, 300, 512, O.BF16)])
 def test_soft_router_stats(K, G, S, N, dtype):

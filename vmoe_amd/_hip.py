@@ -27,6 +27,7 @@ EXPORTS = [
     "vmoe_einsum_combine", "vmoe_cast", "vmoe_copy_bytes", "vmoe_mfma_probe", "vmoe_operand_delivery_probe", "vmoe_operand_delivery_probe_k64",
     "vmoe_add_layer_norm", "vmoe_attention", "vmoe_noisy_gates", "vmoe_compact_rows", "vmoe_compact_rows_static",
     "vmoe_combine_backward_data", "vmoe_combine_backward_weights", "vmoe_soft_router_stats",
+    "vmoe_soft_route_stats",
 ]
 
 

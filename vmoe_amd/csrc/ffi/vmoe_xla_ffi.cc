@@ -535,6 +535,37 @@ static ffi::Error SoftRouterStatsImpl(hipStream_t stream, Any combine_w, Any dis
 XLA_FFI_DEFINE_HANDLER_SYMBOL(VmoeSoftRouterStats, SoftRouterStatsImpl,
                               ffi::Ffi::Bind().Ctx<Stream>().Arg<Any>().Arg<Any>().Ret<F32>().Ret<F32>());
 
+// x (G,S,D), mu (D,N) -> dispatch_w, combine_w, logits (G,S,N), workspace, stats (5,) f32, partial (G,4) f32
+static ffi::Error SoftRouteStatsImpl(hipStream_t stream, Any x, Any mu, AnyOut dispatch_w, AnyOut combine_w,
+                                     AnyOut logits, AnyOut workspace, F32Out stats, F32Out partial, float scale,
+                                     bool want_logits) {
+  VmoeSoftRouteParams p{};
+  p.x = x.untyped_data();
+  p.mu = mu.untyped_data();
+  p.scale = scale;
+  p.dispatch_w = dispatch_w->untyped_data();
+  p.combine_w = combine_w->untyped_data();
+  p.logits = want_logits ? logits->untyped_data() : nullptr;
+  p.workspace = workspace->untyped_data();
+  p.workspace_bytes = workspace->size_bytes();
+  p.G = Dim(x, 0); p.S = Dim(x, 1); p.D = Dim(x, 2);
+  p.N = Dim(mu, 1);
+  p.dtype = DType(x.element_type());
+  p.workspace_prepared = 0;
+  VmoeSoftStatsParams st{};
+  st.combine_w = p.combine_w;
+  st.dispatch_w = p.dispatch_w;
+  st.stats = stats->typed_data();
+  st.partial = partial->typed_data();
+  st.G = p.G; st.S = p.S; st.N = p.N;
+  st.dtype = p.dtype;
+  return Status(vmoe_soft_route_stats(&p, &st, stream), "vmoe_soft_route_stats");
+}
+XLA_FFI_DEFINE_HANDLER_SYMBOL(VmoeSoftRouteStats, SoftRouteStatsImpl,
+                              ffi::Ffi::Bind().Ctx<Stream>().Arg<Any>().Arg<Any>().Ret<Any>().Ret<Any>()
+                                  .Ret<Any>().Ret<Any>().Ret<F32>().Ret<F32>().Attr<float>("scale")
+                                  .Attr<bool>("want_logits"));
+
 // w (G,S,E,C), data -> out; dispatch: data (G,S,D) -> (E, G*C, D); combine: data (E, G*C, D) -> (G,S,D)
 static void FillEinsum(VmoeEinsumParams* p, const Any& w, const Any& data, AnyOut& out) {
   p->w = w.untyped_data();

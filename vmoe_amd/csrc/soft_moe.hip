@@ -517,6 +517,27 @@ __device__ __forceinline__ float half_wave_sum(float v) {
   v += dpp_lane<0x140>(v);
   return v + __shfl_xor(v, 16, kWave);
 }
+// The same where only the upper 16 lanes of the half wave need the result: the last step is
+// a DPP broadcast of lane 15 of the lower row into the upper one (row_bcast15 on rows 1
+// and 3), no lane exchange through the LDS unit.
+__device__ __forceinline__ float row_bcast15(float v) {
+  const int x = __builtin_bit_cast(int, v);
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(x, x, 0x142, 0xa, 0xf, false));
+}
+__device__ __forceinline__ float half_wave_min_upper(float v) {
+  v = fminf(v, dpp_lane<0xB1>(v));
+  v = fminf(v, dpp_lane<0x4E>(v));
+  v = fminf(v, dpp_lane<0x141>(v));
+  v = fminf(v, dpp_lane<0x140>(v));
+  return fminf(v, row_bcast15(v));
+}
+__device__ __forceinline__ float half_wave_max_upper(float v) {
+  v = fmaxf(v, dpp_lane<0xB1>(v));
+  v = fmaxf(v, dpp_lane<0x4E>(v));
+  v = fmaxf(v, dpp_lane<0x141>(v));
+  v = fmaxf(v, dpp_lane<0x140>(v));
+  return fmaxf(v, row_bcast15(v));
+}
 __device__ __forceinline__ float half_wave_max(float v) {
   v = fmaxf(v, dpp_lane<0xB1>(v));
   v = fmaxf(v, dpp_lane<0x4E>(v));
@@ -553,7 +574,7 @@ template <int KSW, int ROWS, bool SCALE_X>
 __global__ __launch_bounds__(kSrThreads) void soft_route_roles_kernel(
     const bf16_t* __restrict__ x, const bf16_t* __restrict__ muw, bf16_t* __restrict__ dispatch_w,
     bf16_t* __restrict__ combine_w, bf16_t* __restrict__ logits_out, float scale, int S, int D,
-    int N, int SP, int NP, SoftPipeLds L) {
+    int N, int SP, int NP, SoftPipeLds L, float* __restrict__ stats_partial) {
   constexpr int CP = (KSW + 7) / 8;   // 16-byte pieces of an item row per lane of a half wave
   constexpr int RPW = ROWS / 4;       // rows of a tile per producer wave
   constexpr int PAIRS = RPW / 2;      // a half wave takes one row at a time
@@ -580,6 +601,12 @@ __global__ __launch_bounds__(kSrThreads) void soft_route_roles_kernel(
   // slots.  The producers take them (tile t - 1 while tile t is multiplied): the consumers'
   // iteration is the longer one (its fragment reads keep the LDS busy).
   constexpr int CR = ROWS / 8;    // rows of a tile per half wave: their chains overlap
+  // With `stats_partial` (only where the register-resident dispatch softmax applies) the
+  // launch also leaves the group's partial sums of the router's monitoring scalars: the
+  // sums over the items of the smallest / largest combine weight, and over the slots of the
+  // smallest / largest dispatch weight, taken from the rounded values that are stored.
+  float row_min_sum = 0.f, row_max_sum = 0.f;
+  float* const st_rows = cmx;                         // 4 producer waves x 2 half waves x 2
   auto combine_rows = [&](int s_begin, int s_end) {
     {
       const int s0 = s_begin + (wave & 3) * (ROWS / 4);
@@ -615,9 +642,18 @@ __global__ __launch_bounds__(kSrThreads) void soft_route_roles_kernel(
       for (int r = 0; r < CR; ++r) {
         const int s = s0 + 2 * r + h;
         const float rs = __builtin_amdgcn_rcpf(sum[r]);
+        const uint32_t p0 = pack_bf16x2(e[r][0] * rs, e[r][1] * rs);
+        const uint32_t p1 = pack_bf16x2(e[r][2] * rs, e[r][3] * rs);
         if (s < s_end && c < N)
-          *reinterpret_cast<uint2*>(combine_w + ((size_t)g * S + s) * N + c) = make_uint2(
-              pack_bf16x2(e[r][0] * rs, e[r][1] * rs), pack_bf16x2(e[r][2] * rs, e[r][3] * rs));
+          *reinterpret_cast<uint2*>(combine_w + ((size_t)g * S + s) * N + c) = make_uint2(p0, p1);
+        if (stats_partial != nullptr) {    // smallest and largest stored weight of the row
+          float lo = fminf(fminf(bf_lo(p0), bf_hi(p0)), fminf(bf_lo(p1), bf_hi(p1)));
+          float hi = fmaxf(fmaxf(bf_lo(p0), bf_hi(p0)), fmaxf(bf_lo(p1), bf_hi(p1)));
+          if (c >= N) { lo = INFINITY; hi = -INFINITY; }
+          lo = half_wave_min_upper(lo);     // (lanes 16..31 of the half wave hold the result)
+          hi = half_wave_max_upper(hi);
+          if (s < s_end) { row_min_sum += lo; row_max_sum += hi; }
+        }
       }
     }
   };
@@ -698,6 +734,10 @@ __global__ __launch_bounds__(kSrThreads) void soft_route_roles_kernel(
       }
     }
     combine_rows((row_tiles - 1) * ROWS, S);
+    if (stats_partial != nullptr && m == 31) {
+      st_rows[(wave * 2 + h) * 2] = row_min_sum;
+      st_rows[(wave * 2 + h) * 2 + 1] = row_max_sum;
+    }
   } else {
     // ---- consumers: slots cw * 32 .. + 32 of every tile, and the combine weights
     const int cw = wave - 4;
@@ -854,13 +894,83 @@ __global__ __launch_bounds__(kSrThreads) void soft_route_roles_kernel(
     }
 #pragma unroll
     for (int u = 0; u < 8; ++u) cs[u] = __builtin_amdgcn_rcpf(cs[u]);
+    float dmin[8], dmax[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      dmin[u] = INFINITY;
+      dmax[u] = -INFINITY;
+    }
 #pragma unroll
     for (int j = 0; j < kTailRows; ++j) {
       const int s_ = tr + 32 * j;
+      uint32_t o[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) o[u] = pack_bf16x2(ev[j][2 * u] * cs[2 * u], ev[j][2 * u + 1] * cs[2 * u + 1]);
       if (s_ < S && tc * 8 < N)
-        *reinterpret_cast<uint4*>(dispatch_w + ((size_t)g * S + s_) * N + tc * 8) = make_uint4(
-            pack_bf16x2(ev[j][0] * cs[0], ev[j][1] * cs[1]), pack_bf16x2(ev[j][2] * cs[2], ev[j][3] * cs[3]),
-            pack_bf16x2(ev[j][4] * cs[4], ev[j][5] * cs[5]), pack_bf16x2(ev[j][6] * cs[6], ev[j][7] * cs[7]));
+        *reinterpret_cast<uint4*>(dispatch_w + ((size_t)g * S + s_) * N + tc * 8) =
+            make_uint4(o[0], o[1], o[2], o[3]);
+      if (stats_partial != nullptr && s_ < S) {
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          dmin[2 * u] = fminf(dmin[2 * u], bf_lo(o[u]));
+          dmax[2 * u] = fmaxf(dmax[2 * u], bf_lo(o[u]));
+          dmin[2 * u + 1] = fminf(dmin[2 * u + 1], bf_hi(o[u]));
+          dmax[2 * u + 1] = fmaxf(dmax[2 * u + 1], bf_hi(o[u]));
+        }
+      }
+    }
+    if (stats_partial != nullptr) {
+      // Smallest / largest stored weight of every slot: across the lanes of a wave, across
+      // the waves in LDS, then wave 0 adds up the slots and the producers' row sums.
+      float* st_min = red + 16 * 128;
+      float* st_max = red + 24 * 128;
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        dmin[u] = fminf(dmin[u], __shfl_xor(dmin[u], 16, kWave));
+        dmin[u] = fminf(dmin[u], __shfl_xor(dmin[u], 32, kWave));
+        dmax[u] = fmaxf(dmax[u], __shfl_xor(dmax[u], 16, kWave));
+        dmax[u] = fmaxf(dmax[u], __shfl_xor(dmax[u], 32, kWave));
+      }
+      if (lane < 16) {
+        *reinterpret_cast<float4*>(st_min + wave * 128 + tc * 8) = make_float4(dmin[0], dmin[1], dmin[2], dmin[3]);
+        *reinterpret_cast<float4*>(st_min + wave * 128 + tc * 8 + 4) = make_float4(dmin[4], dmin[5], dmin[6], dmin[7]);
+        *reinterpret_cast<float4*>(st_max + wave * 128 + tc * 8) = make_float4(dmax[0], dmax[1], dmax[2], dmax[3]);
+        *reinterpret_cast<float4*>(st_max + wave * 128 + tc * 8 + 4) = make_float4(dmax[4], dmax[5], dmax[6], dmax[7]);
+      }
+      __syncthreads();
+      if (wave == 0) {
+        float smin = 0.f, smax = 0.f;
+        if (lane < 16) {
+#pragma unroll
+          for (int u = 0; u < 8; ++u) {
+            float lo = INFINITY, hi = -INFINITY;
+            for (int w = 0; w < 8; ++w) {
+              lo = fminf(lo, st_min[w * 128 + lane * 8 + u]);
+              hi = fmaxf(hi, st_max[w * 128 + lane * 8 + u]);
+            }
+            if (lane * 8 + u < N) {
+              smin += lo;
+              smax += hi;
+            }
+          }
+        }
+#pragma unroll
+        for (int o = 8; o > 0; o >>= 1) {
+          smin += __shfl_xor(smin, o, kWave);
+          smax += __shfl_xor(smax, o, kWave);
+        }
+        if (lane == 0) {
+          float rmin = 0.f, rmax = 0.f;
+          for (int q = 0; q < 8; ++q) {
+            rmin += st_rows[2 * q];
+            rmax += st_rows[2 * q + 1];
+          }
+          stats_partial[(size_t)g * 4 + 0] = rmin;
+          stats_partial[(size_t)g * 4 + 1] = rmax;
+          stats_partial[(size_t)g * 4 + 2] = smin;
+          stats_partial[(size_t)g * 4 + 3] = smax;
+        }
+      }
     }
   } else {
     // More items: three passes over the logits in LDS.  For the maxima and sums a column
@@ -1175,7 +1285,10 @@ extern "C" size_t vmoe_soft_route_workspace_bytes(const VmoeSoftRouteParams* p) 
   return std::max((size_t)p->D * p->N * sizeof(float), padded);
 }
 
-extern "C" int vmoe_soft_route(const VmoeSoftRouteParams* p, vmoe_stream_t stream_) {
+// vmoe_soft_route; with `stats_partial` the routing launch also writes the (G, 4) partial
+// sums of the monitoring scalars where it can (`*wrote_partial` says whether it did).
+static int soft_route_launch(const VmoeSoftRouteParams* p, vmoe_stream_t stream_, float* stats_partial,
+                             bool* wrote_partial) {
   if (p == nullptr || p->x == nullptr || p->mu == nullptr || p->dispatch_w == nullptr ||
       p->combine_w == nullptr)
     return VMOE_E_NULL;
@@ -1204,7 +1317,13 @@ extern "C" int vmoe_soft_route(const VmoeSoftRouteParams* p, vmoe_stream_t strea
     const SoftPipeLds PL = soft_pipe_lds_layout(p->D, SP, NP, tile_rows);
     if (p->D <= 768 && PL.total <= 160 * 1024 && getenv("VMOE_SOFT_ROUTE_SINGLE_ROLE") == nullptr) {
       using Kern = void (*)(const bf16_t*, const bf16_t*, bf16_t*, bf16_t*, bf16_t*, float, int, int,
-                            int, int, int, SoftPipeLds);
+                            int, int, int, SoftPipeLds, float*);
+      // (the partial sums come out of the register-resident dispatch softmax only)
+      // (VMOE_SOFT_STATS_SEPARATE=1 in the environment keeps the separate launches: the switch
+      // behind the before / after figures)
+      float* partial_out = SP <= 32 * kTailRows && getenv("VMOE_SOFT_STATS_SEPARATE") == nullptr
+                               ? stats_partial : nullptr;
+      if (wrote_partial != nullptr) *wrote_partial = partial_out != nullptr;
       auto pick = [&](auto ksw) -> Kern {
         constexpr int K = decltype(ksw)::value;
         if (tile_rows == 32)
@@ -1223,7 +1342,7 @@ extern "C" int vmoe_soft_route(const VmoeSoftRouteParams* p, vmoe_stream_t strea
                            p->D / 32);
       hipLaunchKernelGGL(kern, dim3(p->G), dim3(kSrThreads), PL.total, stream, (const bf16_t*)p->x,
                          (const bf16_t*)p->workspace, (bf16_t*)p->dispatch_w, (bf16_t*)p->combine_w,
-                         (bf16_t*)p->logits, p->scale, p->S, p->D, p->N, SP, NP, PL);
+                         (bf16_t*)p->logits, p->scale, p->S, p->D, p->N, SP, NP, PL, partial_out);
       return launch_status();
     }
     if (!p->workspace_prepared)
@@ -1263,6 +1382,10 @@ extern "C" int vmoe_soft_route(const VmoeSoftRouteParams* p, vmoe_stream_t strea
                        (float*)p->logits, p->scale, scale_x, p->S, p->D, p->N, SP, NP);
   }
   return launch_status();
+}
+
+extern "C" int vmoe_soft_route(const VmoeSoftRouteParams* p, vmoe_stream_t stream) {
+  return soft_route_launch(p, stream, nullptr, nullptr);
 }
 
 extern "C" int vmoe_einsum_dispatch(const VmoeEinsumParams* p, vmoe_stream_t stream) {
@@ -1315,5 +1438,20 @@ extern "C" int vmoe_soft_router_stats(const VmoeSoftStatsParams* p, vmoe_stream_
                        p->N);
   hipLaunchKernelGGL(soft_stats_finish_kernel, dim3(1), dim3(256), 0, s, p->partial, p->stats, p->G,
                      1.0f / ((float)p->G * (float)p->S), 1.0f / ((float)p->G * (float)p->N));
+  return launch_status();
+}
+
+extern "C" int vmoe_soft_route_stats(const VmoeSoftRouteParams* route, const VmoeSoftStatsParams* st,
+                                     vmoe_stream_t stream) {
+  if (route == nullptr || st == nullptr || st->partial == nullptr || st->stats == nullptr) return VMOE_E_NULL;
+  if (st->combine_w != route->combine_w || st->dispatch_w != route->dispatch_w || st->G != route->G ||
+      st->S != route->S || st->N != route->N || st->dtype != route->dtype)
+    return VMOE_E_SHAPE;
+  bool wrote = false;
+  const int rc = soft_route_launch(route, stream, st->partial, &wrote);
+  if (rc != VMOE_OK) return rc;
+  if (!wrote) return vmoe_soft_router_stats(st, stream);
+  hipLaunchKernelGGL(soft_stats_finish_kernel, dim3(1), dim3(256), 0, as_stream(stream), st->partial, st->stats,
+                     st->G, 1.0f / ((float)st->G * (float)st->S), 1.0f / ((float)st->G * (float)st->N));
   return launch_status();
 }

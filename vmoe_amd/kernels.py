@@ -335,12 +335,15 @@ def expert_mlp_workspace_bytes(E, R, D, M, dtype, prepacked: bool) -> int:
 
 
 def soft_route(x: torch.Tensor, mu: torch.Tensor, scale: float, return_logits: bool = False,
-               prepared: Optional[dict] = None):
-  """x (G,S,D), mu (D,N) -> dispatch_w (G,S,N), combine_w (G,S,N) [, logits].
+               prepared: Optional[dict] = None, with_stats: bool = False):
+  """x (G,S,D), mu (D,N) -> dispatch_w (G,S,N), combine_w (G,S,N) [, logits] [, stats].
 
   ``prepared``: a dict the caller keeps for as long as mu, scale, dtype and the shapes stay
   the same; the unit-norm, scaled slot parameters are computed on the first call, kept in
-  it, and reused by the later ones."""
+  it, and reused by the later ones.
+
+  ``with_stats``: also the five scalars of soft_router_stats (a tuple of 0-dim float32
+  tensors, last in the result), from the same call."""
   G, S, D = x.shape
   N = mu.shape[1]
   x = x.contiguous()
@@ -362,8 +365,15 @@ def soft_route(x: torch.Tensor, mu: torch.Tensor, scale: float, return_logits: b
     p.workspace_prepared = 1
   p.workspace = H.ptr(ws)
   p.workspace_bytes = ws.numel()
-  H.call("vmoe_soft_route", p)
-  return (dw, cw, logits) if return_logits else (dw, cw)
+  out = (dw, cw, logits) if return_logits else (dw, cw)
+  if not with_stats:
+    H.call("vmoe_soft_route", p)
+    return out
+  buf = _f32(G * 4 + 8, device=x.device)
+  stats = buf[G * 4:G * 4 + 5]
+  H.call_blocks("vmoe_soft_route_stats", p, H.SoftStatsParams(
+      H.ptr(cw), H.ptr(dw), H.ptr(buf), H.ptr(stats), G, S, N, H.dtype_code(x.dtype)))
+  return out + ((stats[0], stats[1], stats[2], stats[3], stats[4]),)
 
 
 def soft_router_stats(combine_w: torch.Tensor, dispatch_w: torch.Tensor):

@@ -63,15 +63,16 @@ class SoftRouter(module.Module):
       raise ValueError(f"mu has shape {tuple(mu.shape)}, expected {(dim, self.num_experts, num_slots)}")
     n, s = self.num_experts, num_slots
     mu_c = self._cast_mu(mu, dtype)
-    dw, cw = K.soft_route(x, mu_c.reshape(dim, n * s), self._scale_value(p["scale"]),
-                          prepared=self._prepared_mu(mu_c, p["scale"]))
+    # (the routing call also returns the scalars of get_metrics that come from the weights)
+    dw, cw, scalars = K.soft_route(x, mu_c.reshape(dim, n * s), self._scale_value(p["scale"]),
+                                   prepared=self._prepared_mu(mu_c, p["scale"]), with_stats=True)
     dispatch_weights = dw.view(G, m, n, s)
     combine_weights = cw.view(G, m, n, s)
     dispatcher = EinsumDispatcher(combine_weights, dispatch_weights,
                                   partition_spec=self.partition_spec,
                                   einsum_precision=self.precision)
     dispatcher = Bfloat16Dispatcher(dispatcher)
-    metrics = self.get_metrics(combine_weights, dispatch_weights, mu_c)
+    metrics = self.get_metrics(combine_weights, dispatch_weights, mu_c, scalars=scalars)
     return dispatcher, metrics
 
   def _cast_mu(self, mu: Array, dtype) -> Array:
@@ -96,10 +97,13 @@ class SoftRouter(module.Module):
     cache = self.__dict__.setdefault("_scale_cache", module.ParamCache())
     return cache.get((scale,), "scale", lambda: float(scale))
 
-  def get_metrics(self, combine_weights: Array, dispatch_weights: Array, mu: Array):
-    """router.py:112-167.  Monitoring scalars; mu is normalised inside cosine_psim."""
+  def get_metrics(self, combine_weights: Array, dispatch_weights: Array, mu: Array, scalars=None):
+    """router.py:112-167.  Monitoring scalars; mu is normalised inside cosine_psim.
+    ``scalars``: the five scalars of the weights where the routing call already took them."""
     g, m, n, p = combine_weights.shape
-    if combine_weights.is_cuda and combine_weights.dtype in (torch.float32, torch.bfloat16):
+    if scalars is not None:
+      cmin, cmax, dmin, dmax, aux = scalars
+    elif combine_weights.is_cuda and combine_weights.dtype in (torch.float32, torch.bfloat16):
       cmin, cmax, dmin, dmax, aux = K.soft_router_stats(
           combine_weights.reshape(g, m, n * p), dispatch_weights.reshape(g, m, n * p))
     else:
