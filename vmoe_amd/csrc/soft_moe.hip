@@ -597,19 +597,19 @@ __global__ __launch_bounds__(kSrThreads) void soft_route_roles_kernel(
   bf16_t* const xtile[2] = {xs, xs + (size_t)ROWS * LDX};
 
   // Combine weights of the item rows [s_begin, s_end) of one tile: softmax over the N slots.
-  // The four waves of a role share the tile; half wave = one row, lane = four consecutive
-  // slots.  The producers take them (tile t - 1 while tile t is multiplied): the consumers'
-  // iteration is the longer one (its fragment reads keep the LDS busy).
-  constexpr int CR = ROWS / 8;    // rows of a tile per half wave: their chains overlap
+  // Each role takes half of the tile's rows (tile t - 1 while tile t is multiplied, which
+  // keeps the two roles' iterations about equally long), its four waves a quarter of those;
+  // half wave = one row, lane = four consecutive slots.
+  constexpr int CR = ROWS / 16;   // rows of a tile per half wave: their chains overlap
   // With `stats_partial` (only where the register-resident dispatch softmax applies) the
   // launch also leaves the group's partial sums of the router's monitoring scalars: the
   // sums over the items of the smallest / largest combine weight, and over the slots of the
   // smallest / largest dispatch weight, taken from the rounded values that are stored.
   float row_min_sum = 0.f, row_max_sum = 0.f;
-  float* const st_rows = cmx;                         // 4 producer waves x 2 half waves x 2
+  float* const st_rows = cmx;                         // 8 waves x 2 half waves x 2
   auto combine_rows = [&](int s_begin, int s_end) {
     {
-      const int s0 = s_begin + (wave & 3) * (ROWS / 4);
+      const int s0 = s_begin + (wave >> 2) * (ROWS / 2) + (wave & 3) * (ROWS / 8);
       const int c = m * 4;
       float l[CR][4], mx[CR];
 #pragma unroll
@@ -734,10 +734,6 @@ __global__ __launch_bounds__(kSrThreads) void soft_route_roles_kernel(
       }
     }
     combine_rows((row_tiles - 1) * ROWS, S);
-    if (stats_partial != nullptr && m == 31) {
-      st_rows[(wave * 2 + h) * 2] = row_min_sum;
-      st_rows[(wave * 2 + h) * 2 + 1] = row_max_sum;
-    }
   } else {
     // ---- consumers: slots cw * 32 .. + 32 of every tile, and the combine weights
     const int cw = wave - 4;
@@ -801,9 +797,16 @@ __global__ __launch_bounds__(kSrThreads) void soft_route_roles_kernel(
     raw_barrier();
     for (int t = 0; t < row_tiles; ++t) {
       multiply(t, xtile[t & 1]);
+      // (the logits of tile t - 1 were complete at the last barrier)
+      if (t > 0) combine_rows((t - 1) * ROWS, min(t * ROWS, S));
       wait_lgkmcnt0();
       raw_barrier();
     }
+    combine_rows((row_tiles - 1) * ROWS, S);
+  }
+  if (stats_partial != nullptr && m == 31) {
+    st_rows[(wave * 2 + h) * 2] = row_min_sum;
+    st_rows[(wave * 2 + h) * 2 + 1] = row_max_sum;
   }
 
   // Thread -> (16-byte piece c of a weights row, rows s = sr, sr + rpp, ...).
@@ -961,7 +964,7 @@ __global__ __launch_bounds__(kSrThreads) void soft_route_roles_kernel(
         }
         if (lane == 0) {
           float rmin = 0.f, rmax = 0.f;
-          for (int q = 0; q < 8; ++q) {
+          for (int q = 0; q < 16; ++q) {
             rmin += st_rows[2 * q];
             rmax += st_rows[2 * q + 1];
           }
