@@ -47,8 +47,14 @@ PEAK_BF16_TFLOPS = 2500.0
 PEAK_FP32_MATRIX_TFLOPS = 157.3
 PEAK_HBM_GBS = 8000.0
 
-# HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc runs
-# (FETCH_SIZE + WRITE_SIZE, scaled by a copy kernel of known size); None until measured.
+# Short passes of the other workloads that the default run attaches to its line.
+OTHER_STEPS, OTHER_WARMUP = 10, 5
+
+# Figures that cannot be measured from inside the run (hardware counters need rocprofv3
+# around the process): copied from the summaries under profiles/, and reported under
+# roofline.from_profile together with the file they come from.
+# HBM bytes per launch of the dominant kernel (FETCH_SIZE + WRITE_SIZE, scaled by a copy
+# kernel of known size).
 MEASURED_TRAFFIC_BYTES = {
     # mean of the two GEMM launches of a layer: (630 + 565 + 1096 + 182) / 2 MiB;
     # FETCH_SIZE x 2.0, WRITE_SIZE x 1.0 (copy-kernel calibration);
@@ -76,6 +82,9 @@ def parse_args():
   ap.add_argument("--no-dispatch-pass", action="store_true",
                   help="skip the extra pass that times dispatcher.dispatch() (for counter runs "
                        "that should see the step's kernels only)")
+  ap.add_argument("--no-other-workloads", action="store_true",
+                  help="headline configuration only: skip the short passes of the other "
+                       "BASELINE configurations")
   ap.add_argument("--cpu-groups", type=int, default=32,
                   help="groups of the workload the CPU baseline is timed on")
   return ap.parse_args()
@@ -160,8 +169,9 @@ def cpu_baseline(cfg, x_np, params_np, bias_np, groups, gpu_out=None):
   }
 
 
-def soft_main(args):
-  """Soft MoE layer (SoftRouter + expert MLPs), same protocol as the sparse layer."""
+def soft_run(args, short=False):
+  """Soft MoE layer (SoftRouter + expert MLPs), same protocol as the sparse layer.  `short`:
+  no CPU leg."""
   import torch
   from vmoe_amd import _hip, configs, kernels, moe
   from vmoe_amd.nn import vit_moe
@@ -270,7 +280,8 @@ def soft_main(args):
                        "host": int(np.argmax(host_step_ms)), "host_ms": float(max(host_step_ms))},
       "cpu_baseline": None,
   }
-  if not args.no_cpu_baseline:
+  result["expert_mlp_status"] = mlp_status(kernels)
+  if not args.no_cpu_baseline and not short:
     # The oracle's Soft MoE layer on the first groups of the same batch (the expert
     # MLPs see `groups` rows each instead of G, all 128 experts' weights are read).
     from oracle import moe_oracle as O
@@ -296,15 +307,15 @@ def soft_main(args):
                    f"groups ({groups * m} tokens, all {n} experts), median of 3 runs of {t:.2f} s; "
                    "NumPy BLAS + torch CPU threads"),
         "host_cpus": os.cpu_count(), "cpu_model": host_cpu_model()}
-  print(json.dumps(result))
+  return result
 
 
-def vit_main(args):
+def vit_run(args, short=False):
   """Full V-MoE B/16 forward at 224 px, batch 512: images/s, time per module kind
-  broken out with events around the modules' apply methods."""
+  broken out with events around the modules' apply methods.  `short`: no CPU leg."""
   import copy
   import torch
-  from vmoe_amd import _hip, configs
+  from vmoe_amd import _hip, configs, kernels
   from vmoe_amd.nn import vit_moe
 
   dev = torch.device("cuda:0")
@@ -436,8 +447,9 @@ def vit_main(args):
       "model_TFLOPs_per_step": flops_total / 1e12,
       "model_TFLOPs_per_s": flops_total / (ms * 1e-3) / 1e12,
       "moe_ms": module_ms.get("moe_layers"), "module_ms": module_ms, "stage_ms": stage_ms,
+      "expert_mlp_status": mlp_status(kernels),
   }
-  if not args.no_cpu_baseline:
+  if not args.no_cpu_baseline and not short:
     from oracle import moe_oracle as O
     from oracle import vit_oracle as V
     n_img = 8                                  # one routing group
@@ -460,24 +472,25 @@ def vit_main(args):
         "host_cpus": os.cpu_count(), "cpu_model": host_cpu_model()}
   else:
     result["cpu_baseline"] = None
-  print(json.dumps(result))
+  return result
 
 
-def main():
-  args = parse_args()
-  if args.gpus != 1:
-    print("bench.py: this build runs on ONE GPU (all experts resident, no collectives); "
-          f"--gpus {args.gpus} is not supported.", file=sys.stderr)
-    sys.exit(2)
-  if args.config == "soft_moe_b16_128x1":
-    return soft_main(args)
-  if args.config == "vmoe_b16_model_E8_k2_224":
-    return vit_main(args)
+def mlp_status(kernels):
+  """Status words of the expert MLP's workspace after the run (vmoe_expert_mlp_status):
+  pieces of the second product's shared round that gave up a wait, launches that found no
+  valid plan.  Anything but zeros means that an output of the run was not the product."""
+  st = kernels.expert_mlp_status()
+  return None if st is None else {"abandoned_waits": st[0], "plan_mismatches": st[1]}
+
+
+def sparse_run(args, name, short=False):
+  """One sparse MoE layer configuration.  `short`: the timed passes only (no CPU leg, no
+  probes, no vendor GEMMs, no graph pass, no reference-layout dispatch pass)."""
   import torch
   from vmoe_amd import _hip, configs, kernels
   from vmoe_amd.nn import vit_moe
 
-  cfg = configs.CONFIGS[args.config]
+  cfg = configs.CONFIGS[name]
   dev = torch.device("cuda:0")
   torch.cuda.set_device(dev)
   tdt = torch.bfloat16 if cfg.dtype == "bfloat16" else torch.float32
@@ -557,7 +570,7 @@ def main():
   ms_per_step = float(np.median(step_ms))
   host_ms_per_step = (t_enqueued - t0) * 1e3 / args.steps
   tokens_per_s = T / (ms_per_step * 1e-3)
-  out0 = step(0)[0].float().cpu().numpy() if not args.no_cpu_baseline else None
+  out0 = step(0)[0].float().cpu().numpy() if not (args.no_cpu_baseline or short) else None
 
   def per_step(pairs_by_name):
     return {name: float(np.mean([a.elapsed_time(b) for a, b in pairs])) * (len(pairs) / args.steps)
@@ -589,7 +602,11 @@ def main():
               "kernel": "gemm_bf16_mixed_kernel (first product) / gemm_bf16_persistent_kernel (second product)" if b == 2 else "gemm_f32_kernel",
               "achieved": achieved_tflops, "peak": peak, "unit": "TFLOP/s",
               "frac": achieved_tflops / peak, "traffic": MEASURED_TRAFFIC_BYTES.get(cfg.name),
-              "mfma_busy": MEASURED_MFMA_BUSY.get(cfg.name),
+              "from_profile": {"traffic_bytes_per_launch": MEASURED_TRAFFIC_BYTES.get(cfg.name),
+                               "traffic_source": "profiles/hbm_traffic__vmoe_b16_layer.md",
+                               "mfma_busy": MEASURED_MFMA_BUSY.get(cfg.name),
+                               "note": "hardware counters from rocprofv3 --pmc runs of this command, "
+                                       "not read by this run"} if cfg.name in MEASURED_TRAFFIC_BYTES else None,
               "launch_ms": gemm_ms, "flops_per_launch": flops_per_launch, "kept_rows": kept,
               "buffer_rows": E * G * C}
 
@@ -599,7 +616,7 @@ def main():
   # runs: reference layout, every slot row written, empty ones zeroed) is timed on its own.
   bytes_dispatch = T * D * b + E * G * C * D * b + 8 * T * K
   dispatch_ms = None
-  if "vmoe_dispatch" not in stage_ms and args.no_dispatch_pass:
+  if "vmoe_dispatch" not in stage_ms and (args.no_dispatch_pass or short):
     pass
   elif "vmoe_dispatch" not in stage_ms:
     # the layer through the dispatcher's own dispatch() / combine(), as a caller of the
@@ -643,7 +660,7 @@ def main():
   del src, dst
   # Measured arithmetic ceiling of the same device: a register-resident MFMA loop
   # on operand fragments taken from the layer's own hidden activations.
-  if b == 2:
+  if b == 2 and not short:
     seed = out.reshape(-1)[: 1 << 20].contiguous()
     kernels.mfma_probe(seed, 256, 500)
     e0.record()
@@ -655,7 +672,7 @@ def main():
   # The vendor library's GEMM on the same two products as dense matrices of the kept
   # rows (torch.nn.functional.linear -> hipBLASLt, no GELU), same run: a reference
   # point for what this part sustains on these shapes.
-  if b == 2:
+  if b == 2 and not short:
     a_up = xs[0].reshape(-1, D)[:1].expand(kept, D).contiguous()
     w_up = torch.randn((M, D), device=dev).to(tdt) * D ** -0.5
     a_dn = torch.randn((kept, M), device=dev).to(tdt)
@@ -703,6 +720,8 @@ def main():
   # serving loop would run the layer; reported beside the eager figure, never as `value`.
   graph_ms = None
   try:
+    if short:
+      raise StopIteration
     side = torch.cuda.Stream()
     side.wait_stream(torch.cuda.current_stream())
     with torch.cuda.stream(side):
@@ -726,6 +745,8 @@ def main():
     if not torch.equal(keep[(args.steps - 1) % n_rot][0], step(args.steps - 1)[0]):
       raise RuntimeError("graph replay and eager step disagree")
     del graphs, keep
+  except StopIteration:
+    pass
   except Exception as e:   # pylint: disable=broad-except
     print(f"bench.py: HIP graph pass skipped: {e}", file=sys.stderr)
     graph_ms = None
@@ -739,7 +760,8 @@ def main():
   hbm["combine_frac_of_peak"] = hbm["combine_GBps"] / PEAK_HBM_GBS
 
   result = {
-      "metric": "MoE-layer tokens/sec at B/16 E=32 k=2 bf16; dispatch/combine HBM GB/s",
+      "metric": ("MoE-layer tokens/sec at B/16 E=32 k=2 bf16; dispatch/combine HBM GB/s" if cfg.name == HEADLINE
+                 else f"MoE-layer tokens/sec, {cfg.name}"),
       "value": tokens_per_s, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
       "warmup": args.warmup, "ms_per_step": ms_per_step, "higher_is_better": True,
       "scaling": "weak", "vs_baseline": None, "dtype": "bf16" if b == 2 else "f32",
@@ -763,8 +785,9 @@ def main():
       "step_ms_p10_p50_p90": [float(np.percentile(step_ms, q)) for q in (10, 50, 90)],
       "step_ms_first_five": [float(v) for v in step_ms[:5]],
       "untimed_steps_before_warmup": COLD_STEPS + INIT_STEPS,
+      "expert_mlp_status": mlp_status(kernels),
   }
-  if not args.no_cpu_baseline:
+  if not args.no_cpu_baseline and not short:
     params_np = {
         "Router": {"dense": {"kernel": router_np}},
         "Mlp": {"Dense_0": {"kernel": w0.float().cpu().numpy(), "bias": b0.float().cpu().numpy()},
@@ -775,8 +798,70 @@ def main():
   else:
     result["cpu_baseline"] = None
     result["parity_checked"] = None
+  return result
+
+
+SOFT_NAME = "soft_moe_b16_128x1"
+MODEL_NAME = "vmoe_b16_model_E8_k2_224"
+HEADLINE = "vmoe_b16_layer_E32_k2_bpr"
+# The other BASELINE configurations, run as short passes behind the headline one.
+OTHER_WORKLOADS = ("vmoe_s32_layer", "vmoe_l16_384_layer_cf0.5", SOFT_NAME, MODEL_NAME)
+
+
+def run_config(args, name, short=False):
+  if name == SOFT_NAME:
+    return soft_run(args, short)
+  if name == MODEL_NAME:
+    return vit_run(args, short)
+  return sparse_run(args, name, short)
+
+
+def other_workloads(args):
+  """Short passes (OTHER_WARMUP warm-up steps behind the initialisation steps, OTHER_STEPS
+  timed steps, no CPU leg) of the BASELINE configurations that are not the headline one."""
+  import copy
+  import torch
+  short_args = copy.copy(args)
+  short_args.steps, short_args.warmup = OTHER_STEPS, OTHER_WARMUP
+  out = []
+  for name in OTHER_WORKLOADS:
+    gc.collect()
+    torch.cuda.empty_cache()
+    try:
+      r = run_config(short_args, name, short=True)
+    except Exception as e:   # pylint: disable=broad-except
+      out.append({"workload": name, "error": f"{type(e).__name__}: {e}"})
+      continue
+    roof = r["roofline"]
+    entry = {"workload": r["config"]["workload"], "metric": r["metric"], "ms_per_step": r["ms_per_step"],
+             "value": r["value"], "unit": r["unit"], "dtype": r["dtype"], "steps": r["steps"],
+             "warmup": r["warmup"],
+             "roofline": {k: roof.get(k) for k in ("bound", "kernel", "achieved", "peak", "unit", "frac", "launch_ms")},
+             "kept_rows": roof.get("kept_rows", roof.get("kept_rows_per_moe_block")),
+             "stage_ms": r.get("stage_ms"), "expert_mlp_status": r.get("expert_mlp_status")}
+    if "moe_ms" in r:
+      entry["moe_ms"] = r["moe_ms"]
+    if "hbm" in r:
+      entry["hbm"] = {k: r["hbm"][k] for k in ("combine_GBps", "gate_topk_GBps", "copy_kernel_GBps")}
+    out.append(entry)
+  return out
+
+
+def main():
+  args = parse_args()
+  if args.gpus != 1:
+    print("bench.py: this build runs on ONE GPU (all experts resident, no collectives); "
+          f"--gpus {args.gpus} is not supported.", file=sys.stderr)
+    sys.exit(2)
+  result = run_config(args, args.config)
+  if args.config == HEADLINE and not args.no_other_workloads:
+    result["other_workloads"] = other_workloads(args)
   print(json.dumps(result))
-  parity = result["parity_checked"]
+  st = result.get("expert_mlp_status")
+  if st and (st["abandoned_waits"] or st["plan_mismatches"]):
+    print(f"bench.py: the expert MLP's status words are not zero: {st}", file=sys.stderr)
+    sys.exit(1)
+  parity = result.get("parity_checked")
   if parity and parity["bad"] > parity["allowed_bad_fraction"] * parity["items"]:
     print(f"bench.py: the timed path's output differs from the oracle on {parity['bad']} of "
           f"{parity['items']} items", file=sys.stderr)

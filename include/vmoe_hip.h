@@ -299,12 +299,18 @@ int vmoe_densify(const VmoeDensifyParams* p, vmoe_stream_t stream);
  * bf16 needs the kernels in K-contiguous order: pass w0t (E,M,D) / w1t (E,D,M)
  * made once by vmoe_pack_expert_weights; if they are null the call packs
  * w0/w1 into `workspace` first (extra HBM pass).  D % 8 == 0 and M % 8 == 0.
- * `workspace` holds the hidden activations (E, R, M), the launch plans of a call with
- * rows_per_expert and, for bf16, 64 MB through which the second product's workgroups
- * exchange float32 partial sums when the tiles of a last, partial round are cut along k
- * (results are deterministic; such a cut reorders one float32 addition per output, so
- * outputs of a call with rows_per_expert may differ from those of a call without by one
- * bfloat16 rounding step).  Calls that share a workspace must not overlap.
+ * `workspace` holds the hidden activations (E, R, M), the call's status words, the launch
+ * plans of a call with rows_per_expert and, for bf16, 64 MB through which the second
+ * product's workgroups exchange float32 partial sums when the tiles of a last, partial round
+ * are cut along k (results are deterministic; such a cut reorders one float32 addition per
+ * output, so outputs of a call with rows_per_expert may differ from those of a call without
+ * by one bfloat16 rounding step).  Calls that share a workspace must not overlap.
+ * That exchange assumes that all 256 workgroups of the second product are resident at the
+ * same time, which holds when the launch has the GPU to itself: a piece waits for pieces
+ * in workgroups placed before its own.  Kernels of other streams that hold compute units
+ * at that moment void the assumption.  The wait is bounded (about two seconds); a piece
+ * that gives up writes NaN instead of sums it did not get, so the affected output rows are
+ * NaN, and it is counted in the status words (vmoe_expert_mlp_status).
  */
 typedef struct {
   const void* x;    /* (E, R, D) dtype */
@@ -342,10 +348,32 @@ int vmoe_expert_mlp(const VmoeExpertMlpParams* p, vmoe_stream_t stream);
  * vmoe_expert_mlp_planned, which takes the launch plans in the workspace as written.
  * VMOE_E_UNSUPPORTED where the compaction needs its two-launch form (E > 256, fewer than 256
  * assignments per group, many groups of few experts) or the MLP plans nothing (float32):
- * make the separate calls.  Results equal those of the separate calls. */
+ * make the separate calls.  Results equal those of the separate calls.
+ * vmoe_expert_mlp_planned may be called any number of times after one
+ * vmoe_compact_rows_planned, as long as the parameter block names the same shapes and
+ * workspace and nothing else wrote the workspace in between (each call resets the exchange
+ * counters it uses).  The plans carry a tag of the shapes they were written for; a call that
+ * does not find its own tag (workspace never planned, or planned for other E, R, D, M)
+ * launches kernels that do nothing, leaves `out` untouched and counts a plan mismatch in the
+ * status words. */
 int vmoe_compact_rows_planned(const VmoeCompactRowsParams* c, const VmoeExpertMlpParams* mlp,
                               vmoe_stream_t stream);
 int vmoe_expert_mlp_planned(const VmoeExpertMlpParams* p, vmoe_stream_t stream);
+
+/* Status words of the expert MLP calls made on p->workspace (no counterpart in the
+ * reference).  *status receives the DEVICE address of VMOE_MLP_STATUS_WORDS int32 inside the
+ * workspace, or null for float32 (those kernels keep no such state); nothing is launched.
+ *   status[VMOE_MLP_STATUS_ABANDONED_WAITS]  pieces of the second product's shared round that
+ *       gave up waiting for another piece's partial sums (their output rows are NaN);
+ *   status[VMOE_MLP_STATUS_PLAN_MISMATCHES]  launches that did not find a plan written for
+ *       their shapes and therefore did nothing.
+ * Both only grow: the first call on a workspace sets them to zero (it recognises a fresh
+ * workspace by a tag word beside them), later calls add.  Read them (hipMemcpy) once the
+ * stream has finished; anything but zero means that an output of some call since then is
+ * not the product it should be. */
+enum { VMOE_MLP_STATUS_ABANDONED_WAITS = 0, VMOE_MLP_STATUS_PLAN_MISMATCHES = 1,
+       VMOE_MLP_STATUS_WORDS = 2 };
+int vmoe_expert_mlp_status(const VmoeExpertMlpParams* p, const int32_t** status);
 
 /* (batch, rows, cols) -> (batch, cols, rows), 2- or 4-byte elements. */
 typedef struct {

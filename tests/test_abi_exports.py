@@ -150,8 +150,15 @@ def test_xla_ffi_shim_covers_every_entry_point():
   header = re.sub(r"/\*.*?\*/", "", open(HEADER).read(), flags=re.S)
   shim = open(FFI_SOURCE).read()
   code = re.sub(r"//[^\n]*", "", shim)
-  entry_points = re.findall(r"\bint\s+(vmoe_[a-z0-9_]+)\s*\(\s*const\s+(Vmoe\w+Params)\s*\*", header)
+  entry_points = [(f, s_) for f, s_ in re.findall(
+      r"\bint\s+(vmoe_[a-z0-9_]+)\s*\(\s*const\s+(Vmoe\w+Params)\s*\*", header)
+                  if f != "vmoe_expert_mlp_status"]      # no launch: the MLP handlers call it themselves
   assert len(entry_points) >= 24
+  assert len(re.findall(r"\bCopyStatus\(stream, p, status\)", code)) == 3, "every MLP handler returns the status words"
+  assert re.search(r"\bvmoe_expert_mlp_status\s*\(\s*&", code)
+  # the fused custom call falls back to the two-launch compaction where the one-launch form does not exist
+  fused = code[code.index("CompactRowsPlannedImpl("):code.index("XLA_FFI_DEFINE_HANDLER_SYMBOL(VmoeCompactRowsPlanned")]
+  assert "VMOE_E_UNSUPPORTED" in fused and "vmoe_compact_rows(&c" in fused and "vmoe_expert_mlp(&p" in fused
   handlers = set(re.findall(r"XLA_FFI_DEFINE_HANDLER_SYMBOL\(\s*(\w+)\s*,", code))
   for fn, _ in entry_points:
     assert _camel(fn) in handlers, f"no XLA FFI handler symbol {_camel(fn)} for {fn}"

@@ -459,9 +459,33 @@ def test_soft_route(K, G, S, D, n, p, dtype):
   assert_close(to_np(lg), wl.reshape(G, S, n * p), tol * (1 if dtype == O.BF16 else 4), "logits")
   assert_close(to_np(dw), wd.reshape(G, S, n * p), tol * 4, "dispatch weights")
   assert_close(to_np(cw), wc.reshape(G, S, n * p), tol * 4, "combine weights")
+  _check_soft_weights_against_own_logits(to_np(lg), to_np(dw), to_np(cw), dtype, "")
   atol = 1e-4 if dtype == O.F32 else 3e-2
   np.testing.assert_allclose(to_np(dw).sum(1), 1.0, atol=atol)
   np.testing.assert_allclose(to_np(cw).sum(2), 1.0, atol=atol)
+
+
+def _check_soft_weights_against_own_logits(lg, dw, cw, dtype, tag):
+  """The two softmaxes themselves.  Against the oracle the weights carry the difference of the
+  logits (a bfloat16 logit that rounds the other way moves a weight by exp(step) - 1, which is
+  why those comparisons are loose); against the float64 softmaxes of the logits that the kernel
+  itself returned -- the values its softmaxes start from -- nothing is left but the softmax
+  arithmetic and one rounding: two units in the last place of the weights' type (bfloat16: 8
+  significant bits; float32: rtol 1e-5 for the float32 exponentials and sums).  A wrong
+  denominator, a missing maximum or a softmax over the wrong axis does not pass."""
+  lg64 = np.asarray(lg, np.float64)
+  for name, got, axis in (("dispatch weights", dw, 1), ("combine weights", cw, 2)):
+    e = np.exp(lg64 - lg64.max(axis=axis, keepdims=True))
+    want = e / e.sum(axis=axis, keepdims=True)
+    got = np.asarray(got, np.float64)
+    if dtype == O.BF16:
+      allowed = 2.0 ** (np.floor(np.log2(np.maximum(want, 1e-300))) - 7 + 1) + 1e-38
+    else:
+      allowed = 1e-5 * want + 1e-30
+    bad = np.abs(got - want) > allowed
+    assert not bad.any(), (f"{name} {tag}: {bad.sum()} of {bad.size} further than two units in the last "
+                           f"place from the softmax of the kernel's own logits; worst ratio "
+                           f"{float((np.abs(got - want) / allowed).max()):.2f}")
 
 
 def test_soft_route_seeded_shapes(K):
@@ -485,6 +509,7 @@ def test_soft_route_seeded_shapes(K):
     assert_close(to_np(lg), wl.reshape(G, S, n), 2e-2, "logits " + tag)
     assert_close(to_np(dw), wd.reshape(G, S, n), 8e-2, "dispatch weights " + tag)
     assert_close(to_np(cw), wc.reshape(G, S, n), 8e-2, "combine weights " + tag)
+    _check_soft_weights_against_own_logits(to_np(lg), to_np(dw), to_np(cw), O.BF16, tag)
     np.testing.assert_allclose(to_np(dw).sum(1), 1.0, atol=3e-2, err_msg=tag)
     np.testing.assert_allclose(to_np(cw).sum(2), 1.0, atol=3e-2, err_msg=tag)
 
@@ -923,6 +948,7 @@ def test_expert_mlp_second_product_shares_partial_round(K, E, R, D, M):
       assert (d <= step + 1e-30).all(), "more than one bfloat16 step from the dense launch"
       differ += int((d > 0).sum())
     assert differ <= 0.02 * max(1, int(rows.sum())) * D, f"{differ} outputs differ from the dense launch"
+  assert K.expert_mlp_status() == (0, 0), "a piece gave up its wait, or a launch found no plan"
 
 
 @pytest.mark.parametrize("E,R,D,M", [(12, 2048, 1024, 512), (3, 500, 768, 1024)])
@@ -950,6 +976,89 @@ def test_shared_partial_round_is_exact_on_exact_operands(K, E, R, D, M):
   for e, n in enumerate(rows):
     np.testing.assert_array_equal(got[e, :n], want[e, :n], err_msg=f"expert {e}")
     assert (got[e, n:] == 7.0).all()
+  assert K.expert_mlp_status() == (0, 0), "a piece gave up its wait, or a launch found no plan"
+
+
+def test_shared_round_wait_that_gives_up_is_loud(K, monkeypatch):
+  """The bounded wait of the shared round, forced from the host: with
+  VMOE_STREAMK_TEST_GIVE_UP the pieces wait (for a handful of polls) for a deposit count that
+  is never reached.  Every kernel still runs to its end; the pieces that gave up are counted
+  in the status words and their outputs are NaN, not sums that were never delivered.  The
+  count stays when later calls on the same workspace go well."""
+  E, R, D, M = 3, 500, 768, 1024           # 2-3 tiles per die: every tile is shared
+  rng = np.random.default_rng(5)
+  args = [to_dev(O.cast(a, O.BF16), O.BF16) for a in (
+      rng.standard_normal((E, R, D)).astype(np.float32),
+      rng.standard_normal((E, D, M)).astype(np.float32) / np.sqrt(D),
+      rng.standard_normal((E, M)).astype(np.float32) * 0.1,
+      rng.standard_normal((E, M, D)).astype(np.float32) / np.sqrt(M),
+      rng.standard_normal((E, D)).astype(np.float32) * 0.1)]
+  ws = torch.zeros(K.expert_mlp_workspace_bytes(E, R, D, M, torch.bfloat16, prepacked=False),
+                   dtype=torch.uint8, device=dev())
+  good = K.expert_mlp(*args, workspace=ws)
+  torch.cuda.synchronize()
+  assert K.expert_mlp_status() == (0, 0)
+  assert not torch.isnan(good).any()
+  monkeypatch.setenv("VMOE_STREAMK_TEST_GIVE_UP", "4")
+  bad = K.expert_mlp(*args, workspace=ws)
+  torch.cuda.synchronize()
+  monkeypatch.delenv("VMOE_STREAMK_TEST_GIVE_UP")
+  abandoned, mismatches = K.expert_mlp_status()
+  assert abandoned >= 1 and mismatches == 0
+  nan_rows = torch.isnan(bad).any(-1)
+  assert nan_rows.any(), "a piece gave up but no output row says so"
+  ok = ~nan_rows
+  assert torch.equal(bad[ok], good[ok]), "rows that are not NaN must be the product"
+  again = K.expert_mlp(*args, workspace=ws)
+  torch.cuda.synchronize()
+  assert torch.equal(again, good)
+  assert K.expert_mlp_status() == (abandoned, 0), "the status words only grow"
+
+
+def test_expert_mlp_planned_is_repeatable_and_checks_its_plan(K):
+  """vmoe_expert_mlp_planned twice after one vmoe_compact_rows_planned (unchanged routing: a
+  serving loop, a graph of the experts alone) gives the same output both times -- each call
+  resets the exchange counters of its shared round -- and a call on a workspace whose plans
+  were never written runs nothing and says so in the status words."""
+  from vmoe_amd import _hip as H
+  G, S, E, k, C, D, M = 4, 1568, 32, 2, 100, 256, 512     # 64 tiles of the second product: shared pieces on every die
+  rng = np.random.default_rng(23)
+  gates = O.softmax(rng.standard_normal((G, S, E)).astype(np.float32) * 2)
+  val, idx = K.topk(to_dev(gates), k)
+  _, token_slot, _, fill = K.route_assign(val, idx, E, C, True)
+  items = to_dev(O.cast(rng.standard_normal((G * S, D)), O.BF16), O.BF16)
+  w0 = to_dev(O.cast(rng.standard_normal((E, D, M)) / np.sqrt(D), O.BF16), O.BF16)
+  w1 = to_dev(O.cast(rng.standard_normal((E, M, D)) / np.sqrt(M), O.BF16), O.BF16)
+  b0 = to_dev(O.cast(rng.standard_normal((E, M)) * 0.1, O.BF16), O.BF16)
+  b1 = to_dev(O.cast(rng.standard_normal((E, D)) * 0.1, O.BF16), O.BF16)
+  w0t, w1t = K.pack_expert_weights(w0), K.pack_expert_weights(w1)
+  first, maps = K.expert_mlp(items, None, b0, None, b1, w0t=w0t, w1t=w1t, compact=(fill, token_slot, C))
+  first = first.clone()
+  rows = to_np(maps[1])
+  for _ in range(2):
+    out = K.expert_mlp_replay_planned()
+    first_np, out_np = to_np(first), to_np(out)
+    for e in range(E):
+      np.testing.assert_array_equal(out_np[e, :rows[e]], first_np[e, :rows[e]], err_msg=f"expert {e}")
+  assert K.expert_mlp_status() == (0, 0)
+  # a workspace that was never planned: every product launch leaves at once
+  R = G * C
+  ws = torch.randint(0, 255, (K.expert_mlp_workspace_bytes(E, R, D, M, torch.bfloat16, prepacked=True) + (1 << 20),),
+                     dtype=torch.uint8, device=dev())
+  out = torch.full((E, R, D), 7.0, dtype=torch.bfloat16, device=dev())
+  p = H.ExpertMlpParams(H.ptr(items), None, H.ptr(b0), None, H.ptr(b1), H.ptr(w0t), H.ptr(w1t), H.ptr(out),
+                        H.ptr(ws), ws.numel(), E, R, D, M, H.BF16, H.GELU_TANH, H.ptr(maps[1]),
+                        H.ptr(maps[2]), G * S)
+  need = H.lib().vmoe_expert_mlp_workspace_bytes(H.ctypes.byref(p))
+  assert need <= ws.numel()
+  H.call("vmoe_expert_mlp_planned", p)
+  torch.cuda.synchronize()
+  addr = H.ctypes.c_void_p()
+  H.check(H.lib().vmoe_expert_mlp_status(H.ctypes.byref(p), H.ctypes.byref(addr)), "vmoe_expert_mlp_status")
+  words = ws[addr.value - ws.data_ptr():][:8].view(torch.int32).cpu()
+  assert int(words[H.MLP_STATUS_PLAN_MISMATCHES]) == 2, "both products must report the missing plan"
+  assert int(words[H.MLP_STATUS_ABANDONED_WAITS]) == 0
+  assert (to_np(out) == 7.0).all(), "a launch without a valid plan must not write"
 
 
 @pytest.mark.parametrize("G,S,D,N", [(6, 196, 768, 128), (3, 250, 768, 128), (2, 37, 384, 40),

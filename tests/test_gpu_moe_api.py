@@ -676,7 +676,25 @@ def test_layer_configs_vs_oracle(name):
   tol = 2e-5 if dtype == O.F32 else 2e-2
   rms = np.sqrt((want ** 2).mean())
   bad_items = (np.abs(got - want) > tol * (rms + np.abs(want))).any(-1)
-  print(f"{name}: items outside tolerance {bad_items.sum()} / {bad_items.size}")
+  # Routing decisions, item by item: the experts chosen and which choices are kept.  A gate
+  # that differs from the oracle's by one rounding step can flip a decision; those items are
+  # counted on their own, every other item must be inside the tolerance.
+  router_mod, _ = layer._modules()
+  xg = to_dev(x, dtype).view(-1, cfg.group_size, cfg.d_model)
+  disp, _ = router_mod.apply({"params": {"dense": {"kernel": to_dev(params["Router"]["dense"]["kernel"])}}}, xg)
+  odisp, _, _ = O.noisy_top_experts_per_item_router(
+      x.reshape(-1, cfg.group_size, cfg.d_model), params["Router"]["dense"]["kernel"],
+      cfg.num_selected_experts, cfg.dispatcher_kwargs(), dtype, logit_bias=bias)
+  gi, oi = to_np(disp.indices), np.asarray(odisp.indices)
+  C = odisp.capacity
+  flipped = ((gi[..., 0] != oi[..., 0]) | ((gi[..., 1] < C) != (oi[..., 1] < C))).any(-1).reshape(-1)
+  print(f"{name}: routing differs on {flipped.sum()} of {flipped.size} items; items outside "
+        f"tolerance {bad_items.sum()}, of which {(bad_items & ~flipped).sum()} with equal routing")
+  assert (bad_items & ~flipped).sum() == 0, "an item routed as in the oracle is outside the tolerance"
+  assert flipped.mean() <= (0.0 if dtype == O.F32 else 0.01)
+  if name == "vmoe_b16_layer_E32_k2_bpr":
+    # observed: 0 of 50 176.  A handful would be rounding; a tenth of a percent is a regression.
+    assert flipped.sum() <= 50, f"{flipped.sum()} routing decisions differ from the oracle"
   assert bad_items.mean() <= (0.0 if dtype == O.F32 else 0.01)
   if name.startswith("vmoe_l16"):
     # capacity factor 0.5: at least half of the assignments are dropped -> many all-zero rows

@@ -336,6 +336,20 @@ def test_softmax_dense_gelu_closed_forms():
   np.testing.assert_allclose(gb, g, rtol=6e-2, atol=2e-3)
 
 
+def test_gelu_vs_torch():
+  """The oracle's two GELUs against torch's CPU implementations (an independent statement of
+  flax.linen.gelu's approximate=True / False forms; several GPU tests use torch's as their
+  reference, so the two must agree).  In the negative tail 1 + tanh (1 + erf) cancels in
+  float32, hence the absolute floor of a few float32 steps of 1."""
+  import torch
+  t = np.concatenate([np.linspace(-9, 9, 2001), [0.0, -0.0, 1e-8, -1e-8, 20.0, -20.0]]).astype(np.float32)
+  tt = torch.from_numpy(t)
+  np.testing.assert_allclose(O.gelu(t), torch.nn.functional.gelu(tt, approximate="tanh").numpy(),
+                             rtol=2e-6, atol=5e-7)
+  np.testing.assert_allclose(O.gelu(t, approximate=False), torch.nn.functional.gelu(tt).numpy(),
+                             rtol=2e-6, atol=1e-6)
+
+
 def test_mlp_block_vs_float64():
   rng = np.random.default_rng(4)
   E, R, D, M = 3, 5, 8, 12

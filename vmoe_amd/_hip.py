@@ -17,12 +17,13 @@ _lib = None
 
 F32, BF16 = 0, 1
 GELU_TANH, GELU_ERF = 0, 1
+MLP_STATUS_ABANDONED_WAITS, MLP_STATUS_PLAN_MISMATCHES, MLP_STATUS_WORDS = 0, 1, 2
 W_F32, W_BF16, W_BOOL = 0, 1, 2
 
 EXPORTS = [
     "vmoe_abi_version", "vmoe_error_string", "vmoe_gate_topk", "vmoe_topk", "vmoe_router_metrics",
     "vmoe_route_assign", "vmoe_route_assign_metrics", "vmoe_top_items_per_expert", "vmoe_indices_to_slots", "vmoe_dispatch", "vmoe_combine", "vmoe_densify",
-    "vmoe_expert_mlp_workspace_bytes", "vmoe_expert_mlp", "vmoe_expert_mlp_planned", "vmoe_compact_rows_planned", "vmoe_pack_expert_weights",
+    "vmoe_expert_mlp_workspace_bytes", "vmoe_expert_mlp", "vmoe_expert_mlp_planned", "vmoe_expert_mlp_status", "vmoe_compact_rows_planned", "vmoe_pack_expert_weights",
     "vmoe_soft_route_workspace_bytes", "vmoe_soft_route", "vmoe_einsum_dispatch",
     "vmoe_einsum_combine", "vmoe_cast", "vmoe_copy_bytes", "vmoe_mfma_probe", "vmoe_operand_delivery_probe", "vmoe_operand_delivery_probe_k64",
     "vmoe_add_layer_norm", "vmoe_attention", "vmoe_noisy_gates", "vmoe_compact_rows", "vmoe_compact_rows_static",

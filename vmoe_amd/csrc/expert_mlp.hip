@@ -243,18 +243,20 @@ __global__ __launch_bounds__(256) void compact_rows_planned_kernel(
     const int32_t* __restrict__ fill, const int32_t* __restrict__ token_slot,
     int32_t* __restrict__ token_row, int32_t* __restrict__ row_token,
     int32_t* __restrict__ rows_per_expert, int G, int E, int C, int per_group, int K, size_t n,
-    unsigned compact_blocks, int R, RaggedGeom ga, RaggedGeom gb, int32_t* __restrict__ clear,
-    int clear_count) {
+    unsigned compact_blocks, int R, RaggedGeom ga, RaggedGeom gb) {
   extern __shared__ int32_t tile_prefix[];
   if (blockIdx.x < compact_blocks)
     compact_rows_fused_block(fill, token_slot, token_row, row_token, rows_per_expert, G, E, C,
                              per_group, K, n, blockIdx.x);
   else
-    plan_ragged_tiles_block(nullptr, fill, G, E, R, ga, gb, clear, clear_count,
-                            blockIdx.x - compact_blocks, tile_prefix);
+    plan_ragged_tiles_block(nullptr, fill, G, E, R, ga, gb, blockIdx.x - compact_blocks, tile_prefix);
 }
 
 size_t align256(size_t v) { return (v + 255) / 256 * 256; }
+
+// The status words of a bfloat16 call sit behind the hidden activations.
+constexpr size_t kStatusBytes = 256;
+static_assert(kStatusWords * sizeof(int32_t) <= kStatusBytes, "status block");
 
 // Which kernel runs the second product (bfloat16).
 //  kDownShared: 256 x 256 tiles walked by one workgroup per CU, the last, partial round of a
@@ -367,9 +369,9 @@ extern "C" size_t vmoe_expert_mlp_workspace_bytes(const VmoeExpertMlpParams* p) 
   if (p == nullptr || p->E < 1 || p->R < 1 || p->D < 1 || p->M < 1) return 0;
   const size_t b = p->dtype == VMOE_BF16 ? 2 : 4;
   size_t bytes = align256((size_t)p->E * p->R * p->M * b);  // hidden activations
-  if (p->dtype == VMOE_BF16) {   // launch plans of the ragged products, stream-K exchange
+  if (p->dtype == VMOE_BF16) {   // status words, launch plans of the ragged products, stream-K exchange
     const MlpPlans m = mlp_plans(p->E, p->R, p->D, p->M, p->rows_per_expert != nullptr);
-    bytes += m.up_bytes + m.down_bytes + m.streamk_bytes;
+    bytes += kStatusBytes + m.up_bytes + m.down_bytes + m.streamk_bytes;
   }
   if (p->dtype == VMOE_BF16) {
     if (p->w0t == nullptr) bytes += align256((size_t)p->E * p->D * p->M * b);
@@ -381,6 +383,7 @@ extern "C" size_t vmoe_expert_mlp_workspace_bytes(const VmoeExpertMlpParams* p) 
 // Where the pieces of a bfloat16 MLP's workspace lie, and what the planning launch is given.
 struct MlpWorkspace {
   void* hidden = nullptr;
+  int32_t* status = nullptr;         // the call's status words (bfloat16 only)
   int4* plan_up = nullptr;
   int4* plan_down = nullptr;
   void* streamk = nullptr;
@@ -397,6 +400,8 @@ MlpWorkspace mlp_workspace(const VmoeExpertMlpParams* p) {
   w.hidden = ws;
   ws += align256((size_t)p->E * p->R * p->M * b);
   if (p->dtype == VMOE_BF16) {
+    w.status = reinterpret_cast<int32_t*>(ws);
+    ws += kStatusBytes;
     w.m = mlp_plans(p->E, p->R, p->D, p->M, p->rows_per_expert != nullptr);
     if (w.m.up_bytes) w.plan_up = reinterpret_cast<int4*>(ws);
     ws += w.m.up_bytes;
@@ -436,13 +441,9 @@ static int run_expert_mlp(const VmoeExpertMlpParams* p, vmoe_stream_t stream_, b
   const MlpPlans& m = w.m;
   unsigned char* ws = w.rest;
   if (planned_already && w.plan_blocks == 0) return VMOE_E_UNSUPPORTED;
-  if (w.plan_blocks > 0 && !planned_already) {
-    using SK = StreamKWorkspace<CfgDownPersistent>;
+  if (w.plan_blocks > 0 && !planned_already)
     hipLaunchKernelGGL(plan_ragged_tiles_kernel, dim3(w.plan_blocks), dim3(256),
-                       plan_ragged_tiles_lds(p->E), stream, p->rows_per_expert, p->E, p->R, w.ga, w.gb,
-                       streamk != nullptr ? SK::flags(streamk) : nullptr,
-                       streamk != nullptr ? SK::kFlags : 0);
-  }
+                       plan_ragged_tiles_lds(p->E), stream, p->rows_per_expert, p->E, p->R, w.ga, w.gb);
   const bool tanh_gelu = p->gelu == VMOE_GELU_TANH;
   if (p->dtype == VMOE_BF16) {
     const void* w0t = p->w0t;
@@ -458,33 +459,34 @@ static int run_expert_mlp(const VmoeExpertMlpParams* p, vmoe_stream_t stream_, b
       if (rc != VMOE_OK) return rc;
       w1t = ws;
     }
-    // The counters of the second product's stream-K exchange are cleared by the planning
-    // launch, or else by the first product's.
+    // The counters of the second product's stream-K exchange are set to zero by the first
+    // product's launch, in every call: a call that finds its plans written
+    // (vmoe_expert_mlp_planned) can be repeated on the same workspace.
     using SK = StreamKWorkspace<CfgDownPersistent>;
-    const bool planned = plan_up != nullptr || plan_down != nullptr;
-    int32_t* clear = streamk != nullptr && !planned ? SK::flags(streamk) : nullptr;
+    int32_t* clear = streamk != nullptr ? SK::flags(streamk) : nullptr;
+    int32_t* status = w.status;
     static_assert(std::is_same<CfgUp, GemmCfg<128, 256, 2, 2, 32, 3, 2>>::value,
                   "launch_gemm_bf16_first runs CfgUp's geometry");
     if (tanh_gelu)
       rc = launch_gemm_bf16_first<kEpiBiasGeluTanh>((const bf16_t*)p->x, (const bf16_t*)w0t,
                                                     (const bf16_t*)p->b0, (bf16_t*)hidden, p->E,
                                                     p->R, p->M, p->D, stream, p->rows_per_expert,
-                                                    plan_up, p->x_rows, p->num_items, clear, SK::kFlags);
+                                                    plan_up, p->x_rows, p->num_items, clear, SK::kFlags, status);
     else
       rc = launch_gemm_bf16_first<kEpiBiasGeluErf>((const bf16_t*)p->x, (const bf16_t*)w0t,
                                                    (const bf16_t*)p->b0, (bf16_t*)hidden, p->E,
                                                    p->R, p->M, p->D, stream, p->rows_per_expert,
-                                                   plan_up, p->x_rows, p->num_items, clear, SK::kFlags);
+                                                   plan_up, p->x_rows, p->num_items, clear, SK::kFlags, status);
     if (rc != VMOE_OK) return rc;
     switch (m.down_kernel) {
       case kDownShared:
         return launch_gemm_bf16_persistent<CfgDownPersistent, kEpiBias>(
             (const bf16_t*)hidden, (const bf16_t*)w1t, (const bf16_t*)p->b1, (bf16_t*)p->out, p->E,
-            p->R, p->D, p->M, stream, plan_down, streamk, /*flags_clear=*/true);
+            p->R, p->D, p->M, stream, plan_down, streamk, status);
       case kDownWide:
         return launch_gemm_bf16_wide<kEpiBias>((const bf16_t*)hidden, (const bf16_t*)w1t,
                                                (const bf16_t*)p->b1, (bf16_t*)p->out, p->E, p->R,
-                                               p->D, p->M, stream, plan_down);
+                                               p->D, p->M, stream, plan_down, nullptr, 0, status);
       case kDownHalf:
         return launch_gemm_bf16<CfgUp, kEpiBias>((const bf16_t*)hidden, (const bf16_t*)w1t,
                                                 (const bf16_t*)p->b1, (bf16_t*)p->out, p->E, p->R,
@@ -492,7 +494,8 @@ static int run_expert_mlp(const VmoeExpertMlpParams* p, vmoe_stream_t stream_, b
       default:
         return launch_gemm_bf16<CfgDown, kEpiBias>((const bf16_t*)hidden, (const bf16_t*)w1t,
                                                   (const bf16_t*)p->b1, (bf16_t*)p->out, p->E, p->R,
-                                                  p->D, p->M, stream, p->rows_per_expert, plan_down);
+                                                  p->D, p->M, stream, p->rows_per_expert, plan_down,
+                                                  nullptr, 0, nullptr, 0, status);
     }
   }
   if (tanh_gelu)
@@ -515,6 +518,19 @@ extern "C" int vmoe_expert_mlp(const VmoeExpertMlpParams* p, vmoe_stream_t strea
 
 extern "C" int vmoe_expert_mlp_planned(const VmoeExpertMlpParams* p, vmoe_stream_t stream) {
   return run_expert_mlp(p, stream, true);
+}
+
+extern "C" int vmoe_expert_mlp_status(const VmoeExpertMlpParams* p, const int32_t** status) {
+  if (status == nullptr) return VMOE_E_NULL;
+  *status = nullptr;
+  int rc = check_mlp(p);
+  if (rc != VMOE_OK) return rc;
+  if (p->dtype != VMOE_BF16) return VMOE_OK;       // the float32 kernels keep no such state
+  if (p->workspace == nullptr || p->workspace_bytes < vmoe_expert_mlp_workspace_bytes(p) ||
+      !aligned16(p->workspace))
+    return VMOE_E_WORKSPACE;
+  *status = mlp_workspace(p).status;
+  return VMOE_OK;
 }
 
 extern "C" int vmoe_compact_rows_planned(const VmoeCompactRowsParams* c,
@@ -540,13 +556,10 @@ extern "C" int vmoe_compact_rows_planned(const VmoeCompactRowsParams* c,
   if (w.plan_blocks == 0) return VMOE_E_UNSUPPORTED;
   const size_t n = (size_t)c->G * c->S * c->K;
   const unsigned compact_blocks = (unsigned)((n + 255) / 256);
-  using SK = StreamKWorkspace<CfgDownPersistent>;
   hipLaunchKernelGGL(compact_rows_planned_kernel, dim3(compact_blocks + (unsigned)w.plan_blocks),
                      dim3(256), plan_ragged_tiles_lds(c->E), as_stream(stream), c->fill,
                      c->token_slot, c->token_row, c->row_token, c->rows_per_expert, c->G, c->E, c->C,
-                     c->S * c->K, c->K, n, compact_blocks, mlp->R, w.ga, w.gb,
-                     w.streamk != nullptr ? SK::flags(w.streamk) : nullptr,
-                     w.streamk != nullptr ? SK::kFlags : 0);
+                     c->S * c->K, c->K, n, compact_blocks, mlp->R, w.ga, w.gb);
   return launch_status();
 }
 

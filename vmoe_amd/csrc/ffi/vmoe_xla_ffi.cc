@@ -366,14 +366,31 @@ XLA_FFI_DEFINE_HANDLER_SYMBOL(VmoeDensify, DensifyImpl,
                                   .Ret<ffi::Buffer<ffi::PRED>>());
 
 // ---------------------------------------------------------------- expert MLP
+// Copies the status words of the MLP call just issued (vmoe_expert_mlp_status: abandoned
+// waits, plan mismatches) from its workspace into the call's `status` result, behind the
+// kernels on the stream: XLA hands out a fresh workspace per call, so the words must leave
+// with the call.  Zeros where the call keeps none (float32).
+static ffi::Error CopyStatus(hipStream_t stream, const VmoeExpertMlpParams& p, S32Out& status) {
+  const int32_t* words = nullptr;
+  ffi::Error e = Status(vmoe_expert_mlp_status(&p, &words), "vmoe_expert_mlp_status");
+  if (e.failure()) return e;
+  const size_t bytes = VMOE_MLP_STATUS_WORDS * sizeof(int32_t);
+  hipError_t h = words != nullptr
+                     ? hipMemcpyAsync(status->typed_data(), words, bytes, hipMemcpyDeviceToDevice, stream)
+                     : hipMemsetAsync(status->typed_data(), 0, bytes, stream);
+  return h == hipSuccess ? ffi::Error::Success()
+                         : ffi::Error(ffi::ErrorCode::kInternal, hipGetErrorString(h));
+}
+
 // x (E,R,D) -- or, with gather, the items (T,D) --, w0, b0 (E,M), w1, b1 (E,D),
 // rows_per_expert (E,), x_rows (E,R) -> out (E,R,D), workspace (bytes; size it with
-// vmoe_expert_mlp_workspace_bytes through ctypes when building the call).  packed: w0 / w1
+// vmoe_expert_mlp_workspace_bytes through ctypes when building the call), status (2,) s32.  packed: w0 / w1
 // are the transposed copies made by vmoe_pack_expert_weights, (E,M,D) / (E,D,M); else the
 // reference's (E,D,M) / (E,M,D) kernels (bfloat16: repacked into the workspace every call).
 static ffi::Error ExpertMlpImpl(hipStream_t stream, Any x, Any w0, Any b0, Any w1, Any b1,
                                 S32 rows_per_expert, S32 x_rows, AnyOut out, AnyOut workspace,
-                                bool packed, bool has_bias, bool ragged, bool gather, int32_t gelu) {
+                                S32Out status, bool packed, bool has_bias, bool ragged, bool gather,
+                                int32_t gelu) {
   VmoeExpertMlpParams p{};
   p.x = x.untyped_data();
   if (packed) {
@@ -397,11 +414,13 @@ static ffi::Error ExpertMlpImpl(hipStream_t stream, Any x, Any w0, Any b0, Any w
   p.rows_per_expert = (ragged || gather) ? rows_per_expert.typed_data() : nullptr;
   p.x_rows = gather ? x_rows.typed_data() : nullptr;
   p.num_items = gather ? (int32_t)(x.element_count() / p.D) : 0;
-  return Status(vmoe_expert_mlp(&p, stream), "vmoe_expert_mlp");
+  ffi::Error e = Status(vmoe_expert_mlp(&p, stream), "vmoe_expert_mlp");
+  if (e.failure()) return e;
+  return CopyStatus(stream, p, status);
 }
 XLA_FFI_DEFINE_HANDLER_SYMBOL(VmoeExpertMlp, ExpertMlpImpl,
                               ffi::Ffi::Bind().Ctx<Stream>().Arg<Any>().Arg<Any>().Arg<Any>().Arg<Any>()
-                                  .Arg<Any>().Arg<S32>().Arg<S32>().Ret<Any>().Ret<Any>()
+                                  .Arg<Any>().Arg<S32>().Arg<S32>().Ret<Any>().Ret<Any>().Ret<S32>()
                                   .Attr<bool>("packed").Attr<bool>("has_bias").Attr<bool>("ragged")
                                   .Attr<bool>("gather").Attr<int32_t>("gelu"));
 
@@ -410,7 +429,7 @@ XLA_FFI_DEFINE_HANDLER_SYMBOL(VmoeExpertMlp, ExpertMlpImpl,
 // (input_output_aliases).  Operands and attributes as VmoeExpertMlp with ragged = gather = true.
 static ffi::Error ExpertMlpPlannedImpl(hipStream_t stream, Any x, Any w0, Any b0, Any w1, Any b1,
                                        S32 rows_per_expert, S32 x_rows, AnyOut out, AnyOut workspace,
-                                       bool packed, bool has_bias, int32_t gelu) {
+                                       S32Out status, bool packed, bool has_bias, int32_t gelu) {
   VmoeExpertMlpParams p{};
   p.x = x.untyped_data();
   if (packed) {
@@ -434,22 +453,28 @@ static ffi::Error ExpertMlpPlannedImpl(hipStream_t stream, Any x, Any w0, Any b0
   p.rows_per_expert = rows_per_expert.typed_data();
   p.x_rows = x_rows.typed_data();
   p.num_items = (int32_t)(x.element_count() / p.D);
-  return Status(vmoe_expert_mlp_planned(&p, stream), "vmoe_expert_mlp_planned");
+  ffi::Error e = Status(vmoe_expert_mlp_planned(&p, stream), "vmoe_expert_mlp_planned");
+  if (e.failure()) return e;
+  return CopyStatus(stream, p, status);
 }
 XLA_FFI_DEFINE_HANDLER_SYMBOL(VmoeExpertMlpPlanned, ExpertMlpPlannedImpl,
                               ffi::Ffi::Bind().Ctx<Stream>().Arg<Any>().Arg<Any>().Arg<Any>().Arg<Any>()
-                                  .Arg<Any>().Arg<S32>().Arg<S32>().Ret<Any>().Ret<Any>()
+                                  .Arg<Any>().Arg<S32>().Arg<S32>().Ret<Any>().Ret<Any>().Ret<S32>()
                                   .Attr<bool>("packed").Attr<bool>("has_bias").Attr<int32_t>("gelu"));
 
 // Row compaction, launch plans and the MLP of the gathered rows as one custom call (the form
 // in which XLA would use the pair vmoe_compact_rows_planned / vmoe_expert_mlp_planned):
 // fill (G,E), token_slot (G,S,K), items (T,D), weights as VmoeExpertMlp -> token_row (G,S,K),
-// rows_per_expert (E,), row_token (E, G*C), out (E, G*C, D), workspace.
+// rows_per_expert (E,), row_token (E, G*C), out (E, G*C, D), workspace, status (2,) s32,
+// prefix (G,E) s32 scratch.  Shapes for which the one-launch form does not exist (more than
+// 256 experts, fewer than 256 assignments per group, very many groups of few experts,
+// float32: vmoe_compact_rows_planned returns VMOE_E_UNSUPPORTED) take vmoe_compact_rows with
+// the `prefix` scratch followed by vmoe_expert_mlp, as the Python host does: same results.
 static ffi::Error CompactRowsPlannedImpl(hipStream_t stream, S32 fill, S32 token_slot, Any x, Any w0,
                                          Any b0, Any w1, Any b1, S32Out token_row,
                                          S32Out rows_per_expert, S32Out row_token, AnyOut out,
-                                         AnyOut workspace, int32_t capacity, bool packed,
-                                         bool has_bias, int32_t gelu) {
+                                         AnyOut workspace, S32Out status, S32Out prefix,
+                                         int32_t capacity, bool packed, bool has_bias, int32_t gelu) {
   VmoeCompactRowsParams c{};
   FillCompact(&c, fill, token_slot, token_row, rows_per_expert, row_token, capacity);
   VmoeExpertMlpParams p{};
@@ -475,14 +500,31 @@ static ffi::Error CompactRowsPlannedImpl(hipStream_t stream, S32 fill, S32 token
   p.rows_per_expert = rows_per_expert->typed_data();
   p.x_rows = row_token->typed_data();
   p.num_items = (int32_t)(x.element_count() / p.D);
-  ffi::Error e = Status(vmoe_compact_rows_planned(&c, &p, stream), "vmoe_compact_rows_planned");
+  const int rc = vmoe_compact_rows_planned(&c, &p, stream);
+  ffi::Error e = ffi::Error::Success();
+  if (rc == VMOE_E_UNSUPPORTED) {
+    c.prefix = prefix->typed_data();
+    e = Status(vmoe_compact_rows(&c, stream), "vmoe_compact_rows");
+    if (e.failure()) return e;
+    if (p.dtype != VMOE_BF16 || p.D % 32 != 0) {
+      // (only the bfloat16 first product gathers its rows: other callers dispatch first and
+      // use VmoeExpertMlp; this custom call is defined for the gathering form)
+      return ffi::Error(ffi::ErrorCode::kInvalidArgument,
+                        "vmoe_compact_rows_planned: the gathering expert MLP needs bfloat16 and D % 32 == 0");
+    }
+    e = Status(vmoe_expert_mlp(&p, stream), "vmoe_expert_mlp");
+  } else {
+    e = Status(rc, "vmoe_compact_rows_planned");
+    if (e.failure()) return e;
+    e = Status(vmoe_expert_mlp_planned(&p, stream), "vmoe_expert_mlp_planned");
+  }
   if (e.failure()) return e;
-  return Status(vmoe_expert_mlp_planned(&p, stream), "vmoe_expert_mlp_planned");
+  return CopyStatus(stream, p, status);
 }
 XLA_FFI_DEFINE_HANDLER_SYMBOL(VmoeCompactRowsPlanned, CompactRowsPlannedImpl,
                               ffi::Ffi::Bind().Ctx<Stream>().Arg<S32>().Arg<S32>().Arg<Any>().Arg<Any>()
                                   .Arg<Any>().Arg<Any>().Arg<Any>().Ret<S32>().Ret<S32>().Ret<S32>()
-                                  .Ret<Any>().Ret<Any>().Attr<int32_t>("capacity").Attr<bool>("packed")
+                                  .Ret<Any>().Ret<Any>().Ret<S32>().Ret<S32>().Attr<int32_t>("capacity").Attr<bool>("packed")
                                   .Attr<bool>("has_bias").Attr<int32_t>("gelu"));
 
 // in (batch, rows, cols) -> out (batch, cols, rows)

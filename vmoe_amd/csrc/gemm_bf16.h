@@ -258,17 +258,16 @@ __device__ __forceinline__ void plan_one(const RaggedGeom& g, const int32_t* til
   g.plan[i] = plan_entry(g, tile_prefix, rows, batch, R, i);
 }
 
-// Entry num_blocks of a plan (one past its last workgroup) holds the number of live row
-// tiles, from which a tile-walking kernel derives the length of its die's run; the
-// planning launch also clears the `clear_count` flags of the stream-K exchange.
+// Entry num_blocks of a plan (one past its last workgroup) is its header: the number of live
+// row tiles, from which a tile-walking kernel derives the length of its die's run, and the
+// tag of the geometry the plan was written for (plan_tag).
 // One workgroup of the planning launch (block = its index among the planning workgroups).
 // With `fill` (G x batch fill counts of the slot assignment) the row counts are its column
 // sums, added up here, and `rows` is not read: the plan then does not wait for the launch
 // that writes the row counts and can share a launch with it.
 __device__ __forceinline__ void plan_ragged_tiles_block(
     const int32_t* __restrict__ rows, const int32_t* __restrict__ fill, int G, int batch, int R,
-    const RaggedGeom& ga, const RaggedGeom& gb, int32_t* __restrict__ clear, int clear_count,
-    unsigned block, int32_t* tile_prefix) {
+    const RaggedGeom& ga, const RaggedGeom& gb, unsigned block, int32_t* tile_prefix) {
   // tile_prefix: 2 x (batch + 1) live row tiles before batch b, then `batch` row counts
   __shared__ int32_t wsum[2][4];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -318,9 +317,10 @@ __device__ __forceinline__ void plan_ragged_tiles_block(
   plan_one(ga, pa, rows_here, batch, R, i);
   plan_one(gb, pb, rows_here, batch, R, i);
   if (block == 0) {
-    if (tid == 0 && ga.plan != nullptr) ga.plan[ga.num_blocks] = PlanEntry{pa[batch], 0, 0, 0};
-    if (tid == 0 && gb.plan != nullptr) gb.plan[gb.num_blocks] = PlanEntry{pb[batch], 0, 0, 0};
-    for (int c = tid; c < clear_count; c += 256) clear[c] = 0;
+    if (tid == 0 && ga.plan != nullptr)
+      ga.plan[ga.num_blocks] = PlanEntry{pa[batch], plan_tag(ga.bm, ga.tiles_n, ga.panel_rows, ga.num_blocks, batch, R), 0, 0};
+    if (tid == 0 && gb.plan != nullptr)
+      gb.plan[gb.num_blocks] = PlanEntry{pb[batch], plan_tag(gb.bm, gb.tiles_n, gb.panel_rows, gb.num_blocks, batch, R), 0, 0};
   }
 }
 
@@ -328,15 +328,48 @@ __device__ __forceinline__ void plan_ragged_tiles_block(
 inline size_t plan_ragged_tiles_lds(int batch) { return ((size_t)2 * (batch + 1) + batch) * sizeof(int32_t); }
 
 __global__ __launch_bounds__(256) void plan_ragged_tiles_kernel(
-    const int32_t* __restrict__ rows, int batch, int R, RaggedGeom ga, RaggedGeom gb,
-    int32_t* __restrict__ clear, int clear_count) {
+    const int32_t* __restrict__ rows, int batch, int R, RaggedGeom ga, RaggedGeom gb) {
   extern __shared__ int32_t tile_prefix[];
-  plan_ragged_tiles_block(rows, nullptr, 0, batch, R, ga, gb, clear, clear_count, blockIdx.x, tile_prefix);
+  plan_ragged_tiles_block(rows, nullptr, 0, batch, R, ga, gb, blockIdx.x, tile_prefix);
 }
 
-__global__ __launch_bounds__(256) void clear_i32_kernel(int32_t* __restrict__ p, int n) {
-  const int i = blockIdx.x * 256 + threadIdx.x;
-  if (i < n) p[i] = 0;
+// A launch plan as a product kernel is given it: the entries, the index of the header entry
+// and the tag that the header must carry (plan_tag of the launch's own geometry).
+struct PlanRef {
+  const int4* entries;
+  int blocks;
+  int32_t tag;
+};
+
+// What the first launch of an expert MLP call does for the launches behind it on the stream
+// (one workgroup's worth of stores, which would otherwise be a launch of their own): the
+// counters of the second product's stream-K exchange start at zero in every call, and the
+// call's status words are set to zero where the tag word does not say that they have been.
+__device__ __forceinline__ void begin_call(int32_t* __restrict__ flags, int num_flags,
+                                           int32_t* __restrict__ status, int tid, int threads) {
+  if (flags != nullptr)
+    for (int c = tid; c < num_flags; c += threads) flags[c] = 0;
+  if (status != nullptr && tid == 0 && status[kStatusTagWord] != kStatusTag) {
+    status[kStatusAbandonedWaits] = 0;
+    status[kStatusPlanMismatches] = 0;
+    status[kStatusTagWord] = kStatusTag;
+  }
+}
+
+__global__ __launch_bounds__(256) void begin_call_kernel(int32_t* __restrict__ flags, int num_flags,
+                                                         int32_t* __restrict__ status) {
+  begin_call(flags, num_flags, status, threadIdx.x, 256);
+}
+
+// Reads a workgroup's plan entry.  False (and nothing may run) where the plan's header does
+// not carry the launch's tag; workgroup 0 then counts the launch among the call's mismatches.
+__device__ __forceinline__ bool read_plan(const PlanRef& ref, int32_t* __restrict__ status, int tid,
+                                          int4& mine) {
+  const int4 hdr = ref.entries[ref.blocks];
+  mine = ref.entries[blockIdx.x];
+  if (hdr.y == ref.tag) return true;
+  if (blockIdx.x == 0 && tid == 0 && status != nullptr) status[kStatusPlanMismatches] += 1;
+  return false;
 }
 
 // Fast path: Kd % BK == 0.  Global tiles go straight into LDS
@@ -348,18 +381,16 @@ __global__ __launch_bounds__(Cfg::kThreads, Cfg::kBlocksPerCu) void gemm_bf16_ke
     const bf16_t* __restrict__ A, const bf16_t* __restrict__ Bt, const bf16_t* __restrict__ bias,
     bf16_t* __restrict__ C, int R, int N, int Kd, int tiles_m, int tiles_n, int num_tiles,
     int tiles_per_xcd, int panel_rows, const int32_t* __restrict__ rows,
-    const int4* __restrict__ plan, const int32_t* __restrict__ a_rows, int a_items,
-    int32_t* __restrict__ clear, int clear_count) {
+    PlanRef plan_ref, const int32_t* __restrict__ a_rows, int a_items,
+    int32_t* __restrict__ clear, int clear_count, int32_t* __restrict__ status) {
 #if defined(__HIP_DEVICE_COMPILE__)   // buffer-resource builtins exist in the device pass only
   extern __shared__ __align__(1024) unsigned char smem[];
   constexpr int BM = Cfg::BM, BN = Cfg::BN, BK = Cfg::BK;
   constexpr int FM = Cfg::FM, FN = Cfg::FN;
   constexpr int RB = Cfg::kRowBytes;
   const int tid = threadIdx.x;
-  // (a few words that the next launch on the stream wants cleared: the counters of its
-  // stream-K exchange, which would otherwise cost a launch of their own)
-  if (clear != nullptr && blockIdx.x == 0)
-    for (int c = tid; c < clear_count; c += Cfg::kThreads) clear[c] = 0;
+  const int4* plan = plan_ref.entries;
+  if (blockIdx.x == 0) begin_call(clear, clear_count, status, tid, Cfg::kThreads);
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave / Cfg::WN, wn = wave % Cfg::WN;
@@ -370,7 +401,8 @@ __global__ __launch_bounds__(Cfg::kThreads, Cfg::kBlocksPerCu) void gemm_bf16_ke
   // have nothing to do, and the last tile stores only its live rows.
   int live = R;
   if (plan != nullptr) {
-    const int4 mine = plan[blockIdx.x];
+    int4 mine;
+    if (!read_plan(plan_ref, status, tid, mine)) return;
     if (mine.x < 0) return;
     b = mine.x;
     tile_m = mine.y;
@@ -649,15 +681,15 @@ __global__ __launch_bounds__(256, 2) void gemm_bf16_mixed_kernel(
     const bf16_t* __restrict__ A, const bf16_t* __restrict__ Bt, const bf16_t* __restrict__ bias,
     bf16_t* __restrict__ C, int R, int N, int Kd, int tiles_m, int tiles_n, int num_tiles,
     int tiles_per_xcd, int panel_rows, const int32_t* __restrict__ rows,
-    const int4* __restrict__ plan, const int32_t* __restrict__ a_rows, int a_items,
-    int32_t* __restrict__ clear, int clear_count) {
+    PlanRef plan_ref, const int32_t* __restrict__ a_rows, int a_items,
+    int32_t* __restrict__ clear, int clear_count, int32_t* __restrict__ status) {
 #if defined(__HIP_DEVICE_COMPILE__)   // buffer-resource builtins exist in the device pass only
   extern __shared__ __align__(1024) unsigned char smem[];
   constexpr int BM = 128, BN = 256, TM = 64, TN = 128, FM = 2, FN = 4, kWaves = 4;
   constexpr int kASlot = BM * 64, kBSlot = BN * 128, kBBase = 2 * kASlot;
   const int tid = threadIdx.x;
-  if (clear != nullptr && blockIdx.x == 0)
-    for (int c = tid; c < clear_count; c += 256) clear[c] = 0;
+  const int4* plan = plan_ref.entries;
+  if (blockIdx.x == 0) begin_call(clear, clear_count, status, tid, 256);
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave >> 1, wn = wave & 1;
@@ -666,7 +698,8 @@ __global__ __launch_bounds__(256, 2) void gemm_bf16_mixed_kernel(
   int b, tile_m, tile_n;
   int live = R;
   if (plan != nullptr) {
-    const int4 mine = plan[blockIdx.x];
+    int4 mine;
+    if (!read_plan(plan_ref, status, tid, mine)) return;
     if (mine.x < 0) return;
     b = mine.x;
     tile_m = mine.y;
@@ -883,8 +916,9 @@ template <typename Cfg, int EPI, bool HAS_BIAS>
 __global__ __launch_bounds__(Cfg::kThreads, 1) void gemm_bf16_persistent_kernel(
     const bf16_t* __restrict__ A, const bf16_t* __restrict__ Bt, const bf16_t* __restrict__ bias,
     bf16_t* __restrict__ C, int R, int N, int Kd, int tiles_m, int tiles_n, int num_tiles,
-    int tiles_per_xcd, int panel_rows, const int4* __restrict__ plan, int plan_blocks,
-    float* __restrict__ sk_partials, int32_t* __restrict__ sk_flags) {
+    int tiles_per_xcd, int panel_rows, PlanRef plan_ref,
+    float* __restrict__ sk_partials, int32_t* __restrict__ sk_flags, int32_t* __restrict__ status,
+    int spin_limit, int wait_bias) {
 #if defined(__HIP_DEVICE_COMPILE__)   // buffer-resource builtins exist in the device pass only
   extern __shared__ __align__(1024) unsigned char smem[];
   constexpr int BM = Cfg::BM, BN = Cfg::BN, BK = Cfg::BK;
@@ -893,6 +927,14 @@ __global__ __launch_bounds__(Cfg::kThreads, 1) void gemm_bf16_persistent_kernel(
   constexpr int NS = Cfg::NSTAGE, PD = NS - 1, L = Cfg::kLoads;
   constexpr int KS = BK / 16;    // k slices (one MFMA deep) per k tile: 2 or 4
   const int tid = threadIdx.x;
+  const int4* plan = plan_ref.entries;
+  const int plan_blocks = plan_ref.blocks;
+  // A plan whose header does not carry this launch's tag was written for other shapes, or
+  // never: nothing runs, and the call's status words say so.
+  if (plan != nullptr && plan[plan_blocks].y != plan_ref.tag) {
+    if (blockIdx.x == 0 && tid == 0 && status != nullptr) atomicAdd(status + kStatusPlanMismatches, 1);
+    return;
+  }
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave / Cfg::WN, wn = wave % Cfg::WN;
@@ -1224,8 +1266,13 @@ __global__ __launch_bounds__(Cfg::kThreads, 1) void gemm_bf16_persistent_kernel(
     // A piece of a shared tile that is not the first to finish adds the sums deposited so
     // far, chunk by chunk in the epilogue below, the loads kAhead chunks ahead of their
     // use.  The other pieces were computed at the same time as this one, in workgroups
-    // with lower indices (placed before this one), so the wait is short; it is bounded
-    // all the same (sk_flags[kCusPerXcd * kNumXcd] counts the waits that gave up).
+    // with lower indices (placed before this one), so the wait is short.  That rests on all
+    // workgroups of the launch being resident at once, which holds on a GPU this launch has
+    // to itself; a kernel of another stream that holds compute units can keep a producer
+    // from starting while its consumer waits.  The wait is therefore bounded, and a piece
+    // that gives up does not pass off what it finds in memory as sums: it counts itself in
+    // the call's status words and turns every sum it would have taken into NaN, which the
+    // pieces behind it and the output rows then carry.
     const int waits = __builtin_amdgcn_readfirstlane(cur.waits);
     const bool adds_sums = waits > 0;
     typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
@@ -1238,19 +1285,24 @@ __global__ __launch_bounds__(Cfg::kThreads, 1) void gemm_bf16_persistent_kernel(
     const int shared_index = xcd * kCusPerXcd + __builtin_amdgcn_readfirstlane(cur.shared);
     const int sums_base = shared_index * (int)(kTileVecs * 16);
     u32x4_t ahead[kAhead];
+    bool poisoned = false;
     if (adds_sums) {
+      const int32_t* f = sk_flags + shared_index;
+      const int awaited = waits + wait_bias;    // (wait_bias: 0 outside the test of this path)
       if (tid == 0) {
-        const int32_t* f = sk_flags + shared_index;
         int spins = 0;
-        while (__hip_atomic_load(f, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < waits) {
+        while (__hip_atomic_load(f, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < awaited) {
           __builtin_amdgcn_s_sleep(16);
-          if (++spins > (1 << 22)) {
-            atomicAdd(sk_flags + kCusPerXcd * kNumXcd, 1);
+          if (++spins > spin_limit) {
+            if (status != nullptr) atomicAdd(status + kStatusAbandonedWaits, 1);
             break;
           }
         }
       }
       __syncthreads();
+      // (every wave looks for itself: the deposits are there, or its sums are poisoned)
+      poisoned = __builtin_amdgcn_readfirstlane(
+          (int)(__hip_atomic_load(f, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < awaited)) != 0;
 #pragma unroll
       for (int c = 0; c < kAhead; ++c)
         ahead[c] = __builtin_amdgcn_raw_buffer_load_b128(sums_rsrc, vec0 * 16, sums_base + c * 1024, kSumsAux);
@@ -1340,6 +1392,10 @@ __global__ __launch_bounds__(Cfg::kThreads, 1) void gemm_bf16_persistent_kernel(
             const int cidx = (i * FN + j) * 4 + q;
             if (adds_sums) {      // uniform over the workgroup
               v += __builtin_bit_cast(floatx4, ahead[cidx % kAhead]);
+              if (poisoned) {
+                const float nan = __builtin_nanf("");
+                v = floatx4{nan, nan, nan, nan};
+              }
               if (cidx + kAhead < kChunks)
                 ahead[cidx % kAhead] = __builtin_amdgcn_raw_buffer_load_b128(
                     sums_rsrc, vec0 * 16, sums_base + (cidx + kAhead) * 1024, kSumsAux);
@@ -1512,17 +1568,28 @@ GemmGeom gemm_geometry(int batch, int R, int N, int Kd) {
   return g;
 }
 
+// The plan of a launch with geometry g as its kernel takes it (tag: what the planner wrote
+// for the same geometry, batch count and rows per batch).
+template <typename Cfg>
+PlanRef plan_ref(const GemmGeom& g, const int4* plan, int batch, int R) {
+  if (plan == nullptr) return PlanRef{nullptr, 0, 0};
+  const int blocks = (int)(g.ragged_slots * kNumXcd);
+  return PlanRef{plan, blocks, plan_tag(Cfg::BM, g.tiles_n, g.panel_rows, blocks, batch, R)};
+}
+
 // `plan`, if given, was filled by plan_ragged_tiles_kernel for this product's geometry.
+// `clear` / `status`: see begin_call.
 template <typename Cfg, int EPI>
 int launch_gemm_bf16(const bf16_t* A, const bf16_t* Bt, const bf16_t* bias, bf16_t* C, int batch,
                      int R, int N, int Kd, hipStream_t stream, const int32_t* rows = nullptr,
                      const int4* plan = nullptr, const int32_t* a_rows = nullptr,
-                     long long a_items = 0, int32_t* clear = nullptr, int clear_count = 0) {
+                     long long a_items = 0, int32_t* clear = nullptr, int clear_count = 0,
+                     int32_t* status = nullptr) {
   const GemmGeom g = gemm_geometry<Cfg>(batch, R, N, Kd);
-  if (clear != nullptr && !g.fast) {
-    hipLaunchKernelGGL(clear_i32_kernel, dim3((clear_count + 255) / 256), dim3(256), 0, stream, clear,
-                       clear_count);
+  if ((clear != nullptr || status != nullptr) && !g.fast) {
+    hipLaunchKernelGGL(begin_call_kernel, dim3(1), dim3(256), 0, stream, clear, clear_count, status);
     clear = nullptr;
+    status = nullptr;
   }
   if (a_rows != nullptr && (!g.fast || rows == nullptr ||
                             (unsigned long long)a_items * Kd * 2 >= (1ull << 32)))
@@ -1542,7 +1609,8 @@ int launch_gemm_bf16(const bf16_t* A, const bf16_t* Bt, const bf16_t* bias, bf16
   if (e != hipSuccess) return (int)e;
   hipLaunchKernelGGL(kern, dim3(blocks), dim3(Cfg::kThreads), Cfg::kLdsBytes, stream, A, Bt, bias,
                      C, R, N, Kd, g.tiles_m, g.tiles_n, (int)g.tiles, g.tiles_per_xcd, g.panel_rows,
-                     rows, plan, a_rows, (int)a_items, clear, clear_count);
+                     rows, plan_ref<Cfg>(g, plan, batch, R), a_rows, (int)a_items, clear, clear_count,
+                     status);
   return launch_status();
 }
 
@@ -1555,7 +1623,7 @@ template <int EPI>
 int launch_gemm_bf16_first(const bf16_t* A, const bf16_t* Bt, const bf16_t* bias, bf16_t* C,
                            int batch, int R, int N, int Kd, hipStream_t stream,
                            const int32_t* rows, const int4* plan, const int32_t* a_rows,
-                           long long a_items, int32_t* clear, int clear_count) {
+                           long long a_items, int32_t* clear, int clear_count, int32_t* status) {
   using Cfg = GemmCfg<128, 256, 2, 2, 32, 3, 2>;
   const GemmGeom g = gemm_geometry<Cfg>(batch, R, N, Kd);
   const bool gather_ok = a_rows == nullptr ||
@@ -1563,7 +1631,7 @@ int launch_gemm_bf16_first(const bf16_t* A, const bf16_t* Bt, const bf16_t* bias
   if (!g.fast || Kd % 64 != 0 || Kd < 128 || !gather_ok || g.tiles > 0x7ffffff0LL ||
       getenv("VMOE_FIRST_PRODUCT_K32") != nullptr)
     return launch_gemm_bf16<Cfg, EPI>(A, Bt, bias, C, batch, R, N, Kd, stream, rows, plan, a_rows,
-                                      a_items, clear, clear_count);
+                                      a_items, clear, clear_count, status);
   constexpr size_t kLds = 2 * 128 * 64 + 2 * 256 * 128;
   static_assert(kLds * 2 <= 160 * 1024, "two workgroups per CU");
   const unsigned blocks = (unsigned)(plan != nullptr ? g.ragged_slots : g.tiles_per_xcd) * kNumXcd;
@@ -1571,8 +1639,8 @@ int launch_gemm_bf16_first(const bf16_t* A, const bf16_t* Bt, const bf16_t* bias
   hipError_t e = allow_dynamic_lds(reinterpret_cast<const void*>(kern), kLds);
   if (e != hipSuccess) return (int)e;
   hipLaunchKernelGGL(kern, dim3(blocks), dim3(256), kLds, stream, A, Bt, bias, C, R, N, Kd,
-                     g.tiles_m, g.tiles_n, (int)g.tiles, g.tiles_per_xcd, g.panel_rows, rows, plan,
-                     a_rows, (int)a_items, clear, clear_count);
+                     g.tiles_m, g.tiles_n, (int)g.tiles, g.tiles_per_xcd, g.panel_rows, rows,
+                     plan_ref<Cfg>(g, plan, batch, R), a_rows, (int)a_items, clear, clear_count, status);
   return launch_status();
 }
 
@@ -1589,12 +1657,12 @@ bool persistent_gemm_ok(int batch, int R, int N, int Kd, const int32_t* rows, co
 }
 
 // Memory of the stream-K exchange of a tile-walking launch: one tile of float32 partial
-// sums per workgroup, then one flag per workgroup and the counter of abandoned waits.
+// sums per workgroup, then one flag per workgroup.
 template <typename Cfg>
 struct StreamKWorkspace {
   static constexpr int kBlocks = kCusPerXcd * kNumXcd;
   static constexpr size_t kPartialBytes = (size_t)kBlocks * Cfg::BM * Cfg::BN * sizeof(float);
-  static constexpr int kFlags = kBlocks + 1;
+  static constexpr int kFlags = kBlocks;
   static constexpr size_t kBytes = kPartialBytes + (size_t)(kFlags + 63) / 64 * 256;
   static float* partials(void* ws) { return static_cast<float*>(ws); }
   static int32_t* flags(void* ws) {
@@ -1606,12 +1674,14 @@ struct StreamKWorkspace {
 // given, was filled by plan_ragged_tiles_kernel for gemm_geometry<Cfg> (BM, BN and
 // workgroups per CU decide it, not the number of stages).  `streamk`, if given, is
 // StreamKWorkspace<Cfg>::kBytes of memory: the die's last, partial round is then shared
-// along k.  `flags_clear`: the planning launch has already cleared its flags.
+// along k; an earlier launch of the call has set its flags to zero (begin_call).  `status`:
+// the call's status words.
+// VMOE_STREAMK_TEST_GIVE_UP=<spins> in the environment (the test of the bounded wait): pieces
+// wait for deposits that never come, for at most that many polls, and give up.
 template <typename Cfg, int EPI>
 int launch_gemm_bf16_persistent(const bf16_t* A, const bf16_t* Bt, const bf16_t* bias, bf16_t* C,
                                 int batch, int R, int N, int Kd, hipStream_t stream,
-                                const int4* plan = nullptr, void* streamk = nullptr,
-                                bool flags_clear = false) {
+                                const int4* plan, void* streamk, int32_t* status) {
   const GemmGeom g = gemm_geometry<Cfg>(batch, R, N, Kd);
   auto kern = bias != nullptr ? gemm_bf16_persistent_kernel<Cfg, EPI, true>
                               : gemm_bf16_persistent_kernel<Cfg, EPI, false>;
@@ -1625,15 +1695,16 @@ int launch_gemm_bf16_persistent(const bf16_t* A, const bf16_t* Bt, const bf16_t*
   if (streamk != nullptr && getenv("VMOE_WHOLE_TILES") == nullptr) {
     partials = SK::partials(streamk);
     flags = SK::flags(streamk);
-    if (!flags_clear)
-      hipLaunchKernelGGL(clear_i32_kernel, dim3((SK::kFlags + 255) / 256), dim3(256), 0, stream,
-                         flags, SK::kFlags);
   }
-  const int plan_blocks = plan != nullptr ? (int)(g.ragged_slots * kNumXcd) : 0;
+  int spin_limit = 1 << 22, wait_bias = 0;     // polls ~0.5 us apart: about two seconds
+  if (const char* t = getenv("VMOE_STREAMK_TEST_GIVE_UP")) {
+    spin_limit = atoi(t) > 0 ? atoi(t) : 1;
+    wait_bias = 1 << 20;
+  }
   hipLaunchKernelGGL(kern, dim3(kCusPerXcd * kNumXcd), dim3(Cfg::kThreads),
                      PersistentLds<Cfg>::kBytes, stream, A, Bt, bias, C, R, N, Kd, g.tiles_m,
-                     g.tiles_n, (int)g.tiles, g.tiles_per_xcd, g.panel_rows, plan, plan_blocks,
-                     partials, flags);
+                     g.tiles_n, (int)g.tiles, g.tiles_per_xcd, g.panel_rows,
+                     plan_ref<Cfg>(g, plan, batch, R), partials, flags, status, spin_limit, wait_bias);
   return launch_status();
 }
 

@@ -55,14 +55,21 @@ template <typename Cfg, int EPI, bool HAS_BIAS, bool GATHER>
 __global__ __launch_bounds__(Cfg::kThreads, 1) void gemm_bf16_wide_kernel(
     const bf16_t* __restrict__ A, const bf16_t* __restrict__ Bt, const bf16_t* __restrict__ bias,
     bf16_t* __restrict__ C, int R, int N, int Kd, int tiles_m, int tiles_n, int num_tiles,
-    int tiles_per_xcd, int panel_rows, const int4* __restrict__ plan, int plan_blocks,
-    const int32_t* __restrict__ a_rows, int a_items) {
+    int tiles_per_xcd, int panel_rows, PlanRef plan_ref,
+    const int32_t* __restrict__ a_rows, int a_items, int32_t* __restrict__ status) {
 #if defined(__HIP_DEVICE_COMPILE__)   // buffer-resource builtins exist in the device pass only
   extern __shared__ __align__(1024) unsigned char smem[];
   constexpr int BM = Cfg::BM, BN = Cfg::BN, BK = Cfg::BK;
   constexpr int RB = Cfg::kRowBytes, NS = Cfg::NSTAGE, L = Cfg::kLoads, STAGE = Cfg::kStageBytes;
   constexpr int CPR = Cfg::kChunksPerRow, RPL = Cfg::kRowsPerLoad;
   const int tid = threadIdx.x;
+  const int4* plan = plan_ref.entries;
+  const int plan_blocks = plan_ref.blocks;
+  // (a plan whose header does not carry this launch's tag: nothing runs, the status words say so)
+  if (plan != nullptr && plan[plan_blocks].y != plan_ref.tag) {
+    if (blockIdx.x == 0 && tid == 0 && status != nullptr) atomicAdd(status + kStatusPlanMismatches, 1);
+    return;
+  }
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave / Cfg::WN, wn = wave % Cfg::WN;
@@ -297,20 +304,21 @@ inline bool wide_gemm_ok(int batch, int R, int N, int Kd, const int32_t* rows, c
 template <int EPI, typename Cfg = WideCfg>
 int launch_gemm_bf16_wide(const bf16_t* A, const bf16_t* Bt, const bf16_t* bias, bf16_t* C, int batch,
                           int R, int N, int Kd, hipStream_t stream, const int4* plan = nullptr,
-                          const int32_t* a_rows = nullptr, long long a_items = 0) {
+                          const int32_t* a_rows = nullptr, long long a_items = 0,
+                          int32_t* status = nullptr) {
   const GemmGeom g = gemm_geometry<Cfg>(batch, R, N, Kd);
   void (*kern)(const bf16_t*, const bf16_t*, const bf16_t*, bf16_t*, int, int, int, int, int, int, int,
-               int, const int4*, int, const int32_t*, int);
+               int, PlanRef, const int32_t*, int, int32_t*);
   if (a_rows != nullptr)
     kern = bias != nullptr ? gemm_bf16_wide_kernel<Cfg, EPI, true, true> : gemm_bf16_wide_kernel<Cfg, EPI, false, true>;
   else
     kern = bias != nullptr ? gemm_bf16_wide_kernel<Cfg, EPI, true, false> : gemm_bf16_wide_kernel<Cfg, EPI, false, false>;
   hipError_t e = allow_dynamic_lds(reinterpret_cast<const void*>(kern), Cfg::kLdsBytes);
   if (e != hipSuccess) return (int)e;
-  const int plan_blocks = plan != nullptr ? (int)(g.ragged_slots * kNumXcd) : 0;
   hipLaunchKernelGGL(kern, dim3(kCusPerXcd * kNumXcd), dim3(Cfg::kThreads), Cfg::kLdsBytes,
                      stream, A, Bt, bias, C, R, N, Kd, g.tiles_m, g.tiles_n, (int)g.tiles,
-                     g.tiles_per_xcd, g.panel_rows, plan, plan_blocks, a_rows, (int)a_items);
+                     g.tiles_per_xcd, g.panel_rows, plan_ref<Cfg>(g, plan, batch, R), a_rows,
+                     (int)a_items, status);
   return launch_status();
 }
 

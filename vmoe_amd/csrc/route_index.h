@@ -88,6 +88,25 @@ struct RaggedGeom {
   int bm, tiles_n, panel_rows, num_blocks;
   PlanEntry* plan;
 };
+// Entry num_blocks of a plan, one past its last workgroup's, is its header: (live row tiles
+// of all batches, tag, 0, 0).  The tag names what the plan was written for -- tile height,
+// column tiles, panel height, workgroups, batches and rows per batch -- and a product kernel
+// that does not find the tag of its own launch there runs nothing: a workspace that was never
+// planned, or was planned for other shapes, cannot drive its addressing.
+VMOE_HD int32_t plan_tag(int bm, int tiles_n, int panel_rows, int num_blocks, int batch, int R) {
+  const int v[6] = {bm, tiles_n, panel_rows, num_blocks, batch, R};
+  uint32_t h = 0x564d4f45u;
+  for (int i = 0; i < 6; ++i) {
+    h = (h ^ (uint32_t)v[i]) * 0x9E3779B1u;
+    h ^= h >> 15;
+  }
+  return (int32_t)(h | 1u);
+}
+// Status words of an expert MLP call (int32, in its workspace).  They only ever grow: the
+// first launch of a call sets them to zero when the tag word does not yet say that it did.
+enum { kStatusAbandonedWaits = 0, kStatusPlanMismatches = 1, kStatusTagWord = 2, kStatusWords = 3 };
+constexpr int32_t kStatusTag = 0x56537461;
+
 VMOE_HD int plan_min(int a, int b) { return a < b ? a : b; }
 VMOE_HD int plan_max(int a, int b) { return a > b ? a : b; }
 

@@ -302,6 +302,7 @@ def expert_mlp(x: torch.Tensor, w0, b0, w1, b1, w0t=None, w1t=None, approximate_
     workspace = torch.empty(need, dtype=torch.uint8, device=x.device)
   p.workspace = H.ptr(workspace)
   p.workspace_bytes = workspace.numel() * workspace.element_size()
+  _note_status_words(p, workspace)
   if compact is None:
     H.call("vmoe_expert_mlp", p)
     return out
@@ -314,11 +315,53 @@ def expert_mlp(x: torch.Tensor, w0, b0, w1, b1, w0t=None, w1t=None, approximate_
     rc = H.call_blocks("vmoe_compact_rows_planned", c, p, accept=(_E_UNSUPPORTED,))
   if rc == 0:
     H.call("vmoe_expert_mlp_planned", p)
+    global _last_planned
+    _last_planned = (p, (x, w0, b0, w1, b1, w0t, w1t, out, workspace) + maps)
   else:
     c.prefix = H.ptr(_i32(G, E, device=fill.device))
     H.call("vmoe_compact_rows", c)
     H.call("vmoe_expert_mlp", p)
   return out, maps
+
+
+_last_planned = None
+
+
+def expert_mlp_replay_planned() -> torch.Tensor:
+  """Issues vmoe_expert_mlp_planned again with the parameter block of the most recent
+  expert_mlp(compact=...) call that planned its launches (same routing, same buffers: what a
+  serving loop or a graph of the experts alone does) and returns that call's output tensor."""
+  if _last_planned is None:
+    raise RuntimeError("no planned expert_mlp call to repeat")
+  p, keep = _last_planned
+  H.call("vmoe_expert_mlp_planned", p)
+  return keep[7]
+
+
+_last_status_words: Optional[torch.Tensor] = None
+
+
+def _note_status_words(p, workspace: torch.Tensor) -> None:
+  """Remembers where the status words of this call's workspace are (vmoe_expert_mlp_status)."""
+  global _last_status_words
+  addr = ctypes.c_void_p()
+  H.check(H.lib().vmoe_expert_mlp_status(ctypes.byref(p), ctypes.byref(addr)), "vmoe_expert_mlp_status")
+  if not addr.value:
+    _last_status_words = None
+    return
+  off = addr.value - workspace.data_ptr()
+  flat = workspace.view(torch.uint8).reshape(-1)
+  _last_status_words = flat[off:off + 4 * H.MLP_STATUS_WORDS].view(torch.int32)
+
+
+def expert_mlp_status() -> Optional[Tuple[int, int]]:
+  """(abandoned waits, plan mismatches) counted so far on the workspace of the most recent
+  expert_mlp call (synchronises); None for float32.  Anything but (0, 0) means that some
+  call on that workspace did not produce the product it should have."""
+  if _last_status_words is None:
+    return None
+  words = _last_status_words.cpu()
+  return int(words[H.MLP_STATUS_ABANDONED_WAITS]), int(words[H.MLP_STATUS_PLAN_MISMATCHES])
 
 
 def expert_mlp_can_gather(dtype: torch.dtype, D: int, num_items: int) -> bool:
