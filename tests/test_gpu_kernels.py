@@ -891,6 +891,52 @@ def test_expert_mlp_second_product_walks_several_tiles(K, with_bias):
     assert (to_np(out[e, n:]) == 7.0).all(), f"expert {e}"
 
 
+@pytest.mark.parametrize("E,R,D,M", [
+    (64, 1100, 768, 256),     # 960 tiles: the kernel's own choice; four k tiles (the shortest k it takes)
+    (40, 1300, 1024, 512),    # 960 tiles, four column tiles
+    (3, 500, 520, 1024),      # forced: a column tile that ends inside the tile, few tiles per die
+    (5, 257, 264, 320),       # forced: one row past a tile, k of five tiles
+])
+def test_expert_mlp_second_product_on_eight_waves(K, monkeypatch, E, R, D, M):
+  """The eight-wave form of the second product (two waves per SIMD, output leaving through lane
+  exchanges instead of LDS) against the four-wave tile-walking kernel with whole tiles: both
+  add the same products in the same order, so the outputs must agree bit for bit; dense and
+  over packed rows with a launch plan (rows past a count are not written)."""
+  rng = np.random.default_rng(E * 100 + M)
+  args = [to_dev(O.cast(a, O.BF16), O.BF16) for a in (
+      rng.standard_normal((E, R, D)).astype(np.float32),
+      rng.standard_normal((E, D, M)).astype(np.float32) / np.sqrt(D),
+      rng.standard_normal((E, M)).astype(np.float32) * 0.1,
+      rng.standard_normal((E, M, D)).astype(np.float32) / np.sqrt(M),
+      rng.standard_normal((E, D)).astype(np.float32) * 0.1)]
+  rows = rng.integers(0, R + 1, E).astype(np.int32)
+  rows[:3] = [R, 0, 257][:min(3, E)]
+  outs = {}
+  for which in ("eight", "shared"):
+    monkeypatch.setenv("VMOE_SECOND_PRODUCT", which)
+    monkeypatch.setenv("VMOE_WHOLE_TILES", "1")
+    dense = K.expert_mlp(*args)
+    ragged = torch.full_like(dense, 7.0)
+    K.expert_mlp(*args, out=ragged, rows_per_expert=to_dev(rows))
+    outs[which] = (to_np(dense), to_np(ragged))
+    assert K.expert_mlp_status() == (0, 0)
+  monkeypatch.delenv("VMOE_SECOND_PRODUCT")
+  monkeypatch.delenv("VMOE_WHOLE_TILES")
+  np.testing.assert_array_equal(outs["eight"][0], outs["shared"][0])
+  for e, n in enumerate(rows):
+    np.testing.assert_array_equal(outs["eight"][1][e, :n], outs["shared"][1][e, :n], err_msg=f"expert {e}")
+    np.testing.assert_array_equal(outs["eight"][1][e, :n], outs["eight"][0][e, :n], err_msg=f"expert {e}")
+    assert (outs["eight"][1][e, n:] == 7.0).all(), f"expert {e}"
+  # and against a float32 restatement of one expert
+  e = E - 1
+  x, w0, b0, w1, b1 = (a[e].float() for a in args)
+  bf = torch.bfloat16
+  h = ((x @ w0).to(bf).float() + b0).to(bf)
+  h = torch.nn.functional.gelu(h.float(), approximate="tanh").to(bf)
+  want = ((h.float() @ w1).to(bf).float() + b1).to(bf)
+  np.testing.assert_allclose(outs["eight"][0][e], to_np(want), rtol=2e-2, atol=2e-2)
+
+
 SHARED_ROUND_CASES = [
     (16, 2321, 520, 1024),    # 60 tiles per die: one round, then 28 tiles shared by 32 workgroups (pieces of 12-16 k tiles)
     (32, 768, 768, 768),      # 36 per die: 4 tiles in pieces of 4 k tiles, chains of three

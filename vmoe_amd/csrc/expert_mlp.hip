@@ -7,6 +7,7 @@
 #include <cstring>
 
 #include "gemm_bf16_wide.h"
+#include "gemm_bf16_w8.h"
 #include "compact_rows.h"
 
 namespace vmoe {
@@ -261,11 +262,14 @@ static_assert(kStatusWords * sizeof(int32_t) <= kStatusBytes, "status block");
 // Which kernel runs the second product (bfloat16).
 //  kDownShared: 256 x 256 tiles walked by one workgroup per CU, the last, partial round of a
 //    die shared along k (stream-K): its time follows the number of tiles, not of rounds.
+//  kDownEightWaves: the same tiles walked by eight waves per workgroup (gemm_bf16_w8.h), the
+//    tiles of a partial round whole: ahead by about 3 % where a die's run is three rounds or
+//    longer, so that a partial round is a small part of it.
 //  kDownWide: 384 x 256 tiles, eight waves; whole rounds of one tile per CU.
 //  kDownHalf: 128 x 256 tiles, two per CU (static launches the tile-walking kernels do not
 //    cover, where whole rounds of 256 x 256 tiles would waste a tenth or more).
 //  kDownPlain: 256 x 256 tiles, one workgroup per tile.
-enum DownKernel { kDownShared, kDownWide, kDownHalf, kDownPlain };
+enum DownKernel { kDownShared, kDownEightWaves, kDownWide, kDownHalf, kDownPlain };
 
 bool down_prefers_half_tiles(int E, int R, int N) {
   constexpr int64_t kNumCu = 256;
@@ -316,7 +320,13 @@ MlpPlans mlp_plans(int E, int R, int D, int M, bool ragged) {
   // figures the wide kernel only runs where the shared one does not apply.
   const double t_wide = 1.5 * 1.04 * std::ceil((double)wide.tiles / kNumCu);
   const double t_shared = (double)square.tiles / kNumCu + 0.05;
-  if (shared_ok && (!wide_ok || t_shared <= t_wide)) m.down_kernel = kDownShared;
+  // Eight waves where they apply and a die's run of tiles is at least three rounds long (the
+  // B/16 layer: 144 - 150 tiles per die, 1.004 -> 0.990 ms per step in three alternating pairs
+  // of runs; the Soft MoE layer's 48 tiles per die gain more from the shared round).
+  const bool w8_ok = w8_gemm_ok(E, R, D, M, rows, bytes(square) ? planned : nullptr) &&
+                     square.tiles >= 3LL * (long long)kNumCu;
+  if (shared_ok && w8_ok) m.down_kernel = kDownEightWaves;
+  else if (shared_ok && (!wide_ok || t_shared <= t_wide)) m.down_kernel = kDownShared;
   else if (wide_ok) m.down_kernel = kDownWide;
   else if (!ragged && down_prefers_half_tiles(E, R, D)) m.down_kernel = kDownHalf;
   else m.down_kernel = kDownPlain;
@@ -324,6 +334,8 @@ MlpPlans mlp_plans(int E, int R, int D, int M, bool ragged) {
   // two where both apply: the switch behind the figures that the model above was fitted to)
   if (const char* force = getenv("VMOE_SECOND_PRODUCT")) {
     if (strcmp(force, "shared") == 0 && shared_ok) m.down_kernel = kDownShared;
+    if (strcmp(force, "eight") == 0 && w8_gemm_ok(E, R, D, M, rows, bytes(square) ? planned : nullptr))
+      m.down_kernel = kDownEightWaves;
     if (strcmp(force, "wide") == 0 && wide_ok) m.down_kernel = kDownWide;
   }
   m.down = m.down_kernel == kDownWide ? wide : square;
@@ -483,6 +495,10 @@ static int run_expert_mlp(const VmoeExpertMlpParams* p, vmoe_stream_t stream_, b
         return launch_gemm_bf16_persistent<CfgDownPersistent, kEpiBias>(
             (const bf16_t*)hidden, (const bf16_t*)w1t, (const bf16_t*)p->b1, (bf16_t*)p->out, p->E,
             p->R, p->D, p->M, stream, plan_down, streamk, status);
+      case kDownEightWaves:
+        return launch_gemm_bf16_w8<kEpiBias>((const bf16_t*)hidden, (const bf16_t*)w1t,
+                                             (const bf16_t*)p->b1, (bf16_t*)p->out, p->E, p->R, p->D,
+                                             p->M, stream, plan_down, nullptr, 0, status);
       case kDownWide:
         return launch_gemm_bf16_wide<kEpiBias>((const bf16_t*)hidden, (const bf16_t*)w1t,
                                                (const bf16_t*)p->b1, (bf16_t*)p->out, p->E, p->R,

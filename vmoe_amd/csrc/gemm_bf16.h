@@ -38,6 +38,7 @@
 #define VMOE_GEMM_BF16_H_
 
 #include <cmath>
+#include <cstdio>
 #include <cstdlib>
 #include <type_traits>
 #include "vmoe_common.h"
@@ -190,13 +191,25 @@ __device__ __forceinline__ void store_tile(floatx16 (&acc)[TM / 32][TN / 32], un
     const uint32_t lane_off = (uint32_t)(orow * N + oc) * 2u;
     const int row_u = __builtin_amdgcn_readfirstlane(wrow0), col_u = __builtin_amdgcn_readfirstlane(wcol0);
     const bool col_ok = oc + 8 <= N - col_u;
+    // (four staged pieces are read before the first of them is stored: the guard behind a
+    // store keeps every later instruction behind it, the reads of later pieces included)
+    constexpr int kBatch = 4;
+    static_assert(TM / kRowsPerPass % kBatch == 0, "passes come in batches of four");
 #pragma unroll
-    for (int r0 = 0; r0 < TM; r0 += kRowsPerPass) {
-      const uint4 v = *reinterpret_cast<const uint4*>(so + (r0 + orow) * OLD + oc);
-      const bool ok = col_ok && orow < live - (row_u + r0);
-      __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4_t, v), c_rsrc,
-                                             ok ? lane_off : 0xfffffff0u,
-                                             ((row_u + r0) * N + col_u) * 2, EPI != kEpiBias ? 2 : 0);
+    for (int r0 = 0; r0 < TM; r0 += kBatch * kRowsPerPass) {
+      uint4 v[kBatch];
+#pragma unroll
+      for (int t = 0; t < kBatch; ++t)
+        v[t] = *reinterpret_cast<const uint4*>(so + (r0 + t * kRowsPerPass + orow) * OLD + oc);
+#pragma unroll
+      for (int t = 0; t < kBatch; ++t) {
+        const int rs = r0 + t * kRowsPerPass;
+        const bool ok = col_ok && orow < live - (row_u + rs);
+        __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4_t, v[t]), c_rsrc,
+                                               ok ? lane_off : 0xfffffff0u,
+                                               ((row_u + rs) * N + col_u) * 2, EPI != kEpiBias ? 2 : 0);
+        store_data_guard();
+      }
     }
     return;
   }
@@ -682,7 +695,7 @@ __global__ __launch_bounds__(256, 2) void gemm_bf16_mixed_kernel(
     bf16_t* __restrict__ C, int R, int N, int Kd, int tiles_m, int tiles_n, int num_tiles,
     int tiles_per_xcd, int panel_rows, const int32_t* __restrict__ rows,
     PlanRef plan_ref, const int32_t* __restrict__ a_rows, int a_items,
-    int32_t* __restrict__ clear, int clear_count, int32_t* __restrict__ status) {
+    int32_t* __restrict__ clear, int clear_count, int32_t* __restrict__ status, int active_xcds) {
 #if defined(__HIP_DEVICE_COMPILE__)   // buffer-resource builtins exist in the device pass only
   extern __shared__ __align__(1024) unsigned char smem[];
   constexpr int BM = 128, BN = 256, TM = 64, TN = 128, FM = 2, FN = 4, kWaves = 4;
@@ -690,6 +703,7 @@ __global__ __launch_bounds__(256, 2) void gemm_bf16_mixed_kernel(
   const int tid = threadIdx.x;
   const int4* plan = plan_ref.entries;
   if (blockIdx.x == 0) begin_call(clear, clear_count, status, tid, 256);
+  if ((int)(blockIdx.x % kNumXcd) >= active_xcds) return;   // (measurement only, see active_units)
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave >> 1, wn = wave & 1;
@@ -918,7 +932,7 @@ __global__ __launch_bounds__(Cfg::kThreads, 1) void gemm_bf16_persistent_kernel(
     bf16_t* __restrict__ C, int R, int N, int Kd, int tiles_m, int tiles_n, int num_tiles,
     int tiles_per_xcd, int panel_rows, PlanRef plan_ref,
     float* __restrict__ sk_partials, int32_t* __restrict__ sk_flags, int32_t* __restrict__ status,
-    int spin_limit, int wait_bias) {
+    int spin_limit, int wait_bias, int active_xcds, int active_slots) {
 #if defined(__HIP_DEVICE_COMPILE__)   // buffer-resource builtins exist in the device pass only
   extern __shared__ __align__(1024) unsigned char smem[];
   constexpr int BM = Cfg::BM, BN = Cfg::BN, BK = Cfg::BK;
@@ -940,6 +954,7 @@ __global__ __launch_bounds__(Cfg::kThreads, 1) void gemm_bf16_persistent_kernel(
   const int wm = wave / Cfg::WN, wn = wave % Cfg::WN;
   const int m = lane & 31, h = lane >> 5;
   const int xcd = blockIdx.x % kNumXcd, slot = blockIdx.x / kNumXcd;
+  if (xcd >= active_xcds || slot >= active_slots) return;   // (measurement only, see active_units)
   constexpr int CPR = Cfg::kChunksPerRow;
   constexpr int RPL = Cfg::kRowsPerLoad;
   const int lrow = lane / CPR;
@@ -1355,16 +1370,23 @@ __global__ __launch_bounds__(Cfg::kThreads, 1) void gemm_bf16_persistent_kernel(
               *reinterpret_cast<uint2*>(so + m * OLD + cl) = make_uint2(p0, p1);
             }
           }
+          // (all staged pieces are read before the first is stored: the guard behind a store
+          // keeps every later instruction behind it)
+          constexpr int kPasses = 32 / kRowsPerPass;
+          uint4 staged[kPasses];
 #pragma unroll
-          for (int r0 = 0; r0 < 32; r0 += kRowsPerPass) {
+          for (int t = 0; t < kPasses; ++t)
+            staged[t] = *reinterpret_cast<const uint4*>(so + (t * kRowsPerPass + orow) * OLD + oc);
+#pragma unroll
+          for (int t = 0; t < kPasses; ++t) {
             // (lane part of the address in the vector offset, which the range check sees;
             // the pass's part, uniform, in the scalar offset)
-            const uint4 v = *reinterpret_cast<const uint4*>(so + (r0 + orow) * OLD + oc);
-            const int row_s = wrow0 + i * 32 + r0, col_s = wcol0 + c0;
+            const int row_s = wrow0 + i * 32 + t * kRowsPerPass, col_s = wcol0 + c0;
             const bool ok = orow < cur.live - row_s && oc + 8 <= N - col_s;
-            __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4_t, v), c_rsrc,
+            __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4_t, staged[t]), c_rsrc,
                                                    ok ? lane_off : 0xfffffff0u,
                                                    (row_s * N + col_s) * 2, EPI != kEpiBias ? 2 : 0);
+            store_data_guard();
           }
         }
       }
@@ -1403,6 +1425,7 @@ __global__ __launch_bounds__(Cfg::kThreads, 1) void gemm_bf16_persistent_kernel(
             if (leaves_sums) {    // uniform over the workgroup
               __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4_t, v), sums_rsrc,
                                                      vec0 * 16, sums_base + cidx * 1024, kSumsAux);
+              store_data_guard();
             } else {
               const uint32_t p0 = epilogue_pair<EPI, HAS_BIAS>(v[0], v[1], bv[0], bv[1]);
               const uint32_t p1 = epilogue_pair<EPI, HAS_BIAS>(v[2], v[3], bv[2], bv[3]);
@@ -1614,6 +1637,22 @@ int launch_gemm_bf16(const bf16_t* A, const bf16_t* Bt, const bf16_t* bias, bf16
   return launch_status();
 }
 
+// Measurement only: VMOE_GEMM_ACTIVE=<dies>x<compute units per die> in the environment makes
+// the workgroups of the other dies (first and second product) and of the other compute units
+// of a die (second product, one workgroup per compute unit) leave at once.  The work of those
+// that left is not done, so the outputs are incomplete; what the launch then shows is the rate
+// of a die or compute unit when its neighbours are idle, i.e. whether the products are held
+// back by something the whole chip shares.  Unset: all 8 x 32.
+struct ActiveUnits { int xcds, slots; };
+inline ActiveUnits active_units() {
+  ActiveUnits a{kNumXcd, 32};
+  if (const char* t = getenv("VMOE_GEMM_ACTIVE")) {
+    int x = 0, c = 0;
+    if (sscanf(t, "%dx%d", &x, &c) == 2 && x >= 1 && x <= kNumXcd && c >= 1 && c <= 32) a = ActiveUnits{x, c};
+  }
+  return a;
+}
+
 // The first product of an MLP: gemm_bf16_mixed_kernel where it applies (k a multiple of 64
 // and at least 128), else gemm_bf16_kernel with the same tiling; launch geometry and plan are
 // those of GemmCfg<128, 256, 2, 2, 32, 3, 2> either way.  VMOE_FIRST_PRODUCT_K32=1 in the
@@ -1640,7 +1679,8 @@ int launch_gemm_bf16_first(const bf16_t* A, const bf16_t* Bt, const bf16_t* bias
   if (e != hipSuccess) return (int)e;
   hipLaunchKernelGGL(kern, dim3(blocks), dim3(256), kLds, stream, A, Bt, bias, C, R, N, Kd,
                      g.tiles_m, g.tiles_n, (int)g.tiles, g.tiles_per_xcd, g.panel_rows, rows,
-                     plan_ref<Cfg>(g, plan, batch, R), a_rows, (int)a_items, clear, clear_count, status);
+                     plan_ref<Cfg>(g, plan, batch, R), a_rows, (int)a_items, clear, clear_count, status,
+                     active_units().xcds);
   return launch_status();
 }
 
@@ -1692,7 +1732,9 @@ int launch_gemm_bf16_persistent(const bf16_t* A, const bf16_t* Bt, const bf16_t*
   int32_t* flags = nullptr;
   // (VMOE_WHOLE_TILES=1 in the environment keeps every tile whole: the switch behind the
   // before / after figures of the shared round)
-  if (streamk != nullptr && getenv("VMOE_WHOLE_TILES") == nullptr) {
+  const ActiveUnits active = active_units();
+  const bool all_active = active.xcds == kNumXcd && active.slots == kCusPerXcd;
+  if (streamk != nullptr && getenv("VMOE_WHOLE_TILES") == nullptr && all_active) {
     partials = SK::partials(streamk);
     flags = SK::flags(streamk);
   }
@@ -1704,7 +1746,8 @@ int launch_gemm_bf16_persistent(const bf16_t* A, const bf16_t* Bt, const bf16_t*
   hipLaunchKernelGGL(kern, dim3(kCusPerXcd * kNumXcd), dim3(Cfg::kThreads),
                      PersistentLds<Cfg>::kBytes, stream, A, Bt, bias, C, R, N, Kd, g.tiles_m,
                      g.tiles_n, (int)g.tiles, g.tiles_per_xcd, g.panel_rows,
-                     plan_ref<Cfg>(g, plan, batch, R), partials, flags, status, spin_limit, wait_bias);
+                     plan_ref<Cfg>(g, plan, batch, R), partials, flags, status, spin_limit, wait_bias,
+                     active.xcds, active.slots);
   return launch_status();
 }
 

@@ -98,6 +98,19 @@ __device__ __forceinline__ void mfma_result_fence() {
   __builtin_amdgcn_sched_barrier(0);
 }
 
+// Gap behind a 16-byte buffer store whose data registers the next instructions overwrite.
+// The store reads its data registers a few cycles after it has issued.  For a store with an
+// immediate scalar offset the compiler leaves the wait states itself; for one whose scalar
+// offset is a register it leaves none, and a VALU result written to a data register in the very
+// next instruction reached memory in place of the stored value in a few lanes (seen with the
+// register-hungry GELU epilogue, where the allocator reuses the registers at once).  Two idle
+// cycles between scheduling barriers close the window.
+__device__ __forceinline__ void store_data_guard() {
+  __builtin_amdgcn_sched_barrier(0);
+  asm volatile("s_nop 1" ::: "memory");
+  __builtin_amdgcn_sched_barrier(0);
+}
+
 inline hipStream_t as_stream(vmoe_stream_t s) { return reinterpret_cast<hipStream_t>(s); }
 
 inline int launch_status() {
