@@ -56,18 +56,18 @@ OTHER_STEPS, OTHER_WARMUP = 10, 5
 # HBM bytes per launch of the dominant kernel (FETCH_SIZE + WRITE_SIZE, scaled by a copy
 # kernel of known size).
 MEASURED_TRAFFIC_BYTES = {
-    # mean of the two GEMM launches of a layer: (630 + 565 + 1096 + 182) / 2 MiB;
+    # mean of the two GEMM launches of a layer: (634 + 565 + 1026 + 141) / 2 MiB;
     # FETCH_SIZE x 2.0, WRITE_SIZE x 1.0 (copy-kernel calibration);
     # profiles/hbm_traffic__vmoe_b16_layer.md.
-    "vmoe_b16_layer_E32_k2_bpr": 1.297e9,
+    "vmoe_b16_layer_E32_k2_bpr": 1.241e9,
 }
 # Share of the launch during which the matrix cores are busy (SQ_VALU_MFMA_BUSY_CYCLES over
 # GRBM_GUI_ACTIVE x 1 024 SIMDs), from the rocprofv3 --pmc runs of this command summarised in
 # profiles/mfma_util__vmoe_b16_layer.md: counters cannot be read from inside the run.
 MEASURED_MFMA_BUSY = {
     "vmoe_b16_layer_E32_k2_bpr": {
-        "first_product": 0.451, "second_product": 0.599, "vendor_gemm_second_product_shape": 0.536,
-        "register_resident_mfma_loop": 0.937,
+        "first_product": 0.456, "second_product": 0.670, "vendor_gemm_second_product_shape": 0.538,
+        "register_resident_mfma_loop": 0.904,
         "source": "profiles/mfma_util__vmoe_b16_layer.md (rocprofv3 --pmc, same command, 5 steps)"},
 }
 
@@ -99,6 +99,19 @@ def device_weights(cfg, torch, dev, seed):
   w0 = (torch.randn((E, D, M), generator=gen, device=dev) / D ** 0.5).to(tdt)
   w1 = (torch.randn((E, M, D), generator=gen, device=dev) / M ** 0.5).to(tdt)
   return w0, w1, torch.zeros((E, M), dtype=tdt, device=dev), torch.zeros((E, D), dtype=tdt, device=dev)
+
+
+_marker_buffers = None
+
+
+def trace_marker(kernels, torch, dev):
+  """A 48-byte launch of the copy kernel, issued right before and right after the timed steps
+  (outside the region the step events bracket): in a kernel trace of the run the dispatches
+  between the two markers are the timed passes."""
+  global _marker_buffers
+  if _marker_buffers is None:
+    _marker_buffers = (torch.zeros(48, dtype=torch.uint8, device=dev), torch.zeros(48, dtype=torch.uint8, device=dev))
+  kernels.copy_bytes(*_marker_buffers)
 
 
 def host_cpu_model():
@@ -227,6 +240,7 @@ def soft_run(args, short=False):
     step(i)
   torch.cuda.synchronize()
   _hip.set_timing_sink(sink)
+  trace_marker(kernels, torch, dev)
   t0 = time.perf_counter()
   marks[0].record()
   host_t[0] = t0
@@ -235,6 +249,7 @@ def soft_run(args, short=False):
     marks[i + 1].record()
     host_t[i + 1] = time.perf_counter()
   t_enqueued = time.perf_counter()
+  trace_marker(kernels, torch, dev)
   torch.cuda.synchronize()
   t1 = time.perf_counter()
   gc.enable()
@@ -360,11 +375,14 @@ def vit_run(args, short=False):
   # steps (events between kernels serialise their hand-over and would slow the pass).
   sink = _hip.TimingSink(pairs=args.steps * 14, only=MLP_CALLS)
   _hip.set_timing_sink(sink)
+  trace_marker(kernels, torch, dev)
+  torch.cuda.synchronize()
   t0 = time.perf_counter()
   for i in range(args.steps):
     logits, metrics = step(i)
   torch.cuda.synchronize()
   t1 = time.perf_counter()
+  trace_marker(kernels, torch, dev)
   ms = (t1 - t0) * 1e3 / args.steps
   full = _hip.TimingSink(pairs=args.steps * 120)     # about 110 entry-point calls per pass
   spans["pool"] = _hip.TimingSink(pairs=args.steps * 24)
@@ -439,7 +457,7 @@ def vit_run(args, short=False):
                  "tokens": T, "blocks": enc["num_layers"], "moe_blocks": list(moe_cfg["layers"]),
                  "experts": moe_cfg["num_experts"], "selected": 2, "group_size": moe_cfg["group_size"],
                  "capacity_factor": 1.05},
-      "roofline": {"bound": "mfma", "kernel": "gemm_bf16_mixed_kernel (first product) / gemm_bf16_persistent_kernel (second product)", "achieved": achieved,
+      "roofline": {"bound": "mfma", "kernel": "gemm_bf16_mixed_kernel (first product) / gemm_bf16_w8_kernel (second product)", "achieved": achieved,
                    "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": achieved / PEAK_BF16_TFLOPS,
                    "traffic": None, "launch_ms": mlp_ms / (2 * enc["num_layers"]),
                    "flops_all_mlps": flops_mlp, "kept_rows_per_moe_block": kept_per_block,
@@ -555,12 +573,14 @@ def sparse_run(args, name, short=False):
     out, metrics = step(i)
   torch.cuda.synchronize()
   _hip.set_timing_sink(sink)
+  trace_marker(kernels, torch, dev)
   t0 = time.perf_counter()
   marks[0].record()
   for i in range(args.steps):
     out, metrics = step(i)
     marks[i + 1].record()
   t_enqueued = time.perf_counter()      # the host has issued everything; the GPU is still running
+  trace_marker(kernels, torch, dev)
   torch.cuda.synchronize()
   t1 = time.perf_counter()
   gc.enable()
@@ -599,7 +619,7 @@ def sparse_run(args, name, short=False):
   achieved_tflops = flops_per_launch / (gemm_ms * 1e-3) / 1e12
   peak = PEAK_BF16_TFLOPS if tdt == torch.bfloat16 else PEAK_FP32_MATRIX_TFLOPS
   roofline = {"bound": "mfma",
-              "kernel": "gemm_bf16_mixed_kernel (first product) / gemm_bf16_persistent_kernel (second product)" if b == 2 else "gemm_f32_kernel",
+              "kernel": "gemm_bf16_mixed_kernel (first product) / gemm_bf16_w8_kernel (second product)" if b == 2 else "gemm_f32_kernel",
               "achieved": achieved_tflops, "peak": peak, "unit": "TFLOP/s",
               "frac": achieved_tflops / peak, "traffic": MEASURED_TRAFFIC_BYTES.get(cfg.name),
               "from_profile": {"traffic_bytes_per_launch": MEASURED_TRAFFIC_BYTES.get(cfg.name),

@@ -42,7 +42,7 @@ __global__ __launch_bounds__(W8Cfg::kThreads, 1) void gemm_bf16_w8_kernel(
     const bf16_t* __restrict__ A, const bf16_t* __restrict__ Bt, const bf16_t* __restrict__ bias,
     bf16_t* __restrict__ C, int R, int N, int Kd, int tiles_m, int tiles_n, int num_tiles,
     int tiles_per_xcd, int panel_rows, PlanRef plan_ref, int32_t* __restrict__ clear,
-    int clear_count, int32_t* __restrict__ status) {
+    int clear_count, int32_t* __restrict__ status, int active_xcds, int active_slots) {
 #if defined(__HIP_DEVICE_COMPILE__)   // buffer-resource builtins exist in the device pass only
   extern __shared__ __align__(1024) unsigned char smem[];
   using Cfg = W8Cfg;
@@ -62,6 +62,7 @@ __global__ __launch_bounds__(W8Cfg::kThreads, 1) void gemm_bf16_w8_kernel(
   const int wm = wave >> 1, wn = wave & 1;
   const int m = lane & 31, h = lane >> 5;
   const int xcd = blockIdx.x % kNumXcd, slot = blockIdx.x / kNumXcd;
+  if (xcd >= active_xcds || slot >= active_slots) return;   // (measurement only, see active_units)
   // A request fills 8 rows x 128 bytes; lane L lands in LDS position L of the request and
   // fetches the 16-byte piece that the XOR swizzle of its row puts there.
   const int lrow = lane >> 3;
@@ -344,7 +345,7 @@ int launch_gemm_bf16_w8(const bf16_t* A, const bf16_t* Bt, const bf16_t* bias, b
   hipLaunchKernelGGL(kern, dim3(kCusPerXcd * kNumXcd), dim3(W8Cfg::kThreads), W8Cfg::kLdsBytes,
                      stream, A, Bt, bias, C, R, N, Kd, g.tiles_m, g.tiles_n, (int)g.tiles,
                      g.tiles_per_xcd, g.panel_rows, plan_ref<W8Cfg>(g, plan, batch, R), clear,
-                     clear_count, status);
+                     clear_count, status, active_units().xcds, active_units().slots);
   return launch_status();
 }
 
