@@ -891,17 +891,19 @@ def test_expert_mlp_second_product_walks_several_tiles(K, with_bias):
     assert (to_np(out[e, n:]) == 7.0).all(), f"expert {e}"
 
 
+@pytest.mark.parametrize("which", ["eight", "narrow"])
 @pytest.mark.parametrize("E,R,D,M", [
-    (64, 1100, 768, 256),     # 960 tiles: the kernel's own choice; four k tiles (the shortest k it takes)
-    (40, 1300, 1024, 512),    # 960 tiles, four column tiles
+    (64, 1100, 768, 256),     # 960 / 1280 tiles: the kernels' own range; four k tiles (the shortest k they take)
+    (40, 1300, 1024, 512),    # four column tiles of 256, five and a third of 192
     (3, 500, 520, 1024),      # forced: a column tile that ends inside the tile, few tiles per die
     (5, 257, 264, 320),       # forced: one row past a tile, k of five tiles
 ])
-def test_expert_mlp_second_product_on_eight_waves(K, monkeypatch, E, R, D, M):
-  """The eight-wave form of the second product (two waves per SIMD, output leaving through lane
-  exchanges instead of LDS) against the four-wave tile-walking kernel with whole tiles: both
-  add the same products in the same order, so the outputs must agree bit for bit; dense and
-  over packed rows with a launch plan (rows past a count are not written)."""
+def test_expert_mlp_second_product_on_eight_waves(K, monkeypatch, E, R, D, M, which):
+  """The eight-wave forms of the second product (two waves per SIMD, output leaving through lane
+  exchanges instead of LDS; "eight": 256 x 256 tiles and 32 x 32 x 16 MFMAs, "narrow": 256 x 192
+  tiles and 16 x 16 x 32 MFMAs) against the four-wave tile-walking kernel with whole tiles:
+  all add the same products in the same order of k, so the outputs must agree bit for bit;
+  dense and over packed rows with a launch plan (rows past a count are not written)."""
   rng = np.random.default_rng(E * 100 + M)
   args = [to_dev(O.cast(a, O.BF16), O.BF16) for a in (
       rng.standard_normal((E, R, D)).astype(np.float32),
@@ -912,21 +914,21 @@ def test_expert_mlp_second_product_on_eight_waves(K, monkeypatch, E, R, D, M):
   rows = rng.integers(0, R + 1, E).astype(np.int32)
   rows[:3] = [R, 0, 257][:min(3, E)]
   outs = {}
-  for which in ("eight", "shared"):
-    monkeypatch.setenv("VMOE_SECOND_PRODUCT", which)
+  for kernel in (which, "shared"):
+    monkeypatch.setenv("VMOE_SECOND_PRODUCT", kernel)
     monkeypatch.setenv("VMOE_WHOLE_TILES", "1")
     dense = K.expert_mlp(*args)
     ragged = torch.full_like(dense, 7.0)
     K.expert_mlp(*args, out=ragged, rows_per_expert=to_dev(rows))
-    outs[which] = (to_np(dense), to_np(ragged))
+    outs[kernel] = (to_np(dense), to_np(ragged))
     assert K.expert_mlp_status() == (0, 0)
   monkeypatch.delenv("VMOE_SECOND_PRODUCT")
   monkeypatch.delenv("VMOE_WHOLE_TILES")
-  np.testing.assert_array_equal(outs["eight"][0], outs["shared"][0])
+  np.testing.assert_array_equal(outs[which][0], outs["shared"][0])
   for e, n in enumerate(rows):
-    np.testing.assert_array_equal(outs["eight"][1][e, :n], outs["shared"][1][e, :n], err_msg=f"expert {e}")
-    np.testing.assert_array_equal(outs["eight"][1][e, :n], outs["eight"][0][e, :n], err_msg=f"expert {e}")
-    assert (outs["eight"][1][e, n:] == 7.0).all(), f"expert {e}"
+    np.testing.assert_array_equal(outs[which][1][e, :n], outs["shared"][1][e, :n], err_msg=f"expert {e}")
+    np.testing.assert_array_equal(outs[which][1][e, :n], outs[which][0][e, :n], err_msg=f"expert {e}")
+    assert (outs[which][1][e, n:] == 7.0).all(), f"expert {e}"
   # and against a float32 restatement of one expert
   e = E - 1
   x, w0, b0, w1, b1 = (a[e].float() for a in args)
@@ -934,7 +936,7 @@ def test_expert_mlp_second_product_on_eight_waves(K, monkeypatch, E, R, D, M):
   h = ((x @ w0).to(bf).float() + b0).to(bf)
   h = torch.nn.functional.gelu(h.float(), approximate="tanh").to(bf)
   want = ((h.float() @ w1).to(bf).float() + b1).to(bf)
-  np.testing.assert_allclose(outs["eight"][0][e], to_np(want), rtol=2e-2, atol=2e-2)
+  np.testing.assert_allclose(outs[which][0][e], to_np(want), rtol=2e-2, atol=2e-2)
 
 
 SHARED_ROUND_CASES = [

@@ -8,6 +8,7 @@
 
 #include "gemm_bf16_wide.h"
 #include "gemm_bf16_w8.h"
+#include "gemm_bf16_w8x.h"
 #include "compact_rows.h"
 
 namespace vmoe {
@@ -265,11 +266,15 @@ static_assert(kStatusWords * sizeof(int32_t) <= kStatusBytes, "status block");
 //  kDownEightWaves: the same tiles walked by eight waves per workgroup (gemm_bf16_w8.h), the
 //    tiles of a partial round whole: ahead by about 3 % where a die's run is three rounds or
 //    longer, so that a partial round is a small part of it.
+//  kDownNarrow: 256 x 192 tiles walked by eight waves per workgroup with 16 x 16 x 32 MFMAs
+//    (gemm_bf16_w8x.h): where that tiling fills the chip's rounds better (768 output columns:
+//    four column tiles instead of three, 6 rounds of 0.75 instead of 5 of 1).
 //  kDownWide: 384 x 256 tiles, eight waves; whole rounds of one tile per CU.
 //  kDownHalf: 128 x 256 tiles, two per CU (static launches the tile-walking kernels do not
 //    cover, where whole rounds of 256 x 256 tiles would waste a tenth or more).
 //  kDownPlain: 256 x 256 tiles, one workgroup per tile.
-enum DownKernel { kDownShared, kDownEightWaves, kDownWide, kDownHalf, kDownPlain };
+enum DownKernel { kDownShared, kDownEightWaves, kDownNarrow, kDownWide, kDownHalf, kDownPlain };
+using CfgDownNarrow = W8xCfg<6>;
 
 bool down_prefers_half_tiles(int E, int R, int N) {
   constexpr int64_t kNumCu = 256;
@@ -330,16 +335,30 @@ MlpPlans mlp_plans(int E, int R, int D, int M, bool ragged) {
   else if (wide_ok) m.down_kernel = kDownWide;
   else if (!ragged && down_prefers_half_tiles(E, R, D)) m.down_kernel = kDownHalf;
   else m.down_kernel = kDownPlain;
-  // (VMOE_SECOND_PRODUCT=shared|wide in the environment overrides the choice between those
-  // two where both apply: the switch behind the figures that the model above was fitted to)
+  // 192-column tiles: 0.75 of a 256 x 256 tile each at about 1.03 of the time per flop, in
+  // whole rounds, where the run is again at least three rounds long.
+  const GemmGeom narrow = gemm_geometry<CfgDownNarrow>(E, R, D, M);
+  const bool narrow_ok = w8x_gemm_ok<6>(E, R, D, M, rows, bytes(narrow) ? planned : nullptr) &&
+                         narrow.tiles >= 3LL * (long long)kNumCu;
+  if (narrow_ok && (m.down_kernel == kDownEightWaves || m.down_kernel == kDownShared)) {
+    const double t_narrow = 0.75 * 1.03 * std::ceil((double)narrow.tiles / kNumCu);
+    const double t_now = m.down_kernel == kDownEightWaves ? std::ceil((double)square.tiles / kNumCu) : t_shared;
+    if (t_narrow < 0.97 * t_now) m.down_kernel = kDownNarrow;
+  }
+  // (VMOE_SECOND_PRODUCT=shared|eight|narrow|wide in the environment overrides the choice
+  // where the named kernel applies: the switch behind the figures that the model above was
+  // fitted to)
   if (const char* force = getenv("VMOE_SECOND_PRODUCT")) {
     if (strcmp(force, "shared") == 0 && shared_ok) m.down_kernel = kDownShared;
     if (strcmp(force, "eight") == 0 && w8_gemm_ok(E, R, D, M, rows, bytes(square) ? planned : nullptr))
       m.down_kernel = kDownEightWaves;
+    if (strcmp(force, "narrow") == 0 && w8x_gemm_ok<6>(E, R, D, M, rows, bytes(narrow) ? planned : nullptr))
+      m.down_kernel = kDownNarrow;
     if (strcmp(force, "wide") == 0 && wide_ok) m.down_kernel = kDownWide;
   }
-  m.down = m.down_kernel == kDownWide ? wide : square;
+  m.down = m.down_kernel == kDownWide ? wide : m.down_kernel == kDownNarrow ? narrow : square;
   m.down_bm = m.down_kernel == kDownWide ? WideCfg::BM : CfgDown::BM;
+  static_assert(CfgDownNarrow::BM == CfgDown::BM, "row tiles of the narrow kernel");
   m.down_bytes = bytes(m.down);
   if (m.down_kernel == kDownShared)
     m.streamk_bytes = align256(StreamKWorkspace<CfgDownPersistent>::kBytes);
@@ -499,6 +518,10 @@ static int run_expert_mlp(const VmoeExpertMlpParams* p, vmoe_stream_t stream_, b
         return launch_gemm_bf16_w8<kEpiBias>((const bf16_t*)hidden, (const bf16_t*)w1t,
                                              (const bf16_t*)p->b1, (bf16_t*)p->out, p->E, p->R, p->D,
                                              p->M, stream, plan_down, nullptr, 0, status);
+      case kDownNarrow:
+        return launch_gemm_bf16_w8x<kEpiBias, 6>((const bf16_t*)hidden, (const bf16_t*)w1t,
+                                                 (const bf16_t*)p->b1, (bf16_t*)p->out, p->E, p->R,
+                                                 p->D, p->M, stream, plan_down, nullptr, 0, status);
       case kDownWide:
         return launch_gemm_bf16_wide<kEpiBias>((const bf16_t*)hidden, (const bf16_t*)w1t,
                                                (const bf16_t*)p->b1, (bf16_t*)p->out, p->E, p->R,
