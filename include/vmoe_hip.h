@@ -219,7 +219,10 @@ int vmoe_compact_rows(const VmoeCompactRowsParams* p, vmoe_stream_t stream);
  * device (256 KiB, held until the process ends).  G * E beyond that returns
  * VMOE_E_WORKSPACE.  The call allocates and frees nothing.  All calls on one device share
  * the array: calls that overlap on one device (two streams, two host threads) race; calls
- * on one stream, or otherwise ordered, do not.  Results equal vmoe_compact_rows'. */
+ * on one stream, or otherwise ordered, do not.  Results equal vmoe_compact_rows'.
+ * The first call on a device looks up the array's device address (hipGetSymbolAddress, once
+ * per device, under a mutex): make one call on each device before the first capture; after
+ * that a call only launches kernels (no memset node) and may be captured into a HIP graph. */
 #define VMOE_COMPACT_ROWS_STATIC_MAX_GE 65536
 int vmoe_compact_rows_static(const VmoeCompactRowsParams* p, vmoe_stream_t stream);
 
@@ -508,6 +511,12 @@ typedef struct {
   int32_t dtype;
 } VmoeAttentionParams;
 int vmoe_attention(const VmoeAttentionParams* p, vmoe_stream_t stream);
+
+/* ---------------------------------------------------------------------------------------
+ * Measurement aids.  Nothing below has a counterpart in the reference and no product path
+ * calls it: these entry points produce the ceilings (copy rate, register-resident MFMA rate,
+ * operand delivery rate) that the bandwidth and arithmetic figures are compared with.
+ * --------------------------------------------------------------------------------------- */
 
 /* Plain device copy kernel of n bytes (n % 16 == 0); the measured HBM ceiling
  * that bandwidth figures are compared with. */

@@ -59,6 +59,51 @@ def test_compact_rows_static_matches_compact_rows():
     assert int(to_np(w[1]).sum()) == int((to_np(w[0]) >= 0).sum()) > 0
 
 
+def test_compact_rows_static_allocates_nothing_and_can_be_captured():
+  """After the one call per device that looks up the array's address, a call changes neither
+  the device's free memory nor torch's allocator statistics (outputs are allocated before the
+  measurement), and a call captured into a HIP graph (kernels only) gives the eager result on
+  every replay, with eager work and synchronisations between the replays."""
+  from vmoe_amd import _hip as H
+  G, S, E, K, C = CASES[0]
+  fill, token_slot = _routed(11, G, S, E, K, C)
+  want = _compact("vmoe_compact_rows", fill, token_slot, C, True)
+  _compact("vmoe_compact_rows_static", fill, token_slot, C, False)      # the address look-up, outside any capture
+  token_row = torch.full((G, S, K), -7, dtype=torch.int32, device=dev())
+  rows = torch.full((E,), -7, dtype=torch.int32, device=dev())
+  row_token = torch.full((E, G * C), -1, dtype=torch.int32, device=dev())
+  p = H.CompactRowsParams(H.ptr(fill), H.ptr(token_slot), H.ptr(token_row), H.ptr(rows),
+                          None, H.ptr(row_token), G, S, E, K, C)
+  torch.cuda.synchronize()
+  free_before, _ = torch.cuda.mem_get_info()
+  reserved_before = torch.cuda.memory_reserved()
+  for _ in range(3):
+    assert H.lib().vmoe_compact_rows_static(ctypes.byref(p), H.stream()) == 0
+  torch.cuda.synchronize()
+  free_after, _ = torch.cuda.mem_get_info()
+  assert free_after == free_before and torch.cuda.memory_reserved() == reserved_before
+  for name, x, y in zip(("token_row", "rows_per_expert", "row_token"), want, (token_row, rows, row_token)):
+    np.testing.assert_array_equal(to_np(y), to_np(x), err_msg=name)
+  # captured: the graph holds the call's kernels and nothing else
+  graph = torch.cuda.CUDAGraph()
+  side = torch.cuda.Stream()
+  side.wait_stream(torch.cuda.current_stream())
+  with torch.cuda.stream(side):
+    with torch.cuda.graph(graph, stream=side):
+      assert H.lib().vmoe_compact_rows_static(ctypes.byref(p), H.stream()) == 0
+  torch.cuda.current_stream().wait_stream(side)
+  for replay in range(3):
+    token_row.fill_(-7)
+    rows.fill_(-7)
+    row_token.fill_(-1)
+    _compact("vmoe_compact_rows_static", *_routed(20 + replay, *CASES[1]), CASES[1][4], False)   # eager work on the shared array in between
+    torch.cuda.synchronize()
+    graph.replay()
+    torch.cuda.synchronize()
+    for name, x, y in zip(("token_row", "rows_per_expert", "row_token"), want, (token_row, rows, row_token)):
+      np.testing.assert_array_equal(to_np(y), to_np(x), err_msg=f"{name}, replay {replay}")
+
+
 def test_compact_rows_static_rejects_oversize_and_null():
   from vmoe_amd import _hip as H
   lib = H.lib()

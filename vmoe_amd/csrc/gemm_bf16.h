@@ -1362,6 +1362,8 @@ __global__ __launch_bounds__(Cfg::kThreads, 1) void gemm_bf16_persistent_kernel(
               const uint2 bp = bias_pk[j * 4 + q];
               const float bv[4] = {bf_lo(bp.x), bf_hi(bp.x), bf_lo(bp.y), bf_hi(bp.y)};
               float v[4];
+              // (inline asm: the compiler's hazard recogniser does not see these reads of MFMA
+              // results, which is why the mfma_result_fence() ahead of this epilogue is mandatory)
 #pragma unroll
               for (int e = 0; e < 4; ++e)
                 asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(v[e]) : "a"(acc[i][j][q * 4 + e]));
@@ -1403,7 +1405,9 @@ __global__ __launch_bounds__(Cfg::kThreads, 1) void gemm_bf16_persistent_kernel(
             const uint2 bp = bias_pk[j * 4 + q];
             const float bv[4] = {bf_lo(bp.x), bf_hi(bp.x), bf_lo(bp.y), bf_hi(bp.y)};
             // (read here and nowhere earlier: hoisted above the branches below, the reads
-            // of all 64 groups would need 256 registers at once)
+            // of all 64 groups would need 256 registers at once; being inline asm they are
+            // invisible to the compiler's hazard recogniser, so the mfma_result_fence() ahead
+            // of this epilogue is what keeps them behind the last MFMA's write)
             floatx4 v;
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
