@@ -457,7 +457,7 @@ def vit_run(args, short=False):
                  "tokens": T, "blocks": enc["num_layers"], "moe_blocks": list(moe_cfg["layers"]),
                  "experts": moe_cfg["num_experts"], "selected": 2, "group_size": moe_cfg["group_size"],
                  "capacity_factor": 1.05},
-      "roofline": {"bound": "mfma", "kernel": "gemm_bf16_mixed_kernel (first product) / gemm_bf16_w8_kernel (second product)", "achieved": achieved,
+      "roofline": {"bound": "mfma", "kernel": "gemm_bf16_mixed_kernel (first product) / gemm_bf16_w8_kernel<0, true, 8> (second product)", "achieved": achieved,
                    "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": achieved / PEAK_BF16_TFLOPS,
                    "traffic": None, "launch_ms": mlp_ms / (2 * enc["num_layers"]),
                    "flops_all_mlps": flops_mlp, "kept_rows_per_moe_block": kept_per_block,
@@ -619,7 +619,7 @@ def sparse_run(args, name, short=False):
   achieved_tflops = flops_per_launch / (gemm_ms * 1e-3) / 1e12
   peak = PEAK_BF16_TFLOPS if tdt == torch.bfloat16 else PEAK_FP32_MATRIX_TFLOPS
   roofline = {"bound": "mfma",
-              "kernel": "gemm_bf16_mixed_kernel (first product) / gemm_bf16_w8_kernel (second product)" if b == 2 else "gemm_f32_kernel",
+              "kernel": "gemm_bf16_mixed_kernel (first product) / gemm_bf16_w8_kernel<0, true, 8> (second product)" if b == 2 else "gemm_f32_kernel",
               "achieved": achieved_tflops, "peak": peak, "unit": "TFLOP/s",
               "frac": achieved_tflops / peak, "traffic": MEASURED_TRAFFIC_BYTES.get(cfg.name),
               "from_profile": {"traffic_bytes_per_launch": MEASURED_TRAFFIC_BYTES.get(cfg.name),

@@ -8,7 +8,6 @@
 
 #include "gemm_bf16_wide.h"
 #include "gemm_bf16_w8.h"
-#include "gemm_bf16_w8x.h"
 #include "compact_rows.h"
 
 namespace vmoe {
@@ -263,18 +262,19 @@ static_assert(kStatusWords * sizeof(int32_t) <= kStatusBytes, "status block");
 // Which kernel runs the second product (bfloat16).
 //  kDownShared: 256 x 256 tiles walked by one workgroup per CU, the last, partial round of a
 //    die shared along k (stream-K): its time follows the number of tiles, not of rounds.
-//  kDownEightWaves: the same tiles walked by eight waves per workgroup (gemm_bf16_w8.h), the
+//  kDownEightWaves: the same tiles walked by eight waves per workgroup with 16 x 16 x 32 MFMAs
+//    (gemm_bf16_w8.h), the
 //    tiles of a partial round whole: ahead by about 3 % where a die's run is three rounds or
 //    longer, so that a partial round is a small part of it.
-//  kDownNarrow: 256 x 192 tiles walked by eight waves per workgroup with 16 x 16 x 32 MFMAs
-//    (gemm_bf16_w8x.h): where that tiling fills the chip's rounds better (768 output columns:
+//  kDownNarrow: the same kernel on 256 x 192 tiles: where that tiling fills the chip's rounds
+//    better (768 output columns:
 //    four column tiles instead of three, 6 rounds of 0.75 instead of 5 of 1).
 //  kDownWide: 384 x 256 tiles, eight waves; whole rounds of one tile per CU.
 //  kDownHalf: 128 x 256 tiles, two per CU (static launches the tile-walking kernels do not
 //    cover, where whole rounds of 256 x 256 tiles would waste a tenth or more).
 //  kDownPlain: 256 x 256 tiles, one workgroup per tile.
 enum DownKernel { kDownShared, kDownEightWaves, kDownNarrow, kDownWide, kDownHalf, kDownPlain };
-using CfgDownNarrow = W8xCfg<6>;
+using CfgDownNarrow = W8Cfg<6>;
 
 bool down_prefers_half_tiles(int E, int R, int N) {
   constexpr int64_t kNumCu = 256;
@@ -326,9 +326,10 @@ MlpPlans mlp_plans(int E, int R, int D, int M, bool ragged) {
   const double t_wide = 1.5 * 1.04 * std::ceil((double)wide.tiles / kNumCu);
   const double t_shared = (double)square.tiles / kNumCu + 0.05;
   // Eight waves where they apply and a die's run of tiles is at least three rounds long (the
-  // B/16 layer: 144 - 150 tiles per die, 1.004 -> 0.990 ms per step in three alternating pairs
-  // of runs; the Soft MoE layer's 48 tiles per die gain more from the shared round).
-  const bool w8_ok = w8_gemm_ok(E, R, D, M, rows, bytes(square) ? planned : nullptr) &&
+  // B/16 layer: 144 - 150 tiles per die, 1.004 -> 0.990 ms per step with 32 x 32 x 16 MFMAs and
+  // on to 0.985 with 16 x 16 x 32 ones, each in three alternating pairs of runs; the Soft MoE
+  // layer's 48 tiles per die gain more from the shared round).
+  const bool w8_ok = w8_gemm_ok<8>(E, R, D, M, rows, bytes(square) ? planned : nullptr) &&
                      square.tiles >= 3LL * (long long)kNumCu;
   if (shared_ok && w8_ok) m.down_kernel = kDownEightWaves;
   else if (shared_ok && (!wide_ok || t_shared <= t_wide)) m.down_kernel = kDownShared;
@@ -338,7 +339,7 @@ MlpPlans mlp_plans(int E, int R, int D, int M, bool ragged) {
   // 192-column tiles: 0.75 of a 256 x 256 tile each at about 1.03 of the time per flop, in
   // whole rounds, where the run is again at least three rounds long.
   const GemmGeom narrow = gemm_geometry<CfgDownNarrow>(E, R, D, M);
-  const bool narrow_ok = w8x_gemm_ok<6>(E, R, D, M, rows, bytes(narrow) ? planned : nullptr) &&
+  const bool narrow_ok = w8_gemm_ok<6>(E, R, D, M, rows, bytes(narrow) ? planned : nullptr) &&
                          narrow.tiles >= 3LL * (long long)kNumCu;
   if (narrow_ok && (m.down_kernel == kDownEightWaves || m.down_kernel == kDownShared)) {
     const double t_narrow = 0.75 * 1.03 * std::ceil((double)narrow.tiles / kNumCu);
@@ -350,9 +351,9 @@ MlpPlans mlp_plans(int E, int R, int D, int M, bool ragged) {
   // fitted to)
   if (const char* force = getenv("VMOE_SECOND_PRODUCT")) {
     if (strcmp(force, "shared") == 0 && shared_ok) m.down_kernel = kDownShared;
-    if (strcmp(force, "eight") == 0 && w8_gemm_ok(E, R, D, M, rows, bytes(square) ? planned : nullptr))
+    if (strcmp(force, "eight") == 0 && w8_gemm_ok<8>(E, R, D, M, rows, bytes(square) ? planned : nullptr))
       m.down_kernel = kDownEightWaves;
-    if (strcmp(force, "narrow") == 0 && w8x_gemm_ok<6>(E, R, D, M, rows, bytes(narrow) ? planned : nullptr))
+    if (strcmp(force, "narrow") == 0 && w8_gemm_ok<6>(E, R, D, M, rows, bytes(narrow) ? planned : nullptr))
       m.down_kernel = kDownNarrow;
     if (strcmp(force, "wide") == 0 && wide_ok) m.down_kernel = kDownWide;
   }
@@ -515,11 +516,11 @@ static int run_expert_mlp(const VmoeExpertMlpParams* p, vmoe_stream_t stream_, b
             (const bf16_t*)hidden, (const bf16_t*)w1t, (const bf16_t*)p->b1, (bf16_t*)p->out, p->E,
             p->R, p->D, p->M, stream, plan_down, streamk, status);
       case kDownEightWaves:
-        return launch_gemm_bf16_w8<kEpiBias>((const bf16_t*)hidden, (const bf16_t*)w1t,
-                                             (const bf16_t*)p->b1, (bf16_t*)p->out, p->E, p->R, p->D,
-                                             p->M, stream, plan_down, nullptr, 0, status);
+        return launch_gemm_bf16_w8<kEpiBias, 8>((const bf16_t*)hidden, (const bf16_t*)w1t,
+                                                (const bf16_t*)p->b1, (bf16_t*)p->out, p->E, p->R,
+                                                p->D, p->M, stream, plan_down, nullptr, 0, status);
       case kDownNarrow:
-        return launch_gemm_bf16_w8x<kEpiBias, 6>((const bf16_t*)hidden, (const bf16_t*)w1t,
+        return launch_gemm_bf16_w8<kEpiBias, 6>((const bf16_t*)hidden, (const bf16_t*)w1t,
                                                  (const bf16_t*)p->b1, (bf16_t*)p->out, p->E, p->R,
                                                  p->D, p->M, stream, plan_down, nullptr, 0, status);
       case kDownWide:
