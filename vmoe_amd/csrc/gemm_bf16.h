@@ -41,11 +41,25 @@
 #include <cstdio>
 #include <cstdlib>
 #include <type_traits>
+#include <utility>
 #include "vmoe_common.h"
 
 namespace vmoe {
 
 enum { kEpiBias = 0, kEpiBiasGeluTanh = 1, kEpiBiasGeluErf = 2 };
+
+// f(integral_constant<int, 0>) ... f(integral_constant<int, N - 1>), in order: a loop whose
+// index is a constant in the body (register arrays, if constexpr).
+template <int I>
+using IntC = std::integral_constant<int, I>;
+template <typename F, int... Is>
+__device__ __forceinline__ void static_for_impl(F&& f, std::integer_sequence<int, Is...>) {
+  (f(IntC<Is>{}), ...);
+}
+template <int N, typename F>
+__device__ __forceinline__ void static_for(F&& f) {
+  static_for_impl(f, std::make_integer_sequence<int, N>{});
+}
 
 
 // 0.5 x (1 + tanh(c (x + 0.044715 x^3))) = x * sigmoid(2 c (x + 0.044715 x^3)),
@@ -142,35 +156,13 @@ __device__ __forceinline__ void load_bias(uint2 (&bias_pk)[TN / 8], const bf16_t
   }
 }
 
+// The staged wave tile (TM rows of TN + 8 bfloat16 at `so`) to memory as 16-byte
+// row-contiguous pieces.
 template <int EPI, int TM, int TN>
-__device__ __forceinline__ void store_tile(floatx16 (&acc)[TM / 32][TN / 32], unsigned char* smem,
-                                           int wave, int lane, const uint2 (&bias_pk)[TN / 8],
-                                           bool has_bias, bf16_t* __restrict__ C, int b, int R,
-                                           int live, int N, int wrow0, int wcol0) {
-  constexpr int FM = TM / 32, FN = TN / 32, OLD = TN + 8;
-  const int m = lane & 31, h = lane >> 5;
+__device__ __forceinline__ void store_staged_tile(const bf16_t* so, int lane, bf16_t* __restrict__ C,
+                                                  int b, int R, int live, int N, int wrow0, int wcol0) {
+  constexpr int OLD = TN + 8;
   bf16_t* Cb = C + (size_t)b * R * N;
-  bf16_t* so = reinterpret_cast<bf16_t*>(smem) + (size_t)wave * TM * OLD;
-  auto stage = [&](auto has_bias_c) {
-    constexpr bool kHasBias = decltype(has_bias_c)::value;
-#pragma unroll
-    for (int j = 0; j < FN; ++j) {
-#pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const int cl = j * 32 + q * 8 + h * 4;          // column inside the wave tile
-        const uint2 bp = bias_pk[j * 4 + q];
-        const float bv[4] = {bf_lo(bp.x), bf_hi(bp.x), bf_lo(bp.y), bf_hi(bp.y)};
-#pragma unroll
-        for (int i = 0; i < FM; ++i) {
-          const uint32_t p0 = epilogue_pair<EPI, kHasBias>(acc[i][j][q * 4], acc[i][j][q * 4 + 1], bv[0], bv[1]);
-          const uint32_t p1 = epilogue_pair<EPI, kHasBias>(acc[i][j][q * 4 + 2], acc[i][j][q * 4 + 3], bv[2], bv[3]);
-          *reinterpret_cast<uint2*>(so + (i * 32 + m) * OLD + cl) = make_uint2(p0, p1);
-        }
-      }
-    }
-  };
-  if (has_bias) stage(std::true_type{});
-  else stage(std::false_type{});
   // Each wave reads back only what it wrote (LDS operations of a wave complete in order).
   constexpr int kChunksOut = TN / 8;                  // 16-byte chunks per staged row
   constexpr int kRowsPerPass = 64 / kChunksOut;
@@ -234,6 +226,37 @@ __device__ __forceinline__ void store_tile(floatx16 (&acc)[TM / 32][TN / 32], un
       }
     }
   }
+}
+
+template <int EPI, int TM, int TN>
+__device__ __forceinline__ void store_tile(floatx16 (&acc)[TM / 32][TN / 32], unsigned char* smem,
+                                           int wave, int lane, const uint2 (&bias_pk)[TN / 8],
+                                           bool has_bias, bf16_t* __restrict__ C, int b, int R,
+                                           int live, int N, int wrow0, int wcol0) {
+  constexpr int FM = TM / 32, FN = TN / 32, OLD = TN + 8;
+  const int m = lane & 31, h = lane >> 5;
+  bf16_t* so = reinterpret_cast<bf16_t*>(smem) + (size_t)wave * TM * OLD;
+  auto stage = [&](auto has_bias_c) {
+    constexpr bool kHasBias = decltype(has_bias_c)::value;
+#pragma unroll
+    for (int j = 0; j < FN; ++j) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int cl = j * 32 + q * 8 + h * 4;          // column inside the wave tile
+        const uint2 bp = bias_pk[j * 4 + q];
+        const float bv[4] = {bf_lo(bp.x), bf_hi(bp.x), bf_lo(bp.y), bf_hi(bp.y)};
+#pragma unroll
+        for (int i = 0; i < FM; ++i) {
+          const uint32_t p0 = epilogue_pair<EPI, kHasBias>(acc[i][j][q * 4], acc[i][j][q * 4 + 1], bv[0], bv[1]);
+          const uint32_t p1 = epilogue_pair<EPI, kHasBias>(acc[i][j][q * 4 + 2], acc[i][j][q * 4 + 3], bv[2], bv[3]);
+          *reinterpret_cast<uint2*>(so + (i * 32 + m) * OLD + cl) = make_uint2(p0, p1);
+        }
+      }
+    }
+  };
+  if (has_bias) stage(std::true_type{});
+  else stage(std::false_type{});
+  store_staged_tile<EPI, TM, TN>(so, lane, C, b, R, live, N, wrow0, wcol0);
 }
 
 // XCD-aware workgroup -> (batch, tile_m, tile_n); returns false for padding workgroups.
@@ -680,15 +703,51 @@ __global__ __launch_bounds__(Cfg::kThreads, Cfg::kBlocksPerCu) void gemm_bf16_ke
 // does not hold two 64-wide stages of both operands, but it holds them for the B rows (the
 // weights: two thirds of the requests): B sits in two slots of 64-wide k tiles (128-byte
 // segments, 2 x 32 KB), A in two slots of 32-wide ones (64-byte segments, 2 x 8 KB).
-// Iterations are 32 wide; the pair 2 J, 2 J + 1 multiplies B slot J mod 2.
-//   iteration 2 J      slice 0: second half of the B rows of pair J + 1
+// Iterations are 32 wide, one v_mfma_f32_16x16x32_bf16 deep: eight units of four MFMAs (the
+// wave's four row blocks times one of its eight column blocks); a barrier stands in front of
+// the first unit that reads fragments of the next k tile (unit 5).  The pair 2 J, 2 J + 1
+// multiplies B slot J mod 2.
+//   iteration 2 J      units 0-4: second half of the B rows of pair J + 1
 //                      wait (that half may stay in flight), barrier
-//                      slice 1: A rows of k tile 2 J + 2
-//   iteration 2 J + 1  slice 0: nothing
+//                      units 5-7: A rows of k tile 2 J + 2
+//   iteration 2 J + 1  units 0-4: nothing
 //                      wait for everything, barrier (B slot J mod 2 is free from here on)
-//                      slice 1: A rows of k tile 2 J + 3, first half of the B rows of pair J + 2
+//                      units 5-7: A rows of k tile 2 J + 3, first half of the B rows of pair J + 2
 // A load-only model of the launch: 350 us with 64-byte segments for both operands, 271 - 287
-// with this mix.
+// with this mix.  The MFMA shape: the chip runs this product at its power limit, where the
+// 16x16x32 instruction sustains about 14 % more flops than the 32x32x16 one; the same kernel
+// written with 32x32x16 MFMAs (two slices of eight per iteration, barrier between them) took
+// 0.970 - 0.977 ms per step of the B/16 layer against 0.949 - 0.957 (three alternating pairs).
+// store_tile for sums in the layout of v_mfma_f32_16x16x32_bf16 with the B fragment first:
+// acc[i][j][v] = C[row i * 16 + lane % 16][column j * 16 + (lane / 16) * 4 + v].
+template <int EPI, int TM, int TN>
+__device__ __forceinline__ void store_tile16(floatx4 (&acc)[TM / 16][TN / 16], unsigned char* smem,
+                                             int wave, int lane, const uint2 (&bias_pk)[TN / 16],
+                                             bool has_bias, bf16_t* __restrict__ C, int b, int R,
+                                             int live, int N, int wrow0, int wcol0) {
+  constexpr int FM = TM / 16, FN = TN / 16, OLD = TN + 8;
+  const int n16 = lane & 15, g4 = lane >> 4;
+  bf16_t* so = reinterpret_cast<bf16_t*>(smem) + (size_t)wave * TM * OLD;
+  auto stage = [&](auto has_bias_c) {
+    constexpr bool kHasBias = decltype(has_bias_c)::value;
+#pragma unroll
+    for (int j = 0; j < FN; ++j) {
+      const int cl = j * 16 + g4 * 4;          // column inside the wave tile
+      const uint2 bp = bias_pk[j];
+      const float bv[4] = {bf_lo(bp.x), bf_hi(bp.x), bf_lo(bp.y), bf_hi(bp.y)};
+#pragma unroll
+      for (int i = 0; i < FM; ++i) {
+        const uint32_t p0 = epilogue_pair<EPI, kHasBias>(acc[i][j][0], acc[i][j][1], bv[0], bv[1]);
+        const uint32_t p1 = epilogue_pair<EPI, kHasBias>(acc[i][j][2], acc[i][j][3], bv[2], bv[3]);
+        *reinterpret_cast<uint2*>(so + (i * 16 + n16) * OLD + cl) = make_uint2(p0, p1);
+      }
+    }
+  };
+  if (has_bias) stage(std::true_type{});
+  else stage(std::false_type{});
+  store_staged_tile<EPI, TM, TN>(so, lane, C, b, R, live, N, wrow0, wcol0);
+}
+
 template <int EPI>
 __global__ __launch_bounds__(256, 2) void gemm_bf16_mixed_kernel(
     const bf16_t* __restrict__ A, const bf16_t* __restrict__ Bt, const bf16_t* __restrict__ bias,
@@ -698,7 +757,7 @@ __global__ __launch_bounds__(256, 2) void gemm_bf16_mixed_kernel(
     int32_t* __restrict__ clear, int clear_count, int32_t* __restrict__ status, int active_xcds) {
 #if defined(__HIP_DEVICE_COMPILE__)   // buffer-resource builtins exist in the device pass only
   extern __shared__ __align__(1024) unsigned char smem[];
-  constexpr int BM = 128, BN = 256, TM = 64, TN = 128, FM = 2, FN = 4, kWaves = 4;
+  constexpr int BM = 128, BN = 256, TM = 64, TN = 128, FM = 4, FN = 8, kWaves = 4;   // FM x FN MFMA tiles of 16 x 16 per wave
   constexpr int kASlot = BM * 64, kBSlot = BN * 128, kBBase = 2 * kASlot;
   const int tid = threadIdx.x;
   const int4* plan = plan_ref.entries;
@@ -707,7 +766,7 @@ __global__ __launch_bounds__(256, 2) void gemm_bf16_mixed_kernel(
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave >> 1, wn = wave & 1;
-  const int m = lane & 31, h = lane >> 5;
+  const int n16 = lane & 15, g4 = lane >> 4;
 
   int b, tile_m, tile_n;
   int live = R;
@@ -784,60 +843,90 @@ __global__ __launch_bounds__(256, 2) void gemm_bf16_mixed_kernel(
   using Half0 = std::integral_constant<int, 0>;
   using Half1 = std::integral_constant<int, 1>;
 
-  floatx16 acc[FM][FN];
+  floatx4 acc[FM][FN];
 #pragma unroll
   for (int i = 0; i < FM; ++i)
 #pragma unroll
     for (int j = 0; j < FN; ++j)
 #pragma unroll
-      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
-  bf16x8 fa[2][FM], fb[2][FN];
-  const int a_row_off = (wm * TM + m) * 64;
-  const int b_row_off = kBBase + (wn * TN + m) * 128;
-  const int swz_a = (m >> 2) & 3, swz_b = (m >> 1) & 7;
-  // Fragments of slice ks (0, 1) of k tile kt.
-  auto load_frags = [&](int buf, int kt, int ks) {
-    const unsigned char* pa = smem + (kt & 1) * kASlot + a_row_off + (((2 * ks + h) ^ swz_a) * 16);
-    const unsigned char* pb = smem + ((kt >> 1) & 1) * kBSlot + b_row_off +
-                              ((((kt & 1) * 4 + 2 * ks + h) ^ swz_b) * 16);
-#pragma unroll
-    for (int i = 0; i < FM; ++i)
-      fa[buf][i] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(pa + i * 32 * 64));
-#pragma unroll
-    for (int j = 0; j < FN; ++j)
-      fb[buf][j] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(pb + j * 32 * 128));
+      for (int v = 0; v < 4; ++v) acc[i][j][v] = 0.f;
+  // v_mfma_f32_16x16x32_bf16: a lane supplies 8 consecutive k of one row (row = lane % 16,
+  // k = 8 * (lane / 16) of the 32-wide iteration).  An iteration is FN units, one per column
+  // block: four MFMAs (the wave's four row blocks times that column block).  The wave holds
+  // the A fragments of the iteration, reads those of the next one during its last two units,
+  // and keeps the B fragments of the next kLook units in flight.
+  constexpr int kLook = 3, kRing = kLook + 1;
+  static_assert(FN % kRing == 0, "fragment ring");
+  constexpr int kBarrierUnit = FN - kLook;      // first unit that reads from the next k tile
+  bf16x8 fa[2][FM], fb[kRing];
+  const int a_row_off = (wm * TM + n16) * 64;
+  const int b_row_off = kBBase + (wn * TN + n16) * 128;
+  const int swz_a = (n16 >> 2) & 3, swz_b = (n16 >> 1) & 7;
+  auto read_a = [&](int buf, int kt, int i) {
+    fa[buf][i] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(
+        smem + (kt & 1) * kASlot + a_row_off + i * 16 * 64 + ((g4 ^ swz_a) * 16)));
   };
-  auto mfma_slice = [&](int buf) {
-#pragma unroll
-    for (int i = 0; i < FM; ++i)
-#pragma unroll
-      for (int j = 0; j < FN; ++j)
-        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[buf][j], fa[buf][i], acc[i][j], 0, 0, 0);
+  auto read_b = [&](int buf, int kt, int j) {
+    fb[buf] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(
+        smem + ((kt >> 1) & 1) * kBSlot + b_row_off + j * 16 * 128 + ((((kt & 1) * 4 + g4) ^ swz_b) * 16)));
   };
-  // Issue order inside a slice as in gemm_bf16_kernel: the fragment reads of the next slice
-  // behind the first MFMAs, the DMA requests spread over the rest.
-  constexpr int kReads = FM + FN, kMfmas = FM * FN;
-  auto slice_schedule = [&](auto vmem_c) {
-    constexpr int vmem = decltype(vmem_c)::value;
-    constexpr int kLead = kReads < kMfmas ? kReads : kMfmas;
-    constexpr int kRest = kMfmas - kLead;
+  uint2 bias_pk[FN];
 #pragma unroll
-    for (int g = 0; g < kLead; ++g) {
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-    }
-    if constexpr (vmem > 0) {
+  for (int j = 0; j < FN; ++j) {
+    bias_pk[j] = make_uint2(0, 0);
+    if (bias != nullptr) {
+      const int col = col0 + wn * TN + j * 16 + g4 * 4;
+      const bf16_t* src = bias + (size_t)b * N;
+      if ((N & 3) == 0) {
+        bias_pk[j] = *reinterpret_cast<const uint2*>(src + min(col, N - 4));
+      } else {
+        uint32_t v[4];
 #pragma unroll
-      for (int g = 0; g < kRest; ++g) {
-        if (g * vmem / kRest != (g + 1) * vmem / kRest)
-          __builtin_amdgcn_sched_group_barrier(0x020, (vmem + kRest - 1) / kRest, 0);
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        for (int t = 0; t < 4; ++t) v[t] = src[min(col + t, N - 1)];
+        bias_pk[j] = make_uint2(v[0] | (v[1] << 16), v[2] | (v[3] << 16));
       }
     }
+  }
+
+  // Units lo .. hi - 1 of iteration kt (fragment set par = kt & 1 as a constant); `next`: the
+  // k tile kt + 1 exists, so the units from kBarrierUnit on read its first fragments; `dma`
+  // requests go out under these units, spread evenly.
+  auto units = [&](auto lo_c, auto hi_c, auto par_c, int kt, auto next_c, auto dma_c) __attribute__((always_inline)) {
+    constexpr int lo = decltype(lo_c)::value, hi = decltype(hi_c)::value, par = decltype(par_c)::value;
+    constexpr bool next = decltype(next_c)::value;
+    constexpr int dma = decltype(dma_c)::value;
+    static_for<hi - lo>([&](auto c) __attribute__((always_inline)) {
+      constexpr int j = lo + decltype(c)::value;
+      constexpr int jl = j + kLook;
+      constexpr bool rb = jl < FN || next;
+      constexpr bool ra = next && j >= FN - 2;
+      if constexpr (jl < FN) read_b(jl % kRing, kt, jl);
+      else if constexpr (next) read_b(jl % kRing, kt + 1, jl - FN);
+      if constexpr (ra) {
+        read_a(par ^ 1, kt + 1, 2 * (j - (FN - 2)));
+        read_a(par ^ 1, kt + 1, 2 * (j - (FN - 2)) + 1);
+      }
+#pragma unroll
+      for (int i = 0; i < FM; ++i)
+        acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fb[j % kRing], fa[par][i], acc[i][j], 0, 0, 0);
+      constexpr int u = j - lo, n = hi - lo;
+      constexpr int dma_here = (u + 1) * dma / n - u * dma / n;
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      if constexpr (rb) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      if constexpr (ra) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      if constexpr (ra) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+      if constexpr (dma_here > 0) __builtin_amdgcn_sched_group_barrier(0x020, dma_here, 0);
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+    });
     __builtin_amdgcn_sched_barrier(0);
   };
-  uint2 bias_pk[TN / 8];
-  load_bias<TN>(bias_pk, bias, b, N, col0 + wn * TN, lane);
+  using U0 = std::integral_constant<int, 0>;
+  using UB = std::integral_constant<int, kBarrierUnit>;
+  using UN = std::integral_constant<int, FN>;
+  using P0 = std::integral_constant<int, 0>;
+  using P1 = std::integral_constant<int, 1>;
 
   const int nk = Kd / 32;          // even, at least 4: the launcher checks
   load_a(0, 0);
@@ -847,45 +936,46 @@ __global__ __launch_bounds__(256, 2) void gemm_bf16_mixed_kernel(
   load_b_half(1, 1, Half0{});
   wait_vmcnt<2 + kBFirst>();       // k tile 0 has landed: A rows of k tile 1 and the first part of a B slot may be in flight
   raw_barrier();
-  load_frags(0, 0, 0);
-  // B1: pair J + 1 exists; A2 / A3: k tiles 2 J + 2 / 2 J + 3 exist; B2: pair J + 2 exists.
-#define VMOE_MIXED_PAIR(J, B1, A2, A3, B2) do { \
-    const int kt_ = 2 * (J); \
-    load_frags(1, kt_, 1); \
-    if constexpr (B1) load_b_half(((J) + 1) & 1, (J) + 1, Half1{}); \
-    mfma_slice(0); \
-    slice_schedule(std::integral_constant<int, (B1) ? 8 - kBFirst : 0>{}); \
-    wait_vmcnt<(B1) ? 8 - kBFirst : 0>(); \
-    wait_lgkmcnt0(); \
-    raw_barrier(); \
-    load_frags(0, kt_ + 1, 0); \
-    if constexpr (A2) load_a(0, kt_ + 2); \
-    mfma_slice(1); \
-    slice_schedule(std::integral_constant<int, (A2) ? 2 : 0>{}); \
-    load_frags(1, kt_ + 1, 1); \
-    mfma_slice(0); \
-    slice_schedule(std::integral_constant<int, 0>{}); \
-    if constexpr (A2) { \
-      wait_vmcnt<0>(); \
-      wait_lgkmcnt0(); \
-      raw_barrier(); \
-      load_frags(0, kt_ + 2, 0); \
-    } \
-    if constexpr (A3) load_a(1, kt_ + 3); \
-    if constexpr (B2) load_b_half((J) & 1, (J) + 2, Half0{}); \
-    mfma_slice(1); \
-    slice_schedule(std::integral_constant<int, ((A3) ? 2 : 0) + ((B2) ? kBFirst : 0)>{}); \
-  } while (0)
+#pragma unroll
+  for (int i = 0; i < FM; ++i) read_a(0, 0, i);
+#pragma unroll
+  for (int u = 0; u < kLook; ++u) read_b(u, 0, u);
+  // Pair J = iterations 2 J and 2 J + 1 (B slot J mod 2).  B1: pair J + 1 exists; A2 / A3: k
+  // tiles 2 J + 2 / 2 J + 3 exist; B2: pair J + 2 exists.  Requests and barriers as described
+  // above the kernel; a barrier stands in front of the first unit that reads from the next k tile.
+  auto pair = [&](int J, auto b1_c, auto a2_c, auto a3_c, auto b2_c) __attribute__((always_inline)) {
+    constexpr bool B1 = decltype(b1_c)::value, A2 = decltype(a2_c)::value;
+    constexpr bool A3 = decltype(a3_c)::value, B2 = decltype(b2_c)::value;
+    const int kt = 2 * J;
+    if constexpr (B1) load_b_half((J + 1) & 1, J + 1, Half1{});
+    units(U0{}, UB{}, P0{}, kt, std::true_type{}, std::integral_constant<int, B1 ? 8 - kBFirst : 0>{});
+    wait_vmcnt<B1 ? 8 - kBFirst : 0>();
+    wait_lgkmcnt0();
+    raw_barrier();
+    if constexpr (A2) load_a(0, kt + 2);
+    units(UB{}, UN{}, P0{}, kt, std::true_type{}, std::integral_constant<int, A2 ? 2 : 0>{});
+    units(U0{}, UB{}, P1{}, kt + 1, std::bool_constant<A2>{}, U0{});
+    if constexpr (A2) {
+      wait_vmcnt<0>();
+      wait_lgkmcnt0();
+      raw_barrier();
+    }
+    if constexpr (A3) load_a(1, kt + 3);
+    if constexpr (B2) load_b_half(J & 1, J + 2, Half0{});
+    units(UB{}, UN{}, P1{}, kt + 1, std::bool_constant<A2>{},
+          std::integral_constant<int, (A3 ? 2 : 0) + (B2 ? kBFirst : 0)>{});
+  };
+  using T = std::true_type;
+  using F = std::false_type;
   const int npairs = nk / 2;
-  for (int J = 0; J < npairs - 2; ++J) VMOE_MIXED_PAIR(J, true, true, true, true);
-  VMOE_MIXED_PAIR(npairs - 2, true, true, true, false);
-  VMOE_MIXED_PAIR(npairs - 1, false, false, false, false);
-#undef VMOE_MIXED_PAIR
+  for (int J = 0; J < npairs - 2; ++J) pair(J, T{}, T{}, T{}, T{});
+  pair(npairs - 2, T{}, T{}, T{}, F{});
+  pair(npairs - 1, F{}, F{}, F{}, F{});
   wait_lgkmcnt0();
   __syncthreads();   // all waves are done with the operand tiles: LDS is reused below
   mfma_result_fence();
-  store_tile<EPI, TM, TN>(acc, smem, wave, lane, bias_pk, bias != nullptr, C, b, R, live, N,
-                          row0 + wm * TM, col0 + wn * TN);
+  store_tile16<EPI, TM, TN>(acc, smem, wave, lane, bias_pk, bias != nullptr, C, b, R, live, N,
+                            row0 + wm * TM, col0 + wn * TN);
 #endif
 }
 

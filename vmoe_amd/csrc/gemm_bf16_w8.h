@@ -75,17 +75,6 @@ struct W8Cfg {
   static_assert(kLdsBytes <= 160 * 1024, "LDS budget");
 };
 
-template <int I>
-using IntC = std::integral_constant<int, I>;
-template <typename F, int... Is>
-__device__ __forceinline__ void static_for_impl(F&& f, std::integer_sequence<int, Is...>) {
-  (f(IntC<Is>{}), ...);
-}
-template <int N, typename F>
-__device__ __forceinline__ void static_for(F&& f) {
-  static_for_impl(f, std::make_integer_sequence<int, N>{});
-}
-
 // A is (batch, R, Kd).  `clear` / `status`: begin_call.
 template <int EPI, bool HAS_BIAS, int FN_>
 __global__ __launch_bounds__(512, 1) void gemm_bf16_w8_kernel(
