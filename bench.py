@@ -720,8 +720,8 @@ def sparse_run(args, name, short=False):
     w_e = (torch.randn((E, D, M), device=dev) * M ** -0.5).to(tdt)
     delivery = {}
     for name, k_tile, seg, fpb, what in (
-        ("first_product", 32, 64, 2.0 * 128 * 256 / ((128 + 256) * 2), "128 x 256 tiles"),
-        ("second_product", 64, 128, 2.0 * 256 * 256 / ((256 + 256) * 2), "256 x 256 tiles")):
+        ("segments_64B", 32, 64, 2.0 * 128 * 256 / ((128 + 256) * 2), "32-wide k tiles; flop per byte of 128 x 256 tiles"),
+        ("segments_128B", 64, 128, 2.0 * 256 * 256 / ((256 + 256) * 2), "64-wide k tiles; flop per byte of 256 x 256 tiles")):
       for _ in range(3):
         kernels.operand_delivery_probe(a_e, w_e, k_tile=k_tile)
       e0.record()
@@ -733,7 +733,9 @@ def sparse_run(args, name, short=False):
       delivery[name] = {"row_segment_bytes": seg, "TBps": tbps, "tiling": what, "flop_per_byte": fpb,
                         "ceiling_TFLOPs": tbps * fpb}
     delivery["note"] = ("load-only kernel on 256 x 256 tiles of the second product's operands; the rate depends "
-                        "on the shape of the requests, the ceiling on the product's own flop per operand byte")
+                        "on the shape of the requests, the ceiling on the flop per operand byte of the tiling named; "
+                        "the second product requests 128-byte segments, the first product 128-byte segments for its "
+                        "weights (two thirds of its requests) and 64-byte ones for its rows")
     roofline["operand_delivery"] = delivery
     del a_up, a_dn, w_up, w_dn, a_e, w_e
   # The same K steps replayed from HIP graphs (one per rotating input buffer), as a
