@@ -263,12 +263,10 @@ static_assert(kStatusWords * sizeof(int32_t) <= kStatusBytes, "status block");
 //  kDownShared: 256 x 256 tiles walked by one workgroup per CU, the last, partial round of a
 //    die shared along k (stream-K): its time follows the number of tiles, not of rounds.
 //  kDownEightWaves: the same tiles walked by eight waves per workgroup with 16 x 16 x 32 MFMAs
-//    (gemm_bf16_w8.h), the
-//    tiles of a partial round whole: ahead by about 3 % where a die's run is three rounds or
-//    longer, so that a partial round is a small part of it.
+//    (gemm_bf16_w8.h), the tiles of a partial round whole: ahead where a die's run is long
+//    enough that a partial round is a small part of it.
 //  kDownNarrow: the same kernel on 256 x 192 tiles: where that tiling fills the chip's rounds
-//    better (768 output columns:
-//    four column tiles instead of three, 6 rounds of 0.75 instead of 5 of 1).
+//    better (768 output columns: four column tiles instead of three).
 //  kDownWide: 384 x 256 tiles, eight waves; whole rounds of one tile per CU.
 //  kDownHalf: 128 x 256 tiles, two per CU (static launches the tile-walking kernels do not
 //    cover, where whole rounds of 256 x 256 tiles would waste a tenth or more).
@@ -318,43 +316,35 @@ MlpPlans mlp_plans(int E, int R, int D, int M, bool ragged) {
       E, R, D, M, rows, bytes(square) ? planned : nullptr) && M / CfgDownPersistent::BK % kStreamKGranule == 0;
   const bool wide_ok = wide_gemm_ok(E, R, D, M, nullptr, nullptr, nullptr, 0) && (!ragged || bytes(wide));
   constexpr double kNumCu = kCusPerXcd * kNumXcd;
-  // Time in units of one 256 x 256 tile on one CU.  The wide kernel's tile is 1.5 of them
-  // at about 1.04 of the time per flop (0.92 before the 256 x 256 kernel kept its A rows
-  // in a ring of three slots), in whole rounds; the shared kernel pays for its tiles (the
-  // padding of the last row tile of a batch included) plus the exchange.  With these
-  // figures the wide kernel only runs where the shared one does not apply.
+  // Time in units of one 256 x 256 tile of the four-wave kernel on one CU, fitted to alternating
+  // bench runs of the layer configurations (B/16 layer, Soft MoE layer, L/16 layer at capacity
+  // 0.5, B/16 model): the shared kernel pays for its tiles (the padding of the last row tile
+  // of a batch included) plus the exchange; the eight-wave kernel runs whole rounds at 0.95
+  // per tile (two waves per SIMD, 16 x 16 x 32 MFMAs); its 192-column form whole rounds of
+  // tiles three quarters the size at 0.97 of the time per flop, taken only where it wins by
+  // 3 % (Soft MoE: 512 tiles = 2 rounds instead of 1.5 shared ones, 417 -> 397 us for the
+  // MLP; the B/16 model's 13 rounds against 10: 0.2 ms slower); the wide kernel's tile is 1.5
+  // of them at 1.04 of the time per flop, in whole rounds.
+  const GemmGeom narrow = gemm_geometry<CfgDownNarrow>(E, R, D, M);
+  const bool eight_ok = w8_gemm_ok<8>(E, R, D, M, rows, bytes(square) ? planned : nullptr);
+  const bool narrow_ok = w8_gemm_ok<6>(E, R, D, M, rows, bytes(narrow) ? planned : nullptr);
   const double t_wide = 1.5 * 1.04 * std::ceil((double)wide.tiles / kNumCu);
   const double t_shared = (double)square.tiles / kNumCu + 0.05;
-  // Eight waves where they apply and a die's run of tiles is at least three rounds long (the
-  // B/16 layer: 144 - 150 tiles per die, 1.004 -> 0.990 ms per step with 32 x 32 x 16 MFMAs and
-  // on to 0.985 with 16 x 16 x 32 ones, each in three alternating pairs of runs; the Soft MoE
-  // layer's 48 tiles per die gain more from the shared round).
-  const bool w8_ok = w8_gemm_ok<8>(E, R, D, M, rows, bytes(square) ? planned : nullptr) &&
-                     square.tiles >= 3LL * (long long)kNumCu;
-  if (shared_ok && w8_ok) m.down_kernel = kDownEightWaves;
-  else if (shared_ok && (!wide_ok || t_shared <= t_wide)) m.down_kernel = kDownShared;
-  else if (wide_ok) m.down_kernel = kDownWide;
-  else if (!ragged && down_prefers_half_tiles(E, R, D)) m.down_kernel = kDownHalf;
-  else m.down_kernel = kDownPlain;
-  // 192-column tiles: 0.75 of a 256 x 256 tile each at about 1.03 of the time per flop, in
-  // whole rounds, where the run is again at least three rounds long.
-  const GemmGeom narrow = gemm_geometry<CfgDownNarrow>(E, R, D, M);
-  const bool narrow_ok = w8_gemm_ok<6>(E, R, D, M, rows, bytes(narrow) ? planned : nullptr) &&
-                         narrow.tiles >= 3LL * (long long)kNumCu;
-  if (narrow_ok && (m.down_kernel == kDownEightWaves || m.down_kernel == kDownShared)) {
-    const double t_narrow = 0.75 * 1.03 * std::ceil((double)narrow.tiles / kNumCu);
-    const double t_now = m.down_kernel == kDownEightWaves ? std::ceil((double)square.tiles / kNumCu) : t_shared;
-    if (t_narrow < 0.97 * t_now) m.down_kernel = kDownNarrow;
-  }
+  const double t_eight = 0.95 * std::ceil((double)square.tiles / kNumCu);
+  const double t_narrow = 0.75 * 0.97 * std::ceil((double)narrow.tiles / kNumCu);
+  double t_best = 1e300;
+  m.down_kernel = !ragged && down_prefers_half_tiles(E, R, D) ? kDownHalf : kDownPlain;
+  if (wide_ok) { m.down_kernel = kDownWide; t_best = t_wide; }
+  if (shared_ok && t_shared <= t_best) { m.down_kernel = kDownShared; t_best = t_shared; }
+  if (eight_ok && t_eight <= t_best) { m.down_kernel = kDownEightWaves; t_best = t_eight; }
+  if (narrow_ok && t_narrow < 0.97 * t_best) { m.down_kernel = kDownNarrow; t_best = t_narrow; }
   // (VMOE_SECOND_PRODUCT=shared|eight|narrow|wide in the environment overrides the choice
   // where the named kernel applies: the switch behind the figures that the model above was
   // fitted to)
   if (const char* force = getenv("VMOE_SECOND_PRODUCT")) {
     if (strcmp(force, "shared") == 0 && shared_ok) m.down_kernel = kDownShared;
-    if (strcmp(force, "eight") == 0 && w8_gemm_ok<8>(E, R, D, M, rows, bytes(square) ? planned : nullptr))
-      m.down_kernel = kDownEightWaves;
-    if (strcmp(force, "narrow") == 0 && w8_gemm_ok<6>(E, R, D, M, rows, bytes(narrow) ? planned : nullptr))
-      m.down_kernel = kDownNarrow;
+    if (strcmp(force, "eight") == 0 && eight_ok) m.down_kernel = kDownEightWaves;
+    if (strcmp(force, "narrow") == 0 && narrow_ok) m.down_kernel = kDownNarrow;
     if (strcmp(force, "wide") == 0 && wide_ok) m.down_kernel = kDownWide;
   }
   m.down = m.down_kernel == kDownWide ? wide : m.down_kernel == kDownNarrow ? narrow : square;
