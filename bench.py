@@ -741,6 +741,7 @@ def sparse_run(args, name, short=False):
   # The same K steps replayed from HIP graphs (one per rotating input buffer), as a
   # serving loop would run the layer; reported beside the eager figure, never as `value`.
   graph_ms = None
+  graph_many_ms = None
   try:
     if short:
       raise StopIteration
@@ -767,6 +768,21 @@ def sparse_run(args, name, short=False):
     if not torch.equal(keep[(args.steps - 1) % n_rot][0], step(args.steps - 1)[0]):
       raise RuntimeError("graph replay and eager step disagree")
     del graphs, keep
+    # One graph that holds n_rot steps: what a replay costs at its boundaries shows as the
+    # difference between this figure and the one above.
+    many = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(many):
+      keep = [step(i) for i in range(n_rot)]
+    for _ in range(max(1, args.warmup // n_rot)):
+      many.replay()
+    torch.cuda.synchronize()
+    reps = max(1, args.steps // n_rot)
+    tg0 = time.perf_counter()
+    for _ in range(reps):
+      many.replay()
+    torch.cuda.synchronize()
+    graph_many_ms = (time.perf_counter() - tg0) * 1e3 / (reps * n_rot)
+    del many, keep
   except StopIteration:
     pass
   except Exception as e:   # pylint: disable=broad-except
@@ -798,6 +814,7 @@ def sparse_run(args, name, short=False):
                         f"{stage_ms_instrumented_mlp:.4f} ms)"),
       "hbm": hbm,
       "hip_graph_ms_per_step": graph_ms,
+      "hip_graph_ms_per_step_four_steps_per_graph": graph_many_ms,
       "host_enqueue_ms_per_step": host_ms_per_step,
       "wall_ms_per_step": wall_ms_per_step,
       "ms_per_step_note": ("ms_per_step and value: median of the K per-step times between events "
