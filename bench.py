@@ -56,18 +56,18 @@ OTHER_STEPS, OTHER_WARMUP = 10, 5
 # HBM bytes per launch of the dominant kernel (FETCH_SIZE + WRITE_SIZE, scaled by a copy
 # kernel of known size).
 MEASURED_TRAFFIC_BYTES = {
-    # mean of the two GEMM launches of a layer: (634 + 565 + 1026 + 141) / 2 MiB;
+    # mean of the two GEMM launches of a layer: (630 + 565 + 1034 + 148) / 2 MiB;
     # FETCH_SIZE x 2.0, WRITE_SIZE x 1.0 (copy-kernel calibration);
     # profiles/hbm_traffic__vmoe_b16_layer.md.
-    "vmoe_b16_layer_E32_k2_bpr": 1.241e9,
+    "vmoe_b16_layer_E32_k2_bpr": 1.246e9,
 }
 # Share of the launch during which the matrix cores are busy (SQ_VALU_MFMA_BUSY_CYCLES over
 # GRBM_GUI_ACTIVE x 1 024 SIMDs), from the rocprofv3 --pmc runs of this command summarised in
 # profiles/mfma_util__vmoe_b16_layer.md: counters cannot be read from inside the run.
 MEASURED_MFMA_BUSY = {
     "vmoe_b16_layer_E32_k2_bpr": {
-        "first_product": 0.456, "second_product": 0.670, "vendor_gemm_second_product_shape": 0.538,
-        "register_resident_mfma_loop": 0.904,
+        "first_product": 0.444, "second_product": 0.611, "vendor_gemm_second_product_shape": 0.527,
+        "register_resident_mfma_loop": 0.897,
         "source": "profiles/mfma_util__vmoe_b16_layer.md (rocprofv3 --pmc, same command, 5 steps)"},
 }
 
