@@ -18,15 +18,17 @@ namespace {
 // v_mfma_f32_32x32x2_f32 (IEEE float32 multiply-add).  64x64 tile, 4 waves,
 // B is consumed in the reference's (in, out) order: a lane's B operand is one
 // scalar B[k][n], so no transposition is needed.
-constexpr int kF32Tile = 64, kF32BK = 16;
+constexpr int kF32Tile = 64, kF32BK = 32;
 
 template <int EPI>
 __global__ __launch_bounds__(256) void gemm_f32_kernel(
     const float* __restrict__ A, const float* __restrict__ B, const float* __restrict__ bias,
     float* __restrict__ C, int R, int N, int Kd, int tiles_m, int tiles_n,
     const int32_t* __restrict__ rows) {
-  __shared__ float sa[kF32Tile][kF32BK + 1];
-  __shared__ float sb[kF32BK][kF32Tile + 4];
+  // Two LDS stages of a 32-wide k tile: the global loads of k tile t + 1 are issued before the
+  // MFMAs of k tile t and written to the other stage behind them, one barrier per k tile.
+  __shared__ float sa[2][kF32Tile][kF32BK + 1];
+  __shared__ float sb[2][kF32BK][kF32Tile + 4];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave >> 1, wn = wave & 1;
   const int m = lane & 31, h = lane >> 5;
@@ -45,27 +47,46 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(
   floatx16 acc;
 #pragma unroll
   for (int v = 0; v < 16; ++v) acc[v] = 0.f;
-  const int ar = tid >> 2, akc = (tid & 3) * 4;   // A: 64 rows x 4 float4
-  const int bk = tid >> 4, bn = (tid & 15) * 4;   // B: 16 rows x 16 float4
-  for (int k0 = 0; k0 < Kd; k0 += kF32BK) {
-    float4 va = make_float4(0.f, 0.f, 0.f, 0.f), vb = va;
-    {
-      int gr = row0 + ar;
-      if (gr >= R) gr = R - 1;
-      if (k0 + akc + 4 <= Kd) va = *reinterpret_cast<const float4*>(Ab + (size_t)gr * Kd + k0 + akc);
-      int gk = k0 + bk, gn = col0 + bn;
-      if (gk < Kd && gn + 4 <= N) vb = *reinterpret_cast<const float4*>(Bb + (size_t)gk * N + gn);
+  // A: 64 rows x 8 float4 per k tile, B: 32 rows x 16 float4: two float4 of each per thread.
+  const int ar = tid >> 3, akc = (tid & 7) * 4;    // rows ar, ar + 32
+  const int bk = tid >> 4, bn = (tid & 15) * 4;    // k rows bk, bk + 16
+  float4 va[2], vb[2];
+  auto fetch = [&](int k0) {
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      va[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+      vb[u] = va[u];
+      const int gr = min(row0 + ar + u * 32, R - 1);
+      if (k0 + akc + 4 <= Kd) va[u] = *reinterpret_cast<const float4*>(Ab + (size_t)gr * Kd + k0 + akc);
+      const int gk = k0 + bk + u * 16, gn = col0 + bn;
+      if (gk < Kd && gn + 4 <= N) vb[u] = *reinterpret_cast<const float4*>(Bb + (size_t)gk * N + gn);
     }
-    __syncthreads();
-    sa[ar][akc + 0] = va.x; sa[ar][akc + 1] = va.y; sa[ar][akc + 2] = va.z; sa[ar][akc + 3] = va.w;
-    sb[bk][bn + 0] = vb.x; sb[bk][bn + 1] = vb.y; sb[bk][bn + 2] = vb.z; sb[bk][bn + 3] = vb.w;
-    __syncthreads();
+  };
+  auto stage = [&](int s_) {
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      float* pa = &sa[s_][ar + u * 32][akc];
+      pa[0] = va[u].x; pa[1] = va[u].y; pa[2] = va[u].z; pa[3] = va[u].w;
+      float* pb = &sb[s_][bk + u * 16][bn];
+      pb[0] = vb[u].x; pb[1] = vb[u].y; pb[2] = vb[u].z; pb[3] = vb[u].w;
+    }
+  };
+  fetch(0);
+  stage(0);
+  __syncthreads();
+  int cur = 0;
+  for (int k0 = 0; k0 < Kd; k0 += kF32BK) {
+    const bool more = k0 + kF32BK < Kd;
+    if (more) fetch(k0 + kF32BK);
 #pragma unroll
     for (int ks = 0; ks < kF32BK / 2; ++ks) {
-      float a = sa[wm * 32 + m][ks * 2 + h];
-      float bb = sb[ks * 2 + h][wn * 32 + m];
+      float a = sa[cur][wm * 32 + m][ks * 2 + h];
+      float bb = sb[cur][ks * 2 + h][wn * 32 + m];
       acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a, bb, acc, 0, 0, 0);
     }
+    if (more) stage(cur ^ 1);
+    __syncthreads();
+    cur ^= 1;
   }
   mfma_result_fence();
   const int col = col0 + wn * 32 + m;
