@@ -357,6 +357,8 @@ MLP_CASES = [
     # E, R, D, M, dtype
     (2, 40, 64, 128, O.F32),
     (8, 512, 512, 2048, O.F32),       # S/32-style layer, full size
+    (3, 100, 96, 200, O.F32),         # column tile that ends inside the matrix; second product's k not whole tiles
+    (3, 100, 96, 160, O.F32),         # both products through the LDS-DMA kernel, ragged rows and columns
     (3, 100, 72, 136, O.BF16),        # ragged everything
     (2, 300, 256, 512, O.BF16),
     (3, 300, 64, 192, O.BF16),        # shortest second product the tile-walking kernel takes (6 k tiles)

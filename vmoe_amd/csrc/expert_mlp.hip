@@ -8,6 +8,7 @@
 
 #include "gemm_bf16_wide.h"
 #include "gemm_bf16_w8.h"
+#include "gemm_f32.h"
 #include "compact_rows.h"
 
 namespace vmoe {
@@ -106,6 +107,15 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(
 template <int EPI>
 int launch_gemm_f32(const float* A, const float* B, const float* bias, float* C, int batch, int R,
                     int N, int Kd, hipStream_t stream, const int32_t* rows = nullptr) {
+  // The DMA kernel where its shapes allow: 64 x 128 tiles when they outnumber the CUs twice
+  // over, 64 x 64 otherwise.  VMOE_F32_GEMM=plain keeps the register-staged kernel below.
+  const char* which = getenv("VMOE_F32_GEMM");
+  if (gemm_f32_dma_ok(A, B, R, N, Kd) && !(which != nullptr && strcmp(which, "plain") == 0)) {
+    const long long wide_tiles = (long long)batch * ((R + 63) / 64) * ((N + 127) / 128);
+    if (wide_tiles >= 2 * kCusPerXcd * kNumXcd && !(which != nullptr && strcmp(which, "64") == 0))
+      return launch_gemm_f32_dma<EPI, 128>(A, B, bias, C, batch, R, N, Kd, stream, rows);
+    return launch_gemm_f32_dma<EPI, 64>(A, B, bias, C, batch, R, N, Kd, stream, rows);
+  }
   const int tiles_m = (R + kF32Tile - 1) / kF32Tile, tiles_n = (N + kF32Tile - 1) / kF32Tile;
   const long long blocks = (long long)batch * tiles_m * tiles_n;
   if (blocks > 0x7fffffffLL) return VMOE_E_OVERFLOW;
