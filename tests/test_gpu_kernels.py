@@ -617,6 +617,42 @@ def test_compact_rows(K, G, S, E, Kk, C, bpr):
     assert sorted(mine) == list(range(f.sum(0)[ee]))
 
 
+@pytest.mark.parametrize("E,R,D,M", [
+    (8, 416, 512, 2048),      # the S/32 layer: one expert per die
+    (5, 700, 512, 1024),      # runs that begin and end inside an expert
+    (3, 1000, 512, 1536),
+])
+def test_expert_mlp_float32_products_on_the_dma_kernel(K, monkeypatch, E, R, D, M):
+  """The float32 products on the LDS-DMA kernel (64 x 128 or 64 x 64 tiles, one run of the tile
+  list per die, rows past a count skipped in blocks of 32) against the register-staged kernel
+  and against the oracle; dense and over ragged rows."""
+  rng = np.random.default_rng(E + R)
+  x = rng.standard_normal((E, R, D)).astype(np.float32)
+  w0 = (rng.standard_normal((E, D, M)) / np.sqrt(D)).astype(np.float32)
+  b0 = (rng.standard_normal((E, M)) * 0.1).astype(np.float32)
+  w1 = (rng.standard_normal((E, M, D)) / np.sqrt(M)).astype(np.float32)
+  b1 = (rng.standard_normal((E, D)) * 0.1).astype(np.float32)
+  args = [to_dev(a) for a in (x, w0, b0, w1, b1)]
+  rows = rng.integers(0, R + 1, E).astype(np.int32)
+  rows[:3] = [R, 0, 33]
+  want = O.mlp_block(x, w0, b0, w1, b1, O.F32)
+  outs = {}
+  for form in ("dma", "64", "plain"):
+    if form != "dma":
+      monkeypatch.setenv("VMOE_F32_GEMM", form)
+    dense = to_np(K.expert_mlp(*args))
+    ragged = torch.full((E, R, D), 7.0, dtype=torch.float32, device=dev())
+    K.expert_mlp(*args, out=ragged, rows_per_expert=to_dev(rows))
+    outs[form] = (dense, to_np(ragged))
+    assert_close(dense, want, 1e-5, f"{form}: dense")
+    for e, n in enumerate(rows):
+      np.testing.assert_array_equal(outs[form][1][e, :n], dense[e, :n], err_msg=f"{form}: expert {e}")
+      assert (outs[form][1][e, n:] == 7.0).all(), f"{form}: expert {e} wrote past its rows"
+  monkeypatch.delenv("VMOE_F32_GEMM")
+  assert_close(outs["dma"][0], outs["plain"][0], 1e-5, "dma against plain")   # other order of k
+  np.testing.assert_array_equal(outs["dma"][0], outs["64"][0])              # same order of k
+
+
 @pytest.mark.parametrize("dtype", [O.F32, O.BF16])
 @pytest.mark.parametrize("E", [5, 20])      # fewer / more experts than dies in the launch plan
 def test_expert_mlp_rows_per_expert(K, dtype, E):

@@ -111,6 +111,10 @@ __global__ __launch_bounds__(256) void gemm_f32_dma_kernel(
   bool block_live[Cfg::FM];
 #pragma unroll
   for (int i = 0; i < Cfg::FM; ++i) block_live[i] = row0 + (wm * Cfg::FM + i) * 32 < live;
+  // the bias is fetched ahead of the loop: its latency would otherwise open the epilogue
+  const int col = col0 + wn * 32 + m;
+  const bool col_ok = col < N;
+  const float bv = (bias != nullptr && col_ok) ? bias[(size_t)b * N + col] : 0.f;
   floatx16 acc[Cfg::FM];
 #pragma unroll
   for (int i = 0; i < Cfg::FM; ++i)
@@ -192,9 +196,6 @@ __global__ __launch_bounds__(256) void gemm_f32_dma_kernel(
   }
   mfma_result_fence();
 
-  const int col = col0 + wn * 32 + m;
-  const bool col_ok = col < N;
-  const float bv = (bias != nullptr && col_ok) ? bias[(size_t)b * N + col] : 0.f;
   float* Cb = C + (size_t)b * R * N;
 #pragma unroll
   for (int i = 0; i < Cfg::FM; ++i) {
@@ -203,7 +204,7 @@ __global__ __launch_bounds__(256) void gemm_f32_dma_kernel(
     for (int v = 0; v < 16; ++v) {
       const int row = row0 + (wm * Cfg::FM + i) * 32 + (v >> 2) * 8 + h * 4 + (v & 3);
       float o = acc[i][v] + bv;
-      if (EPI == kEpiBiasGeluTanh) o = gelu_tanh(o);
+      if (EPI == kEpiBiasGeluTanh) o = gelu_tanh_fast(o);   // hardware exp2 and reciprocal: ~1e-7 relative
       if (EPI == kEpiBiasGeluErf) o = gelu_erf(o);
       if (row < live && col_ok) Cb[(size_t)row * N + col] = o;
     }
