@@ -95,6 +95,38 @@ def test_gate_topk_logit_bias(K):
   assert_close(to_np(gates), O.router_gates(x, w, O.BF16, b), 2e-2, "gates with bias")
 
 
+@pytest.mark.parametrize("n,D,E", [(1568, 512, 8), (45, 64, 5), (4100, 384, 32), (33, 1024, 24)])
+def test_gate_topk_float32_split_k_form(K, monkeypatch, n, D, E):
+  """float32 gating over few items deals the k range of a tile to the four waves of a workgroup
+  (partial logits added in wave order): against the one-wave-per-tile form
+  (VMOE_GATE_NO_SPLIT_K=1) bit for bit on operands whose partial sums are exact, within float32
+  rounding otherwise; logits output and logit bias included."""
+  rng = np.random.default_rng(n + D)
+  xi = rng.integers(-2, 3, (1, n, D)).astype(np.float32)
+  wi = rng.integers(-2, 3, (D, E)).astype(np.float32) / 64
+  b = (rng.integers(-8, 9, E) / 4).astype(np.float32)
+  xr = rng.standard_normal((1, n, D)).astype(np.float32)
+  wr = (rng.standard_normal((D, E)) / np.sqrt(D)).astype(np.float32)
+  for x, w, exact in ((xi, wi, True), (xr, wr, False)):
+    monkeypatch.delenv("VMOE_GATE_NO_SPLIT_K", raising=False)
+    g_s, v_s, i_s, l_s = K.gate_topk(to_dev(x), to_dev(w), 2, logit_bias=to_dev(b), return_logits=True)
+    g_p, v_p, i_p = K.gate_topk(to_dev(x), to_dev(w), 2)
+    monkeypatch.setenv("VMOE_GATE_NO_SPLIT_K", "1")
+    g_d, v_d, i_d, l_d = K.gate_topk(to_dev(x), to_dev(w), 2, logit_bias=to_dev(b), return_logits=True)
+    monkeypatch.delenv("VMOE_GATE_NO_SPLIT_K")
+    want = x[0].astype(np.float64) @ w.astype(np.float64) + b
+    np.testing.assert_allclose(to_np(l_s)[0], want, rtol=1e-5, atol=1e-5)
+    assert_close(to_np(g_p), O.router_gates(x, w, O.F32), 1e-5, "gates without bias")
+    if exact:
+      np.testing.assert_array_equal(to_np(l_s), to_np(l_d))
+      np.testing.assert_array_equal(to_np(g_s), to_np(g_d))
+      np.testing.assert_array_equal(to_np(i_s), to_np(i_d))
+      np.testing.assert_array_equal(to_np(v_s), to_np(v_d))
+    else:
+      np.testing.assert_allclose(to_np(l_s), to_np(l_d), rtol=1e-5, atol=1e-5)
+      np.testing.assert_allclose(to_np(g_s), to_np(g_d), rtol=1e-5, atol=1e-6)
+
+
 def test_gate_topk_streaming_and_direct_loads_agree(K, monkeypatch):
   """The two forms of the bfloat16 gating kernel (item rows through LDS by DMA, or by direct
   loads: VMOE_GATE_DIRECT_LOADS=1) add the same products in a different order of k: equal

@@ -69,7 +69,7 @@ template <typename T> __host__ __device__ constexpr int w_stride(int kc, int epa
   return sizeof(T) == 2 ? kc + 8 : epad;
 }
 
-template <typename T, int NT, bool LOGITS, int WAVES>
+template <typename T, int NT, bool LOGITS, int WAVES, bool SPLITK = false>
 __global__ __launch_bounds__(WAVES * kWave) void gate_topk_kernel(
     const T* __restrict__ x, const T* __restrict__ w, const float* __restrict__ bias,
     T* __restrict__ gates, float* __restrict__ logits, float* __restrict__ topk_val,
@@ -87,11 +87,16 @@ __global__ __launch_bounds__(WAVES * kWave) void gate_topk_kernel(
   const int m = lane & 31;
   const int h = lane >> 5;
   const int stride = w_stride<T>(KC, EP);
-  const int tiles_per_iter = gridDim.x * kGateWaves;
+  // SPLITK (float32, few items): the four waves of a workgroup share one tile of 32 items and
+  // a quarter of D each, and meet in the logits tiles of the epilogue: a launch of a few dozen
+  // tiles is as long as its longest chain of loads and MFMAs, which this cuts in four.
+  static_assert(!SPLITK || (sizeof(T) == 4 && WAVES == 4), "split-k form");
+  const int tiles_per_iter = SPLITK ? gridDim.x : gridDim.x * kGateWaves;
   const int iters = (num_tiles + tiles_per_iter - 1) / tiles_per_iter;
 
   for (int it = 0; it < iters; ++it) {
-    const int tile = it * tiles_per_iter + blockIdx.x * kGateWaves + wave;
+    const int tile = SPLITK ? it * tiles_per_iter + blockIdx.x
+                            : it * tiles_per_iter + blockIdx.x * kGateWaves + wave;
     const bool active = tile < num_tiles;
     const int row0 = tile * 32;
     int r = row0 + m;
@@ -246,25 +251,50 @@ __global__ __launch_bounds__(WAVES * kWave) void gate_topk_kernel(
           mfma_result_fence();
         }
       } else {
+        // float32: the item rows are loaded four 16-wide k steps at a time, two such batches in
+        // flight (a batch is refilled as soon as its MFMAs are issued).
         const int nkb = KC / 16;
-        for (int kb = 0; kb < nkb; ++kb) {
-          const int kl = kb * 16 + h * 8;
-          float a[8];
+        int kb_lo = 0, kb_hi = nkb;
+        if (SPLITK) {
+          kb_lo = wave * (nkb / kGateWaves);
+          kb_hi = kb_lo + nkb / kGateWaves;
+        }
+        constexpr int FB = 4;
+        float4 va[2][FB][2];
+        auto load_f = [&](const int u, int kb0) {
 #pragma unroll
-          for (int j = 0; j < 2; ++j) {
-            int kg = k0 + kl + j * 4;
-            float4 v = (kg + 4 <= D) ? *reinterpret_cast<const float4*>(xrow + kg)
-                                     : make_float4(0.f, 0.f, 0.f, 0.f);
-            a[j * 4 + 0] = v.x; a[j * 4 + 1] = v.y; a[j * 4 + 2] = v.z; a[j * 4 + 3] = v.w;
-          }
+          for (int t = 0; t < FB; ++t)
 #pragma unroll
-          for (int i = 0; i < 8; ++i) {
+            for (int j = 0; j < 2; ++j) {
+              const int kg = k0 + (kb0 + t) * 16 + h * 8 + j * 4;
+              va[u][t][j] = (kb0 + t < kb_hi && kg + 4 <= D) ? *reinterpret_cast<const float4*>(xrow + kg)
+                                                             : make_float4(0.f, 0.f, 0.f, 0.f);
+            }
+        };
+        auto mma_f = [&](const int u, int kb0) {
 #pragma unroll
-            for (int nt = 0; nt < NT; ++nt) {
-              float b = wl[(kl + i) * stride + nt * 32 + m];
-              acc[nt] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], b, acc[nt], 0, 0, 0);
+          for (int t = 0; t < FB; ++t) {
+            if (kb0 + t >= kb_hi) break;
+            const int kl = (kb0 + t) * 16 + h * 8;
+            const float a[8] = {va[u][t][0].x, va[u][t][0].y, va[u][t][0].z, va[u][t][0].w,
+                                va[u][t][1].x, va[u][t][1].y, va[u][t][1].z, va[u][t][1].w};
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+#pragma unroll
+              for (int nt = 0; nt < NT; ++nt) {
+                float b = wl[(kl + i) * stride + nt * 32 + m];
+                acc[nt] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], b, acc[nt], 0, 0, 0);
+              }
             }
           }
+        };
+        load_f(0, kb_lo);
+        load_f(1, kb_lo + FB);
+        for (int kb0 = kb_lo; kb0 < kb_hi; kb0 += 2 * FB) {
+          mma_f(0, kb0);
+          load_f(0, kb0 + 2 * FB);
+          mma_f(1, kb0 + FB);
+          load_f(1, kb0 + 3 * FB);
           mfma_result_fence();
         }
       }
@@ -289,8 +319,11 @@ __global__ __launch_bounds__(WAVES * kWave) void gate_topk_kernel(
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
           const int rl = (i >> 2) * 8 + h * 4 + (i & 3);
-          float v = Elt<T>::round(acc[nt][i]);
-          if (bias != nullptr) v = Elt<T>::round(v + bn[nt]);
+          float v = acc[nt][i];
+          if (!SPLITK) {
+            v = Elt<T>::round(v);
+            if (bias != nullptr) v = Elt<T>::round(v + bn[nt]);
+          }
           st[rl * (EP + 1) + nt * 32 + m] = v;
         }
     }
@@ -299,12 +332,26 @@ __global__ __launch_bounds__(WAVES * kWave) void gate_topk_kernel(
     const int n0 = h * CNT;
     float g[CNT];
     float mx = -INFINITY;
+    if (SPLITK) {
+      // the four waves' partial logits meet here, added in wave order; wave 0 finishes the tile
+      __syncthreads();
+      if (wave != 0) {
+        __syncthreads();          // the tiles are free again once wave 0 has read them
+        continue;
+      }
+    }
 #pragma unroll
     for (int j = 0; j < CNT; ++j) {
-      const float v = st[m * (EP + 1) + n0 + j];
+      float v = st[m * (EP + 1) + n0 + j];
+      if (SPLITK) {
+#pragma unroll
+        for (int ww = 1; ww < kGateWaves; ++ww) v += st[(ww * 32 + m) * (EP + 1) + n0 + j];
+        if (bias != nullptr && n0 + j < E) v += bias[n0 + j];
+      }
       g[j] = (n0 + j < E) ? v : -INFINITY;
       mx = fmaxf(mx, g[j]);
     }
+    if (SPLITK) __syncthreads();
     if (LOGITS && row < num_items) {
 #pragma unroll
       for (int j = 0; j < CNT; ++j)
@@ -699,6 +746,11 @@ int launch_gate(const VmoeGateTopkParams* p, hipStream_t stream) {
       return three ? srun(gate_topk_stream_kernel<3, 8>) : srun(gate_topk_stream_kernel<2, 8>);
     }
   }
+  // float32, up to 32 experts, at most two tiles of items per CU: a tile per workgroup, its k
+  // range dealt to the four waves.
+  const bool split_k = sizeof(T) == 4 && nt == 1 && waves == 4 && num_tiles <= 512 && kc % 64 == 0 &&
+                       getenv("VMOE_GATE_NO_SPLIT_K") == nullptr;
+  if (split_k) blocks = num_tiles;
   auto run = [&](auto kern) {
     hipError_t e = allow_dynamic_lds(reinterpret_cast<const void*>(kern), lds);
     if (e != hipSuccess) return (int)e;
@@ -710,6 +762,11 @@ int launch_gate(const VmoeGateTopkParams* p, hipStream_t stream) {
   };
   // The logits output is a separate instantiation: its extra live pointer costs
   // the common one a wave of occupancy.
+  if constexpr (sizeof(T) == 4) {
+    if (split_k)
+      return p->logits != nullptr ? run(gate_topk_kernel<T, 1, true, 4, true>)
+                                  : run(gate_topk_kernel<T, 1, false, 4, true>);
+  }
   if (p->logits != nullptr) {
     switch (nt) {
       case 1: return waves == 8 ? run(gate_topk_kernel<T, 1, true, 8>) : run(gate_topk_kernel<T, 1, true, 4>);
