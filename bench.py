@@ -619,7 +619,7 @@ def sparse_run(args, name, short=False):
   achieved_tflops = flops_per_launch / (gemm_ms * 1e-3) / 1e12
   peak = PEAK_BF16_TFLOPS if tdt == torch.bfloat16 else PEAK_FP32_MATRIX_TFLOPS
   roofline = {"bound": "mfma",
-              "kernel": "gemm_bf16_mixed_kernel (first product) / gemm_bf16_w8_kernel<0, true, 8> (second product)" if b == 2 else "gemm_f32_kernel",
+              "kernel": "gemm_bf16_mixed_kernel (first product) / gemm_bf16_w8_kernel<0, true, 8> (second product)" if b == 2 else "gemm_f32_dma_kernel<1, 128> (first product) / gemm_f32_dma_kernel<0, 64> (second product)",
               "achieved": achieved_tflops, "peak": peak, "unit": "TFLOP/s",
               "frac": achieved_tflops / peak, "traffic": MEASURED_TRAFFIC_BYTES.get(cfg.name),
               "from_profile": {"traffic_bytes_per_launch": MEASURED_TRAFFIC_BYTES.get(cfg.name),
