@@ -1019,13 +1019,14 @@ SHARED_ROUND_CASES = [
 
 
 @pytest.mark.parametrize("E,R,D,M", SHARED_ROUND_CASES)
-def test_expert_mlp_second_product_shares_partial_round(K, E, R, D, M):
+def test_expert_mlp_second_product_shares_partial_round(K, monkeypatch, E, R, D, M):
   """The tile-walking second product cuts the tiles of a die's last, partial round along k
   among the die's workgroups; the float32 sums travel from piece to piece through memory.
   Against the same experts computed one at a time and against a float32 restatement: a cut
   changes the order of one float32 addition per output, so an output may differ from the
   uncut computation by one bfloat16 step (few do); dense and over packed rows with a launch
   plan (random row counts move the cuts); rows past a count are not written."""
+  monkeypatch.setenv("VMOE_SECOND_PRODUCT", "shared")      # whatever the launch geometry would choose
   rng = np.random.default_rng(E * 1000 + R)
   bf = torch.bfloat16
   x = to_dev(O.cast(rng.standard_normal((E, R, D)).astype(np.float32), O.BF16), O.BF16)
@@ -1070,10 +1071,11 @@ def test_expert_mlp_second_product_shares_partial_round(K, E, R, D, M):
 
 
 @pytest.mark.parametrize("E,R,D,M", [(12, 2048, 1024, 512), (3, 500, 768, 1024)])
-def test_shared_partial_round_is_exact_on_exact_operands(K, E, R, D, M):
+def test_shared_partial_round_is_exact_on_exact_operands(K, monkeypatch, E, R, D, M):
   """The same cuts on operands whose every product, sum and rounding step is exact (small
   integers, GELU the identity): whatever the order of the additions, the result must
   equal the float64 answer bit for bit, dense and over packed rows."""
+  monkeypatch.setenv("VMOE_SECOND_PRODUCT", "shared")      # whatever the launch geometry would choose
   rng = np.random.default_rng(D + M)
   x = rng.integers(-1, 2, (E, R, D)).astype(np.float32)
   w0 = _sparse_signs(rng, (E, D, M), 8, axis=1)
@@ -1103,6 +1105,7 @@ def test_shared_round_wait_that_gives_up_is_loud(K, monkeypatch):
   is never reached.  Every kernel still runs to its end; the pieces that gave up are counted
   in the status words and their outputs are NaN, not sums that were never delivered.  The
   count stays when later calls on the same workspace go well."""
+  monkeypatch.setenv("VMOE_SECOND_PRODUCT", "shared")      # whatever the launch geometry would choose
   E, R, D, M = 3, 500, 768, 1024           # 2-3 tiles per die: every tile is shared
   rng = np.random.default_rng(5)
   args = [to_dev(O.cast(a, O.BF16), O.BF16) for a in (

@@ -360,7 +360,9 @@ MlpPlans mlp_plans(int E, int R, int D, int M, bool ragged) {
   const bool eight_ok = w8_gemm_ok<8>(E, R, D, M, rows, bytes(square) ? planned : nullptr);
   const bool narrow_ok = w8_gemm_ok<6>(E, R, D, M, rows, bytes(narrow) ? planned : nullptr);
   const double t_wide = 1.5 * 1.04 * std::ceil((double)wide.tiles / kNumCu);
-  const double t_shared = (double)square.tiles / kNumCu + 0.05;
+  // the shared form balances a partial round but runs 32x32x16 MFMAs and exchanges sums: on the
+  // L/16 half-capacity layer (0.8 tiles per CU) it measures 2 % behind eight waves
+  const double t_shared = 1.12 * (double)square.tiles / kNumCu + 0.1;
   const double t_eight = 0.95 * std::ceil((double)square.tiles / kNumCu);
   const double t_narrow = 0.75 * 0.97 * std::ceil((double)narrow.tiles / kNumCu);
   double t_best = 1e300;
