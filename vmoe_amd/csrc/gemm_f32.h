@@ -4,17 +4,22 @@
 // C[b] = epilogue(A[b] (R x Kd) . B[b] (Kd x N) + bias[b]); B in the reference's (in, out)
 // order, so a lane's B operand is one scalar B[k][n] and nothing is transposed.
 //
-// What bounds a float32 product here is not the matrix cores' operand appetite (a 32x32x2 MFMA
-// takes 64 clocks for one A and one B scalar per lane) but how often the operands cross from
-// L2 to the CUs and how evenly few, long tiles fall on 256 CUs:
+// The matrix cores' operand appetite is small here (a 32x32x2 MFMA takes 64 clocks for one A and
+// one B scalar per lane, and a register-resident loop of them runs at 0.99 of the float32 matrix
+// peak), so the design is about the traffic between L2 and the CUs and about how few, long
+// tiles fall on 256 CUs:
 //   * a 64 x 64 tile fetches 512 bytes per 8 192 flops, 9.8 TB/s at the float32 matrix peak; the
-//     first product therefore takes 64 x 128 tiles;
+//     first product therefore takes 64 x 128 tiles where those still outnumber the CUs twice;
 //   * the tile list is cut into eight contiguous runs, one per XCD (a workgroup's XCD is its
 //     index modulo 8), batch-major and column-panel-major inside a run: with eight experts each
-//     die multiplies one expert, whose activations stay in its L2 while the weights stream
-//     through it once;
+//     die multiplies one expert, and the tiles of a run walk k in step, so that a k slice of
+//     the operands is fetched into the die's L2 once for all of them;
 //   * rows beyond a ragged batch's count cost nothing: a wave skips the 32-row blocks that
 //     hold none, so a tile's time follows its live blocks.
+// With requests, fragment reads and barriers taken out the launches of the S/32 layer last
+// nearly as long as with them: what is left between them and the peak is the 3.4 or 1.75 tiles
+// per CU, and that the workgroups that share a CU, taking turns MFMA by MFMA, also reach their
+// prologues and epilogues together.
 // Loop: k tiles of 32 in a ring of three LDS stages, requested two iterations before their
 // fragments are read, one barrier per k tile.  A rows are stored with their
 // 16-byte pieces XOR-swizzled by (row / 2) % 8, B rows 16..31 with their column halves
