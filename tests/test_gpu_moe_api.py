@@ -633,6 +633,41 @@ def test_soft_moe_b16_shape_vs_oracle(moe):
   assert_close(to_np(out), want, 3e-2, "soft moe b16 shape")
 
 
+def test_soft_moe_full_size_is_equivariant_to_group_order(moe):
+  """The Soft MoE layer at the benchmark's full size (256 groups of 196 tokens, 128 experts x 1
+  slot): every group forms its slots from its own tokens and an expert's output row depends on
+  its own input row only, so permuting the groups permutes the output bit for bit; and the
+  first groups of the full batch match the same groups run on their own to one bfloat16 step (a
+  prefix of the groups is a prefix of every expert's rows)."""
+  from vmoe_amd import configs
+  from vmoe_amd.nn import vit_moe
+  from vmoe_amd.projects.soft_moe import router
+  cfg = configs.SOFT_B16
+  x, params = configs.make_soft_inputs(cfg, seed=4, num_images=cfg.num_images)
+  dtype = O.BF16
+  layer = router.SoftRouter(num_experts=cfg.num_experts, num_slots=cfg.num_slots,
+                            compute_similarity_metrics=False)
+  rp = {"params": {"mu": to_dev(params["Router"]["mu"]), "scale": torch.tensor(1.0, device=dev())}}
+  mlp = moe.sparse_moe_spmd(vit_moe.MlpBlock, variable_axes={"params": 0})(mlp_dim=cfg.mlp_dim)
+  variables = {"params": {k: {kk: to_dev(O.cast(vv, dtype), dtype) for kk, vv in v.items()}
+                          for k, v in params["Mlp"].items()}}
+
+  def run(xd):
+    disp, _ = layer.apply(rp, xd)
+    return mlp.apply(variables, disp, xd)
+
+  xd = to_dev(O.cast(x, dtype), dtype)
+  G = xd.shape[0]
+  assert G == 256
+  out = run(xd)
+  perm = torch.randperm(G, generator=torch.Generator().manual_seed(9)).to(dev())
+  out_p = run(xd[perm].contiguous())
+  assert torch.equal(out_p, out[perm]), f"{(out_p != out[perm]).any(-1).sum().item()} tokens differ"
+  head = run(xd[:8].contiguous())          # other launch geometry: a product cut along k may round one step apart
+  torch.testing.assert_close(head.float(), out[:8].float(), rtol=2.0 ** -7, atol=1e-6)
+  assert torch.isfinite(out.float()).all()
+
+
 # groups of each benchmark configuration that the layer test runs (None = all of them)
 LAYER_CONFIG_GROUPS = {
     "vmoe_s32_layer": None,                 # fp32, full size
@@ -711,6 +746,39 @@ ROUTERS_BY_NAME = {
     "dotted_soft": {"name": "vmoe_amd.projects.soft_moe.router.SoftRouter"},
     "call_syntax": {"name": "NoisyTopExpertsPerItemRouter(num_selected_experts=2)"},
 }
+
+
+@pytest.mark.parametrize("name", ["vmoe_b16_layer_E32_k2_bpr", "vmoe_s32_layer"])
+def test_layer_full_size_is_equivariant_to_group_order(name):
+  """A property that holds at any size, checked at the benchmark configurations' full size: the
+  groups of a layer are routed independently, and an output row of the expert products depends
+  on its own input row only (same order of k whatever tile the row lands in), so permuting the
+  groups of the input permutes the output, bit for bit.  The rows of every expert's buffer,
+  the launch plan and the tiles' contents all change with the permutation."""
+  from vmoe_amd import configs
+  from vmoe_amd.nn import vit_moe
+  cfg = configs.CONFIGS[name]
+  x, params, bias = configs.make_layer_inputs(cfg, seed=11, num_images=cfg.num_images)
+  dtype = O.BF16 if cfg.dtype == "bfloat16" else O.F32
+  rk = dict(num_selected_experts=cfg.num_selected_experts, dispatcher=cfg.dispatcher_kwargs())
+  if bias is not None:
+    rk["logit_bias"] = to_dev(bias)
+  layer = vit_moe.MlpMoeBlock(mlp_dim=cfg.mlp_dim, num_experts=cfg.num_experts,
+                              group_size=cfg.group_size, deterministic=True, router=rk,
+                              dtype=tdtype(dtype))
+  params["Mlp"] = {k: {kk: O.cast(vv, dtype) for kk, vv in v.items()} for k, v in params["Mlp"].items()}
+  dev_params = _params_to_dev(params, dtype)
+  xd = to_dev(O.cast(x, dtype), dtype)
+  G = xd.numel() // (cfg.group_size * cfg.d_model)
+  assert G >= 8
+  out, _ = layer.apply(dev_params, xd)
+  perm = torch.randperm(G, generator=torch.Generator().manual_seed(3)).to(dev())
+  xg = xd.reshape(G, cfg.group_size, cfg.d_model)
+  out_p, _ = layer.apply(dev_params, xg[perm].reshape(xd.shape).contiguous())
+  got = out_p.reshape(G, cfg.group_size, cfg.d_model)
+  want = out.reshape(G, cfg.group_size, cfg.d_model)[perm]
+  assert torch.equal(got, want), f"{(got != want).any(-1).sum().item()} items differ under a permutation of the groups"
+  assert not torch.equal(out_p.reshape(want.shape), out.reshape(want.shape))      # the permutation did something
 
 
 @pytest.mark.parametrize("dtype", [O.F32, O.BF16])
