@@ -336,7 +336,8 @@ typedef struct {
                                      (num_items, D) matrix of items itself and x_rows[e][r] the
                                      item in row r of expert e (row_token of vmoe_compact_rows):
                                      the first product gathers its rows, no dispatched buffer
-                                     is needed.  bf16 with D % 32 == 0 only
+                                     is needed.  D % 32 == 0 (both types), float32 also
+                                     16-byte aligned x and w0 and items within 2 GiB
                                      (VMOE_E_UNSUPPORTED otherwise) */
   int32_t num_items;              /* rows of x when x_rows is given */
 } VmoeExpertMlpParams;

@@ -686,6 +686,36 @@ def test_expert_mlp_float32_products_on_the_dma_kernel(K, monkeypatch, E, R, D, 
 
 
 @pytest.mark.parametrize("dtype", [O.F32, O.BF16])
+def test_expert_mlp_gathers_its_rows_from_the_items(K, dtype):
+  """x_rows: the first product reads row r of expert e from item x_rows[e][r] of the (T, D)
+  matrix of items.  Bit for bit what the same call computes on a buffer built by indexing;
+  entries past an expert's count (here out of range on purpose) are never followed."""
+  rng = np.random.default_rng(17)
+  E, R, D, M, T = 6, 200, 96, 160, 500
+  items = to_dev(O.cast(rng.standard_normal((T, D)).astype(np.float32), dtype), dtype)
+  w0 = to_dev(O.cast(rng.standard_normal((E, D, M)).astype(np.float32) / np.sqrt(D), dtype), dtype)
+  w1 = to_dev(O.cast(rng.standard_normal((E, M, D)).astype(np.float32) / np.sqrt(M), dtype), dtype)
+  b0 = to_dev(O.cast(rng.standard_normal((E, M)).astype(np.float32) * 0.1, dtype), dtype)
+  b1 = to_dev(O.cast(rng.standard_normal((E, D)).astype(np.float32) * 0.1, dtype), dtype)
+  rows = np.asarray([200, 0, 1, 65, 128, 199], np.int32)
+  x_rows = np.full((E, R), 2 ** 30, np.int32)
+  for e, n in enumerate(rows):
+    x_rows[e, :n] = rng.integers(0, T, n)
+  assert K.expert_mlp_can_gather(tdtype(dtype), D, T)
+  got = torch.full((E, R, D), 7.0, dtype=tdtype(dtype), device=dev())
+  K.expert_mlp(items, w0, b0, w1, b1, out=got, rows_per_expert=to_dev(rows), x_rows=to_dev(x_rows))
+  buf = items[torch.from_numpy(np.where(x_rows < T, x_rows, 0)).to(dev()).long()]      # (E, R, D)
+  want = torch.full((E, R, D), 7.0, dtype=tdtype(dtype), device=dev())
+  K.expert_mlp(buf, w0, b0, w1, b1, out=want, rows_per_expert=to_dev(rows))
+  assert torch.equal(got, want)
+  for e, n in enumerate(rows):
+    assert (to_np(got[e, n:]) == 7.0).all()
+  full = O.mlp_block(to_np(buf).astype(np.float32), to_np(w0), to_np(b0), to_np(w1), to_np(b1), dtype)
+  for e, n in enumerate(rows):
+    assert_close(to_np(got[e, :n]), full[e, :n], 1e-5 if dtype == O.F32 else 2e-2, f"expert {e}")
+
+
+@pytest.mark.parametrize("dtype", [O.F32, O.BF16])
 @pytest.mark.parametrize("E", [5, 20])      # fewer / more experts than dies in the launch plan
 def test_expert_mlp_rows_per_expert(K, dtype, E):
   """Leading rows equal the full computation bit for bit; the other rows are not written."""

@@ -106,16 +106,20 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(
 
 template <int EPI>
 int launch_gemm_f32(const float* A, const float* B, const float* bias, float* C, int batch, int R,
-                    int N, int Kd, hipStream_t stream, const int32_t* rows = nullptr) {
+                    int N, int Kd, hipStream_t stream, const int32_t* rows = nullptr,
+                    const int32_t* a_rows = nullptr, int a_items = 0) {
   // The DMA kernel where its shapes allow: 64 x 128 tiles when they outnumber the CUs twice
   // over, 64 x 64 otherwise.  VMOE_F32_GEMM=plain keeps the register-staged kernel below.
   const char* which = getenv("VMOE_F32_GEMM");
-  if (gemm_f32_dma_ok(A, B, R, N, Kd) && !(which != nullptr && strcmp(which, "plain") == 0)) {
+  // (gathered rows are the DMA kernel's alone: check_mlp has made sure that it applies)
+  if (gemm_f32_dma_ok(A, B, R, N, Kd, a_items) &&
+      (a_rows != nullptr || !(which != nullptr && strcmp(which, "plain") == 0))) {
     const long long wide_tiles = (long long)batch * ((R + 63) / 64) * ((N + 127) / 128);
     if (wide_tiles >= 2 * kCusPerXcd * kNumXcd && !(which != nullptr && strcmp(which, "64") == 0))
-      return launch_gemm_f32_dma<EPI, 128>(A, B, bias, C, batch, R, N, Kd, stream, rows);
-    return launch_gemm_f32_dma<EPI, 64>(A, B, bias, C, batch, R, N, Kd, stream, rows);
+      return launch_gemm_f32_dma<EPI, 128>(A, B, bias, C, batch, R, N, Kd, stream, rows, a_rows, a_items);
+    return launch_gemm_f32_dma<EPI, 64>(A, B, bias, C, batch, R, N, Kd, stream, rows, a_rows, a_items);
   }
+  if (a_rows != nullptr) return VMOE_E_UNSUPPORTED;
   const int tiles_m = (R + kF32Tile - 1) / kF32Tile, tiles_n = (N + kF32Tile - 1) / kF32Tile;
   const long long blocks = (long long)batch * tiles_m * tiles_n;
   if (blocks > 0x7fffffffLL) return VMOE_E_OVERFLOW;
@@ -401,7 +405,10 @@ static int check_mlp(const VmoeExpertMlpParams* p) {
   if (p->x_rows != nullptr) {
     if (p->rows_per_expert == nullptr) return VMOE_E_NULL;
     if (p->num_items < 1) return VMOE_E_SHAPE;
-    if (p->dtype != VMOE_BF16) return VMOE_E_UNSUPPORTED;
+    // float32: the LDS-DMA kernel gathers (whole 32-wide k tiles, 16-byte aligned operands)
+    if (p->dtype != VMOE_BF16 &&
+        !gemm_f32_dma_ok((const float*)p->x, (const float*)p->w0, p->R, p->M, p->D, p->num_items))
+      return VMOE_E_UNSUPPORTED;
   }
   if (p->gelu != VMOE_GELU_TANH && p->gelu != VMOE_GELU_ERF) return VMOE_E_DTYPE;
   if (p->dtype == VMOE_BF16) {
@@ -564,11 +571,11 @@ static int run_expert_mlp(const VmoeExpertMlpParams* p, vmoe_stream_t stream_, b
   if (tanh_gelu)
     rc = launch_gemm_f32<kEpiBiasGeluTanh>((const float*)p->x, (const float*)p->w0,
                                            (const float*)p->b0, (float*)hidden, p->E, p->R, p->M,
-                                           p->D, stream, p->rows_per_expert);
+                                           p->D, stream, p->rows_per_expert, p->x_rows, p->num_items);
   else
     rc = launch_gemm_f32<kEpiBiasGeluErf>((const float*)p->x, (const float*)p->w0,
                                           (const float*)p->b0, (float*)hidden, p->E, p->R, p->M,
-                                          p->D, stream, p->rows_per_expert);
+                                          p->D, stream, p->rows_per_expert, p->x_rows, p->num_items);
   if (rc != VMOE_OK) return rc;
   return launch_gemm_f32<kEpiBias>((const float*)hidden, (const float*)p->w1, (const float*)p->b1,
                                    (float*)p->out, p->E, p->R, p->D, p->M, stream,

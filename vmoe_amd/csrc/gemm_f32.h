@@ -52,7 +52,7 @@ template <int EPI, int BN_>
 __global__ __launch_bounds__(256) void gemm_f32_dma_kernel(
     const float* __restrict__ A, const float* __restrict__ B, const float* __restrict__ bias,
     float* __restrict__ C, int batch, int R, int N, int Kd, int tiles_m, int tiles_n, int per_xcd,
-    const int32_t* __restrict__ rows) {
+    const int32_t* __restrict__ rows, const int32_t* __restrict__ a_rows, int a_items) {
 #if defined(__HIP_DEVICE_COMPILE__)   // buffer-resource builtins exist in the device pass only
   using Cfg = F32Cfg<BN_>;
   extern __shared__ __align__(1024) unsigned char smem[];
@@ -82,7 +82,14 @@ __global__ __launch_bounds__(256) void gemm_f32_dma_kernel(
     for (int i = 0; i < Cfg::kAIssues; ++i) {
       const int r = (i * Cfg::kWaves + wave) * 8 + lrow;
       const int piece = pos ^ ((r >> 1) & 7);
-      a_goff[i] = (uint32_t)min(row0 + r, R - 1) * (uint32_t)Kd * 4u + piece * 16;
+      // a_rows: A is the matrix of items (a_items x Kd) and a_rows[b][row] names the item of a
+      // row (rows past the count hold no index: they read the last live row's item)
+      int arow = min(row0 + r, (a_rows != nullptr ? live : R) - 1);
+      if (a_rows != nullptr) {
+        arow = a_rows[(size_t)b * R + arow];
+        arow = (unsigned)arow < (unsigned)a_items ? arow : 0;
+      }
+      a_goff[i] = (uint32_t)arow * (uint32_t)Kd * 4u + piece * 16;
     }
   }
   {
@@ -97,7 +104,8 @@ __global__ __launch_bounds__(256) void gemm_f32_dma_kernel(
   // Reads past the end of a batch's operand return zero (the last column tile of the last k
   // row reaches there when N is not a multiple of the tile).
   const __amdgpu_buffer_rsrc_t a_rsrc = __builtin_amdgcn_make_buffer_rsrc(
-      const_cast<float*>(A + (size_t)b * R * Kd), 0, (int)((uint32_t)R * (uint32_t)Kd * 4u), 0x00020000);
+      const_cast<float*>(a_rows != nullptr ? A : A + (size_t)b * R * Kd), 0,
+      (int)((uint32_t)(a_rows != nullptr ? a_items : R) * (uint32_t)Kd * 4u), 0x00020000);
   const __amdgpu_buffer_rsrc_t b_rsrc = __builtin_amdgcn_make_buffer_rsrc(
       const_cast<float*>(B + (size_t)b * Kd * N), 0, (int)((uint32_t)Kd * (uint32_t)N * 4u), 0x00020000);
   auto request = [&](int stage, int kt) {
@@ -219,15 +227,18 @@ __global__ __launch_bounds__(256) void gemm_f32_dma_kernel(
 
 // Shapes the DMA kernel takes: whole 32-wide k tiles, operand rows that are whole 16-byte
 // pieces at 16-byte aligned addresses, a batch's operands within reach of 32-bit offsets.
-inline bool gemm_f32_dma_ok(const float* A, const float* B, int R, int N, int Kd) {
+// (a_items: rows of the matrix of items when the rows are gathered, else 0)
+inline bool gemm_f32_dma_ok(const float* A, const float* B, int R, int N, int Kd, int a_items = 0) {
   return Kd % 32 == 0 && N % 4 == 0 && R > 0 && (reinterpret_cast<uintptr_t>(A) & 15u) == 0 &&
-         (reinterpret_cast<uintptr_t>(B) & 15u) == 0 && (int64_t)R * Kd * 4 < ((int64_t)1 << 31) &&
+         (reinterpret_cast<uintptr_t>(B) & 15u) == 0 &&
+         (int64_t)(a_items > R ? a_items : R) * Kd * 4 < ((int64_t)1 << 31) &&
          (int64_t)Kd * N * 4 < ((int64_t)1 << 31);
 }
 
 template <int EPI, int BN_>
 int launch_gemm_f32_dma(const float* A, const float* B, const float* bias, float* C, int batch,
-                        int R, int N, int Kd, hipStream_t stream, const int32_t* rows) {
+                        int R, int N, int Kd, hipStream_t stream, const int32_t* rows,
+                        const int32_t* a_rows = nullptr, int a_items = 0) {
   using Cfg = F32Cfg<BN_>;
   const int tiles_m = (R + Cfg::BM - 1) / Cfg::BM, tiles_n = (N + Cfg::BN - 1) / Cfg::BN;
   const long long total = (long long)batch * tiles_m * tiles_n;
@@ -237,7 +248,7 @@ int launch_gemm_f32_dma(const float* A, const float* B, const float* bias, float
   hipError_t e = allow_dynamic_lds(reinterpret_cast<const void*>(kern), Cfg::kLds);
   if (e != hipSuccess) return (int)e;
   hipLaunchKernelGGL(kern, dim3((unsigned)per_xcd * 8), dim3(Cfg::kThreads), Cfg::kLds, stream, A, B,
-                     bias, C, batch, R, N, Kd, tiles_m, tiles_n, per_xcd, rows);
+                     bias, C, batch, R, N, Kd, tiles_m, tiles_n, per_xcd, rows, a_rows, a_items);
   return launch_status();
 }
 

@@ -311,7 +311,7 @@ def expert_mlp(x: torch.Tensor, w0, b0, w1, b1, w0t=None, w1t=None, approximate_
   # (VMOE_PLAN_SEPARATE_LAUNCH=1 in the environment keeps the planning launch apart: the
   # switch behind the before / after figures)
   rc = _E_UNSUPPORTED
-  if not os.environ.get("VMOE_PLAN_SEPARATE_LAUNCH"):
+  if x.dtype == torch.bfloat16 and not os.environ.get("VMOE_PLAN_SEPARATE_LAUNCH"):   # float32 products keep no plan
     rc = H.call_blocks("vmoe_compact_rows_planned", c, p, accept=(_E_UNSUPPORTED,))
   if rc == 0:
     H.call("vmoe_expert_mlp_planned", p)
@@ -366,6 +366,8 @@ def expert_mlp_status() -> Optional[Tuple[int, int]]:
 
 def expert_mlp_can_gather(dtype: torch.dtype, D: int, num_items: int) -> bool:
   """Whether expert_mlp can take the items themselves plus x_rows (no dispatched buffer)."""
+  if dtype == torch.float32:
+    return D % 32 == 0 and num_items * D * 4 < (1 << 31)
   return dtype == torch.bfloat16 and D % 32 == 0 and num_items * D * 2 < (1 << 32)
 
 

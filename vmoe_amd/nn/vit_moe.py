@@ -75,7 +75,7 @@ class MlpBlock(module.Module):
   def can_gather(self, items: Array) -> bool:
     """Whether apply_experts_gathered covers these items (dtype and width of the kernel)."""
     dtype = self.dtype or items.dtype
-    return (items.is_cuda and dtype == torch.bfloat16 and items.dtype == torch.bfloat16
+    return (items.is_cuda and dtype in (torch.bfloat16, torch.float32) and items.dtype == dtype
             and K.expert_mlp_can_gather(dtype, items.shape[-1], items.numel() // items.shape[-1]))
 
   def apply_experts_gathered(self, variables, items: Array, row_token: Array,
@@ -89,6 +89,10 @@ class MlpBlock(module.Module):
     w1, b1 = p["Dense_1"]["kernel"], p["Dense_1"].get("bias")
     module.require_no_grad("MlpBlock", items, w0, b0, w1, b1)
     cast = lambda t: None if t is None else K.cast(t, dtype)
+    if dtype != torch.bfloat16:      # float32 reads the kernels in the reference's layout
+      return K.expert_mlp(K.cast(items, dtype), cast(w0), cast(b0), cast(w1), cast(b1),
+                          approximate_gelu=self.approximate_gelu, rows_per_expert=rows_per_expert,
+                          x_rows=row_token)
     return K.expert_mlp(K.cast(items, dtype), None, cast(b0), None, cast(b1),
                         w0t=self._pack(w0, dtype), w1t=self._pack(w1, dtype),
                         approximate_gelu=self.approximate_gelu, rows_per_expert=rows_per_expert,
@@ -106,6 +110,10 @@ class MlpBlock(module.Module):
     w1, b1 = p["Dense_1"]["kernel"], p["Dense_1"].get("bias")
     module.require_no_grad("MlpBlock", items, w0, b0, w1, b1)
     cast = lambda t: None if t is None else K.cast(t, dtype)
+    if dtype != torch.bfloat16:
+      return K.expert_mlp(K.cast(items, dtype), cast(w0), cast(b0), cast(w1), cast(b1),
+                          approximate_gelu=self.approximate_gelu,
+                          compact=(fill, token_slot, capacity))
     return K.expert_mlp(K.cast(items, dtype), None, cast(b0), None, cast(b1),
                         w0t=self._pack(w0, dtype), w1t=self._pack(w1, dtype),
                         approximate_gelu=self.approximate_gelu,
