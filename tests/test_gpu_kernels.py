@@ -620,7 +620,9 @@ def test_einsum_golden_and_bool_weights(K, goldens):
 # ------------------------------------------------------------------ packed expert rows
 @pytest.mark.parametrize("G,S,E,Kk,C,bpr", [(4, 64, 4, 2, 20, True), (8, 50, 8, 2, 16, False), (8, 128, 8, 2, 30, False), (32, 1568, 32, 2, 100, True),
                                             (3, 33, 5, 1, 8, True), (300, 16, 4, 2, 6, False),
-                                            (64, 128, 4, 2, 6, True), (9, 300, 7, 2, 40, True), (2, 200, 300, 2, 3, False)])
+                                            (64, 128, 4, 2, 6, True), (9, 300, 7, 2, 40, True), (2, 200, 300, 2, 3, False),
+                                            (32, 49, 8, 2, 16, False),      # S/32 layer: a block of 256 assignments touches four groups
+                                            (40, 19, 8, 2, 6, True)])        # 38 per group: eight groups per block, the most the one-launch form takes
 def test_compact_rows(K, G, S, E, Kk, C, bpr):
   """token_row = e*G*C + (kept items of expert e in the groups before g) + position."""
   rng = np.random.default_rng(G * S + E)

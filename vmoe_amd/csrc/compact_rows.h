@@ -6,19 +6,24 @@
 
 namespace vmoe {
 
+// Groups that one block of 256 consecutive assignments may touch (first group included).
+constexpr int kCompactMaxSpan = 8;
+
 // token_slot = e*G*C + r(g, c)  ->  token_row = e*G*C + rows of expert e before group g + c,
-// for the 256 assignments block * 256 .. block * 256 + 255.  For E <= 256 and at least 256
-// assignments per group (a workgroup then touches at most two groups): the workgroup adds up
-// the fill counts of the groups before its first group itself -- 256 / E threads per expert,
-// each a strided share of the groups, joined in LDS.  Workgroup 0 also writes the experts'
-// row counts.
+// for the 256 assignments block * 256 .. block * 256 + 255.  For E <= 256 and groups of at
+// least 37 assignments (a workgroup then touches at most kCompactMaxSpan groups): the
+// workgroup adds up the fill counts of the groups before its first group itself -- 256 / E
+// threads per expert, each a strided share of the groups, joined in LDS -- and then, per
+// expert, the counts of the groups it touches.  Workgroup 0 also writes the experts' row
+// counts.
+
 __device__ __forceinline__ void compact_rows_fused_block(
     const int32_t* __restrict__ fill, const int32_t* __restrict__ token_slot,
     int32_t* __restrict__ token_row, int32_t* __restrict__ row_token,
     int32_t* __restrict__ rows_per_expert, int G, int E, int C, int per_group, int K, size_t n,
     unsigned block) {
   __shared__ int32_t part[256];
-  __shared__ int32_t before[2][256];
+  __shared__ int32_t before[kCompactMaxSpan][256];   // rows of expert e before group g_lo + j
   const int tid = threadIdx.x;
   const size_t i0 = (size_t)block * 256;
   const int g_lo = (int)(i0 / per_group);
@@ -38,8 +43,12 @@ __device__ __forceinline__ void compact_rows_fused_block(
   };
   const int lo = column_sum(g_lo);
   if (tid < E) {
-    before[0][tid] = lo;
-    before[1][tid] = lo + (g_lo < G ? fill[(size_t)g_lo * E + tid] : 0);
+    int acc = lo;
+#pragma unroll
+    for (int j = 0; j < kCompactMaxSpan; ++j) {      // the groups that the block's 256 assignments touch
+      before[j][tid] = acc;
+      if (g_lo + j < G) acc += fill[(size_t)(g_lo + j) * E + tid];
+    }
   }
   if (block == 0) {
     const int total = column_sum(G);
@@ -58,10 +67,13 @@ __device__ __forceinline__ void compact_rows_fused_block(
   token_row[i] = row;
 }
 
-// Whether the one-launch form applies (else a prefix launch goes first).
+// Whether the one-launch form applies (else a prefix launch goes first): a block's 256
+// consecutive assignments lie in at most kCompactMaxSpan groups.
 inline bool compact_rows_fused_ok(int G, int S, int E, int K) {
   const int parts = E <= 256 ? 256 / E : 1;
-  return E <= 256 && (int64_t)S * K >= 256 && (G + parts - 1) / parts <= 16;
+  const int64_t per_group = (int64_t)S * K;
+  return E <= 256 && (255 + per_group - 1) / per_group + 1 <= kCompactMaxSpan &&
+         (G + parts - 1) / parts <= 16;
 }
 
 }  // namespace vmoe
