@@ -166,6 +166,34 @@ __global__ __launch_bounds__(WAVES * kWave) void gate_topk_kernel(
       }
     }
 
+    // float32: the item rows are loaded four 16-wide k steps at a time, two such batches in
+    // flight (a batch is refilled as soon as its MFMAs are issued); the first two go out before
+    // the router kernel is staged.
+    constexpr int FB = 4;
+    float4 va[kBf16 ? 1 : 2][kBf16 ? 1 : FB][2];
+    int kb_lo = 0, kb_hi = KC / 16;
+    if (SPLITK) {
+      kb_lo = wave * (KC / 16 / kGateWaves);
+      kb_hi = kb_lo + KC / 16 / kGateWaves;
+    }
+    auto load_f = [&](const int u, int k0, int kb0) {
+#pragma unroll
+      for (int t = 0; t < (kBf16 ? 1 : FB); ++t)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+          const int kg = k0 + (kb0 + t) * 16 + h * 8 + j * 4;
+          va[u][t][j] = (kb0 + t < kb_hi && kg + 4 <= D)
+                            ? *reinterpret_cast<const float4*>(reinterpret_cast<const float*>(xrow) + kg)
+                            : make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+    };
+    if constexpr (!kBf16) {
+      if (active) {
+        load_f(0, 0, kb_lo);
+        load_f(1, 0, kb_lo + FB);
+      }
+    }
+
     for (int c = 0; c < num_chunks; ++c) {
       const int k0 = c * KC;
       if (num_chunks > 1 || it == 0) {
@@ -251,26 +279,6 @@ __global__ __launch_bounds__(WAVES * kWave) void gate_topk_kernel(
           mfma_result_fence();
         }
       } else {
-        // float32: the item rows are loaded four 16-wide k steps at a time, two such batches in
-        // flight (a batch is refilled as soon as its MFMAs are issued).
-        const int nkb = KC / 16;
-        int kb_lo = 0, kb_hi = nkb;
-        if (SPLITK) {
-          kb_lo = wave * (nkb / kGateWaves);
-          kb_hi = kb_lo + nkb / kGateWaves;
-        }
-        constexpr int FB = 4;
-        float4 va[2][FB][2];
-        auto load_f = [&](const int u, int kb0) {
-#pragma unroll
-          for (int t = 0; t < FB; ++t)
-#pragma unroll
-            for (int j = 0; j < 2; ++j) {
-              const int kg = k0 + (kb0 + t) * 16 + h * 8 + j * 4;
-              va[u][t][j] = (kb0 + t < kb_hi && kg + 4 <= D) ? *reinterpret_cast<const float4*>(xrow + kg)
-                                                             : make_float4(0.f, 0.f, 0.f, 0.f);
-            }
-        };
         auto mma_f = [&](const int u, int kb0) {
 #pragma unroll
           for (int t = 0; t < FB; ++t) {
@@ -288,13 +296,15 @@ __global__ __launch_bounds__(WAVES * kWave) void gate_topk_kernel(
             }
           }
         };
-        load_f(0, kb_lo);
-        load_f(1, kb_lo + FB);
+        if (c > 0) {
+          load_f(0, k0, kb_lo);
+          load_f(1, k0, kb_lo + FB);
+        }
         for (int kb0 = kb_lo; kb0 < kb_hi; kb0 += 2 * FB) {
           mma_f(0, kb0);
-          load_f(0, kb0 + 2 * FB);
+          load_f(0, k0, kb0 + 2 * FB);
           mma_f(1, kb0 + FB);
-          load_f(1, kb0 + 3 * FB);
+          load_f(1, k0, kb0 + 3 * FB);
           mfma_result_fence();
         }
       }
