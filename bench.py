@@ -732,10 +732,29 @@ def sparse_run(args, name, short=False):
       tbps = moved * 10 / (e0.elapsed_time(e1) * 1e-3) / 1e12
       delivery[name] = {"row_segment_bytes": seg, "TBps": tbps, "tiling": what, "flop_per_byte": fpb,
                         "ceiling_TFLOPs": tbps * fpb}
+    # ... and the same kind of requests over tiles that the workgroups share: 64 tiles (201 MB:
+    # they stay in L2 and the Infinity Cache, 16 workgroups per tile and launch) and all 188
+    # tiles of the buffer (592 MB: more than the caches hold).  What the request path delivers
+    # when no request waits for HBM, and what is left when most do.
+    flat = a_dn.view(torch.uint8).view(-1)
+    for name, seg, tiles in (("cached_128B", 128, 64), ("cached_64B", 64, 64), ("beyond_caches_128B", 128, 188)):
+      resident = flat[: tiles * 512 * M * 2]
+      for _ in range(3):
+        kernels.resident_delivery_probe(resident, M * 2, M * 2 // 128, 4, seg)
+      e0.record()
+      for _ in range(10):
+        moved = kernels.resident_delivery_probe(resident, M * 2, M * 2 // 128, 4, seg)
+      e1.record()
+      torch.cuda.synchronize()
+      delivery[name] = {"row_segment_bytes": seg, "TBps": moved * 10 / (e0.elapsed_time(e1) * 1e-3) / 1e12,
+                        "operands": f"{tiles} tiles of 512 rows x {M * 2} bytes shared by 256 workgroups, "
+                                    "two k tiles of 64 KB in flight per workgroup"}
     delivery["note"] = ("load-only kernel on 256 x 256 tiles of the second product's operands; the rate depends "
                         "on the shape of the requests, the ceiling on the flop per operand byte of the tiling named; "
                         "the second product requests 128-byte segments, the first product 128-byte segments for its "
-                        "weights (two thirds of its requests) and 64-byte ones for its rows")
+                        "weights (two thirds of its requests) and 64-byte ones for its rows; cached_* / beyond_caches_*: "
+                        "requests of the same shapes over shared tiles that stay in the caches, or do not: the products' "
+                        "own rates lie between them, set by their misses at the depth of their rings")
     roofline["operand_delivery"] = delivery
     del a_up, a_dn, w_up, w_dn, a_e, w_e
   # The same K steps replayed from HIP graphs (one per rotating input buffer), as a

@@ -546,6 +546,18 @@ int vmoe_operand_delivery_probe(const void* a, const void* bt, int32_t batch, in
 int vmoe_operand_delivery_probe_k64(const void* a, const void* bt, int32_t batch, int32_t rows,
                                     int32_t n, int32_t kd, double* bytes, vmoe_stream_t stream);
 
+/* The same kind of requests over tiles that the workgroups share (no counterpart in the reference;
+ * measurement aid): 256 workgroups walk tiles_per_workgroup tiles each, taken round robin
+ * from the buf_bytes / (512 * row_bytes) tiles of 512 rows x row_bytes that `buf` holds, in
+ * k_tiles steps of 128 bytes per row (k_tiles * 128 <= row_bytes), two steps in flight;
+ * segment_bytes = 128: a request is 8 rows x 128 bytes, 64: 16 rows x 64 bytes.  *bytes is
+ * set to the bytes moved into LDS.  With few tiles in `buf` (less than the caches hold)
+ * hardly a request waits for HBM: bytes / time against the other delivery probes' rates is
+ * what the products' misses cost at their ring depth. */
+int vmoe_resident_delivery_probe(const void* buf, size_t buf_bytes, int32_t row_bytes,
+                                 int32_t k_tiles, int32_t tiles_per_workgroup,
+                                 int32_t segment_bytes, double* bytes, vmoe_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

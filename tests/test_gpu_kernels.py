@@ -870,6 +870,22 @@ def test_gating_logits_are_read_whole(K):
     np.testing.assert_array_equal(got, ref.reshape(G * S, E), err_msg=dtype)
 
 
+def test_resident_delivery_probe(K):
+  """The load-only kernel over shared, L2-resident tiles runs to its end for both request shapes
+  and reports the bytes it moved; bad arguments come back as error codes."""
+  from vmoe_amd import _hip as H
+  buf = torch.zeros(3 * 512 * 1024 + 100, dtype=torch.uint8, device=dev())      # three tiles and a bit
+  for seg in (128, 64):
+    assert K.resident_delivery_probe(buf, 1024, 8, 2, seg) == 256 * 2 * 8 * 65536
+  torch.cuda.synchronize()
+  with pytest.raises(H.VmoeError, match="invalid sizes"):
+    K.resident_delivery_probe(buf, 1024, 9, 2, 128)          # 9 k tiles of 128 bytes > row
+  with pytest.raises(H.VmoeError, match="invalid sizes"):
+    K.resident_delivery_probe(buf, 1024, 8, 2, 32)
+  with pytest.raises(H.VmoeError, match="invalid sizes"):
+    K.resident_delivery_probe(buf[:1000], 1024, 8, 2, 128)   # not one whole tile
+
+
 def test_operand_delivery_probe(K):
   """The load-only measurement kernel reports the operand bytes of the 256 x 256 tiling
   and refuses what the tiling refuses."""

@@ -25,7 +25,7 @@ EXPORTS = [
     "vmoe_route_assign", "vmoe_route_assign_metrics", "vmoe_top_items_per_expert", "vmoe_indices_to_slots", "vmoe_dispatch", "vmoe_combine", "vmoe_densify",
     "vmoe_expert_mlp_workspace_bytes", "vmoe_expert_mlp", "vmoe_expert_mlp_planned", "vmoe_expert_mlp_status", "vmoe_compact_rows_planned", "vmoe_pack_expert_weights",
     "vmoe_soft_route_workspace_bytes", "vmoe_soft_route", "vmoe_einsum_dispatch",
-    "vmoe_einsum_combine", "vmoe_cast", "vmoe_copy_bytes", "vmoe_mfma_probe", "vmoe_operand_delivery_probe", "vmoe_operand_delivery_probe_k64",
+    "vmoe_einsum_combine", "vmoe_cast", "vmoe_copy_bytes", "vmoe_mfma_probe", "vmoe_operand_delivery_probe", "vmoe_operand_delivery_probe_k64", "vmoe_resident_delivery_probe",
     "vmoe_add_layer_norm", "vmoe_attention", "vmoe_noisy_gates", "vmoe_compact_rows", "vmoe_compact_rows_static",
     "vmoe_combine_backward_data", "vmoe_combine_backward_weights", "vmoe_soft_router_stats",
     "vmoe_soft_route_stats",

@@ -664,6 +664,72 @@ extern "C" int vmoe_operand_delivery_probe_k64(const void* a, const void* bt, in
   return launch_operand_delivery_probe<CfgDownPersistent>(a, bt, batch, rows, n, kd, bytes, stream);
 }
 
+// The same requests over tiles that the workgroups share: kNumCu workgroups of 256 threads walk
+// `tiles_per_workgroup` tiles each, taken round robin from the `distinct` tiles of 512 rows
+// that `buf` holds (with few tiles, many workgroups per tile and hardly a miss), k tile by k
+// tile of 64 KB, at most two k tiles in flight.  SEG = 128: a request is 8 rows x 128 bytes;
+// SEG = 64: 16 rows x 64 bytes, two requests per row and k tile.  What it moves per time is what
+// the request path delivers when latency is that of the caches: the gap to the other delivery probes
+// is what misses cost at this ring depth.
+template <int SEG>
+__global__ __launch_bounds__(256, 1) void resident_delivery_probe_kernel(
+    const unsigned char* __restrict__ buf, int distinct, int k_tiles, int tiles_per_workgroup,
+    uint32_t row_bytes) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  extern __shared__ __align__(1024) unsigned char smem[];
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  constexpr int kRowsPerRequest = 1024 / SEG, kLanesPerRow = SEG / 16;
+  const uint32_t lane_off = (uint32_t)(lane / kLanesPerRow) * row_bytes + (lane % kLanesPerRow) * 16;
+  for (int t = 0; t < tiles_per_workgroup; ++t) {
+    const size_t tile = ((size_t)blockIdx.x * tiles_per_workgroup + t) % distinct;
+    const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<unsigned char*>(buf + tile * 512 * row_bytes), 0, -1, 0x00020000);
+    for (int kt = 0; kt < k_tiles; ++kt) {
+      unsigned char* s = smem + (kt & 1) * 65536;
+#pragma unroll
+      for (int part = 0; part < 128 / SEG; ++part)
+#pragma unroll
+        for (int i = 0; i < 512 / kRowsPerRequest / 4; ++i) {
+          const int request = i * 4 + wave;
+          __builtin_amdgcn_raw_ptr_buffer_load_lds(
+              rsrc, (lds_ptr_t)(s + (part * (512 / kRowsPerRequest) + request) * 1024), 16,
+              lane_off + (uint32_t)request * kRowsPerRequest * row_bytes, kt * 128 + part * SEG, 0, 0);
+        }
+      wait_vmcnt<16>();     // the k tile before this one has landed
+    }
+  }
+  wait_vmcnt<0>();
+#endif
+}
+
+extern "C" int vmoe_resident_delivery_probe(const void* buf, size_t buf_bytes, int32_t row_bytes,
+                                            int32_t k_tiles, int32_t tiles_per_workgroup,
+                                            int32_t segment_bytes, double* bytes,
+                                            vmoe_stream_t stream) {
+  if (buf == nullptr || bytes == nullptr) return VMOE_E_NULL;
+  if (row_bytes < 128 || k_tiles < 1 || tiles_per_workgroup < 1 || (int64_t)k_tiles * 128 > row_bytes)
+    return VMOE_E_SHAPE;
+  if (segment_bytes != 64 && segment_bytes != 128) return VMOE_E_SHAPE;
+  if (!aligned16(buf) || row_bytes % 16 != 0) return VMOE_E_ALIGN;
+  const size_t tile_bytes = (size_t)512 * row_bytes;
+  if (tile_bytes >= ((size_t)1 << 32)) return VMOE_E_OVERFLOW;
+  const size_t distinct = buf_bytes / tile_bytes;
+  if (distinct < 1 || distinct > 0x7fffffff) return VMOE_E_SHAPE;
+  constexpr int kLds = 2 * 65536;
+  auto launch = [&](auto kern) -> int {
+    hipError_t e = allow_dynamic_lds(reinterpret_cast<const void*>(kern), kLds);
+    if (e != hipSuccess) return (int)e;
+    hipLaunchKernelGGL(kern, dim3(kCusPerXcd * kNumXcd), dim3(256), kLds, as_stream(stream),
+                       static_cast<const unsigned char*>(buf), (int)distinct, k_tiles,
+                       tiles_per_workgroup, (uint32_t)row_bytes);
+    return launch_status();
+  };
+  *bytes = (double)(kCusPerXcd * kNumXcd) * tiles_per_workgroup * k_tiles * 65536.0;
+  return segment_bytes == 128 ? launch(resident_delivery_probe_kernel<128>)
+                              : launch(resident_delivery_probe_kernel<64>);
+}
+
 extern "C" int vmoe_pack_expert_weights(const VmoeTransposeParams* p, vmoe_stream_t stream) {
   if (p == nullptr || p->in == nullptr || p->out == nullptr) return VMOE_E_NULL;
   if (p->batch < 1 || p->rows < 1 || p->cols < 1 || p->batch > 65535) return VMOE_E_SHAPE;

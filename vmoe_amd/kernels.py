@@ -576,6 +576,20 @@ def operand_delivery_probe(a: torch.Tensor, bt: torch.Tensor, k_tile: int = 32) 
   return float(moved.value)
 
 
+def resident_delivery_probe(buf: torch.Tensor, row_bytes: int, k_tiles: int,
+                            tiles_per_workgroup: int = 4, segment_bytes: int = 128) -> float:
+  """Launches the load-only kernel whose 256 workgroups share the few tiles of 512 rows x
+  row_bytes that `buf` (contiguous, any dtype) holds (few tiles: hardly a request waits for HBM);
+  returns the bytes it moves into LDS (time it with events)."""
+  moved = H.ctypes.c_double(0.0)
+  n = buf.numel() * buf.element_size()
+  H.check(H.lib().vmoe_resident_delivery_probe(H.ptr(buf), H.c_size_t(n), row_bytes, k_tiles,
+                                               tiles_per_workgroup, segment_bytes,
+                                               H.ctypes.byref(moved), H.stream()),
+          "vmoe_resident_delivery_probe")
+  return float(moved.value)
+
+
 def mfma_probe(seed: torch.Tensor, blocks: int = 256, iters: int = 2000) -> float:
   """Launches the register-resident MFMA loop on operands read from `seed`;
   returns the floating-point operations it issues (time it with events)."""
