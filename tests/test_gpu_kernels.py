@@ -687,6 +687,35 @@ def test_expert_mlp_float32_products_on_the_dma_kernel(K, monkeypatch, E, R, D, 
   np.testing.assert_array_equal(outs["dma"][0], outs["64"][0])              # same order of k
 
 
+def test_expert_mlp_float32_seeded_shapes(K):
+  """A seeded sweep of float32 expert MLPs over odd shapes (rows short of a block, widths that
+  end inside a tile, k that is or is not whole 32-wide tiles, many or few experts), dense and
+  over ragged rows, against the oracle at 1e-5: whichever kernel the shape takes."""
+  rng = np.random.default_rng(2024)
+  for case in range(14):
+    E = int(rng.choice([1, 2, 3, 8, 11, 40]))
+    R = int(rng.choice([1, 7, 31, 33, 64, 65, 130, 257]))
+    D = int(rng.choice([32, 36, 64, 96, 100, 160, 224]))
+    M = int(rng.choice([32, 40, 64, 128, 132, 192, 288]))
+    x = rng.standard_normal((E, R, D)).astype(np.float32)
+    w0 = (rng.standard_normal((E, D, M)) / np.sqrt(D)).astype(np.float32)
+    b0 = (rng.standard_normal((E, M)) * 0.1).astype(np.float32)
+    w1 = (rng.standard_normal((E, M, D)) / np.sqrt(M)).astype(np.float32)
+    b1 = (rng.standard_normal((E, D)) * 0.1).astype(np.float32)
+    rows = rng.integers(0, R + 1, E).astype(np.int32)
+    rows[0] = R
+    want = O.mlp_block(x, w0, b0, w1, b1, O.F32)
+    args = [to_dev(a) for a in (x, w0, b0, w1, b1)]
+    dense = to_np(K.expert_mlp(*args))
+    assert_close(dense, want, 1e-5, f"case {case}: E={E} R={R} D={D} M={M} dense")
+    ragged = torch.full((E, R, D), 7.0, dtype=torch.float32, device=dev())
+    K.expert_mlp(*args, out=ragged, rows_per_expert=to_dev(rows))
+    ragged = to_np(ragged)
+    for e, n in enumerate(rows):
+      np.testing.assert_array_equal(ragged[e, :n], dense[e, :n], err_msg=f"case {case}: E={E} R={R} D={D} M={M} expert {e}")
+      assert (ragged[e, n:] == 7.0).all(), f"case {case}: expert {e} wrote past its rows"
+
+
 @pytest.mark.parametrize("dtype", [O.F32, O.BF16])
 def test_expert_mlp_gathers_its_rows_from_the_items(K, dtype):
   """x_rows: the first product reads row r of expert e from item x_rows[e][r] of the (T, D)
