@@ -716,6 +716,48 @@ def test_expert_mlp_float32_seeded_shapes(K):
       assert (ragged[e, n:] == 7.0).all(), f"case {case}: expert {e} wrote past its rows"
 
 
+def test_expert_mlp_bfloat16_seeded_shapes(K):
+  """The same sweep in bfloat16 (widths in multiples of 8): dense against the oracle, ragged
+  rows bit for bit against the dense call and nothing written past them, and, where the shape
+  allows it, rows gathered from the items bit for bit against rows indexed beforehand."""
+  rng = np.random.default_rng(2025)
+  gathered = 0
+  for case in range(14):
+    E = int(rng.choice([1, 2, 3, 8, 11, 40]))
+    R = int(rng.choice([1, 7, 31, 33, 64, 65, 130, 257, 300]))
+    D = int(rng.choice([32, 40, 64, 96, 104, 160, 256]))
+    M = int(rng.choice([32, 48, 64, 128, 136, 192, 512]))
+    T = int(rng.choice([R, 3 * R + 5]))
+    name = f"case {case}: E={E} R={R} D={D} M={M} T={T}"
+    items = O.cast(rng.standard_normal((T, D)).astype(np.float32), O.BF16)
+    w0 = O.cast((rng.standard_normal((E, D, M)) / np.sqrt(D)).astype(np.float32), O.BF16)
+    b0 = O.cast((rng.standard_normal((E, M)) * 0.1).astype(np.float32), O.BF16)
+    w1 = O.cast((rng.standard_normal((E, M, D)) / np.sqrt(M)).astype(np.float32), O.BF16)
+    b1 = O.cast((rng.standard_normal((E, D)) * 0.1).astype(np.float32), O.BF16)
+    rows = rng.integers(0, R + 1, E).astype(np.int32)
+    rows[0] = R
+    x_rows = rng.integers(0, T, (E, R)).astype(np.int32)
+    x = items[x_rows]                                                      # (E, R, D)
+    want = O.mlp_block(x, w0, b0, w1, b1, O.BF16)
+    wd = [to_dev(a, O.BF16) for a in (w0, b0, w1, b1)]
+    dense = K.expert_mlp(to_dev(x, O.BF16), *wd)
+    assert_close(to_np(dense), want, 2e-2, name + " dense")
+    ragged = torch.full((E, R, D), 7.0, dtype=torch.bfloat16, device=dev())
+    K.expert_mlp(to_dev(x, O.BF16), *wd, out=ragged, rows_per_expert=to_dev(rows))
+    for e, n in enumerate(rows):
+      assert torch.equal(ragged[e, :n], dense[e, :n]), name + f" expert {e}"
+      assert (to_np(ragged[e, n:]) == 7.0).all(), name + f": expert {e} wrote past its rows"
+    if K.expert_mlp_can_gather(torch.bfloat16, D, T):
+      gathered += 1
+      for e, n in enumerate(rows):
+        x_rows[e, n:] = 2 ** 30                                            # never followed
+      got = torch.full((E, R, D), 7.0, dtype=torch.bfloat16, device=dev())
+      K.expert_mlp(to_dev(items, O.BF16), *wd, out=got, rows_per_expert=to_dev(rows),
+                   x_rows=to_dev(x_rows))
+      assert torch.equal(got, ragged), name + " gathered"
+  assert gathered >= 4
+
+
 @pytest.mark.parametrize("dtype", [O.F32, O.BF16])
 def test_expert_mlp_gathers_its_rows_from_the_items(K, dtype):
   """x_rows: the first product reads row r of expert e from item x_rows[e][r] of the (T, D)
